@@ -1,0 +1,98 @@
+"""ctypes binding of ``libd3gs_hip.so`` (declared in ``include/d3gs_hip.h``).
+
+The library is built in-tree by ``csrc/Makefile`` (``build()`` below drives it).
+There is no CPU fallback: loading fails loudly when the shared object is
+missing, and every entry point raises ``RuntimeError`` on a non-zero status.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_CSRC = os.path.join(_HERE, "csrc")
+LIB_PATH = os.path.join(_CSRC, "libd3gs_hip.so")
+
+ABI_VERSION = 1
+
+
+class Params(C.Structure):
+    """Mirror of ``d3gs_params``."""
+    _fields_ = [
+        ("n", C.c_int32), ("width", C.c_int32), ("height", C.c_int32),
+        ("tiles_x", C.c_int32), ("tiles_y", C.c_int32),
+        ("sh_degree", C.c_int32), ("sh_stride", C.c_int32), ("has_sh_base", C.c_int32),
+        ("filter_algo", C.c_int32), ("training", C.c_int32),
+        ("fx", C.c_float), ("fy", C.c_float), ("cx", C.c_float), ("cy", C.c_float),
+        ("tan_fovx", C.c_float), ("tan_fovy", C.c_float),
+        ("w2c", C.c_float * 9), ("cam_center", C.c_float * 3),
+        ("z_near", C.c_float), ("z_far", C.c_float), ("eps", C.c_float),
+        ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
+        ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
+        ("scale_global", C.c_float), ("bg", C.c_float * 3),
+    ]
+
+
+_VP = C.c_void_p
+_SIGNATURES = {
+    "d3gs_abi_version": (C.c_int, []),
+    "d3gs_last_error_string": (C.c_char_p, []),
+    "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
+    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 14 + [_VP]),
+    "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
+    "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
+    "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 7 + [C.c_int64, _VP]),
+    "d3gs_sort_workspace_bytes": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
+    "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
+                                  C.POINTER(C.c_int), _VP]),
+    "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP]),
+    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 8 + [_VP]),
+    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 14 + [_VP]),
+    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 13 + [C.c_int32] + [_VP] * 6 + [_VP]),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def build(force: bool = True) -> str:
+    """Compile every HIP source for gfx950 into ``csrc/libd3gs_hip.so``."""
+    cmd = ["make", "-C", _CSRC, "-j8"]
+    if force:
+        cmd.append("-B")
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {_CSRC}` (hipcc, gfx950). "
+                "There is no CPU fallback for the rasterizer.")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        if L.d3gs_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"libd3gs_hip.so ABI {L.d3gs_abi_version()} != expected {ABI_VERSION}")
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().d3gs_last_error_string()
+        raise RuntimeError(f"{what} failed ({rc}): {msg.decode() if msg else ''}")
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (None -> NULL)."""
+    if t is None:
+        return None
+    assert t.is_contiguous(), "tensor passed to the HIP library must be contiguous"
+    return C.c_void_p(t.data_ptr())

@@ -1,0 +1,370 @@
+// Tile binning: prefix scan of per-gaussian tile counts, (tile, depth) key
+// expansion, stable LSD radix sort of (u64 key, i32 value) pairs, and tile-range
+// extraction.  All stages are HBM-bandwidth-bound integer work.
+//
+// Reference: d3sim/algos/d3gs/render.py:694-695 (cumsum), 739-840 (keys),
+// 845-887 + d3sim/csrc/devsort.py:38-149 (CUB radix sort), 896-939 (ranges).
+#include "device_math.h"
+
+namespace d3gs {
+
+// ---------------------------------------------------------------------------
+// Inclusive scan, int32, three phases (chunk sums -> scan of sums -> chunk scan).
+// ---------------------------------------------------------------------------
+constexpr int kScanItems = 8;                      // per thread
+constexpr int kScanChunk = kBlock * kScanItems;    // 2048 per block
+
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int t = __shfl_up(v, off, 64);
+        if (lane >= off) v += t;
+    }
+    return v;
+}
+
+// block-wide exclusive scan of one int per thread; returns exclusive prefix and the block total
+__device__ __forceinline__ int block_excl_scan(int v, int& total, int* smem /* >= 4 ints */) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = wave_incl_scan(v, lane);
+    if (lane == 63) smem[wave] = incl;
+    __syncthreads();
+    int w0 = smem[0], w1 = smem[1], w2 = smem[2], w3 = smem[3];
+    __syncthreads();
+    int base = (wave > 0 ? w0 : 0) + (wave > 1 ? w1 : 0) + (wave > 2 ? w2 : 0);
+    total = w0 + w1 + w2 + w3;
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_chunk_sums_kernel(const int32_t* __restrict__ in, int n,
+                                                                  int32_t* __restrict__ sums) {
+    __shared__ int smem[4];
+    const int base = blockIdx.x * kScanChunk + threadIdx.x * kScanItems;
+    int s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) s += (base + k < n) ? in[base + k] : 0;
+    int total;
+    block_excl_scan(s, total, smem);
+    if (threadIdx.x == 0) sums[blockIdx.x] = total;
+}
+
+// single block: exclusive scan of `sums` in place (int32), grand total as int64
+__global__ __launch_bounds__(kBlock) void scan_sums_kernel(int32_t* __restrict__ sums, int nchunks,
+                                                            int64_t* __restrict__ total_out) {
+    __shared__ int smem[4];
+    long long carry = 0;
+    for (int start = 0; start < nchunks; start += kBlock) {
+        int idx = start + threadIdx.x;
+        int v = idx < nchunks ? sums[idx] : 0;
+        int total;
+        int ex = block_excl_scan(v, total, smem);
+        if (idx < nchunks) sums[idx] = (int)(carry + ex);
+        carry += total;
+    }
+    if (threadIdx.x == 0 && total_out) *total_out = carry;
+}
+
+__global__ __launch_bounds__(kBlock) void scan_apply_kernel(int32_t* __restrict__ data, int n,
+                                                             const int32_t* __restrict__ chunk_prefix) {
+    __shared__ int smem[4];
+    const int base = blockIdx.x * kScanChunk + threadIdx.x * kScanItems;
+    int v[kScanItems];
+    int s = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+        v[k] = (base + k < n) ? data[base + k] : 0;
+        s += v[k];
+    }
+    int total;
+    int ex = block_excl_scan(s, total, smem) + chunk_prefix[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+        ex += v[k];
+        if (base + k < n) data[base + k] = ex;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Key expansion: one thread per gaussian, emits its (tile << 32 | depth bits)
+// keys at the offset the scan assigned (render.py:745-840).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, const int32_t* __restrict__ radii,
+                                                            const float* __restrict__ uvs,
+                                                            const float* __restrict__ conic_opacity,
+                                                            const float* __restrict__ depths,
+                                                            const int32_t* __restrict__ offsets,
+                                                            uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
+                                                            long long m) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= P.n) return;
+    const int r = radii[i];
+    if (r <= 0) return;
+    long long off = i == 0 ? 0 : offsets[i - 1];
+    const long long end = offsets[i];
+    if (end > m) return;  // caller passed a smaller buffer than the scan total: never write past it
+    const uint32_t dbits = __float_as_uint(depths[i]);
+    const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
+    const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
+    TileWalkIn g{uv.x, uv.y, (float)r, co.x, co.y, co.z, co.w};
+    const int tiles_x = P.tiles_x;
+    tile_walk(P, g, [&](int x, int y) {
+        if (off < end) {
+            uint64_t key = (uint64_t)(uint32_t)(y * tiles_x + x);
+            keys[off] = (key << 32) | dbits;
+            vals[off] = i;
+        }
+        ++off;
+    });
+}
+
+// ---------------------------------------------------------------------------
+// Radix sort, 8-bit digits, per pass: block histograms -> scan -> stable scatter.
+// A block owns a contiguous run of kSortTile keys; wave w of the block owns the
+// w-th quarter, processed 64 keys at a time, so (wave, round, lane) order equals
+// input order and ranks computed from it are stable.
+// ---------------------------------------------------------------------------
+constexpr int kSortItems = 16;
+constexpr int kSortTile = kBlock * kSortItems;  // 4096 keys per block
+constexpr int kRadix = 256;
+
+__global__ __launch_bounds__(kBlock) void sort_hist_kernel(const uint64_t* __restrict__ keys, long long m, int shift,
+                                                            uint32_t mask, int nblocks,
+                                                            int32_t* __restrict__ hist /* [kRadix][nblocks] */) {
+    __shared__ int h[kRadix];
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const long long base = (long long)blockIdx.x * kSortTile;
+#pragma unroll 4
+    for (int k = 0; k < kSortItems; ++k) {
+        long long idx = base + k * kBlock + threadIdx.x;
+        if (idx < m) {
+            uint32_t d = (uint32_t)(keys[idx] >> shift) & mask;
+            atomicAdd(&h[d], 1);
+        }
+    }
+    __syncthreads();
+    hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = h[threadIdx.x];
+}
+
+__global__ __launch_bounds__(kBlock) void sort_scatter_kernel(const uint64_t* __restrict__ keys_in,
+                                                               const int32_t* __restrict__ vals_in,
+                                                               uint64_t* __restrict__ keys_out,
+                                                               int32_t* __restrict__ vals_out, long long m, int shift,
+                                                               uint32_t mask, int nblocks,
+                                                               const int32_t* __restrict__ offsets /* scanned hist */) {
+    __shared__ int wave_cnt[4][kRadix];   // running / final per-wave digit counts
+    __shared__ int digit_base[kRadix];    // global output offset of this block's first key of each digit
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int k = threadIdx.x; k < 4 * kRadix; k += kBlock) (&wave_cnt[0][0])[k] = 0;
+    __syncthreads();
+
+    const long long base = (long long)blockIdx.x * kSortTile + wave * (kSortTile / 4);
+    uint64_t key[kSortItems];
+    int rank[kSortItems];
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int k = 0; k < kSortItems; ++k) {
+        const long long idx = base + k * 64 + lane;
+        const bool in = idx < m;
+        key[k] = in ? keys_in[idx] : ~0ull;
+        const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
+        // lanes holding the same digit
+        uint64_t peers = __ballot(in);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint64_t bal = __ballot((d >> b) & 1u);
+            peers &= ((d >> b) & 1u) ? bal : ~bal;
+        }
+        int before = 0;
+        if (in) before = wave_cnt[wave][d];
+        __builtin_amdgcn_wave_barrier();
+        if (in && (peers & lt_mask) == 0) wave_cnt[wave][d] = before + __popcll(peers);
+        __builtin_amdgcn_wave_barrier();
+        rank[k] = before + __popcll(peers & lt_mask);
+    }
+    __syncthreads();
+    {
+        // thread t owns digit t: exclusive prefix over waves + the block's global base
+        const int d = threadIdx.x;
+        int c0 = wave_cnt[0][d], c1 = wave_cnt[1][d], c2 = wave_cnt[2][d], c3 = wave_cnt[3][d];
+        // `offsets` is the inclusive scan of the (digit-major) block histograms
+        digit_base[d] = offsets[(size_t)d * nblocks + blockIdx.x] - (c0 + c1 + c2 + c3);
+        wave_cnt[0][d] = 0;
+        wave_cnt[1][d] = c0;
+        wave_cnt[2][d] = c0 + c1;
+        wave_cnt[3][d] = c0 + c1 + c2;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kSortItems; ++k) {
+        const long long idx = base + k * 64 + lane;
+        if (idx < m) {
+            const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
+            const long long pos = (long long)digit_base[d] + wave_cnt[wave][d] + rank[k];
+            keys_out[pos] = key[k];
+            vals_out[pos] = vals_in[idx];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Tile ranges (render.py:897-939)
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const uint64_t* __restrict__ keys, long long m,
+                                                              int32_t* __restrict__ ranges, int num_tiles) {
+    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= m) return;
+    const uint32_t t = (uint32_t)(keys[i] >> 32);
+    if (t >= (uint32_t)num_tiles) return;  // corrupt key: never write outside the table
+    if (i == 0) {
+        ranges[2 * t] = 0;
+    } else {
+        const uint32_t tp = (uint32_t)(keys[i - 1] >> 32);
+        if (t != tp) {
+            if (tp < (uint32_t)num_tiles) ranges[2 * tp + 1] = (int32_t)i;
+            ranges[2 * t] = (int32_t)i;
+        }
+    }
+    if (i == m - 1) ranges[2 * t + 1] = (int32_t)m;
+}
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+static inline int scan_chunks(long long n) { return (int)((n + kScanChunk - 1) / kScanChunk); }
+
+// workspace for scanning `n` ints: chunk sums
+static size_t scan_ws_bytes(long long n) { return align_up((size_t)std::max(1, scan_chunks(n)) * sizeof(int32_t), 256); }
+
+static int launch_scan(int32_t* data, long long n, void* ws, int64_t* total_dev, hipStream_t s) {
+    const int nchunks = scan_chunks(n);
+    int32_t* sums = (int32_t*)ws;
+    hipLaunchKernelGGL(scan_chunk_sums_kernel, dim3(nchunks), dim3(kBlock), 0, s, data, (int)n, sums);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, sums, nchunks, total_dev);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nchunks), dim3(kBlock), 0, s, data, (int)n, sums);
+    return hipGetLastError() == hipSuccess ? D3GS_OK : D3GS_ERR_LAUNCH;
+}
+
+}  // namespace d3gs
+
+using namespace d3gs;
+
+extern "C" int d3gs_scan_workspace_bytes(int32_t n, size_t* bytes_out_host) {
+    if (n < 0 || !bytes_out_host) { set_error("d3gs_scan_workspace_bytes: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+    *bytes_out_host = scan_ws_bytes(n);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t workspace_bytes,
+                               int64_t* total_dev, d3gs_stream_t stream) {
+    if (n < 0 || !total_dev) { set_error("d3gs_scan_tiles: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (n == 0) {
+        // a one-thread kernel rather than a memset node: safe under stream capture
+        hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, (int32_t*)nullptr, 0,
+                           total_dev);
+        return D3GS_OK;
+    }
+    if (!tiles_touched || !workspace) { set_error("d3gs_scan_tiles: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (workspace_bytes < scan_ws_bytes(n)) {
+        set_error("d3gs_scan_tiles: workspace %zu < required %zu", workspace_bytes, scan_ws_bytes(n));
+        return D3GS_ERR_WORKSPACE_TOO_SMALL;
+    }
+    int rc = launch_scan(tiles_touched, n, workspace, total_dev, (hipStream_t)stream);
+    if (rc) set_error("d3gs_scan_tiles: launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return rc;
+}
+
+extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                              const float* depths, const int32_t* offsets, uint64_t* keys, int32_t* gaussian_idx,
+                              int64_t m, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_make_keys");
+    if (rc) return rc;
+    if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (p->n == 0 || m == 0) return D3GS_OK;
+    if (!radii || !uvs || !conic_opacity || !depths || !offsets || !keys || !gaussian_idx) {
+        set_error("d3gs_make_keys: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(make_keys_kernel, dim3((p->n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, *p,
+                       radii, uvs, conic_opacity, depths, offsets, keys, gaussian_idx, (long long)m);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+static int sort_blocks(int64_t m) { return (int)((m + kSortTile - 1) / kSortTile); }
+
+extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* bytes_out_host) {
+    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !bytes_out_host) {
+        set_error("d3gs_sort_workspace_bytes: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const size_t hist_elems = (size_t)kRadix * std::max(1, sort_blocks(m));
+    *bytes_out_host = align_up(hist_elems * sizeof(int32_t), 256) + scan_ws_bytes((long long)hist_elems);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                               size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                               d3gs_stream_t stream) {
+    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !result_in_b_host) {
+        set_error("d3gs_sort_pairs: bad argument (m=%lld bits=[%d,%d))", (long long)m, begin_bit, end_bit);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (m >= (1ll << 31)) { set_error("d3gs_sort_pairs: m >= 2^31 is not supported"); return D3GS_ERR_UNSUPPORTED; }
+    *result_in_b_host = 0;
+    if (m == 0 || begin_bit == end_bit) return D3GS_OK;
+    if (!keys_a || !keys_b || !vals_a || !vals_b || !workspace) {
+        set_error("d3gs_sort_pairs: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    size_t need = 0;
+    d3gs_sort_workspace_bytes(m, begin_bit, end_bit, &need);
+    if (workspace_bytes < need) {
+        set_error("d3gs_sort_pairs: workspace %zu < required %zu", workspace_bytes, need);
+        return D3GS_ERR_WORKSPACE_TOO_SMALL;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int nblocks = sort_blocks(m);
+    const size_t hist_elems = (size_t)kRadix * nblocks;
+    int32_t* hist = (int32_t*)workspace;
+    void* scan_ws = (char*)workspace + align_up(hist_elems * sizeof(int32_t), 256);
+    uint64_t* kin = keys_a;
+    uint64_t* kout = keys_b;
+    int32_t* vin = vals_a;
+    int32_t* vout = vals_b;
+    int in_b = 0;
+    for (int bit = begin_bit; bit < end_bit; bit += 8) {
+        const int nb = std::min(8, end_bit - bit);
+        const uint32_t mask = (1u << nb) - 1u;
+        hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(kBlock), 0, s, kin, (long long)m, bit, mask, nblocks, hist);
+        // inclusive scan of the digit-major histogram table, in place; the scatter kernel
+        // subtracts its own count to get the exclusive offset
+        {
+            const int nchunks = scan_chunks((long long)hist_elems);
+            int32_t* sums = (int32_t*)scan_ws;
+            hipLaunchKernelGGL(scan_chunk_sums_kernel, dim3(nchunks), dim3(kBlock), 0, s, hist, (int)hist_elems, sums);
+            hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, sums, nchunks, (int64_t*)nullptr);
+            hipLaunchKernelGGL(scan_apply_kernel, dim3(nchunks), dim3(kBlock), 0, s, hist, (int)hist_elems, sums);
+        }
+        hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(kBlock), 0, s, kin, vin, kout, vout, (long long)m, bit,
+                           mask, nblocks, hist);
+        std::swap(kin, kout);
+        std::swap(vin, vout);
+        in_b ^= 1;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_sort_pairs: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    *result_in_b_host = in_b;
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
+                                d3gs_stream_t stream) {
+    if (m < 0 || num_tiles < 0) { set_error("d3gs_tile_ranges: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (m == 0) return D3GS_OK;
+    if (!keys_sorted || !workload_ranges) { set_error("d3gs_tile_ranges: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
+    hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       (hipStream_t)stream, keys_sorted, (long long)m, workload_ranges, (int)num_tiles);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_tile_ranges: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}

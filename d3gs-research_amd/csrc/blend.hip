@@ -1,0 +1,354 @@
+// Per-tile alpha blending, forward and backward.
+//
+// One 256-thread workgroup (4 wave64) per 16x16 tile; wave w owns the 8x8 pixel
+// patch (w & 1, w >> 1) of the tile so that a wavefront covers a compact square
+// and whole-wave culling of a gaussian is likely.  The tile's depth-sorted
+// gaussians are staged 256 at a time into LDS by the whole workgroup and read
+// back with wave-uniform (broadcast) addresses.
+//
+// Culling that keeps results exact: a gaussian contributes to a pixel only if
+// alpha = min(0.99, o * exp(power)) >= alpha_eps.  Each staged gaussian carries
+// thr = ln(alpha_eps / o) - 1e-3; power < thr implies alpha < alpha_eps with a
+// margin four orders of magnitude above any rounding error, so a wavefront whose
+// 64 pixels all have power < thr skips the gaussian without evaluating exp.
+// Every pixel that passes the coarse test goes through the exact sequence.
+//
+// Reference: d3sim/algos/d3gs/render.py:1466-1570 (prologue), 1677-1923 (loop),
+// 1924-2019 (gradients), 2020-2210 (reduction + atomics), 2222-2294 (epilogue).
+#include "device_math.h"
+
+namespace d3gs {
+
+struct __attribute__((aligned(16))) StagedGaussian {
+    float x, y, thr, pad;   // pixel-space centre, cull threshold
+    float a, b, c, o;       // conic (a, b, c) and opacity
+};
+
+// Tile index for a workgroup.  Consecutive workgroup ids are dealt round-robin
+// to the 8 XCDs, each with its own L2; give every XCD a contiguous band of tiles
+// so neighbouring tiles (which share gaussians) hit the same L2.
+__device__ __forceinline__ int tile_for_block(int bid, int ntiles) {
+    const int per = (ntiles + 7) >> 3;
+    return (bid & 7) * per + (bid >> 3);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    // butterfly inside each row of 16 lanes with DPP, then add the 4 row sums
+    int x = __float_as_int(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    x = __float_as_int(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    x = __float_as_int(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, false));  // row_half_mirror
+    x = __float_as_int(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, false));  // row_mirror
+    x = __float_as_int(v);
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(x, 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(x, 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(x, 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(x, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ int wave_max_i32(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+__device__ __forceinline__ void stage_gaussian(const d3gs_params& P, int g, const float* __restrict__ uvs,
+                                               const float* __restrict__ conic_opacity, StagedGaussian* dst) {
+    const float2 xy = *reinterpret_cast<const float2*>(uvs + 2 * g);
+    const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * g);
+    StagedGaussian s;
+    s.x = xy.x;
+    s.y = xy.y;
+    s.thr = __logf(P.alpha_eps / co.w) - 1.0e-3f;
+    s.pad = 0.0f;
+    s.a = co.x;
+    s.b = co.y;
+    s.c = co.z;
+    s.o = co.w;
+    *dst = s;
+}
+
+__global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, const int32_t* __restrict__ ranges,
+                                                            const int32_t* __restrict__ idx_sorted,
+                                                            const float* __restrict__ uvs,
+                                                            const float* __restrict__ conic_opacity,
+                                                            const float* __restrict__ rgb_g, float* __restrict__ color,
+                                                            float* __restrict__ final_T,
+                                                            int32_t* __restrict__ n_contrib) {
+    __shared__ StagedGaussian s_g[kBlock];
+    __shared__ float4 s_rgb[kBlock];
+
+    const int ntiles = P.tiles_x * P.tiles_y;
+    const int tile = tile_for_block(blockIdx.x, ntiles);
+    if (tile >= ntiles) return;
+    const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
+    const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
+    const bool inside = px < P.width && py < P.height;
+    const float pxf = (float)px, pyf = (float)py;
+
+    const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
+    const int len = r1 - r0;
+    const int rounds = (len + kBlock - 1) / kBlock;
+
+    bool done = !inside;
+    float T = 1.0f;
+    float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f;
+    int contributor = 0;
+
+    for (int round = 0; round < rounds; ++round) {
+        if (__syncthreads_count(done) == kBlock) break;
+        const int src = r0 + round * kBlock + tid;
+        if (src < r1) {
+            const int g = idx_sorted[src];
+            stage_gaussian(P, g, uvs, conic_opacity, &s_g[tid]);
+            s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+        }
+        __syncthreads();
+        if (__all(done)) continue;
+        const int cnt = min(kBlock, len - round * kBlock);
+        for (int j = 0; j < cnt; ++j) {
+            const StagedGaussian sg = s_g[j];
+            const float dx = sg.x - pxf, dy = sg.y - pyf;
+            const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
+            const bool cand = !done && power >= sg.thr;
+            if (!__any(cand)) continue;
+            if (cand) {
+                const float G = det_expf(power);
+                const float alpha = fminf(0.99f, sg.o * G);
+                if (alpha >= P.alpha_eps) {
+                    const float nextT = T * (1.0f - alpha);
+                    const bool should_done = nextT < P.transmittance_eps;
+                    if (power > 0.0f || should_done) {
+                        done = should_done;
+                    } else {
+                        const float w = alpha * T;
+                        T = nextT;
+                        contributor = round * kBlock + j;
+                        const float4 c = s_rgb[j];
+                        acc0 = acc0 + w * c.x;
+                        acc1 = acc1 + w * c.y;
+                        acc2 = acc2 + w * c.z;
+                    }
+                }
+            }
+        }
+    }
+
+    if (inside) {
+        const size_t pid = (size_t)py * P.width + px;
+        final_T[pid] = T;
+        n_contrib[pid] = contributor;
+        if (P.training) {
+            color[3 * pid + 0] = acc0;
+            color[3 * pid + 1] = acc1;
+            color[3 * pid + 2] = acc2;
+        } else {
+            color[3 * pid + 0] = fminf(fmaxf(acc0 + T * P.bg[0], 0.0f), 1.0f);
+            color[3 * pid + 1] = fminf(fmaxf(acc1 + T * P.bg[1], 0.0f), 1.0f);
+            color[3 * pid + 2] = fminf(fmaxf(acc2 + T * P.bg[2], 0.0f), 1.0f);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Backward: front-to-back recompute; per gaussian the nine partial derivatives
+// are summed over the wavefront, then over the tile's four wavefronts in LDS,
+// and only then added to global memory: one atomic per value per (tile, gaussian).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
+    const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
+    const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
+    const float* __restrict__ final_T, const int32_t* __restrict__ n_contrib, const float* __restrict__ color,
+    const float* __restrict__ drgb, const float* __restrict__ dT, float* __restrict__ duv, float* __restrict__ dconic,
+    float* __restrict__ dopacity, float* __restrict__ dcolor) {
+    __shared__ StagedGaussian s_g[kBlock];
+    __shared__ float4 s_rgb[kBlock];
+    __shared__ int s_id[kBlock];
+    __shared__ float s_grad[9][kBlock];
+    __shared__ int s_wmax[4];
+
+    const int ntiles = P.tiles_x * P.tiles_y;
+    const int tile = tile_for_block(blockIdx.x, ntiles);
+    if (tile >= ntiles) return;
+    const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
+    const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
+    const bool inside = px < P.width && py < P.height;
+    const float pxf = (float)px, pyf = (float)py;
+    const size_t pid = (size_t)py * P.width + px;
+
+    const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
+    const int len = r1 - r0;
+    if (len <= 0) return;
+
+    int contributor = 0;
+    float render_T = 0.0f, dT_val = 0.0f;
+    float rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f, dr0 = 0.0f, dr1 = 0.0f, dr2 = 0.0f;
+    if (inside) {
+        contributor = min(n_contrib[pid] + 1, len);
+        render_T = final_T[pid];
+        dT_val = dT[pid];
+        rr0 = color[3 * pid + 0];
+        rr1 = color[3 * pid + 1];
+        rr2 = color[3 * pid + 2];
+        dr0 = drgb[3 * pid + 0];
+        dr1 = drgb[3 * pid + 1];
+        dr2 = drgb[3 * pid + 2];
+    }
+    const float dT_term = (-dT_val) * render_T;
+    const int wave_todo = wave_max_i32(contributor);
+    if (lane == 0) s_wmax[wave] = wave_todo;
+    __syncthreads();
+    const int block_todo = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
+    const int rounds = (block_todo + kBlock - 1) / kBlock;
+
+    float T = 1.0f;
+    for (int round = 0; round < rounds; ++round) {
+        __syncthreads();  // previous round's flush has read s_grad / s_id
+        const int src = r0 + round * kBlock + tid;
+        if (src < r1) {
+            const int g = idx_sorted[src];
+            s_id[tid] = g;
+            stage_gaussian(P, g, uvs, conic_opacity, &s_g[tid]);
+            s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+        }
+#pragma unroll
+        for (int k = 0; k < 9; ++k) s_grad[k][tid] = 0.0f;
+        __syncthreads();
+        const int cnt = min(kBlock, wave_todo - round * kBlock);
+        for (int j = 0; j < cnt; ++j) {
+            const StagedGaussian sg = s_g[j];
+            const float dx = sg.x - pxf, dy = sg.y - pyf;
+            const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
+            const bool cand = (round * kBlock + j < contributor) && power >= sg.thr && power <= 0.0f;
+            if (!__any(cand)) continue;
+            float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, g3 = 0.0f, g4 = 0.0f, g5 = 0.0f, g6 = 0.0f, g7 = 0.0f, g8 = 0.0f;
+            bool valid = false;
+            if (cand) {
+                const float G = det_expf(power);
+                const float alpha = fminf(0.99f, sg.o * G);
+                if (alpha >= P.alpha_eps) {
+                    valid = true;
+                    const float nextT = T * (1.0f - alpha);
+                    const float w = alpha * T;
+                    T = nextT;
+                    const float4 c = s_rgb[j];
+                    rr0 = rr0 - w * c.x;
+                    rr1 = rr1 - w * c.y;
+                    rr2 = rr2 - w * c.z;
+                    float dl = ((dr0 * (T * c.x - rr0) + dr1 * (T * c.y - rr1)) + dr2 * (T * c.z - rr2));
+                    dl = dl + dT_term;
+                    const float dL_dalpha = dl / (1.0f - alpha);
+                    const float dL_dG = sg.o * dL_dalpha;
+                    const float gdx = G * dx, gdy = G * dy;
+                    const float dG_du = (-gdx) * sg.a - gdy * sg.b;
+                    const float dG_dv = (-gdy) * sg.c - gdx * sg.b;
+                    g0 = dL_dG * dG_du;
+                    g1 = dL_dG * dG_dv;
+                    g2 = ((-0.5f) * gdx) * dx * dL_dG;
+                    g3 = ((-gdx) * dy) * dL_dG;
+                    g4 = ((-0.5f) * gdy) * dy * dL_dG;
+                    g5 = dL_dalpha * G;
+                    g6 = w * dr0;
+                    g7 = w * dr1;
+                    g8 = w * dr2;
+                }
+            }
+            if (!__any(valid)) continue;
+            g0 = wave_sum(g0);
+            g1 = wave_sum(g1);
+            g2 = wave_sum(g2);
+            g3 = wave_sum(g3);
+            g4 = wave_sum(g4);
+            g5 = wave_sum(g5);
+            g6 = wave_sum(g6);
+            g7 = wave_sum(g7);
+            g8 = wave_sum(g8);
+            if (lane == 0) {
+                atomicAdd(&s_grad[0][j], g0);
+                atomicAdd(&s_grad[1][j], g1);
+                atomicAdd(&s_grad[2][j], g2);
+                atomicAdd(&s_grad[3][j], g3);
+                atomicAdd(&s_grad[4][j], g4);
+                atomicAdd(&s_grad[5][j], g5);
+                atomicAdd(&s_grad[6][j], g6);
+                atomicAdd(&s_grad[7][j], g7);
+                atomicAdd(&s_grad[8][j], g8);
+            }
+        }
+        __syncthreads();
+        if (round * kBlock + tid < len) {
+            float v[9];
+            bool any = false;
+#pragma unroll
+            for (int k = 0; k < 9; ++k) {
+                v[k] = s_grad[k][tid];
+                any = any || v[k] != 0.0f;
+            }
+            if (any) {
+                const int g = s_id[tid];
+                unsafeAtomicAdd(duv + 2 * g + 0, v[0]);
+                unsafeAtomicAdd(duv + 2 * g + 1, v[1]);
+                unsafeAtomicAdd(dconic + 3 * g + 0, v[2]);
+                unsafeAtomicAdd(dconic + 3 * g + 1, v[3]);
+                unsafeAtomicAdd(dconic + 3 * g + 2, v[4]);
+                unsafeAtomicAdd(dopacity + g, v[5]);
+                unsafeAtomicAdd(dcolor + 3 * g + 0, v[6]);
+                unsafeAtomicAdd(dcolor + 3 * g + 1, v[7]);
+                unsafeAtomicAdd(dcolor + 3 * g + 2, v[8]);
+            }
+        }
+    }
+}
+
+}  // namespace d3gs
+
+using namespace d3gs;
+
+static int blend_grid(const d3gs_params* p) {
+    const int ntiles = p->tiles_x * p->tiles_y;
+    return ((ntiles + 7) / 8) * 8;
+}
+
+extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                              const float* uvs, const float* conic_opacity, const float* rgb_gaussian, float* color,
+                              float* final_T, int32_t* n_contrib, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_blend_fwd");
+    if (rc) return rc;
+    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib) {
+        set_error("d3gs_blend_fwd: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(blend_fwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
+                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, color, final_T, n_contrib);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_blend_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                              const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                              const float* final_T, const int32_t* n_contrib, const float* color, const float* drgb,
+                              const float* dT, float* duv, float* dconic, float* dopacity, float* dcolor,
+                              d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_blend_bwd");
+    if (rc) return rc;
+    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb ||
+        !dT || !duv || !dconic || !dopacity || !dcolor) {
+        set_error("d3gs_blend_bwd: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(blend_bwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
+                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, final_T, n_contrib, color, drgb, dT,
+                       duv, dconic, dopacity, dcolor);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_blend_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}

@@ -1,0 +1,279 @@
+// Device-side math shared by the gfx950 kernels.
+//
+// Everything here is float32 written as explicit single operations; the
+// translation units are compiled with -ffp-contract=off so that a fused
+// multiply-add appears only where __builtin_fmaf is spelled out.  That fixed
+// operation order is what makes the integer outputs of the pipeline (radii,
+// tile counts, sort keys) reproducible against a CPU evaluation of the same
+// formulas.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/d3gs_hip.h"
+
+namespace d3gs {
+
+constexpr int kTile = 16;          // tile edge in pixels (config tile_size, config_def.py:79)
+constexpr int kBlock = 256;        // threads per tile / per 1-D block (csrc/inliner.py:38)
+
+// exp with a fixed operation sequence (Cephes single-precision scheme): the
+// same sequence on any IEEE-754 machine gives the same bits.  The reference
+// calls CUDA's approximate __expf here (render.py:1768); its rounding is
+// unspecified, this one is < 1 ulp from the true value.
+__device__ __forceinline__ float det_expf(float x) {
+    if (!(x == x)) return x;
+    if (x < -86.0f) return 0.0f;
+    if (x > 88.0f) return __builtin_inff();
+    float kf = __builtin_rintf(x * 1.44269504088896341f);
+    float r = __builtin_fmaf(kf, -0.693359375f, x);
+    r = __builtin_fmaf(kf, 2.12194440e-4f, r);
+    float z = r * r;
+    float p = 1.9875691500e-4f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+    float e = __builtin_fmaf(p, z, r) + 1.0f;
+    return __builtin_ldexpf(e, (int)kf);
+}
+
+// Same, for arguments already known to lie in [-86, 88] and not NaN.
+__device__ __forceinline__ float det_expf_inrange(float x) {
+    float kf = __builtin_rintf(x * 1.44269504088896341f);
+    float r = __builtin_fmaf(kf, -0.693359375f, x);
+    r = __builtin_fmaf(kf, 2.12194440e-4f, r);
+    float z = r * r;
+    float p = 1.9875691500e-4f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+    float e = __builtin_fmaf(p, z, r) + 1.0f;
+    return __builtin_ldexpf(e, (int)kf);
+}
+
+__device__ __forceinline__ float det_logf(float x) {
+    if (!(x > 0.0f)) return -__builtin_inff();
+    if (x < 1.17549435e-38f) x = 1.17549435e-38f;
+    uint32_t ix = __float_as_uint(x);
+    int e = (int)(ix >> 23) - 126;
+    float m = __uint_as_float((ix & 0x007fffffu) | 0x3f000000u);
+    if (m < 0.707106781186547524f) {
+        e -= 1;
+        m = (m + m) - 1.0f;
+    } else {
+        m = m - 1.0f;
+    }
+    float z = m * m;
+    float y = 7.0376836292e-2f;
+    y = __builtin_fmaf(y, m, -1.1514610310e-1f);
+    y = __builtin_fmaf(y, m, 1.1676998740e-1f);
+    y = __builtin_fmaf(y, m, -1.2420140846e-1f);
+    y = __builtin_fmaf(y, m, 1.4249322787e-1f);
+    y = __builtin_fmaf(y, m, -1.6668057665e-1f);
+    y = __builtin_fmaf(y, m, 2.0000714765e-1f);
+    y = __builtin_fmaf(y, m, -2.4999993993e-1f);
+    y = __builtin_fmaf(y, m, 3.3333331174e-1f);
+    y = (y * m) * z;
+    float fe = (float)e;
+    y = y + (-2.12194440e-4f * fe);
+    y = y + (-0.5f * z);
+    float r = m + y;
+    r = r + (0.693359375f * fe);
+    return r;
+}
+
+__device__ __forceinline__ float det_sigmoid(float x) { return 1.0f / (1.0f + det_expf(-x)); }
+
+__device__ __forceinline__ float dot3(const float* a, const float* b) { return (a[0] * b[0] + a[1] * b[1]) + a[2] * b[2]; }
+
+// Tile coordinate from a pixel-space float: truncate toward zero like the
+// reference's cast (render.py:472-473), clamped to [0, hi].  The float clamp
+// first keeps the conversion defined for huge or non-finite inputs.
+__device__ __forceinline__ int tile_coord(float v, int hi) {
+    v = fminf(fmaxf(v, -1.0f), 1.0e6f);
+    int t = (int)v;
+    return t < 0 ? 0 : (t > hi ? hi : t);
+}
+
+// Unit quaternion in (x,y,z,w) memory order -> rotation matrix, row major.
+__device__ __forceinline__ void quat_to_rot(const float q[4], float R[9]) {
+    float x = q[0], y = q[1], z = q[2], w = q[3];
+    float xx = x * x, yy = y * y, zz = z * z;
+    float xy = x * y, xz = x * z, yz = y * z;
+    float wx = w * x, wy = w * y, wz = w * z;
+    R[0] = 1.0f - 2.0f * (yy + zz);
+    R[1] = 2.0f * (xy - wz);
+    R[2] = 2.0f * (xz + wy);
+    R[3] = 2.0f * (xy + wz);
+    R[4] = 1.0f - 2.0f * (xx + zz);
+    R[5] = 2.0f * (yz - wx);
+    R[6] = 2.0f * (xz - wy);
+    R[7] = 2.0f * (yz + wx);
+    R[8] = 1.0f - 2.0f * (xx + yy);
+}
+
+// Sigma3 = (R diag s)(R diag s)^T as [00,01,02,11,12,22]   (gs3d.py:368-385)
+__device__ __forceinline__ void cov3d_from_scale_rot(const float s[3], const float R[9], float c6[6]) {
+    float M[9];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) M[i * 3 + j] = R[i * 3 + j] * s[j];
+    c6[0] = dot3(M + 0, M + 0);
+    c6[1] = dot3(M + 0, M + 3);
+    c6[2] = dot3(M + 0, M + 6);
+    c6[3] = dot3(M + 3, M + 3);
+    c6[4] = dot3(M + 3, M + 6);
+    c6[5] = dot3(M + 6, M + 6);
+}
+
+__device__ __forceinline__ void sym3_mv(const float c6[6], const float v[3], float out[3]) {
+    out[0] = (c6[0] * v[0] + c6[1] * v[1]) + c6[2] * v[2];
+    out[1] = (c6[1] * v[0] + c6[3] * v[1]) + c6[4] * v[2];
+    out[2] = (c6[2] * v[0] + c6[4] * v[1]) + c6[5] * v[2];
+}
+
+// Rows of T = J W for the EWA projection (gs3d.py:436-456); tx,ty are the
+// frustum-clamped camera-space x,y.
+__device__ __forceinline__ void ewa_rows(const d3gs_params& P, const float pc[3], float t0[3], float t1[3], float& tx,
+                                         float& ty) {
+    float limx = fabsf((P.tan_fovx * P.clamp_factor) * pc[2]);
+    float limy = fabsf((P.tan_fovy * P.clamp_factor) * pc[2]);
+    tx = fminf(fmaxf(pc[0], -limx), limx);
+    ty = fminf(fmaxf(pc[1], -limy), limy);
+    float zz = pc[2] * pc[2];
+    float j00 = P.fx / pc[2];
+    float j11 = P.fy / pc[2];
+    float j02 = -(tx * P.fx) / zz;
+    float j12 = -(ty * P.fy) / zz;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        t0[k] = j00 * P.w2c[0 + k] + j02 * P.w2c[6 + k];
+        t1[k] = j11 * P.w2c[3 + k] + j12 * P.w2c[6 + k];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Tiles touched by one gaussian (render.py:1017-1327).  Visits kept tiles in
+// row-major order (y outer, x inner) and calls f(x, y); returns the count.
+// The preprocess kernel counts with it and the key-expansion kernel emits with
+// it, from the same stored (uv, radius, conic, opacity), so both make identical
+// decisions.
+// ---------------------------------------------------------------------------
+struct TileWalkIn {
+    float u, v;
+    float radius;
+    float conic0, conic1, conic2;
+    float opacity;
+};
+
+__device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1, float by1, float w, float h, float s,
+                                                 float c, float cu, float cv) {
+    // 4-axis separating-axis test (gs3d.py:1254-1322).  With NaN sin/cos every
+    // "<=" below is false, so the tile is kept.
+    float l1x = (bx1 - bx0) / 2.0f, l1y = (by1 - by0) / 2.0f;
+    float l2x = w / 2.0f, l2y = h / 2.0f;
+    float lx = (bx1 + bx0) / 2.0f - cu, ly = (by1 + by0) / 2.0f - cv;
+    float r1, r2, r3, r4;
+    r1 = l1x * 1.0f; r2 = l1y * 0.0f; r3 = l2x * fabsf(c); r4 = l2y * fabsf(-s);
+    if (((r1 + r2) + r3) + r4 <= fabsf(lx)) return false;
+    r1 = l1x * 0.0f; r2 = l1y * 1.0f; r3 = l2x * fabsf(s); r4 = l2y * fabsf(c);
+    if (((r1 + r2) + r3) + r4 <= fabsf(ly)) return false;
+    r1 = l1x * fabsf(c); r2 = l1y * fabsf(s); r3 = l2x * fabsf(c * c + s * s); r4 = l2y * fabsf((-s) * c + c * s);
+    if (((r1 + r2) + r3) + r4 <= fabsf(lx * c + ly * s)) return false;
+    r1 = l1x * fabsf(-s); r2 = l1y * fabsf(c); r3 = l2x * fabsf(c * (-s) + s * c); r4 = l2y * fabsf((-s) * (-s) + c * c);
+    if (((r1 + r2) + r3) + r4 <= fabsf(lx * (-s) + ly * c)) return false;
+    return true;
+}
+
+template <class F>
+__device__ __forceinline__ int tile_walk(const d3gs_params& P, const TileWalkIn& g, F&& f) {
+    const int TX = P.tiles_x, TY = P.tiles_y;
+    int rminx = tile_coord((g.u - g.radius) / 16.0f, TX);
+    int rminy = tile_coord((g.v - g.radius) / 16.0f, TY);
+    int rmaxx = tile_coord((((g.u + g.radius) + 16.0f) - 1.0f) / 16.0f, TX);
+    int rmaxy = tile_coord((((g.v + g.radius) + 16.0f) - 1.0f) / 16.0f, TY);
+    int count = 0;
+    if (P.filter_algo == D3GS_FILTER_NONE) {
+        for (int y = rminy; y < rmaxy; ++y)
+            for (int x = rminx; x < rmaxx; ++x) { f(x, y); ++count; }
+        return count;
+    }
+    // half extents of the exact alpha >= alpha_eps ellipse (gs3d.py:710-742)
+    float bound = 2.0f * det_logf(P.alpha_eps / g.opacity);
+    float D = g.conic0 * g.conic2 - g.conic1 * g.conic1;
+    float vx = ((-bound) * g.conic2) * D;
+    float vy = ((-bound) * g.conic0) * D;
+    float bx = sqrtf(fmaxf(0.0f, vx)) / D;
+    float by = sqrtf(fmaxf(0.0f, vy)) / D;
+    bx = vx > 0.0f ? bx : 0.0f;
+    by = vy > 0.0f ? by : 0.0f;
+    bx = fabsf(bx);
+    by = fabsf(by);
+    int bminx = tile_coord((g.u - bx) / 16.0f, TX);
+    int bminy = tile_coord((g.v - by) / 16.0f, TY);
+    int bmaxx = tile_coord(ceilf((g.u + bx) / 16.0f), TX);
+    int bmaxy = tile_coord(ceilf((g.v + by) / 16.0f), TY);
+    float uo = g.u - (float)bminx * 16.0f;
+    float vo = g.v - (float)bminy * 16.0f;
+    float ow = 0.0f, oh = 0.0f, os = 0.0f, oc = 0.0f;
+    const bool use_obb = P.filter_algo == D3GS_FILTER_OBB || P.filter_algo == D3GS_FILTER_OBB_DFVT;
+    if (use_obb) {
+        // oriented bounding box of the ellipse x^T Q x = 1, Q = -conic / bound (gs3d.py:761-791, 981-987)
+        float eA = (-g.conic0) / bound, eC = (-g.conic2) / bound, eB = (-g.conic1) / bound;
+        float det = eA * eC - eB * eB;
+        float mid = 0.5f * (eA + eC);
+        float sq = sqrtf(fmaxf(0.0f, mid * mid - det));
+        float e1 = mid + sq, e2 = mid - sq;
+        float s1 = e1 > 0.0f ? 1.0f : -1.0f, s2 = e2 > 0.0f ? 1.0f : -1.0f;
+        float v2x = e2 - eC, v2y = eB;
+        float len = sqrtf(v2x * v2x + v2y * v2y);
+        v2x = v2x / len;
+        v2y = v2y / len;
+        float minor = 1.0f / sqrtf(e1 * s1);
+        float major = 1.0f / sqrtf(e2 * s2);
+        ow = major * 2.0f;
+        oh = minor * 2.0f;
+        os = v2y;
+        oc = v2x;
+    }
+    for (int y = bminy; y < bmaxy; ++y) {
+        float py0 = (float)((y - bminy) * 16);
+        float py1 = py0 + 16.0f;
+        for (int x = bminx; x < bmaxx; ++x) {
+            float px0 = (float)((x - bminx) * 16);
+            float px1 = px0 + 16.0f;
+            bool keep;
+            if (!use_obb) {
+                bool xo = (uo - bx) <= px1 && (uo + bx) >= px0;
+                bool yo = (vo - by) <= py1 && (vo + by) >= py0;
+                keep = xo && yo;
+            } else {
+                keep = obb_overlaps_box(px0, py0, px1, py1, ow, oh, os, oc, uo, vo);
+            }
+            keep = keep && x >= rminx && x < rmaxx && y >= rminy && y < rmaxy;
+            if (keep) { f(x, y); ++count; }
+        }
+    }
+    return count;
+}
+
+constexpr float kShC0 = 0.28209479177387814f;
+constexpr float kShC1 = 0.4886025119029199f;
+__device__ constexpr float kShC2[5] = {1.0925484305920792f, -1.0925484305920792f, 0.31539156525252005f,
+                                       -1.0925484305920792f, 0.5462742152960396f};
+__device__ constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f, -0.4570457994644658f,
+                                       0.3731763325901154f, -0.4570457994644658f, 1.445305721320277f,
+                                       -0.5900435899266435f};
+
+// Thread-local error string helpers live in capi.hip.
+void set_error(const char* fmt, ...);
+// Validates sizes / enum values of a params block (defined in preprocess.hip).
+int check_params(const d3gs_params* p, const char* who);
+
+}  // namespace d3gs

@@ -1,0 +1,433 @@
+// Per-gaussian kernels: preprocess forward (projection, EWA covariance, conic,
+// radius, tile count, SH colour) and preprocess backward (chain rule back to the
+// raw model tensors).  One thread per gaussian, 256-thread blocks; both are
+// single streaming passes bound by HBM bandwidth.
+//
+// Reference: d3sim/algos/d3gs/render.py:421-476, 569-619 (forward) and
+// 3217-3356 (backward); math in d3sim/csrc/gs3d.py and d3sim/csrc/camera.py.
+#include "device_math.h"
+
+namespace d3gs {
+
+// SH -> RGB for one channel (gs3d.py:151-201); `rest` points at coefficient 1.
+__device__ __forceinline__ float sh_channel(int degree, float x, float y, float z, float base, const float* rest, int ch) {
+    float r = kShC0 * base;
+    if (degree > 0) {
+        r = ((r - (kShC1 * y) * rest[0 * 3 + ch]) + (kShC1 * z) * rest[1 * 3 + ch]) - (kShC1 * x) * rest[2 * 3 + ch];
+        if (degree > 1) {
+            float xx = x * x, yy = y * y, zz = z * z;
+            float xy = x * y, yz = y * z, xz = x * z;
+            r = r + (kShC2[0] * xy) * rest[3 * 3 + ch];
+            r = r + (kShC2[1] * yz) * rest[4 * 3 + ch];
+            r = r + (kShC2[2] * ((2.0f * zz - xx) - yy)) * rest[5 * 3 + ch];
+            r = r + (kShC2[3] * xz) * rest[6 * 3 + ch];
+            r = r + (kShC2[4] * (xx - yy)) * rest[7 * 3 + ch];
+            if (degree > 2) {
+                r = r + ((kShC3[0] * y) * (3.0f * xx - yy)) * rest[8 * 3 + ch];
+                r = r + ((kShC3[1] * xy) * z) * rest[9 * 3 + ch];
+                r = r + ((kShC3[2] * y) * ((4.0f * zz - xx) - yy)) * rest[10 * 3 + ch];
+                r = r + ((kShC3[3] * z) * ((2.0f * zz - 3.0f * xx) - 3.0f * yy)) * rest[11 * 3 + ch];
+                r = r + ((kShC3[4] * x) * ((4.0f * zz - xx) - yy)) * rest[12 * 3 + ch];
+                r = r + ((kShC3[5] * z) * (xx - yy)) * rest[13 * 3 + ch];
+                r = r + ((kShC3[6] * x) * (xx - 3.0f * yy)) * rest[14 * 3 + ch];
+            }
+        }
+    }
+    return r + 0.5f;
+}
+
+__global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
+    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
+    const float* __restrict__ sh_base, float* __restrict__ depths, int32_t* __restrict__ radii,
+    float* __restrict__ uvs, float* __restrict__ conic_opacity, int32_t* __restrict__ tiles_touched,
+    float* __restrict__ rgb_out, float* __restrict__ cov2d_out, uint8_t* __restrict__ ne0_out) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= P.n) return;
+
+    bool valid = true;
+    float z = 0.0f, u = 0.0f, v = 0.0f, con0 = 0.0f, con1 = 0.0f, con2 = 0.0f, op = 0.0f;
+    float a = 0.0f, b = 0.0f, c = 0.0f, radius = 0.0f;
+    int count = 0;
+    float rgb[3] = {0.0f, 0.0f, 0.0f};
+    uint32_t ne0 = 0;
+
+    float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+    float pc[3] = {dot3(P.w2c + 0, d), dot3(P.w2c + 3, d), dot3(P.w2c + 6, d)};
+    z = pc[2];
+    valid = (z >= P.z_near && z <= P.z_far);
+    if (valid) {
+        u = ((pc[0] / z) * P.fx + P.cx) - 0.5f;
+        v = ((pc[1] / z) * P.fy + P.cy) - 0.5f;
+
+        const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
+        float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
+        float q[4] = {qr.x / qn, qr.y / qn, qr.z / qn, qr.w / qn};
+        float s[3] = {det_expf(scale[3 * i]), det_expf(scale[3 * i + 1]), det_expf(scale[3 * i + 2])};
+        if (!P.training) {
+            s[0] = s[0] * P.scale_global;
+            s[1] = s[1] * P.scale_global;
+            s[2] = s[2] * P.scale_global;
+        }
+        float R[9], c6[6];
+        quat_to_rot(q, R);
+        cov3d_from_scale_rot(s, R, c6);
+
+        float t0[3], t1[3], tx, ty;
+        ewa_rows(P, pc, t0, t1, tx, ty);
+        float v0[3], v1[3];
+        sym3_mv(c6, t0, v0);
+        sym3_mv(c6, t1, v1);
+        a = dot3(t0, v0) + P.lowpass;
+        b = dot3(t0, v1);
+        c = dot3(t1, v1) + P.lowpass;
+
+        float det = a * c - b * b;
+        float det_inv = 1.0f / (det + P.eps);
+        con0 = c * det_inv;
+        con1 = (-b) * det_inv;
+        con2 = a * det_inv;
+        op = det_sigmoid(opacity[i]);
+
+        float mid = 0.5f * (a + c);
+        float sq = sqrtf(fmaxf(P.radii_eigen_eps, mid * mid - det));
+        float l1 = mid + sq, l2 = mid - sq;
+        radius = ceilf(P.std_sigma * sqrtf(fmaxf(l1, l2)));
+
+        int rminx = tile_coord((u - radius) / 16.0f, P.tiles_x);
+        int rminy = tile_coord((v - radius) / 16.0f, P.tiles_y);
+        int rmaxx = tile_coord((((u + radius) + 16.0f) - 1.0f) / 16.0f, P.tiles_x);
+        int rmaxy = tile_coord((((v + radius) + 16.0f) - 1.0f) / 16.0f, P.tiles_y);
+        int area = (rmaxx - rminx) * (rmaxy - rminy);
+        valid = (det > 0.0f) && area != 0 && (op > P.alpha_eps);
+    }
+    if (valid) {
+        TileWalkIn g{u, v, radius, con0, con1, con2, op};
+        count = tile_walk(P, g, [](int, int) {});
+
+        float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
+        float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
+        const float* shp = sh + (size_t)i * P.sh_stride * 3;
+        const float* base = P.has_sh_base ? sh_base + 3 * i : shp;
+        const float* rest = P.has_sh_base ? shp : shp + 3;
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch) rgb[ch] = sh_channel(P.sh_degree, dx, dy, dz, base[ch], rest, ch);
+        ne0 = ((rgb[0] < 0.0f) << 2) | ((rgb[1] < 0.0f) << 1) | (rgb[2] < 0.0f);
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch) rgb[ch] = fmaxf(rgb[ch], 0.0f);
+    } else {
+        z = u = v = con0 = con1 = con2 = op = a = b = c = radius = 0.0f;
+    }
+
+    depths[i] = z;
+    radii[i] = (int)radius;
+    *reinterpret_cast<float2*>(uvs + 2 * i) = make_float2(u, v);
+    *reinterpret_cast<float4*>(conic_opacity + 4 * i) = make_float4(con0, con1, con2, op);
+    tiles_touched[i] = count;
+    rgb_out[3 * i + 0] = rgb[0];
+    rgb_out[3 * i + 1] = rgb[1];
+    rgb_out[3 * i + 2] = rgb[2];
+    if (cov2d_out) {
+        cov2d_out[3 * i + 0] = a;
+        cov2d_out[3 * i + 1] = b;
+        cov2d_out[3 * i + 2] = c;
+    }
+    if (ne0_out) ne0_out[i] = (uint8_t)ne0;
+}
+
+// ---------------------------------------------------------------------------
+// Preprocess backward.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
+    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
+    const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
+    const float* __restrict__ duv, const float* __restrict__ dconic, const float* dopacity_in /* may alias dopacity_out */,
+    const float* __restrict__ dcolor, const float* __restrict__ dz_in, const int sh_mask_compat,
+    float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale,
+    float* dopacity_out, float* __restrict__ dsh, float* __restrict__ dsh_base) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= P.n) return;
+    const int K = P.sh_stride;
+    float* dshp = dsh + (size_t)i * K * 3;
+
+    if (radii[i] == 0) {
+        dxyz[3 * i] = dxyz[3 * i + 1] = dxyz[3 * i + 2] = 0.0f;
+        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        dscale[3 * i] = dscale[3 * i + 1] = dscale[3 * i + 2] = 0.0f;
+        dopacity_out[i] = 0.0f;
+        for (int k = 0; k < K * 3; ++k) dshp[k] = 0.0f;
+        if (dsh_base) dsh_base[3 * i] = dsh_base[3 * i + 1] = dsh_base[3 * i + 2] = 0.0f;
+        return;
+    }
+
+    const float* W = P.w2c;
+    float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+    float pc[3] = {dot3(W + 0, d), dot3(W + 3, d), dot3(W + 6, d)};
+    float z = pc[2];
+    // pinhole backward (camera.py:357-369)
+    float gu = duv[2 * i] * P.fx, gv = duv[2 * i + 1] * P.fy;
+    float zi = 1.0f / z, zi2 = 1.0f / (z * z);
+    float dzin = dz_in ? dz_in[i] : 0.0f;
+    float dpc[3] = {gu * zi, gv * zi, (dzin + ((-gu) * pc[0]) * zi2) + ((-gv) * pc[1]) * zi2};
+
+    // conic -> cov2d backward (gs3d.py:571-586)
+    float a = cov2d[3 * i], b = cov2d[3 * i + 1], c = cov2d[3 * i + 2];
+    float g0 = dconic[3 * i], g1 = dconic[3 * i + 1], g2 = dconic[3 * i + 2];
+    float det = a * c - b * b;
+    float k2 = 1.0f / (det * det + 1e-8f);
+    float da = k2 * ((((-c) * c) * g0 + (b * c) * g1) + (det - a * c) * g2);
+    float db = (k2 * 2.0f) * (((b * c) * g0 - (det / 2.0f + b * b) * g1) + (a * b) * g2);
+    float dc = k2 * ((((-a) * a) * g2 + (a * b) * g1) + (det - a * c) * g0);
+
+    const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
+    float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
+    float q[4] = {qr.x / qn, qr.y / qn, qr.z / qn, qr.w / qn};
+    float s[3] = {det_expf(scale[3 * i]), det_expf(scale[3 * i + 1]), det_expf(scale[3 * i + 2])};
+    float R[9], c6[6];
+    quat_to_rot(q, R);
+    cov3d_from_scale_rot(s, R, c6);
+
+    // EWA backward (gs3d.py:490-530): cov2d = T Sigma3 T^T with T = J W
+    float t0[3], t1[3], tx, ty;
+    ewa_rows(P, pc, t0, t1, tx, ty);
+    float limx = fabsf((P.tan_fovx * P.clamp_factor) * z), limy = fabsf((P.tan_fovy * P.clamp_factor) * z);
+    float mx = (pc[0] < -limx || pc[0] > limx) ? 0.0f : 1.0f;
+    float my = (pc[1] < -limy || pc[1] > limy) ? 0.0f : 1.0f;
+    float G00 = da, G01 = 0.5f * db, G11 = dc;
+    float u0[3], u1[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        u0[k] = G00 * t0[k] + G01 * t1[k];
+        u1[k] = G01 * t0[k] + G11 * t1[k];
+    }
+    float dS[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) dS[r * 3 + k] = t0[r] * u0[k] + t1[r] * u1[k];
+    float dT0[3], dT1[3];
+    sym3_mv(c6, u0, dT0);
+    sym3_mv(c6, u1, dT1);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        dT0[k] = 2.0f * dT0[k];
+        dT1[k] = 2.0f * dT1[k];
+    }
+    float dJ00 = dot3(dT0, W + 0), dJ02 = dot3(dT0, W + 6);
+    float dJ11 = dot3(dT1, W + 3), dJ12 = dot3(dT1, W + 6);
+    float zz = z * z;
+    float zzi = 1.0f / zz;
+    float z3 = (z * z) * z;
+    float txf = tx * P.fx, tyf = ty * P.fy;
+    float dmean[3];
+    dmean[0] = ((mx * (-dJ02)) * P.fx) * zzi;
+    dmean[1] = ((my * (-dJ12)) * P.fy) * zzi;
+    dmean[2] = (-(P.fx * dJ00 + P.fy * dJ11)) * zzi + (2.0f * (dJ02 * txf + dJ12 * tyf)) / z3;
+    float tot[3] = {dpc[0] + dmean[0], dpc[1] + dmean[1], dpc[2] + dmean[2]};
+    float gx[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) gx[k] = (W[0 + k] * tot[0] + W[3 + k] * tot[1]) + W[6 + k] * tot[2];
+
+    // cov3d backward (gs3d.py:400-416)
+    float M[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) M[r * 3 + k] = R[r * 3 + k] * s[k];
+    float dM[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+            dM[r * 3 + k] = 2.0f * ((dS[r * 3 + 0] * M[0 + k] + dS[r * 3 + 1] * M[3 + k]) + dS[r * 3 + 2] * M[6 + k]);
+    float ds[3], dR[9];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) ds[k] = (dM[0 + k] * R[0 + k] + dM[3 + k] * R[3 + k]) + dM[6 + k] * R[6 + k];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) dR[r * 3 + k] = dM[r * 3 + k] * s[k];
+    float qx = q[0], qy = q[1], qz = q[2], qw = q[3];
+    float dq[4];
+    dq[0] = 2.0f * (((qy * (dR[1] + dR[3]) + qz * (dR[2] + dR[6])) - (2.0f * qx) * (dR[4] + dR[8])) + qw * (dR[7] - dR[5]));
+    dq[1] = 2.0f * (((qx * (dR[1] + dR[3]) - (2.0f * qy) * (dR[0] + dR[8])) + qz * (dR[5] + dR[7])) + qw * (dR[2] - dR[6]));
+    dq[2] = 2.0f * (((qx * (dR[2] + dR[6]) + qy * (dR[5] + dR[7])) - (2.0f * qz) * (dR[0] + dR[4])) + qw * (dR[3] - dR[1]));
+    dq[3] = 2.0f * ((qz * (dR[3] - dR[1]) + qy * (dR[2] - dR[6])) + qx * (dR[7] - dR[5]));
+    // activation backward: exp, normalize, sigmoid (origin/model.py:332-383)
+    dscale[3 * i + 0] = ds[0] * s[0];
+    dscale[3 * i + 1] = ds[1] * s[1];
+    dscale[3 * i + 2] = ds[2] * s[2];
+    float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
+    *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
+                                                            (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
+    float o = det_sigmoid(opacity[i]);
+    dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+
+    // SH backward (gs3d.py:262-364)
+    float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
+    float x = d[0] / dn, y = d[1] / dn, zd = d[2] / dn;
+    uint32_t m = ne0[i];
+    float cg[3];
+    if (sh_mask_compat) {
+        cg[0] = dcolor[3 * i + 0] * ((m & 1) ? 0.0f : 1.0f);
+        cg[1] = dcolor[3 * i + 1] * ((m & 2) ? 0.0f : 1.0f);
+        cg[2] = dcolor[3 * i + 2] * ((m & 4) ? 0.0f : 1.0f);
+    } else {
+        cg[0] = dcolor[3 * i + 0] * ((m & 4) ? 0.0f : 1.0f);
+        cg[1] = dcolor[3 * i + 1] * ((m & 2) ? 0.0f : 1.0f);
+        cg[2] = dcolor[3 * i + 2] * ((m & 1) ? 0.0f : 1.0f);
+    }
+    const float* shp = sh + (size_t)i * K * 3;
+    const float* rest = P.has_sh_base ? shp : shp + 3;
+    float* drest = P.has_sh_base ? dshp : dshp + 3;
+    float* dbase = P.has_sh_base ? dsh_base + 3 * i : dshp;
+    const int deg = P.sh_degree;
+    // coefficients above the evaluated degree receive zero gradient
+    const int used = (deg + 1) * (deg + 1) - 1;
+    for (int k = used; k < K - (P.has_sh_base ? 0 : 1); ++k) {
+        drest[k * 3 + 0] = 0.0f;
+        drest[k * 3 + 1] = 0.0f;
+        drest[k * 3 + 2] = 0.0f;
+    }
+    float ddir[3] = {0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ch = 0; ch < 3; ++ch) {
+        float gch = cg[ch];
+        dbase[ch] = kShC0 * gch;
+        float dx_ = 0.0f, dy_ = 0.0f, dz_ = 0.0f;
+        if (deg > 0) {
+            drest[0 * 3 + ch] = (-kShC1 * y) * gch;
+            drest[1 * 3 + ch] = (kShC1 * zd) * gch;
+            drest[2 * 3 + ch] = (-kShC1 * x) * gch;
+            dx_ = -kShC1 * rest[2 * 3 + ch];
+            dy_ = -kShC1 * rest[0 * 3 + ch];
+            dz_ = kShC1 * rest[1 * 3 + ch];
+            if (deg > 1) {
+                float xx = x * x, yy = y * y, zz2 = zd * zd, xy = x * y, yz = y * zd, xz = x * zd;
+                drest[3 * 3 + ch] = (kShC2[0] * xy) * gch;
+                drest[4 * 3 + ch] = (kShC2[1] * yz) * gch;
+                drest[5 * 3 + ch] = (kShC2[2] * ((2.0f * zz2 - xx) - yy)) * gch;
+                drest[6 * 3 + ch] = (kShC2[3] * xz) * gch;
+                drest[7 * 3 + ch] = (kShC2[4] * (xx - yy)) * gch;
+                float s3 = rest[3 * 3 + ch], s4 = rest[4 * 3 + ch], s5 = rest[5 * 3 + ch], s6 = rest[6 * 3 + ch],
+                      s7 = rest[7 * 3 + ch];
+                dx_ += kShC2[0] * y * s3 + kShC2[2] * 2.0f * (-x) * s5 + kShC2[3] * zd * s6 + kShC2[4] * 2.0f * x * s7;
+                dy_ += kShC2[0] * x * s3 + kShC2[1] * zd * s4 + kShC2[2] * 2.0f * (-y) * s5 + kShC2[4] * 2.0f * (-y) * s7;
+                dz_ += kShC2[1] * y * s4 + kShC2[2] * 2.0f * 2.0f * zd * s5 + kShC2[3] * x * s6;
+                if (deg > 2) {
+                    drest[8 * 3 + ch] = ((kShC3[0] * y) * (3.0f * xx - yy)) * gch;
+                    drest[9 * 3 + ch] = ((kShC3[1] * xy) * zd) * gch;
+                    drest[10 * 3 + ch] = ((kShC3[2] * y) * ((4.0f * zz2 - xx) - yy)) * gch;
+                    drest[11 * 3 + ch] = ((kShC3[3] * zd) * ((2.0f * zz2 - 3.0f * xx) - 3.0f * yy)) * gch;
+                    drest[12 * 3 + ch] = ((kShC3[4] * x) * ((4.0f * zz2 - xx) - yy)) * gch;
+                    drest[13 * 3 + ch] = ((kShC3[5] * zd) * (xx - yy)) * gch;
+                    drest[14 * 3 + ch] = ((kShC3[6] * x) * (xx - 3.0f * yy)) * gch;
+                    float s8 = rest[8 * 3 + ch], s9 = rest[9 * 3 + ch], s10 = rest[10 * 3 + ch],
+                          s11 = rest[11 * 3 + ch], s12 = rest[12 * 3 + ch], s13 = rest[13 * 3 + ch],
+                          s14 = rest[14 * 3 + ch];
+                    dx_ += kShC3[0] * s8 * 3.0f * 2.0f * xy + kShC3[1] * s9 * yz + kShC3[2] * s10 * (-2.0f) * xy +
+                           kShC3[3] * s11 * (-3.0f) * 2.0f * xz + kShC3[4] * s12 * ((-3.0f) * xx + 4.0f * zz2 - yy) +
+                           kShC3[5] * s13 * 2.0f * xz + kShC3[6] * s14 * 3.0f * (xx - yy);
+                    dy_ += kShC3[0] * s8 * 3.0f * (xx - yy) + kShC3[1] * s9 * xz +
+                           kShC3[2] * s10 * ((-3.0f) * yy + 4.0f * zz2 - xx) + kShC3[3] * s11 * (-3.0f) * 2.0f * yz +
+                           kShC3[4] * s12 * (-2.0f) * xy + kShC3[5] * s13 * (-2.0f) * yz +
+                           kShC3[6] * s14 * (-3.0f) * 2.0f * xy;
+                    dz_ += kShC3[1] * s9 * xy + kShC3[2] * s10 * 4.0f * 2.0f * yz +
+                           kShC3[3] * s11 * 3.0f * ((2.0f * zz2 - xx) - yy) + kShC3[4] * s12 * 4.0f * 2.0f * xz +
+                           kShC3[5] * s13 * (xx - yy);
+                }
+            }
+        }
+        ddir[0] += dx_ * gch;
+        ddir[1] += dy_ * gch;
+        ddir[2] += dz_ * gch;
+    }
+    float dirv[3] = {x, y, zd};
+    float dd = (dirv[0] * ddir[0] + dirv[1] * ddir[1]) + dirv[2] * ddir[2];
+    dxyz[3 * i + 0] = gx[0] + (ddir[0] - dirv[0] * dd) / dn;
+    dxyz[3 * i + 1] = gx[1] + (ddir[1] - dirv[1] * dd) / dn;
+    dxyz[3 * i + 2] = gx[2] + (ddir[2] - dirv[2] * dd) / dn;
+}
+
+int check_params(const d3gs_params* p, const char* who) {
+    if (!p) { set_error("%s: params is NULL", who); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (p->n < 0 || p->width <= 0 || p->height <= 0) {
+        set_error("%s: bad sizes n=%d width=%d height=%d", who, p->n, p->width, p->height);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p->tiles_x != (p->width + kTile - 1) / kTile || p->tiles_y != (p->height + kTile - 1) / kTile) {
+        set_error("%s: tiles_x/tiles_y do not match ceil(width/16), ceil(height/16)", who);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p->sh_degree < 0 || p->sh_degree > 3) {
+        set_error("%s: sh_degree %d outside [0,3]", who, p->sh_degree);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    int need = (p->sh_degree + 1) * (p->sh_degree + 1) - (p->has_sh_base ? 1 : 0);
+    if (p->sh_stride < need) {
+        set_error("%s: sh_stride %d holds fewer coefficients than degree %d needs (%d)", who, p->sh_stride,
+                  p->sh_degree, need);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p->filter_algo == D3GS_FILTER_ELLIPSE) {
+        set_error("%s: early_filter_algo ELLIPSE is not implemented", who);
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    if (p->filter_algo < 0 || p->filter_algo > 4) {
+        set_error("%s: unknown early_filter_algo %d", who, p->filter_algo);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    return D3GS_OK;
+}
+
+}  // namespace d3gs
+
+using namespace d3gs;
+
+extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
+                                   const float* scale, const float* opacity, const float* color_sh,
+                                   const float* color_sh_base, float* depths, int32_t* radii, float* uvs,
+                                   float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
+                                   float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_preprocess_fwd");
+    if (rc) return rc;
+    if (p->n == 0) return D3GS_OK;
+    if (!xyz || !quaternion_xyzw || !scale || !opacity || !color_sh || !depths || !radii || !uvs || !conic_opacity ||
+        !tiles_touched || !rgb_gaussian || (p->has_sh_base && !color_sh_base)) {
+        set_error("d3gs_preprocess_fwd: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
+    hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
+                       opacity, color_sh, color_sh_base, depths, radii, uvs, conic_opacity, tiles_touched,
+                       rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
+                                   const float* scale, const float* opacity, const float* color_sh,
+                                   const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
+                                   const float* duv, const float* dconic, const float* dopacity_in,
+                                   const float* dcolor, const float* dz, int32_t sh_mask_compat, float* dxyz,
+                                   float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
+                                   float* dcolor_sh_base, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_preprocess_bwd");
+    if (rc) return rc;
+    if (p->n == 0) return D3GS_OK;
+    if (!xyz || !quaternion_xyzw || !scale || !opacity || !color_sh || !radii || !cov2d_vecs || !sh_to_rgb_ne_0 ||
+        !duv || !dconic || !dopacity_in || !dcolor || !dxyz || !dquaternion_xyzw || !dscale || !dopacity_out ||
+        !dcolor_sh || (p->has_sh_base && !dcolor_sh_base)) {
+        set_error("d3gs_preprocess_bwd: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
+    hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
+                       opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, duv, dconic, dopacity_in, dcolor, dz,
+                       (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}

@@ -1,0 +1,79 @@
+"""Gaussian model containers with the reference's tensor layout.
+
+``GaussianModelOriginFused`` mirrors d3sim/algos/d3gs/origin/model.py:34-48 and
+435-465: raw (pre-activation) tensors whose activations — exp for scale,
+normalize for the quaternion, sigmoid for opacity — are applied inside the
+preprocess kernel.  Quaternions are stored (x, y, z, w).
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+
+import torch
+
+
+@dataclasses.dataclass(kw_only=True)
+class GaussianModelOriginBase:
+    xyz: torch.Tensor                    # [N, 3] f32
+    quaternion_xyzw: torch.Tensor        # [N, 4] f32
+    scale: torch.Tensor                  # [N, 3] f32 (log-scale)
+    opacity: torch.Tensor                # [N]    f32 (logit)
+    color_sh: torch.Tensor               # [N, K, 3] f32
+    color_sh_base: torch.Tensor | None = None   # [N, 3] f32 when the DC term is split off
+    instance_id: torch.Tensor | None = None
+    act_applied: bool = False
+    cur_sh_degree: int = 0
+
+    def __len__(self):
+        return self.xyz.shape[0]
+
+    @property
+    def color_sh_degree(self) -> int:
+        dim = self.color_sh.shape[1]
+        if self.color_sh_base is not None:
+            dim += 1
+        res = int(math.sqrt(dim)) - 1
+        assert (res + 1) * (res + 1) == dim
+        return res
+
+    def get_proxy_field_dict(self):
+        res = {"xyz": self.xyz, "quaternion_xyzw": self.quaternion_xyzw, "scale": self.scale,
+               "opacity": self.opacity, "color_sh": self.color_sh}
+        if self.color_sh_base is not None:
+            res["color_sh_base"] = self.color_sh_base
+        return res
+
+    def set_requires_grad(self, requires_grad: bool):
+        for t in self.get_proxy_field_dict().values():
+            t.requires_grad_(requires_grad)
+
+    def clear_grad(self):
+        for t in self.get_proxy_field_dict().values():
+            t.grad = None
+
+    def create_model_with_act(self):
+        if self.act_applied:
+            return dataclasses.replace(self)
+        return dataclasses.replace(self, act_applied=True)
+
+    def to_device(self, device):
+        kw = {k: v.to(device) for k, v in self.get_proxy_field_dict().items()}
+        return dataclasses.replace(self, **kw)
+
+
+@dataclasses.dataclass(kw_only=True)
+class GaussianModelOriginFused(GaussianModelOriginBase):
+    """Activations fused into the kernels (origin/model.py:435-465)."""
+
+    @property
+    def fused_quaternion_xyzw_act_op(self):
+        return ("normalize", "normalize_grad_out")
+
+    @property
+    def fused_scale_act_op(self):
+        return ("exponential", "exponential_grad_out")
+
+    @property
+    def fused_opacity_act_op(self):
+        return ("sigmoid", "sigmoid_grad_out")

@@ -1,0 +1,447 @@
+"""Rasterize operator: the reference's Python surface over the gfx950 library.
+
+Mirrors d3sim/algos/d3gs/render.py: the dataclasses (35-150), ``GaussianSplatOp``
+with ``forward`` (169-1015), ``rasterize_forward_backward`` (1329-2316) and
+``backward`` (2779-3374), the autograd glue (3376-3587) and the user entry point
+``rasterize_gaussians`` (3783-3838).  Where the reference assembles CUDA source
+text and JIT-compiles it, this module allocates with torch and calls the
+ahead-of-time HIP library through ``_capi`` on torch's current stream.
+
+Scope: one camera per call (batch 1), RGB output in NHWC, early filters NONE /
+AABB / OBB / OBB_DFVT (the latter computed as the OBB tile set), the default
+backward algorithm.  Options outside that scope raise ``NotImplementedError``.
+"""
+from __future__ import annotations
+
+import contextlib
+import copy
+import ctypes as C
+import dataclasses
+
+import numpy as np
+import torch
+
+from . import _capi
+from .camera import BasicPinholeCamera
+from .config_def import EarlyFilterAlgo, GaussianSplatConfig, RasterizeBackwardAlgo
+from .model import GaussianModelOriginBase, GaussianModelOriginFused
+
+
+def div_up(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+@dataclasses.dataclass
+class GaussianSplatOpContext:
+    """render.py:57-72"""
+    conic_opacity: torch.Tensor
+    radii: torch.Tensor
+    uvs: torch.Tensor
+    rgb_gaussian: torch.Tensor | None
+    gaussian_idx_sorted: torch.Tensor
+    workload_ranges: torch.Tensor
+    image_shape_wh: tuple[int, int]
+    depths: torch.Tensor
+    cov2d_vecs: torch.Tensor | None = None
+    sh_to_rgb_ne_0: torch.Tensor | None = None
+    per_gaussian_snap: None = None
+
+
+@dataclasses.dataclass
+class GaussianSplatOutput:
+    """render.py:74-100"""
+    custom_features: torch.Tensor | None
+    T: torch.Tensor
+    color: torch.Tensor
+    depth: torch.Tensor | None = None
+    n_contrib: torch.Tensor | None = None
+    radii: torch.Tensor | None = None
+    sparse_gaussian_ids: torch.Tensor | None = None
+    sparse_batch_ids: torch.Tensor | None = None
+
+    @property
+    def image_shape_wh(self) -> tuple[int, int]:
+        return (self.T.shape[2], self.T.shape[1])
+
+    def select_batch(self, batch_idx: int):
+        s = slice(batch_idx, batch_idx + 1)
+        return GaussianSplatOutput(
+            custom_features=None if self.custom_features is None else self.custom_features[s],
+            T=self.T[s], color=self.color[s], depth=None if self.depth is None else self.depth[s],
+            n_contrib=None if self.n_contrib is None else self.n_contrib[s], radii=self.radii)
+
+
+@dataclasses.dataclass
+class RasterizeGradientOutput:
+    """render.py:103-111"""
+    duv: torch.Tensor
+    dconic: torch.Tensor
+    dopacity: torch.Tensor
+    dcolor: torch.Tensor | None
+    dcustom_features: torch.Tensor | None = None
+    dz: torch.Tensor | None = None
+
+
+@dataclasses.dataclass
+class GaussianSplatGradients:
+    """render.py:113-120"""
+    drgb: torch.Tensor
+    dT: torch.Tensor
+    ddepth: torch.Tensor | None = None
+    dcustom_features: torch.Tensor | None = None
+
+
+@dataclasses.dataclass
+class CameraParamBundle:
+    focal_xy_ppoint: torch.Tensor
+    image_shape_wh: tuple[int, int]
+    frame_ids: torch.Tensor | None
+
+
+@dataclasses.dataclass
+class CameraBundle(CameraParamBundle):
+    """render.py:129-150; only bundles holding one camera are accepted here."""
+    cam2world_T: torch.Tensor = None
+
+    @classmethod
+    def from_pinhole_cams(cls, cams: list[BasicPinholeCamera], device="cuda"):
+        c2w = np.stack([np.ascontiguousarray(c.pose.to_world[:3].T) for c in cams], 0).reshape(-1, 4, 3)
+        fpp = np.stack([np.concatenate([c.focal_length, c.principal_point]) for c in cams], 0).reshape(-1, 4)
+        return cls(torch.from_numpy(fpp.astype(np.float32)).to(device), cams[0].image_shape_wh, None,
+                   torch.from_numpy(c2w.astype(np.float32)).to(device))
+
+
+class GaussianSplatOp:
+    """render.py:152-159: one op per config; the config is frozen at construction."""
+
+    def __init__(self, cfg: GaussianSplatConfig) -> None:
+        self._cfg = copy.deepcopy(cfg)
+        self._lib = _capi.lib()  # fails loudly when the HIP library is not built
+        self._check_supported()
+        # optional per-stage timing: set to a dict to collect torch.cuda.Event pairs
+        self.stage_events: dict[str, list] | None = None
+        self.last_num_rendered = 0
+
+    # ------------------------------------------------------------------ utils
+    def _check_supported(self):
+        c = self._cfg
+        unsupported = {
+            "tile_size != (16, 16)": tuple(c.tile_size) != (16, 16),
+            "enable_32bit_sort": c.enable_32bit_sort, "render_depth": c.render_depth,
+            "render_inv_depth": c.render_inv_depth, "enable_anti_aliasing": c.enable_anti_aliasing,
+            "use_nchw": c.use_nchw, "render_rgba": c.render_rgba,
+            "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
+            "disable_builtin_rgb": c.disable_builtin_rgb,
+            "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
+            "use_int64_tile_touched": c.use_int64_tile_touched,
+            "rasterize_backward_algo=PER_GAUSSIAN": c.rasterize_backward_algo != RasterizeBackwardAlgo.DEFAULT,
+            "early_filter_algo=ELLIPSE": c.early_filter_algo == EarlyFilterAlgo.ELLIPSE,
+        }
+        bad = [k for k, v in unsupported.items() if v]
+        if bad:
+            raise NotImplementedError("GaussianSplatOp (gfx950 build): unsupported config options: " + ", ".join(bad))
+
+    @property
+    def is_nchw(self):
+        return self._cfg.use_nchw
+
+    @property
+    def is_rgba(self):
+        return self._cfg.render_rgba
+
+    @contextlib.contextmanager
+    def _stage(self, name: str):
+        if self.stage_events is None:
+            yield
+            return
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        yield
+        b.record()
+        self.stage_events.setdefault(name, []).append((a, b))
+
+    @staticmethod
+    def _stream():
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def _camera_arrays(self, cameras):
+        if isinstance(cameras, BasicPinholeCamera):
+            intrinsic = cameras.intrinsic
+            focal = np.array([intrinsic[0, 0], intrinsic[1, 1]], np.float32)
+            pp = np.array([intrinsic[0, 2], intrinsic[1, 2]], np.float32)
+            c2w_T = np.ascontiguousarray(np.asarray(cameras.pose.to_world)[:3].T).astype(np.float32)
+        elif isinstance(cameras, CameraBundle):
+            if cameras.cam2world_T.shape[0] != 1:
+                raise NotImplementedError("camera bundles with more than one camera are not supported")
+            fpp = cameras.focal_xy_ppoint[0].detach().cpu().numpy().astype(np.float32)
+            focal, pp = fpp[:2], fpp[2:]
+            c2w_T = cameras.cam2world_T[0].detach().cpu().numpy().astype(np.float32).reshape(4, 3)
+        else:
+            raise TypeError(f"unsupported camera type {type(cameras)}")
+        return focal, pp, c2w_T, cameras.image_shape_wh
+
+    def make_params(self, model: GaussianModelOriginBase, cameras, training: bool) -> _capi.Params:
+        """Scalars the reference bakes into kernel source (render.py:198-230, 333-358)."""
+        c = self._cfg
+        focal, pp, c2w_T, (width, height) = self._camera_arrays(cameras)
+        P = _capi.Params()
+        P.n = len(model)
+        P.width, P.height = int(width), int(height)
+        P.tiles_x, P.tiles_y = div_up(width, 16), div_up(height, 16)
+        P.sh_degree = int(model.cur_sh_degree)
+        P.sh_stride = int(model.color_sh.shape[1])
+        P.has_sh_base = int(model.color_sh_base is not None)
+        P.filter_algo = int(c.early_filter_algo)
+        P.training = int(bool(training))
+        P.fx, P.fy, P.cx, P.cy = float(focal[0]), float(focal[1]), float(pp[0]), float(pp[1])
+        tan_fov = np.float32(0.5) * np.array([width, height], np.float32) / focal
+        P.tan_fovx, P.tan_fovy = float(tan_fov[0]), float(tan_fov[1])
+        P.w2c[:] = [float(v) for v in c2w_T[:3].reshape(-1)]
+        P.cam_center[:] = [float(v) for v in c2w_T[3]]
+        P.z_near, P.z_far, P.eps = float(c.near), float(c.far), float(c.eps)
+        P.radii_eigen_eps = float(c.cov2d_radii_eigen_eps)
+        P.clamp_factor = float(c.projected_clamp_factor)
+        P.std_sigma = float(c.gaussian_std_sigma)
+        P.lowpass = float(c.gaussian_lowpass_filter)
+        P.alpha_eps = float(c.alpha_eps)
+        P.transmittance_eps = float(c.transmittance_eps)
+        P.scale_global = float(c.scale_global)
+        P.bg[:] = [float(v) for v in np.asarray(c.bg_color, np.float32).reshape(3)]
+        return P
+
+    @staticmethod
+    def _check_model(model: GaussianModelOriginBase):
+        n = len(model)
+        exp = {"xyz": (n, 3), "quaternion_xyzw": (n, 4), "scale": (n, 3), "opacity": (n,)}
+        for name, shape in exp.items():
+            t = getattr(model, name)
+            assert t.is_cuda and t.dtype == torch.float32 and tuple(t.shape) == shape and t.is_contiguous(), \
+                f"model.{name} must be a contiguous float32 cuda tensor of shape {shape}"
+        sh = model.color_sh
+        assert sh.is_cuda and sh.dtype == torch.float32 and sh.ndim == 3 and sh.shape[0] == n and sh.shape[2] == 3 \
+            and sh.is_contiguous(), "model.color_sh must be a contiguous float32 cuda tensor [N, K, 3]"
+        if model.color_sh_base is not None:
+            b = model.color_sh_base
+            assert b.is_cuda and b.dtype == torch.float32 and tuple(b.shape) == (n, 3) and b.is_contiguous()
+        assert 0 <= model.cur_sh_degree <= min(3, model.color_sh_degree), "cur_sh_degree out of range"
+
+    # ---------------------------------------------------------------- forward
+    def forward(self, model: GaussianModelOriginBase, cameras, training: bool = False, instance2world_T=None,
+                custom_features=None, mask=None, prep_user_inputs=None):
+        """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
+        assert model.act_applied, "model must be activated before render"
+        if instance2world_T is not None or custom_features is not None or mask is not None or prep_user_inputs:
+            raise NotImplementedError("instance2world_T / custom_features / mask / prep_user_inputs are not supported")
+        if not isinstance(model, GaussianModelOriginFused):
+            raise NotImplementedError("only GaussianModelOriginFused (in-kernel activations) is supported")
+        self._check_model(model)
+        L = self._lib
+        P = self.make_params(model, cameras, training)
+        n, dev = P.n, model.xyz.device
+        width, height = P.width, P.height
+        num_tiles = P.tiles_x * P.tiles_y
+        s = self._stream()
+        f32, i32 = torch.float32, torch.int32
+
+        with self._stage("preprocess"):
+            depths = torch.empty(n, dtype=f32, device=dev)
+            radii = torch.empty(n, dtype=i32, device=dev)
+            uvs = torch.empty((n, 2), dtype=f32, device=dev)
+            conic_opacity = torch.empty((n, 4), dtype=f32, device=dev)
+            tiles_touched = torch.empty(n, dtype=i32, device=dev)
+            rgb_gaussian = torch.empty((n, 3), dtype=f32, device=dev)
+            cov2d_vecs = torch.empty((n, 3), dtype=f32, device=dev) if training else None
+            ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
+            _capi.check(L.d3gs_preprocess_fwd(
+                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+                _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
+                _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                _capi.ptr(tiles_touched), _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs), _capi.ptr(ne0), s),
+                "d3gs_preprocess_fwd")
+
+        with self._stage("scan"):
+            ws_bytes = C.c_size_t(0)
+            _capi.check(L.d3gs_scan_workspace_bytes(n, C.byref(ws_bytes)), "d3gs_scan_workspace_bytes")
+            scan_ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
+            total = torch.empty(1, dtype=torch.int64, device=dev)
+            _capi.check(L.d3gs_scan_tiles(_capi.ptr(tiles_touched), n, _capi.ptr(scan_ws), ws_bytes.value,
+                                          _capi.ptr(total), s), "d3gs_scan_tiles")
+            num_rendered = int(total.item())  # host sync: sizes the next allocations (render.py:695)
+        self.last_num_rendered = num_rendered
+
+        final_T = torch.empty((1, height, width), dtype=f32, device=dev)
+        n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
+        out_color = torch.empty((1, height, width, 3), dtype=f32, device=dev)
+        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=None, n_contrib=n_contrib,
+                                  radii=radii)
+        if num_rendered == 0:
+            # the reference returns uninitialised buffers here (render.py:706-729); fill with the
+            # values an empty scene renders to instead
+            final_T.fill_(1.0)
+            n_contrib.zero_()
+            if training:
+                out_color.zero_()
+            else:
+                bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=dev).clamp(0, 1)
+                out_color[:] = bg
+            return out, None
+
+        with self._stage("make_keys"):
+            keys = torch.empty(num_rendered, dtype=torch.int64, device=dev)
+            gaussian_idx = torch.empty(num_rendered, dtype=i32, device=dev)
+            _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                                         _capi.ptr(depths), _capi.ptr(tiles_touched), _capi.ptr(keys),
+                                         _capi.ptr(gaussian_idx), num_rendered, s), "d3gs_make_keys")
+
+        with self._stage("sort"):
+            end_bit = 32 + L.d3gs_higher_msb(num_tiles)
+            keys_b = torch.empty_like(keys)
+            vals_b = torch.empty_like(gaussian_idx)
+            _capi.check(L.d3gs_sort_workspace_bytes(num_rendered, 0, end_bit, C.byref(ws_bytes)),
+                        "d3gs_sort_workspace_bytes")
+            sort_ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
+            in_b = C.c_int(0)
+            _capi.check(L.d3gs_sort_pairs(_capi.ptr(keys), _capi.ptr(keys_b), _capi.ptr(gaussian_idx),
+                                          _capi.ptr(vals_b), _capi.ptr(sort_ws), ws_bytes.value, num_rendered, 0,
+                                          end_bit, C.byref(in_b), s), "d3gs_sort_pairs")
+            keys_sorted, gaussian_idx_sorted = (keys_b, vals_b) if in_b.value else (keys, gaussian_idx)
+
+        with self._stage("tile_ranges"):
+            workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+            _capi.check(L.d3gs_tile_ranges(_capi.ptr(keys_sorted), num_rendered, _capi.ptr(workload_ranges),
+                                           num_tiles, s), "d3gs_tile_ranges")
+
+        ctx = GaussianSplatOpContext(
+            conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
+            gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
+            image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths)
+        self._last_keys_sorted = keys_sorted  # kept for parity tests (sorted key order)
+        with self._stage("blend_fwd"):
+            self.rasterize_forward_backward(model, ctx, out, training=training, _params=P)
+        if not training:
+            ctx = None
+        return out, ctx
+
+    # ------------------------------------------------------- blend fwd / bwd
+    def rasterize_forward_backward(self, model, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
+                                   grad: GaussianSplatGradients | None = None, training: bool = False,
+                                   render_depth: bool = False, custom_features=None, _params=None, _cameras=None):
+        """render.py:1329-2316: blend forward when ``grad`` is None, else blend backward."""
+        if render_depth or custom_features is not None:
+            raise NotImplementedError("render_depth / custom_features are not supported")
+        L = self._lib
+        P = _params
+        if P is None:
+            assert _cameras is not None, "camera needed to rebuild kernel parameters"
+            P = self.make_params(model, _cameras, training)
+        s = self._stream()
+        n, dev = P.n, ctx.uvs.device
+        if grad is None:
+            _capi.check(L.d3gs_blend_fwd(
+                C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(out.color), _capi.ptr(out.T),
+                _capi.ptr(out.n_contrib), s), "d3gs_blend_fwd")
+            return None
+        drgb = grad.drgb
+        assert drgb.is_contiguous(), "drgb must be contiguous"
+        assert grad.dT.is_contiguous(), "dT must be contiguous"
+        duv = torch.zeros((n, 2), dtype=torch.float32, device=dev)
+        dconic = torch.zeros((n, 3), dtype=torch.float32, device=dev)
+        dopacity = torch.zeros(n, dtype=torch.float32, device=dev)
+        dcolor = torch.zeros((n, 3), dtype=torch.float32, device=dev)
+        _capi.check(L.d3gs_blend_bwd(
+            C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
+            _capi.ptr(out.color), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(duv), _capi.ptr(dconic),
+            _capi.ptr(dopacity), _capi.ptr(dcolor), s), "d3gs_blend_bwd")
+        return RasterizeGradientOutput(duv=duv, dconic=dconic, dopacity=dopacity, dcolor=dcolor)
+
+    # --------------------------------------------------------------- backward
+    def backward(self, model: GaussianModelOriginBase, cameras, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
+                 grad: GaussianSplatGradients, return_uv_grad: bool = False, instance2world_T=None,
+                 custom_features=None, prep_user_inputs=None):
+        """render.py:2779-3374.  Returns ``(grad_model, duv | None, dcustom_features)``; ``grad_model``
+        is a model-shaped dataclass holding the gradients of the raw tensors."""
+        if instance2world_T is not None or custom_features is not None or prep_user_inputs:
+            raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
+        if grad.ddepth is not None or grad.dcustom_features is not None:
+            raise NotImplementedError("depth / custom feature gradients are not supported")
+        L = self._lib
+        P = self.make_params(model, cameras, True)
+        s = self._stream()
+        n, dev = P.n, model.xyz.device
+        with self._stage("blend_bwd"):
+            g = self.rasterize_forward_backward(model, ctx, out, grad, training=True, _params=P)
+        with self._stage("preprocess_bwd"):
+            dxyz = torch.empty_like(model.xyz)
+            dquat = torch.empty_like(model.quaternion_xyzw)
+            dscale = torch.empty_like(model.scale)
+            dsh = torch.empty_like(model.color_sh)
+            dsh_base = torch.empty_like(model.color_sh_base) if model.color_sh_base is not None else None
+            # opacity gradient is finished in place in the buffer the blend accumulated into
+            # (render.py:2918 external_tensors={"opacity": dopacity})
+            _capi.check(L.d3gs_preprocess_bwd(
+                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+                _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
+                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.duv), _capi.ptr(g.dconic), _capi.ptr(g.dopacity),
+                _capi.ptr(g.dcolor), None, int(self._cfg.compat_ref_sh_mask_bitorder), _capi.ptr(dxyz),
+                _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(g.dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), s),
+                "d3gs_preprocess_bwd")
+        grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=g.dopacity,
+                                         color_sh=dsh, color_sh_base=dsh_base)
+        self.last_raster_grads = g
+        if return_uv_grad:
+            return grad_model, g.duv.view(1, -1, 2), None
+        return grad_model, None, None
+
+
+class _RasterizeGaussians(torch.autograd.Function):
+    """render.py:3376-3587, with saved tensors addressed by name."""
+
+    @staticmethod
+    def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, model_cls, cameras,
+                training, op: GaussianSplatOp, uv_grad_holder=None):
+        model = model_cls(xyz=xyz, color_sh=color_sh, color_sh_base=color_sh_base, scale=scale,
+                          quaternion_xyzw=quaternion_xyzw, opacity=opacity, cur_sh_degree=cur_sh_degree,
+                          act_applied=True)
+        out, fwd_ctx = op.forward(model, cameras, training)
+        ctx.has_ctx = fwd_ctx is not None
+        if fwd_ctx is not None:
+            ctx.fwd_ctx = fwd_ctx
+            ctx.out = out
+        ctx.model = model
+        ctx.op = op
+        ctx.cameras = cameras
+        ctx.return_uv_grad = uv_grad_holder is not None
+        ctx.mark_non_differentiable(out.n_contrib, out.radii)
+        return out.color, out.T, out.n_contrib, out.radii
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, drgb, dT, dn_contrib, dradii):
+        if not ctx.has_ctx:
+            return (None,) * 12
+        if drgb is None:
+            drgb = torch.zeros_like(ctx.out.color)
+        if dT is None:
+            dT = torch.zeros_like(ctx.out.T)
+        grads = GaussianSplatGradients(drgb=drgb.contiguous(), dT=dT.contiguous())
+        gm, duv, _ = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
+                                     return_uv_grad=ctx.return_uv_grad)
+        return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, None, None,
+                None, None, duv)
+
+
+def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSplatOp, training=False,
+                        uv_grad_holder: torch.Tensor | None = None, instance2world_T=None, custom_features=None,
+                        mask=None) -> GaussianSplatOutput:
+    """render.py:3783-3838."""
+    if instance2world_T is not None or custom_features is not None or mask is not None:
+        raise NotImplementedError("instance2world_T / custom_features / mask are not supported")
+    model = model.create_model_with_act()
+    res = _RasterizeGaussians.apply(model.xyz, model.color_sh, model.color_sh_base, model.scale,
+                                    model.quaternion_xyzw, model.opacity, model.cur_sh_degree, type(model), cameras,
+                                    training, op, uv_grad_holder)
+    return GaussianSplatOutput(color=res[0], depth=None, custom_features=None, T=res[1], n_contrib=res[2],
+                               radii=res[3])

@@ -1,0 +1,154 @@
+/*
+ * d3gs_hip.h — C ABI of libd3gs_hip.so, the MI355X (gfx950) implementation of
+ * the 3D-Gaussian-splatting rasterize forward/backward path.
+ *
+ * The reference reaches its GPU code through two native boundaries:
+ *   (1) JIT kernel launches  `self._inliner.kernel_1d / kernel_raw(name, ..., code)`
+ *       (d3sim/csrc/inliner.py:35-43; call sites listed per entry point below);
+ *   (2) the pybind module    `d3sim.d3sim_thtools.device_sort.DeviceSort`
+ *       (d3sim/csrc/devsort.py:20-149, stubs d3sim_thtools/device_sort.pyi:3-38).
+ * Every entry point below replaces one of those call sites.
+ *
+ * Conventions
+ *   - all pointers are DEVICE pointers unless the name ends in `_host`;
+ *   - the caller owns every buffer (outputs, accumulators, workspaces); nothing
+ *     here allocates or frees device memory;
+ *   - every call enqueues work on `stream` (a hipStream_t passed as void*) and
+ *     returns without synchronising;
+ *   - return value 0 = success; negative = error (D3GS_ERR_*), with a message
+ *     available from d3gs_last_error_string() (thread local);
+ *   - accumulators written with atomics (duv, dconic, dopacity, dcolor) and the
+ *     tile range table must be zero-filled by the caller, as in the reference
+ *     (render.py:897, 1388-1411).
+ */
+#ifndef D3GS_HIP_H_
+#define D3GS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define D3GS_ABI_VERSION 1
+
+#define D3GS_OK 0
+#define D3GS_ERR_INVALID_ARGUMENT (-1)
+#define D3GS_ERR_UNSUPPORTED (-2)
+#define D3GS_ERR_WORKSPACE_TOO_SMALL (-3)
+#define D3GS_ERR_LAUNCH (-4)
+
+/* EarlyFilterAlgo, d3sim/algos/d3gs/config_def.py:59-70 */
+#define D3GS_FILTER_NONE 0
+#define D3GS_FILTER_AABB 1
+#define D3GS_FILTER_ELLIPSE 2 /* not implemented: returns D3GS_ERR_UNSUPPORTED */
+#define D3GS_FILTER_OBB 3
+#define D3GS_FILTER_OBB_DFVT 4 /* computed as the OBB tile set */
+
+typedef void* d3gs_stream_t;
+
+/* Scalars the reference bakes into the JIT source text (render.py:198-230,
+ * 333-358; config_def.py:77-151). Plain data, passed by pointer from the host. */
+typedef struct d3gs_params {
+    int32_t n;           /* number of gaussians */
+    int32_t width, height;
+    int32_t tiles_x, tiles_y; /* ceil(width/16), ceil(height/16) */
+    int32_t sh_degree;   /* evaluated SH degree (cur_sh_degree), 0..3 */
+    int32_t sh_stride;   /* coefficients per gaussian stored in color_sh */
+    int32_t has_sh_base; /* DC coefficient lives in color_sh_base */
+    int32_t filter_algo; /* D3GS_FILTER_* */
+    int32_t training;
+    float fx, fy, cx, cy;
+    float tan_fovx, tan_fovy; /* 0.5 * (W,H) / focal */
+    float w2c[9];        /* rows 0..2 of cam2world_T = world->camera rotation */
+    float cam_center[3]; /* row 3 of cam2world_T */
+    float z_near, z_far;
+    float eps;
+    float radii_eigen_eps;
+    float clamp_factor;
+    float std_sigma;
+    float lowpass;
+    float alpha_eps;
+    float transmittance_eps;
+    float scale_global;
+    float bg[3];
+} d3gs_params;
+
+int d3gs_abi_version(void);
+const char* d3gs_last_error_string(void);
+
+/* DeviceSort.get_higher_msb — devsort.py:131-149: bit length of n. */
+int d3gs_higher_msb(uint32_t n);
+
+/* K1 — replaces kernel_raw("gs3d_preprocess_...") at render.py:629-681 (body
+ * 421-476, 569-619).  One pass over the gaussians: fused activations, projection,
+ * EWA covariance, conic, radius, tile rect, validity, tile count under the chosen
+ * early filter, SH colour.  Outputs of rejected gaussians are written as zeros.
+ * cov2d_vecs and sh_to_rgb_ne_0 may be NULL (inference). sh_base may be NULL. */
+int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
+                        const float* opacity, const float* color_sh, const float* color_sh_base, float* depths,
+                        int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
+                        float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
+
+/* K2 — replaces `tiles_touched.cumsum_(0)` + `.item()` at render.py:694-695.
+ * In-place inclusive scan; the grand total is written to *total_dev (device
+ * int64).  Workspace size from d3gs_scan_workspace_bytes. */
+int d3gs_scan_workspace_bytes(int32_t n, size_t* bytes_out_host);
+int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t workspace_bytes, int64_t* total_dev,
+                    d3gs_stream_t stream);
+
+/* K3 — replaces kernel_1d("prepare_sort_data_...") at render.py:739-840.
+ * offsets = the inclusive scan from d3gs_scan_tiles; m = its total. */
+int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                   const float* depths, const int32_t* offsets, uint64_t* keys, int32_t* gaussian_idx, int64_t m,
+                   d3gs_stream_t stream);
+
+/* K4 — replaces DeviceSort.get_sort_workspace_size / do_radix_sort_with_bit_range
+ * (devsort.py:38-129; call site render.py:846-887).  Stable LSD radix sort of
+ * (uint64 key, int32 value) pairs on key bits [begin_bit, end_bit), ping-ponging
+ * between the a and b buffers.  *result_in_b_host (host int) tells which pair of
+ * buffers holds the result, like the reference's (key_swap, value_swap). */
+int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* bytes_out_host);
+int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                    size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                    d3gs_stream_t stream);
+
+/* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
+ * ranges[num_tiles][2] must be zero-filled by the caller. */
+int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
+                     d3gs_stream_t stream);
+
+/* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
+ * color [H,W,3], final_T [H,W], n_contrib [H,W]. */
+int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, float* color,
+                   float* final_T, int32_t* n_contrib, d3gs_stream_t stream);
+
+/* K7 — replaces kernel_raw("rasterize_True_...") (same generator, grad != None,
+ * render.py:1341, 1589-1676, 1774-2210).  Produces the complete gradient (the
+ * reference's backward_reduction_balanced_factor <= 0 branch, render.py:2024-2050,
+ * 2182-2210).  duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3] are
+ * accumulated with atomics: zero-fill them first. */
+int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* final_T,
+                   const int32_t* n_contrib, const float* color, const float* drgb, const float* dT, float* duv,
+                   float* dconic, float* dopacity, float* dcolor, d3gs_stream_t stream);
+
+/* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
+ * (body 3217-3356).  Chain rule from (duv, dconic, dopacity, dcolor[, dz]) to
+ * the raw model tensors, including the fused activation gradients.  Gradients
+ * of gaussians with radii == 0 are written as zeros.  dz and the *_base
+ * pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
+ * reference's reversed bit order (render.py:3344-3350). */
+int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
+                        const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                        const uint8_t* sh_to_rgb_ne_0, const float* duv, const float* dconic,
+                        const float* dopacity_in, const float* dcolor, const float* dz, int32_t sh_mask_compat,
+                        float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
+                        float* dcolor_sh_base, d3gs_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* D3GS_HIP_H_ */

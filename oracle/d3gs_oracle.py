@@ -1,0 +1,233 @@
+"""numpy front end of the CPU oracle (``libd3gs_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: tests, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this module; the product
+package never does.  Every function here is a thin ctypes call into
+``d3gs_oracle.cpp``, whose header lists the reference lines each stage restates.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libd3gs_oracle.so")
+
+FILTER_NONE, FILTER_AABB, FILTER_ELLIPSE, FILTER_OBB, FILTER_OBB_DFVT = 0, 1, 2, 3, 4
+
+
+class OracleParams(C.Structure):
+    _fields_ = [
+        ("n", C.c_int32), ("width", C.c_int32), ("height", C.c_int32),
+        ("tiles_x", C.c_int32), ("tiles_y", C.c_int32),
+        ("sh_degree", C.c_int32), ("sh_stride", C.c_int32), ("has_sh_base", C.c_int32),
+        ("filter_algo", C.c_int32), ("training", C.c_int32),
+        ("fx", C.c_float), ("fy", C.c_float), ("cx", C.c_float), ("cy", C.c_float),
+        ("tan_fovx", C.c_float), ("tan_fovy", C.c_float),
+        ("w2c", C.c_float * 9), ("cam_center", C.c_float * 3),
+        ("z_near", C.c_float), ("z_far", C.c_float), ("eps", C.c_float),
+        ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
+        ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
+        ("scale_global", C.c_float), ("bg", C.c_float * 3),
+    ]
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with the Makefile next to this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-B" if force else "-s", "libd3gs_oracle.so"], check=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_expf.restype = C.c_float
+        _lib.orc_expf.argtypes = [C.c_float]
+        _lib.orc_logf.restype = C.c_float
+        _lib.orc_logf.argtypes = [C.c_float]
+        _lib.orc_scan.restype = C.c_int64
+        _lib.orc_higher_msb.restype = C.c_int32
+        _lib.orc_higher_msb.argtypes = [C.c_uint32]
+        _lib.orc_num_threads.restype = C.c_int32
+    return _lib
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_degree, sh_stride,
+                has_sh_base=False, filter_algo=FILTER_NONE, training=True, near=0.2, far=10000.0, eps=1e-6,
+                radii_eigen_eps=0.1, clamp_factor=1.3, std_sigma=3.0, lowpass=0.3, alpha_eps=1.0 / 255.0,
+                transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0)) -> OracleParams:
+    """cam2world_T is the 4x3 matrix ``to_world[:3].T`` (render.py:205-206)."""
+    P = OracleParams()
+    P.n, P.width, P.height = int(n), int(width), int(height)
+    P.tiles_x, P.tiles_y = (width + 15) // 16, (height + 15) // 16
+    P.sh_degree, P.sh_stride, P.has_sh_base = int(sh_degree), int(sh_stride), int(bool(has_sh_base))
+    P.filter_algo, P.training = int(filter_algo), int(bool(training))
+    f = np.asarray(focal_xy, np.float32)
+    pp = np.asarray(principal_point, np.float32)
+    P.fx, P.fy, P.cx, P.cy = float(f[0]), float(f[1]), float(pp[0]), float(pp[1])
+    # tan_fov = 0.5 * resolution / focal in float32 (render.py:358, 3274)
+    tf = np.float32(0.5) * np.array([width, height], np.float32) / f
+    P.tan_fovx, P.tan_fovy = float(tf[0]), float(tf[1])
+    c2w = np.ascontiguousarray(np.asarray(cam2world_T, np.float32).reshape(4, 3))
+    P.w2c[:] = [float(v) for v in c2w[:3].reshape(-1)]
+    P.cam_center[:] = [float(v) for v in c2w[3]]
+    P.z_near, P.z_far, P.eps = float(near), float(far), float(eps)
+    P.radii_eigen_eps, P.clamp_factor, P.std_sigma = float(radii_eigen_eps), float(clamp_factor), float(std_sigma)
+    P.lowpass, P.alpha_eps, P.transmittance_eps = float(lowpass), float(alpha_eps), float(transmittance_eps)
+    P.scale_global = float(scale_global)
+    P.bg[:] = [float(v) for v in bg]
+    return P
+
+
+def expf(x):
+    L = lib()
+    return np.array([L.orc_expf(float(v)) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
+def logf(x):
+    L = lib()
+    return np.array([L.orc_logf(float(v)) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
+def higher_msb(n: int) -> int:
+    return int(lib().orc_higher_msb(int(n)))
+
+
+def set_num_threads(n: int):
+    lib().orc_set_num_threads(C.c_int32(int(n)))
+
+
+def num_threads() -> int:
+    return int(lib().orc_num_threads())
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, np.float32)
+
+
+def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None):
+    n = P.n
+    out = dict(
+        depths=np.empty(n, np.float32), radii=np.empty(n, np.int32), uvs=np.empty((n, 2), np.float32),
+        conic_opacity=np.empty((n, 4), np.float32), tiles_touched=np.empty(n, np.int32),
+        rgb_gaussian=np.empty((n, 3), np.float32), cov2d_vecs=np.empty((n, 3), np.float32),
+        sh_to_rgb_ne_0=np.empty(n, np.uint8))
+    xyz, quat, scale, opacity, sh, sh_base = map(_f32, (xyz, quat, scale, opacity, sh, sh_base))
+    rc = lib().orc_preprocess_fwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(sh_base),
+                                  _p(out["depths"]), _p(out["radii"]), _p(out["uvs"]), _p(out["conic_opacity"]),
+                                  _p(out["tiles_touched"]), _p(out["rgb_gaussian"]), _p(out["cov2d_vecs"]),
+                                  _p(out["sh_to_rgb_ne_0"]))
+    if rc != 0:
+        raise ValueError("oracle: unsupported early_filter_algo")
+    return out
+
+
+def scan(tiles_touched):
+    t = np.ascontiguousarray(tiles_touched, np.int32).copy()
+    total = lib().orc_scan(_p(t), C.c_int32(t.shape[0]))
+    return t, int(total)
+
+
+def make_keys(P, radii, uvs, conic_opacity, depths, offsets, m):
+    keys = np.zeros(m, np.uint64)
+    vals = np.zeros(m, np.int32)
+    lib().orc_make_keys(C.byref(P), _p(radii), _p(uvs), _p(conic_opacity), _p(depths), _p(offsets), _p(keys), _p(vals))
+    return keys, vals
+
+
+def sort_pairs(keys, vals, begin_bit, end_bit):
+    keys = np.ascontiguousarray(keys, np.uint64)
+    vals = np.ascontiguousarray(vals, np.int32)
+    ko, vo = np.empty_like(keys), np.empty_like(vals)
+    lib().orc_sort_pairs(_p(keys), _p(vals), _p(ko), _p(vo), C.c_int64(keys.shape[0]), C.c_int32(begin_bit),
+                         C.c_int32(end_bit))
+    return ko, vo
+
+
+def tile_ranges(keys_sorted, num_tiles):
+    r = np.zeros((num_tiles, 2), np.int32)
+    lib().orc_tile_ranges(_p(keys_sorted), C.c_int64(keys_sorted.shape[0]), _p(r), C.c_int32(num_tiles))
+    return r
+
+
+def blend_fwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb):
+    H, W = P.height, P.width
+    color = np.zeros((H, W, 3), np.float32)
+    T = np.zeros((H, W), np.float32)
+    nc = np.zeros((H, W), np.int32)
+    lib().orc_blend_fwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(color), _p(T),
+                        _p(nc))
+    return color, T, nc
+
+
+def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib, color, drgb, dT):
+    n = P.n
+    duv = np.zeros((n, 2), np.float64)
+    dconic = np.zeros((n, 3), np.float64)
+    dop = np.zeros(n, np.float64)
+    dcol = np.zeros((n, 3), np.float64)
+    drgb, dT = _f32(drgb), _f32(dT)
+    lib().orc_blend_bwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(final_T),
+                        _p(n_contrib), _p(color), _p(drgb), _p(dT), _p(duv), _p(dconic), _p(dop), _p(dcol))
+    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol)
+
+
+def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dconic, dopacity, dcolor, dz=None,
+                   sh_mask_compat=False):
+    n, K = P.n, P.sh_stride
+    xyz, quat, scale, opacity, sh, cov2d, duv, dconic, dopacity, dcolor, dz = map(
+        _f32, (xyz, quat, scale, opacity, sh, cov2d, duv, dconic, dopacity, dcolor, dz))
+    out = dict(dxyz=np.empty((n, 3), np.float32), dquat=np.empty((n, 4), np.float32),
+               dscale=np.empty((n, 3), np.float32), dopacity=np.empty(n, np.float32),
+               dsh=np.empty((n, K, 3), np.float32),
+               dsh_base=np.empty((n, 3), np.float32) if P.has_sh_base else None)
+    lib().orc_preprocess_bwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(radii), _p(cov2d),
+                             _p(ne0), _p(duv), _p(dconic), _p(dopacity), _p(dcolor), _p(dz),
+                             C.c_int32(int(sh_mask_compat)), _p(out["dxyz"]), _p(out["dquat"]), _p(out["dscale"]),
+                             _p(out["dopacity"]), _p(out["dsh"]), _p(out["dsh_base"]))
+    return out
+
+
+def forward(P, xyz, quat, scale, opacity, sh, sh_base=None):
+    """Whole forward: K1 .. K6.  Returns every intermediate the op context holds."""
+    pre = preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base)
+    offsets, m = scan(pre["tiles_touched"])
+    num_tiles = P.tiles_x * P.tiles_y
+    keys, vals = make_keys(P, pre["radii"], pre["uvs"], pre["conic_opacity"], pre["depths"], offsets, m)
+    end_bit = 32 + higher_msb(num_tiles)
+    ks, vs = sort_pairs(keys, vals, 0, end_bit)
+    ranges = tile_ranges(ks, num_tiles)
+    color, T, nc = blend_fwd(P, ranges, vs, pre["uvs"], pre["conic_opacity"], pre["rgb_gaussian"])
+    out = dict(pre)
+    out.update(offsets=offsets, num_rendered=m, keys=keys, vals=vals, keys_sorted=ks, gaussian_idx_sorted=vs,
+               workload_ranges=ranges, color=color, T=T, n_contrib=nc, end_bit=end_bit)
+    return out
+
+
+def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False):
+    """Whole backward: K7 + K9 from the dict ``forward`` returned."""
+    g = blend_bwd(P, fwd["workload_ranges"], fwd["gaussian_idx_sorted"], fwd["uvs"], fwd["conic_opacity"],
+                  fwd["rgb_gaussian"], fwd["T"], fwd["n_contrib"], fwd["color"], drgb, dT)
+    sh_in = sh
+    pb = preprocess_bwd(P, xyz, quat, scale, opacity, sh_in, fwd["radii"], fwd["cov2d_vecs"], fwd["sh_to_rgb_ne_0"],
+                        g["duv"].astype(np.float32), g["dconic"].astype(np.float32),
+                        g["dopacity"].astype(np.float32), g["dcolor"].astype(np.float32),
+                        sh_mask_compat=sh_mask_compat)
+    return g, pb

@@ -1,0 +1,214 @@
+"""GPU parity: every stage of the HIP path against the CPU oracle on identical
+seeded inputs, called through the C ABI (via the operator, which is a thin
+ctypes caller).  Integer / index outputs must be bit-exact; the image is
+bit-exact by construction (same operation sequence) and asserted <= 1e-5 abs;
+gradients within 1e-4 relative (atomic / wavefront reduction order)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import gen_scene, grad_close, op_config, oracle_forward, torch_model
+
+pytestmark = pytest.mark.gpu
+
+NONE, AABB, OBB, DFVT = 0, 1, 3, 4
+
+CASES = [
+    # (config id, n override, (w,h) override, filter)
+    (0, None, None, NONE),
+    (0, None, None, AABB),
+    (0, None, None, OBB),
+    (0, None, None, DFVT),
+    (1, None, None, AABB),
+    (1, 20000, (250, 190), NONE),     # ragged image: W,H not multiples of 16
+    (2, 100000, (640, 360), AABB),
+    (3, 100000, (480, 270), OBB),
+    (4, 30000, (960, 540), AABB),
+]
+
+
+def _run_gpu(scene, filt, training=True):
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    op = GaussianSplatOp(op_config(scene, filt))
+    model = torch_model(scene)
+    out, ctx = op.forward(model, scene.camera(), training=training)
+    torch.cuda.synchronize()
+    return op, model, out, ctx
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt", CASES)
+def test_forward_stages_bit_exact(oracle, cfg_id, n, wh, filt):
+    import torch
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    print(f"case cfg={cfg_id} n={scene.n} wh={scene.width}x{scene.height} filter={filt}", flush=True)
+    P, ref = oracle_forward(oracle, scene, filt)
+    op, model, out, ctx = _run_gpu(scene, filt)
+    assert ctx is not None
+    cpu = lambda t: t.detach().cpu().numpy()
+    # K1
+    assert np.array_equal(cpu(ctx.radii), ref["radii"])
+    assert np.array_equal(cpu(ctx.depths).view(np.uint32), ref["depths"].view(np.uint32))
+    assert np.array_equal(cpu(ctx.uvs).view(np.uint32), ref["uvs"].view(np.uint32))
+    assert np.array_equal(cpu(ctx.conic_opacity).view(np.uint32), ref["conic_opacity"].view(np.uint32))
+    assert np.array_equal(cpu(ctx.rgb_gaussian).view(np.uint32), ref["rgb_gaussian"].view(np.uint32))
+    assert np.array_equal(cpu(ctx.cov2d_vecs).view(np.uint32), ref["cov2d_vecs"].view(np.uint32))
+    assert np.array_equal(cpu(ctx.sh_to_rgb_ne_0), ref["sh_to_rgb_ne_0"])
+    # K2-K5
+    assert op.last_num_rendered == ref["num_rendered"]
+    assert np.array_equal(cpu(op._last_keys_sorted).view(np.uint64), ref["keys_sorted"])
+    assert np.array_equal(cpu(ctx.gaussian_idx_sorted), ref["gaussian_idx_sorted"])
+    assert np.array_equal(cpu(ctx.workload_ranges), ref["workload_ranges"])
+    # K6
+    assert np.array_equal(cpu(out.n_contrib)[0], ref["n_contrib"])
+    assert np.abs(cpu(out.T)[0] - ref["T"]).max() <= 1e-5
+    assert np.abs(cpu(out.color)[0] - ref["color"]).max() <= 1e-5
+    # same operation order on both sides: expected to be identical bits
+    assert np.array_equal(cpu(out.color)[0].view(np.uint32), ref["color"].view(np.uint32))
+    assert np.array_equal(cpu(out.T)[0].view(np.uint32), ref["T"].view(np.uint32))
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt", [(0, None, None, AABB), (1, None, None, AABB),
+                                              (2, 100000, (640, 360), AABB), (4, 30000, (960, 540), NONE)])
+def test_inference_path(oracle, cfg_id, n, wh, filt):
+    scene = gen_scene(cfg_id, n=n, wh=wh, with_grad=False)
+    bg = (0.2, 0.5, 0.7)
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    P, ref = oracle_forward(oracle, scene, filt, training=False, bg=bg, scale_global=0.8)
+    op = GaussianSplatOp(op_config(scene, filt, bg_color=np.array(bg, np.float32), scale_global=0.8))
+    out, ctx = op.forward(torch_model(scene), scene.camera(), training=False)
+    assert ctx is None
+    assert np.array_equal(out.color.cpu().numpy()[0].view(np.uint32), ref["color"].view(np.uint32))
+    assert np.array_equal(out.radii.cpu().numpy(), ref["radii"])
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt", [(0, None, None, AABB), (0, None, None, NONE), (1, None, None, AABB),
+                                              (1, 20000, (250, 190), OBB), (2, 100000, (640, 360), AABB),
+                                              (4, 30000, (960, 540), AABB)])
+def test_backward_parity(oracle, cfg_id, n, wh, filt):
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    print(f"case cfg={cfg_id} n={scene.n} wh={scene.width}x{scene.height} filter={filt}", flush=True)
+    rng = np.random.default_rng(7)
+    dT = rng.standard_normal(scene.dT.shape).astype(np.float32)
+    P, ref = oracle_forward(oracle, scene, filt)
+    g_ref, pb_ref = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                    scene.color_sh, scene.drgb[0], dT[0])
+    op, model, out, ctx = _run_gpu(scene, filt)
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(dT).cuda())
+    gm, duv, _ = op.backward(model, scene.camera(), ctx, out, grads, return_uv_grad=True)
+    torch.cuda.synchronize()
+    g = op.last_raster_grads
+    cpu = lambda t: t.detach().cpu().numpy()
+    # blend backward (dopacity was finished in place by preprocess backward, so compare it via the model grad)
+    for name, got in (("duv", g.duv), ("dconic", g.dconic), ("dcolor", g.dcolor)):
+        ok, worst, nbad = grad_close(cpu(got), g_ref[name])
+        assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+    assert duv.shape == (1, scene.n, 2)
+    # preprocess backward
+    for name, got in (("dxyz", gm.xyz), ("dquat", gm.quaternion_xyzw), ("dscale", gm.scale),
+                      ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
+        ok, worst, nbad = grad_close(cpu(got), pb_ref[name])
+        assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+
+
+def test_autograd_entry_point(oracle):
+    """rasterize_gaussians + loss.backward() gives the same gradients as op.backward."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp, rasterize_gaussians
+    scene = gen_scene(0)
+    op = GaussianSplatOp(op_config(scene, AABB))
+    model = torch_model(scene)
+    model.act_applied = False
+    model.set_requires_grad(True)
+    holder = torch.zeros((1, scene.n, 2), device="cuda", requires_grad=True)
+    out = rasterize_gaussians(model, scene.camera(), op, training=True, uv_grad_holder=holder)
+    drgb = torch.from_numpy(scene.drgb).cuda()
+    (out.color * drgb).sum().backward()
+    P, ref = oracle_forward(oracle, scene, AABB)
+    g_ref, pb_ref = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                    scene.color_sh, scene.drgb[0], scene.dT[0])
+    for name, t in (("dxyz", model.xyz), ("dscale", model.scale), ("dquat", model.quaternion_xyzw),
+                    ("dopacity", model.opacity), ("dsh", model.color_sh)):
+        ok, worst, nbad = grad_close(t.grad.cpu().numpy(), pb_ref[name])
+        assert ok, f"{name}: {nbad} bad (worst {worst:.2f}x)"
+    ok, worst, nbad = grad_close(holder.grad.cpu().numpy()[0], g_ref["duv"])
+    assert ok
+
+
+def test_empty_scene_returns_background():
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(0, n=64, with_grad=False)
+    scene.xyz[:, 2] = -5.0  # everything behind the camera
+    op = GaussianSplatOp(op_config(scene, AABB))
+    out, ctx = op.forward(torch_model(scene), scene.camera(), training=True)
+    assert ctx is None and op.last_num_rendered == 0
+    assert float(out.T.min()) == 1.0 and float(out.color.abs().max()) == 0.0
+    assert int(out.radii.abs().max()) == 0
+
+
+@pytest.mark.parametrize("m,begin,end", [(1, 0, 45), (255, 0, 8), (4096, 0, 45), (4097, 3, 41), (100003, 0, 64),
+                                         (1 << 20, 0, 47), (300000, 32, 45)])
+def test_sort_pairs_c_abi(oracle, m, begin, end):
+    """d3gs_sort_pairs against numpy's stable argsort on the masked key bits; many duplicate keys."""
+    import torch
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    rng = np.random.default_rng(m)
+    keys = rng.integers(0, 1 << 62, size=m, dtype=np.uint64)
+    keys[rng.random(m) < 0.5] &= np.uint64(0x00001FFF000000FF)  # heavy duplication in the sorted bits
+    vals = np.arange(m, dtype=np.int32)
+    width = end - begin
+    masked = (keys >> np.uint64(begin)) & np.uint64((1 << width) - 1 if width < 64 else 0xFFFFFFFFFFFFFFFF)
+    order = np.argsort(masked, kind="stable")
+    ka = torch.from_numpy(keys.view(np.int64)).cuda()
+    va = torch.from_numpy(vals).cuda()
+    kb, vb = torch.empty_like(ka), torch.empty_like(va)
+    nbytes = C.c_size_t(0)
+    _capi.check(L.d3gs_sort_workspace_bytes(m, begin, end, C.byref(nbytes)), "ws")
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device="cuda")
+    in_b = C.c_int(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _capi.check(L.d3gs_sort_pairs(_capi.ptr(ka), _capi.ptr(kb), _capi.ptr(va), _capi.ptr(vb), _capi.ptr(ws),
+                                  nbytes.value, m, begin, end, C.byref(in_b), stream), "sort")
+    torch.cuda.synchronize()
+    ks, vs = (kb, vb) if in_b.value else (ka, va)
+    assert np.array_equal(vs.cpu().numpy(), vals[order])
+    assert np.array_equal(ks.cpu().numpy().view(np.uint64), keys[order])
+    ko, vo = oracle.sort_pairs(keys, vals, begin, end)
+    assert np.array_equal(vo, vals[order])
+
+
+@pytest.mark.parametrize("n", [1, 63, 2048, 2049, 1_000_003])
+def test_scan_c_abi(n):
+    import torch
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    rng = np.random.default_rng(n)
+    x = rng.integers(0, 50, size=n, dtype=np.int32)
+    t = torch.from_numpy(x).cuda()
+    nbytes = C.c_size_t(0)
+    _capi.check(L.d3gs_scan_workspace_bytes(n, C.byref(nbytes)), "ws")
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device="cuda")
+    total = torch.zeros(1, dtype=torch.int64, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _capi.check(L.d3gs_scan_tiles(_capi.ptr(t), n, _capi.ptr(ws), nbytes.value, _capi.ptr(total), stream), "scan")
+    assert np.array_equal(t.cpu().numpy(), np.cumsum(x, dtype=np.int64).astype(np.int32))
+    assert int(total.item()) == int(x.sum())
+
+
+def test_error_codes_without_compute():
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    P = _capi.Params()
+    P.n, P.width, P.height, P.tiles_x, P.tiles_y = 4, 32, 32, 3, 2   # wrong tile counts
+    rc = L.d3gs_blend_fwd(C.byref(P), None, None, None, None, None, None, None, None, None)
+    assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
+    P.tiles_x = 2
+    P.filter_algo = 2
+    rc = L.d3gs_blend_fwd(C.byref(P), None, None, None, None, None, None, None, None, None)
+    assert rc == -2
