@@ -1,0 +1,68 @@
+"""CPU-side checks of the C-ABI shared library: it loads, exports every symbol the
+header declares, and validates arguments without touching a GPU."""
+import ctypes as C
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "d3gs_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(d3gs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    from d3gs_research_amd import _capi
+    lib = C.CDLL(_capi.LIB_PATH)
+    declared = _declared_symbols()
+    assert len(declared) >= 13
+    for sym in declared:
+        assert hasattr(lib, sym), f"{sym} declared in d3gs_hip.h but not exported"
+    assert sorted(_capi.EXPORTED_SYMBOLS) == declared, "ctypes binding and header disagree"
+
+
+def test_params_struct_matches_header_layout():
+    from d3gs_research_amd import _capi
+    # 10 int32 + 6 float + 9 + 3 + 10 float + 3 float
+    assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3)
+
+
+def test_abi_version_and_msb():
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    assert L.d3gs_abi_version() == 1
+    # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
+    assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
+
+
+def test_error_codes_without_compute():
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    P = _capi.Params()
+    P.n, P.width, P.height, P.tiles_x, P.tiles_y, P.sh_stride = 4, 32, 32, 3, 2, 1   # wrong tile counts
+    nul = [None] * 9
+    rc = L.d3gs_blend_fwd(C.byref(P), *nul)
+    assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
+    P.tiles_x = 2
+    P.filter_algo = 2   # ELLIPSE: declared, not implemented
+    assert L.d3gs_blend_fwd(C.byref(P), *nul) == -2
+    P.filter_algo = 1
+    assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"NULL" in L.d3gs_last_error_string()
+    P.sh_degree, P.sh_stride = 3, 4
+    assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"sh_stride" in L.d3gs_last_error_string()
+    n = C.c_size_t(0)
+    assert L.d3gs_sort_workspace_bytes(1000, 0, 65, C.byref(n)) == -1
+    assert L.d3gs_sort_workspace_bytes(1000, 0, 45, C.byref(n)) == 0 and n.value > 0
+    in_b = C.c_int(7)
+    assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 0, 0, 45, C.byref(in_b), None) == 0 and in_b.value == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    import pytest
+    from d3gs_research_amd import _capi
+    monkeypatch.setattr(_capi, "_lib", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _capi.lib()

