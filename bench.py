@@ -1,0 +1,151 @@
+#!/usr/bin/env python3
+"""Benchmark of the rasterize forward+backward path on one MI355X.
+
+One "step" = one view: preprocess -> scan -> key expansion -> radix sort -> tile
+ranges -> blend forward, then blend backward -> preprocess backward, with every
+input already resident in HBM.  Prints ONE JSON line (see the driver contract):
+whole-job ms/view, a roofline object for the dominant kernel and the CPU oracle
+timed on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
+
+# algorithmic HBM bytes per stage: N gaussians, M (tile, gaussian) pairs, P pixels, T tiles
+STAGE_BYTES = {
+    "preprocess": lambda N, M, P, T, passes: 297 * N,
+    "scan": lambda N, M, P, T, passes: 8 * N,
+    "make_keys": lambda N, M, P, T, passes: 36 * N + 12 * M,
+    "sort": lambda N, M, P, T, passes: (8 + 24 * passes) * M,
+    "tile_ranges": lambda N, M, P, T, passes: 8 * M + 8 * T,
+    "blend_fwd": lambda N, M, P, T, passes: 40 * M + 20 * P,
+    "blend_bwd": lambda N, M, P, T, passes: 76 * M + 36 * P,
+    "preprocess_bwd": lambda N, M, P, T, passes: (236 + 50 + 236) * N,
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="BASELINE config id (2 = headline 1M @1080p)")
+    ap.add_argument("--filter", type=str, default="OBB_DFVT", help="early_filter_algo: NONE, AABB, OBB, OBB_DFVT")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="only run a plain 256 MiB -> 256 MiB elementwise copy 5 times (reference reading for "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the rasterize path is single-device); --gpus must be 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    if args.pmc_calibrate:
+        x = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")
+        y = torch.empty_like(x)
+        for _ in range(5):
+            torch.mul(x, 1.0, out=y)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch.mul(x, 1.0, out=y)", "read_bytes": x.numel() * 4,
+                          "write_bytes": y.numel() * 4, "launches": 5}))
+        return
+    from helpers import op_config, oracle_params, torch_model
+    from d3gs_research_amd.config_def import EarlyFilterAlgo
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    from d3gs_research_amd.synthetic import gen_scene
+
+    filt = EarlyFilterAlgo[args.filter]
+    scene = gen_scene(args.config)
+    cam = scene.camera()
+    op = GaussianSplatOp(op_config(scene, filt))
+    model = torch_model(scene, "cuda:0")
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+
+    def step():
+        out, ctx = op.forward(model, cam, training=True)
+        gm, duv, _ = op.backward(model, cam, ctx, out, grads, return_uv_grad=True)
+        return out, gm
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    op.stage_events = {}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    N, P_px, T_tiles = scene.n, scene.width * scene.height, ((scene.width + 15) // 16) * ((scene.height + 15) // 16)
+    M = op.last_num_rendered
+    end_bit = 32 + int(T_tiles).bit_length()
+    passes = (end_bit + 7) // 8
+    stages = {}
+    for name, evs in op.stage_events.items():
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        avg = sum(ts) / len(ts)
+        nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes)
+        stages[name] = {"ms": round(avg, 4), "ms_p50": round(ts[len(ts) // 2], 4), "alg_bytes": int(nbytes),
+                        "gbs": round(nbytes / (avg * 1e-3) / 1e9, 1)}
+    op.stage_events = None
+    gpu_sum = sum(s["ms"] for s in stages.values())
+    dom = max(stages, key=lambda k: stages[k]["ms"])
+    achieved = stages[dom]["gbs"]
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": None,
+                "pair_evals_per_s": round(256.0 * M / (stages[dom]["ms"] * 1e-3), 1)}
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle import d3gs_oracle as O
+        O.build()
+        cs = scene if args.cpu_n in (0, scene.n) else gen_scene(args.config, n=args.cpu_n)
+        Pc = oracle_params(O, cs, int(filt))
+        c0 = time.perf_counter()
+        ref = O.forward(Pc, cs.xyz, cs.quaternion_xyzw, cs.scale, cs.opacity, cs.color_sh)
+        c1 = time.perf_counter()
+        O.backward(Pc, ref, cs.xyz, cs.quaternion_xyzw, cs.scale, cs.opacity, cs.color_sh, cs.drgb[0], cs.dT[0])
+        c2 = time.perf_counter()
+        cpu_baseline = {"value": round((c2 - c0) * 1e3, 1), "unit": "ms/view", "cores": O.num_threads(),
+                        "kind": "port", "fwd_ms": round((c1 - c0) * 1e3, 1), "bwd_ms": round((c2 - c1) * 1e3, 1),
+                        "sample": f"1 view of config {args.config} with {cs.n} gaussians "
+                                  f"({'full workload' if cs.n == scene.n else 'reduced gaussian count'}), "
+                                  f"M={ref['num_rendered']}, OpenMP over {O.num_threads()} threads"}
+
+    ranges_len = None
+    line = {
+        "metric": "fwd+bwd raster ms/view, 1M Gaussians @1080p, 1 MI355X" if args.config == 2
+        else f"fwd+bwd raster ms/view, config {args.config}",
+        "value": round(ms_per_step, 4), "unit": "ms/view", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"config {args.config}: {scene.name}", "gaussians": N, "sh_degree": scene.sh_degree,
+                   "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name, "pairs_M": int(M),
+                   "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles},
+        "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "gpu_stage_sum_ms": round(gpu_sum, 4),
+        "stages": stages,
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
