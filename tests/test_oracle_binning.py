@@ -1,0 +1,120 @@
+"""Pins tile filters, scan, key expansion, sort and tile ranges of the oracle:
+brute force over pixels for the filters' losslessness, numpy cumsum / stable
+argsort for the integer stages, and structural invariants of the result."""
+import numpy as np
+import pytest
+
+from f64_reference import preprocess_f64
+from helpers import gen_scene, oracle_forward
+
+NONE, AABB, OBB, DFVT = 0, 1, 3, 4
+
+
+def _tile_sets(ref, n):
+    tiles = (ref["keys"] >> np.uint64(32)).astype(np.int64)
+    sets = [set() for _ in range(n)]
+    for t, g in zip(tiles.tolist(), ref["vals"].tolist()):
+        sets[g].add(t)
+    return sets
+
+
+@pytest.mark.parametrize("make", [lambda: gen_scene(0, n=1500), lambda: gen_scene(4, n=3000, wh=(480, 270))])
+def test_filters_are_lossless_and_nested(oracle, make):
+    """config_def.py:136-141: AABB / OBB only drop tiles in which no pixel reaches alpha >= 1/255;
+    OBB tiles are a subset of AABB tiles, which are a subset of the 3-sigma rect (NONE)."""
+    scene = make()
+    refs = {f: oracle_forward(oracle, scene, f)[1] for f in (NONE, AABB, OBB, DFVT)}
+    sets = {f: _tile_sets(refs[f], scene.n) for f in refs}
+    pre = refs[NONE]
+    tiles_x = (scene.width + 15) // 16
+    uv = pre["uvs"].astype(np.float64)
+    co = pre["conic_opacity"].astype(np.float64)
+    dropped_checked = 0
+    for g in range(scene.n):
+        s_none, s_aabb, s_obb = sets[NONE][g], sets[AABB][g], sets[OBB][g]
+        assert s_obb <= s_aabb <= s_none
+        assert sets[DFVT][g] == s_obb                      # the author's invariant, render.py:1051-1072
+        for t in s_none - s_obb:
+            tx, ty = t % tiles_x, t // tiles_x
+            xs = np.arange(tx * 16, min(tx * 16 + 16, scene.width), dtype=np.float64)
+            ys = np.arange(ty * 16, min(ty * 16 + 16, scene.height), dtype=np.float64)
+            dx = uv[g, 0] - xs[None, :]
+            dy = uv[g, 1] - ys[:, None]
+            power = -0.5 * (co[g, 0] * dx * dx + co[g, 2] * dy * dy) - co[g, 1] * dx * dy
+            alpha = co[g, 3] * np.exp(power)
+            assert alpha.max() < (1 / 255.0) * (1 + 1e-4), (g, t, alpha.max())
+            dropped_checked += 1
+    assert dropped_checked > 100          # the test did examine dropped tiles
+    # a lossless filter cannot change the image
+    for f in (AABB, OBB, DFVT):
+        assert np.array_equal(refs[f]["color"], refs[NONE]["color"])
+        assert np.array_equal(refs[f]["T"], refs[NONE]["T"])
+
+
+def test_none_filter_is_the_three_sigma_rect(oracle):
+    """render.py:472-473: rect = [int((uv - r)/16), int((uv + r + 15)/16)) clamped to the grid."""
+    scene = gen_scene(0)
+    ref = oracle_forward(oracle, scene, NONE)[1]
+    sets = _tile_sets(ref, scene.n)
+    uv, r = ref["uvs"].astype(np.float64), ref["radii"].astype(np.float64)
+    tiles = 8
+    for g in np.flatnonzero(ref["radii"] > 0)[:800]:
+        lo = np.clip(np.trunc((uv[g] - r[g]) / 16), 0, tiles).astype(int)
+        hi = np.clip(np.trunc((uv[g] + r[g] + 15) / 16), 0, tiles).astype(int)
+        want = {y * tiles + x for y in range(lo[1], hi[1]) for x in range(lo[0], hi[0])}
+        assert sets[g] == want
+        assert len(want) == (ref["tiles_touched"][g])
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt", [(0, None, None, NONE), (1, 30000, None, AABB), (2, 50000, (640, 360), OBB)])
+def test_scan_keys_sort_ranges(oracle, cfg_id, n, wh, filt):
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    ref = oracle_forward(oracle, scene, filt)[1]
+    tt = ref["tiles_touched"]
+    m = ref["num_rendered"]
+    # scan == numpy cumsum
+    assert np.array_equal(ref["offsets"], np.cumsum(tt, dtype=np.int64).astype(np.int32)) and m == int(tt.sum())
+    # keys: emitted at [offset[i-1], offset[i]) with value i, low word = float bits of the depth,
+    # high word = tile id in row-major order (render.py:773, 809, 830-833)
+    starts = np.concatenate([[0], ref["offsets"][:-1]])
+    owner = np.repeat(np.arange(scene.n, dtype=np.int32), tt)
+    assert np.array_equal(ref["vals"], owner)
+    low = (ref["keys"] & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    assert np.array_equal(low, ref["depths"].view(np.uint32)[owner])
+    tile = (ref["keys"] >> np.uint64(32)).astype(np.int64)
+    num_tiles = ((scene.width + 15) // 16) * ((scene.height + 15) // 16)
+    assert tile.min() >= 0 and tile.max() < num_tiles
+    first = np.ones(m, bool)
+    first[1:] = owner[1:] != owner[:-1]
+    assert (np.diff(tile)[~first[1:]] > 0).all()        # row-major ascending within one gaussian
+    # sort == numpy stable argsort on the full key (bits above end_bit are zero)
+    assert ref["end_bit"] == 32 + int(num_tiles).bit_length()
+    order = np.argsort(ref["keys"], kind="stable")
+    assert np.array_equal(ref["keys_sorted"], ref["keys"][order])
+    assert np.array_equal(ref["gaussian_idx_sorted"], ref["vals"][order])
+    # ranges partition [0, m); untouched tiles stay [0, 0)
+    r = ref["workload_ranges"]
+    lens = r[:, 1] - r[:, 0]
+    assert lens.sum() == m and (lens >= 0).all()
+    counts = np.bincount(tile, minlength=num_tiles)
+    assert np.array_equal(lens, counts)
+    assert (r[counts == 0] == 0).all()
+    st = tile[order]
+    for t in np.flatnonzero(counts)[:200]:
+        seg = slice(r[t, 0], r[t, 1])
+        assert (st[seg] == t).all()
+        d = ref["depths"][ref["gaussian_idx_sorted"][seg]]
+        assert (np.diff(d) >= 0).all()                    # front to back
+        ties = np.diff(d) == 0
+        assert (np.diff(ref["gaussian_idx_sorted"][seg])[ties] > 0).all()   # stable: ties keep index order
+
+
+def test_sort_bit_range_and_stability(oracle):
+    rng = np.random.default_rng(5)
+    keys = rng.integers(0, 1 << 40, size=50000, dtype=np.uint64)
+    vals = np.arange(keys.size, dtype=np.int32)
+    for b, e in ((0, 40), (8, 24), (3, 17), (32, 40), (0, 1)):
+        ko, vo = oracle.sort_pairs(keys, vals, b, e)
+        masked = (keys >> np.uint64(b)) & np.uint64((1 << (e - b)) - 1)
+        order = np.argsort(masked, kind="stable")
+        assert np.array_equal(vo, vals[order]) and np.array_equal(ko, keys[order])
