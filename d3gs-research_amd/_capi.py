@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class Params(C.Structure):
@@ -46,9 +46,9 @@ _SIGNATURES = {
     "d3gs_sort_workspace_bytes": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
     "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
                                   C.POINTER(C.c_int), _VP]),
-    "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP]),
-    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 8 + [_VP]),
-    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 14 + [_VP]),
+    "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
+    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [_VP]),
+    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
     "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 13 + [C.c_int32] + [_VP] * 6 + [_VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -228,6 +228,40 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const uint64_t* __r
     if (i == m - 1) ranges[2 * t + 1] = (int32_t)m;
 }
 
+// Tile ids ordered by descending list length (counting sort over 256 length buckets, one
+// workgroup).  Order inside a bucket is arbitrary: the result only steers scheduling.
+__global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t* __restrict__ ranges, int num_tiles,
+                                                          int32_t* __restrict__ order) {
+    __shared__ int s_max;
+    __shared__ int s_bin[256];
+    if (threadIdx.x == 0) s_max = 0;
+    if (threadIdx.x < 256) s_bin[threadIdx.x] = 0;
+    __syncthreads();
+    int mx = 0;
+    for (int t = threadIdx.x; t < num_tiles; t += 1024) mx = max(mx, ranges[2 * t + 1] - ranges[2 * t]);
+    atomicMax(&s_max, mx);
+    __syncthreads();
+    const long long denom = (long long)s_max + 1;
+    for (int t = threadIdx.x; t < num_tiles; t += 1024) {
+        const int len = ranges[2 * t + 1] - ranges[2 * t];
+        atomicAdd(&s_bin[255 - (int)((long long)len * 256 / denom)], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int b = 0; b < 256; ++b) {
+            const int c = s_bin[b];
+            s_bin[b] = acc;
+            acc += c;
+        }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < num_tiles; t += 1024) {
+        const int len = ranges[2 * t + 1] - ranges[2 * t];
+        order[atomicAdd(&s_bin[255 - (int)((long long)len * 256 / denom)], 1)] = t;
+    }
+}
+
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 static inline int scan_chunks(long long n) { return (int)((n + kScanChunk - 1) / kScanChunk); }
 
@@ -358,12 +392,18 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
 }
 
 extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
-                                d3gs_stream_t stream) {
+                                int32_t* tile_order, d3gs_stream_t stream) {
     if (m < 0 || num_tiles < 0) { set_error("d3gs_tile_ranges: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
-    if (m == 0) return D3GS_OK;
-    if (!keys_sorted || !workload_ranges) { set_error("d3gs_tile_ranges: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
-    hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       (hipStream_t)stream, keys_sorted, (long long)m, workload_ranges, (int)num_tiles);
+    if ((m > 0 && !keys_sorted) || (num_tiles > 0 && !workload_ranges)) {
+        set_error("d3gs_tile_ranges: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (m > 0)
+        hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           (hipStream_t)stream, keys_sorted, (long long)m, workload_ranges, (int)num_tiles);
+    if (tile_order && num_tiles > 0)
+        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, workload_ranges,
+                           (int)num_tiles, tile_order);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_tile_ranges: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

@@ -9,9 +9,16 @@
 // Culling that keeps results exact: a gaussian contributes to a pixel only if
 // alpha = min(0.99, o * exp(power)) >= alpha_eps.  Each staged gaussian carries
 // thr = ln(alpha_eps / o) - 1e-3; power < thr implies alpha < alpha_eps with a
-// margin four orders of magnitude above any rounding error, so a wavefront whose
-// 64 pixels all have power < thr skips the gaussian without evaluating exp.
-// Every pixel that passes the coarse test goes through the exact sequence.
+// margin four orders of magnitude above the rounding error of exp and log, so a
+// pixel whose power is below thr never needs exp.  Two levels use it:
+//   1. when a gaussian is staged, the bounding box of its {power >= thr} ellipse
+//      (inflated by a bound on the rounding error of `power` inside this tile) is
+//      tested against each wavefront's 8x8 patch; the four 64-bit ballots become
+//      per-patch bit masks in LDS and a wavefront only visits gaussians whose
+//      bit is set (scalar bit scan, no per-pixel work for the rest);
+//   2. per pixel, `power < thr` skips the exact sequence.
+// Every pixel that passes goes through the exact operation sequence, so the
+// culling never changes a result.
 //
 // Reference: d3sim/algos/d3gs/render.py:1466-1570 (prologue), 1677-1923 (loop),
 // 1924-2019 (gradients), 2020-2210 (reduction + atomics), 2222-2294 (epilogue).
@@ -24,12 +31,12 @@ struct __attribute__((aligned(16))) StagedGaussian {
     float a, b, c, o;       // conic (a, b, c) and opacity
 };
 
-// Tile index for a workgroup.  Consecutive workgroup ids are dealt round-robin
-// to the 8 XCDs, each with its own L2; give every XCD a contiguous band of tiles
-// so neighbouring tiles (which share gaussians) hit the same L2.
-__device__ __forceinline__ int tile_for_block(int bid, int ntiles) {
-    const int per = (ntiles + 7) >> 3;
-    return (bid & 7) * per + (bid >> 3);
+// Tile index for a workgroup.  Tile list lengths are heavily skewed (dense screen regions hold
+// lists 20x the median), so the launch order matters more than L2 locality: with `tile_order`
+// (tiles by descending list length) the long tiles start first and, because consecutive
+// workgroup ids are dealt round-robin to the 8 XCDs, spread evenly over the chip.
+__device__ __forceinline__ int tile_for_block(int bid, const int32_t* __restrict__ tile_order) {
+    return tile_order ? tile_order[bid] : bid;
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -56,8 +63,11 @@ __device__ __forceinline__ int wave_max_i32(int v) {
     return v;
 }
 
-__device__ __forceinline__ void stage_gaussian(const d3gs_params& P, int g, const float* __restrict__ uvs,
-                                               const float* __restrict__ conic_opacity, StagedGaussian* dst) {
+// Stages one gaussian and returns a 4-bit mask: bit q set when the gaussian may reach a pixel of
+// the tile's 8x8 patch q (q & 1 = right half, q >> 1 = lower half).  Conservative by construction.
+__device__ __forceinline__ uint32_t stage_gaussian(const d3gs_params& P, int g, const float* __restrict__ uvs,
+                                                   const float* __restrict__ conic_opacity, float tile_x0,
+                                                   float tile_y0, StagedGaussian* dst) {
     const float2 xy = *reinterpret_cast<const float2*>(uvs + 2 * g);
     const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * g);
     StagedGaussian s;
@@ -70,27 +80,66 @@ __device__ __forceinline__ void stage_gaussian(const d3gs_params& P, int g, cons
     s.c = co.z;
     s.o = co.w;
     *dst = s;
+    // Level set {power >= thr}: a dx^2 + 2 b dx dy + c dy^2 <= R with R = -2 thr.  A pixel of this tile
+    // evaluates `power` with an absolute rounding error below err; widening R by 2 err keeps every pixel
+    // whose computed power can reach thr inside the box.
+    const float X = fabsf(xy.x - (tile_x0 + 7.5f)) + 8.0f, Y = fabsf(xy.y - (tile_y0 + 7.5f)) + 8.0f;
+    const float err = 1.0e-6f * (co.x * X * X + co.z * Y * Y + 2.0f * fabsf(co.y) * X * Y);
+    const float R = -2.0f * s.thr + 2.0f * err + 1.0e-3f;
+    const float D = co.x * co.z - co.y * co.y;
+    // ill-conditioned conic (or not positive definite in float): no box, visit everywhere
+    if (!(D > 1.0e-4f * co.x * co.z) || !(R > 0.0f)) return 0xFu;
+    const float hx = 1.01f * __fsqrt_rn(R * co.z / D) + 0.01f;
+    const float hy = 1.01f * __fsqrt_rn(R * co.x / D) + 0.01f;
+    const bool left = xy.x - hx <= tile_x0 + 7.0f, right = xy.x + hx >= tile_x0 + 8.0f;
+    const bool top = xy.y - hy <= tile_y0 + 7.0f, bottom = xy.y + hy >= tile_y0 + 8.0f;
+    const bool in_x = xy.x + hx >= tile_x0 && xy.x - hx <= tile_x0 + 15.0f;
+    const bool in_y = xy.y + hy >= tile_y0 && xy.y - hy <= tile_y0 + 15.0f;
+    if (!(in_x && in_y)) return 0u;
+    return (uint32_t)(left && top) | ((uint32_t)(right && top) << 1) | ((uint32_t)(left && bottom) << 2) |
+           ((uint32_t)(right && bottom) << 3);
+}
+
+// Publishes the four per-patch ballots of this staging wavefront's 64 gaussians.
+__device__ __forceinline__ void publish_masks(uint32_t bits, int wave, int lane, unsigned long long (*s_mask)[4]) {
+    const unsigned long long m0 = __ballot(bits & 1u), m1 = __ballot(bits & 2u), m2 = __ballot(bits & 4u),
+                             m3 = __ballot(bits & 8u);
+    if (lane == 0) {
+        s_mask[0][wave] = m0;
+        s_mask[1][wave] = m1;
+        s_mask[2][wave] = m2;
+        s_mask[3][wave] = m3;
+    }
+}
+
+__device__ __forceinline__ unsigned long long uniform_u64(unsigned long long v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((unsigned long long)hi << 32) | lo;
 }
 
 __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, const int32_t* __restrict__ ranges,
                                                             const int32_t* __restrict__ idx_sorted,
                                                             const float* __restrict__ uvs,
                                                             const float* __restrict__ conic_opacity,
-                                                            const float* __restrict__ rgb_g, float* __restrict__ color,
-                                                            float* __restrict__ final_T,
+                                                            const float* __restrict__ rgb_g,
+                                                            const int32_t* __restrict__ tile_order,
+                                                            float* __restrict__ color, float* __restrict__ final_T,
                                                             int32_t* __restrict__ n_contrib) {
     __shared__ StagedGaussian s_g[kBlock];
     __shared__ float4 s_rgb[kBlock];
+    __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 
     const int ntiles = P.tiles_x * P.tiles_y;
-    const int tile = tile_for_block(blockIdx.x, ntiles);
-    if (tile >= ntiles) return;
+    const int tile = tile_for_block(blockIdx.x, tile_order);
+    if (tile < 0 || tile >= ntiles) return;
     const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
     const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
     const bool inside = px < P.width && py < P.height;
     const float pxf = (float)px, pyf = (float)py;
+    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
     const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
     const int len = r1 - r0;
@@ -104,37 +153,46 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
     for (int round = 0; round < rounds; ++round) {
         if (__syncthreads_count(done) == kBlock) break;
         const int src = r0 + round * kBlock + tid;
+        uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            stage_gaussian(P, g, uvs, conic_opacity, &s_g[tid]);
+            bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
             s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
         }
+        publish_masks(bits, wave, lane, s_mask);
         __syncthreads();
         if (__all(done)) continue;
-        const int cnt = min(kBlock, len - round * kBlock);
-        for (int j = 0; j < cnt; ++j) {
-            const StagedGaussian sg = s_g[j];
-            const float dx = sg.x - pxf, dy = sg.y - pyf;
-            const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
-            const bool cand = !done && power >= sg.thr;
-            if (!__any(cand)) continue;
-            if (cand) {
-                const float G = det_expf(power);
-                const float alpha = fminf(0.99f, sg.o * G);
-                if (alpha >= P.alpha_eps) {
-                    const float nextT = T * (1.0f - alpha);
-                    const bool should_done = nextT < P.transmittance_eps;
-                    if (power > 0.0f || should_done) {
-                        done = should_done;
-                    } else {
-                        const float w = alpha * T;
-                        T = nextT;
-                        contributor = round * kBlock + j;
-                        const float4 c = s_rgb[j];
-                        acc0 = acc0 + w * c.x;
-                        acc1 = acc1 + w * c.y;
-                        acc2 = acc2 + w * c.z;
+        bool wave_done = false;
+        for (int chunk = 0; chunk < 4 && !wave_done; ++chunk) {
+            unsigned long long m = uniform_u64(s_mask[wave][chunk]);
+            while (m) {
+                const int j = chunk * 64 + __builtin_ctzll(m);
+                m &= m - 1;
+                const StagedGaussian sg = s_g[j];
+                const float dx = sg.x - pxf, dy = sg.y - pyf;
+                const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
+                if (!done && power >= sg.thr) {
+                    const float G = det_expf(power);
+                    const float alpha = fminf(0.99f, sg.o * G);
+                    if (alpha >= P.alpha_eps) {
+                        const float nextT = T * (1.0f - alpha);
+                        const bool should_done = nextT < P.transmittance_eps;
+                        if (power > 0.0f || should_done) {
+                            done = should_done;
+                        } else {
+                            const float w = alpha * T;
+                            T = nextT;
+                            contributor = round * kBlock + j;
+                            const float4 c = s_rgb[j];
+                            acc0 = acc0 + w * c.x;
+                            acc1 = acc1 + w * c.y;
+                            acc2 = acc2 + w * c.z;
+                        }
                     }
+                }
+                if (__all(done)) {
+                    wave_done = true;
+                    break;
                 }
             }
         }
@@ -164,7 +222,8 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
 __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
     const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
-    const float* __restrict__ final_T, const int32_t* __restrict__ n_contrib, const float* __restrict__ color,
+    const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
+    const int32_t* __restrict__ n_contrib, const float* __restrict__ color,
     const float* __restrict__ drgb, const float* __restrict__ dT, float* __restrict__ duv, float* __restrict__ dconic,
     float* __restrict__ dopacity, float* __restrict__ dcolor) {
     __shared__ StagedGaussian s_g[kBlock];
@@ -172,16 +231,18 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     __shared__ int s_id[kBlock];
     __shared__ float s_grad[9][kBlock];
     __shared__ int s_wmax[4];
+    __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 
     const int ntiles = P.tiles_x * P.tiles_y;
-    const int tile = tile_for_block(blockIdx.x, ntiles);
-    if (tile >= ntiles) return;
+    const int tile = tile_for_block(blockIdx.x, tile_order);
+    if (tile < 0 || tile >= ntiles) return;
     const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
     const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
     const bool inside = px < P.width && py < P.height;
     const float pxf = (float)px, pyf = (float)py;
+    const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
     const size_t pid = (size_t)py * P.width + px;
 
     const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
@@ -213,17 +274,24 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     for (int round = 0; round < rounds; ++round) {
         __syncthreads();  // previous round's flush has read s_grad / s_id
         const int src = r0 + round * kBlock + tid;
+        uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
             s_id[tid] = g;
-            stage_gaussian(P, g, uvs, conic_opacity, &s_g[tid]);
+            bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
             s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
         }
+        publish_masks(bits, wave, lane, s_mask);
 #pragma unroll
         for (int k = 0; k < 9; ++k) s_grad[k][tid] = 0.0f;
         __syncthreads();
         const int cnt = min(kBlock, wave_todo - round * kBlock);
-        for (int j = 0; j < cnt; ++j) {
+        for (int chunk = 0; chunk < 4 && chunk * 64 < cnt; ++chunk) {
+          unsigned long long m = uniform_u64(s_mask[wave][chunk]);
+          if (cnt - chunk * 64 < 64) m &= (1ull << (cnt - chunk * 64)) - 1ull;
+          while (m) {
+            const int j = chunk * 64 + __builtin_ctzll(m);
+            m &= m - 1;
             const StagedGaussian sg = s_g[j];
             const float dx = sg.x - pxf, dy = sg.y - pyf;
             const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
@@ -282,6 +350,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
                 atomicAdd(&s_grad[7][j], g7);
                 atomicAdd(&s_grad[8][j], g8);
             }
+          }
         }
         __syncthreads();
         if (round * kBlock + tid < len) {
@@ -312,14 +381,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
 
 using namespace d3gs;
 
-static int blend_grid(const d3gs_params* p) {
-    const int ntiles = p->tiles_x * p->tiles_y;
-    return ((ntiles + 7) / 8) * 8;
-}
+static int blend_grid(const d3gs_params* p) { return p->tiles_x * p->tiles_y; }
 
 extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
-                              const float* uvs, const float* conic_opacity, const float* rgb_gaussian, float* color,
-                              float* final_T, int32_t* n_contrib, d3gs_stream_t stream) {
+                              const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                              const int32_t* tile_order, float* color, float* final_T, int32_t* n_contrib,
+                              d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_fwd");
     if (rc) return rc;
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib) {
@@ -327,7 +394,7 @@ extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_rang
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     hipLaunchKernelGGL(blend_fwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
-                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, color, final_T, n_contrib);
+                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, color, final_T, n_contrib);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_blend_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
@@ -335,9 +402,9 @@ extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_rang
 
 extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                               const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                              const float* final_T, const int32_t* n_contrib, const float* color, const float* drgb,
-                              const float* dT, float* duv, float* dconic, float* dopacity, float* dcolor,
-                              d3gs_stream_t stream) {
+                              const int32_t* tile_order, const float* final_T, const int32_t* n_contrib,
+                              const float* color, const float* drgb, const float* dT, float* duv, float* dconic,
+                              float* dopacity, float* dcolor, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_bwd");
     if (rc) return rc;
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb ||
@@ -346,8 +413,8 @@ extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_rang
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     hipLaunchKernelGGL(blend_bwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
-                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, final_T, n_contrib, color, drgb, dT,
-                       duv, dconic, dopacity, dcolor);
+                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, final_T, n_contrib, color,
+                       drgb, dT, duv, dconic, dopacity, dcolor);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_blend_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

@@ -45,6 +45,8 @@ class GaussianSplatOpContext:
     cov2d_vecs: torch.Tensor | None = None
     sh_to_rgb_ne_0: torch.Tensor | None = None
     per_gaussian_snap: None = None
+    # not in the reference: tile ids by descending list length, the blend kernels' launch order
+    tile_order: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -309,13 +311,15 @@ class GaussianSplatOp:
 
         with self._stage("tile_ranges"):
             workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+            tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
             _capi.check(L.d3gs_tile_ranges(_capi.ptr(keys_sorted), num_rendered, _capi.ptr(workload_ranges),
-                                           num_tiles, s), "d3gs_tile_ranges")
+                                           num_tiles, _capi.ptr(tile_order), s), "d3gs_tile_ranges")
 
         ctx = GaussianSplatOpContext(
             conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
             gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
-            image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths)
+            image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
+            tile_order=tile_order)
         self._last_keys_sorted = keys_sorted  # kept for parity tests (sorted key order)
         with self._stage("blend_fwd"):
             self.rasterize_forward_backward(model, ctx, out, training=training, _params=P)
@@ -340,8 +344,8 @@ class GaussianSplatOp:
         if grad is None:
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(out.color), _capi.ptr(out.T),
-                _capi.ptr(out.n_contrib), s), "d3gs_blend_fwd")
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order),
+                _capi.ptr(out.color), _capi.ptr(out.T), _capi.ptr(out.n_contrib), s), "d3gs_blend_fwd")
             return None
         drgb = grad.drgb
         assert drgb.is_contiguous(), "drgb must be contiguous"
@@ -352,9 +356,9 @@ class GaussianSplatOp:
         dcolor = torch.zeros((n, 3), dtype=torch.float32, device=dev)
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
-            _capi.ptr(out.color), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(duv), _capi.ptr(dconic),
-            _capi.ptr(dopacity), _capi.ptr(dcolor), s), "d3gs_blend_bwd")
+            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
+            _capi.ptr(out.n_contrib), _capi.ptr(out.color), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(duv),
+            _capi.ptr(dconic), _capi.ptr(dopacity), _capi.ptr(dcolor), s), "d3gs_blend_bwd")
         return RasterizeGradientOutput(duv=duv, dconic=dconic, dopacity=dopacity, dcolor=dcolor)
 
     # --------------------------------------------------------------- backward

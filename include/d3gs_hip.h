@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 1
+#define D3GS_ABI_VERSION 2
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -115,14 +115,18 @@ int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t
                     d3gs_stream_t stream);
 
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
- * ranges[num_tiles][2] must be zero-filled by the caller. */
+ * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],
+ * may be NULL) receives the tile ids sorted by descending list length: a launch order
+ * for the blend kernels that starts the longest tiles first (no counterpart in the
+ * reference, which launches tiles in raster order; it changes scheduling, not results). */
 int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
-                     d3gs_stream_t stream);
+                     int32_t* tile_order, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
  * color [H,W,3], final_T [H,W], n_contrib [H,W]. */
 int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
-                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, float* color,
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                   const int32_t* tile_order /* from d3gs_tile_ranges, or NULL for raster order */, float* color,
                    float* final_T, int32_t* n_contrib, d3gs_stream_t stream);
 
 /* K7 — replaces kernel_raw("rasterize_True_...") (same generator, grad != None,
@@ -131,9 +135,10 @@ int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const i
  * 2182-2210).  duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3] are
  * accumulated with atomics: zero-fill them first. */
 int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
-                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* final_T,
-                   const int32_t* n_contrib, const float* color, const float* drgb, const float* dT, float* duv,
-                   float* dconic, float* dopacity, float* dcolor, d3gs_stream_t stream);
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                   const int32_t* tile_order /* or NULL */, const float* final_T, const int32_t* n_contrib,
+                   const float* color, const float* drgb, const float* dT, float* duv, float* dconic,
+                   float* dopacity, float* dcolor, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from (duv, dconic, dopacity, dcolor[, dz]) to
