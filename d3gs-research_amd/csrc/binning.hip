@@ -95,26 +95,22 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             const int32_t* __restrict__ offsets,
                                                             uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= P.n) return;
+    // no early return: every lane takes part in the cooperative emission of large gaussians
+    const int i_raw = blockIdx.x * kBlock + threadIdx.x;
+    const bool in_range = i_raw < P.n;
+    const int i = in_range ? i_raw : P.n - 1;
     const int r = radii[i];
-    if (r <= 0) return;
     long long off = i == 0 ? 0 : offsets[i - 1];
     const long long end = offsets[i];
-    if (end > m) return;  // caller passed a smaller buffer than the scan total: never write past it
+    // a caller that passed a smaller buffer than the scan total must never be written past
+    const bool active = in_range && r > 0 && end <= m;
     const uint32_t dbits = __float_as_uint(depths[i]);
     const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
     const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
     TileWalkIn g{uv.x, uv.y, (float)r, co.x, co.y, co.z, co.w};
-    const int tiles_x = P.tiles_x;
-    tile_walk(P, g, [&](int x, int y) {
-        if (off < end) {
-            uint64_t key = (uint64_t)(uint32_t)(y * tiles_x + x);
-            keys[off] = (key << 32) | dbits;
-            vals[off] = i;
-        }
-        ++off;
-    });
+    TileWalk walk = {};
+    if (active) walk = tile_walk_setup(P, g);
+    wave_tile_emit(P.filter_algo, active, walk, P.tiles_x, dbits, i, off, end, keys, vals);
 }
 
 // ---------------------------------------------------------------------------

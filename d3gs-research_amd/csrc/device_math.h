@@ -159,17 +159,33 @@ __device__ __forceinline__ void ewa_rows(const d3gs_params& P, const float pc[3]
 }
 
 // ---------------------------------------------------------------------------
-// Tiles touched by one gaussian (render.py:1017-1327).  Visits kept tiles in
-// row-major order (y outer, x inner) and calls f(x, y); returns the count.
-// The preprocess kernel counts with it and the key-expansion kernel emits with
-// it, from the same stored (uv, radius, conic, opacity), so both make identical
-// decisions.
+// Tiles touched by one gaussian (render.py:1017-1327).
+//
+// tile_walk_setup() evaluates, once per gaussian, everything the per-tile test
+// needs; tile_keep() is the per-tile predicate.  The preprocess kernel counts
+// kept tiles and the key-expansion kernel emits them, both from the same stored
+// (uv, radius, conic, opacity), in row-major order (y outer, x inner), so both
+// make identical decisions.
+//
+// Tile counts per gaussian are heavy-tailed (median 4, maximum ~1000 at the
+// benchmark scene), so a plain one-thread-per-gaussian loop leaves 63 lanes idle
+// behind the largest gaussian of each wavefront.  wave_tile_count()/wave_tile_emit()
+// let each lane walk its own gaussian only when it is small, and process the
+// large ones cooperatively: the owner's setup is broadcast with v_readlane and
+// the 64 lanes test 64 candidate tiles per step.
 // ---------------------------------------------------------------------------
 struct TileWalkIn {
     float u, v;
     float radius;
     float conic0, conic1, conic2;
     float opacity;
+};
+
+struct TileWalk {
+    int rminx, rminy, rmaxx, rmaxy;  // 3-sigma tile rect
+    int bminx, bminy, bw, bh;        // candidate rect (origin, size); the 3-sigma rect when no filter
+    float uo, vo, bx, by;            // centre relative to the candidate rect origin, AABB half extents
+    float ow, oh, os, oc;            // oriented box: width, height, sin, cos
 };
 
 __device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1, float by1, float w, float h, float s,
@@ -191,18 +207,20 @@ __device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1
     return true;
 }
 
-template <class F>
-__device__ __forceinline__ int tile_walk(const d3gs_params& P, const TileWalkIn& g, F&& f) {
+__device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const TileWalkIn& g) {
     const int TX = P.tiles_x, TY = P.tiles_y;
-    int rminx = tile_coord((g.u - g.radius) / 16.0f, TX);
-    int rminy = tile_coord((g.v - g.radius) / 16.0f, TY);
-    int rmaxx = tile_coord((((g.u + g.radius) + 16.0f) - 1.0f) / 16.0f, TX);
-    int rmaxy = tile_coord((((g.v + g.radius) + 16.0f) - 1.0f) / 16.0f, TY);
-    int count = 0;
+    TileWalk w;
+    w.rminx = tile_coord((g.u - g.radius) / 16.0f, TX);
+    w.rminy = tile_coord((g.v - g.radius) / 16.0f, TY);
+    w.rmaxx = tile_coord((((g.u + g.radius) + 16.0f) - 1.0f) / 16.0f, TX);
+    w.rmaxy = tile_coord((((g.v + g.radius) + 16.0f) - 1.0f) / 16.0f, TY);
+    w.uo = w.vo = w.bx = w.by = w.ow = w.oh = w.os = w.oc = 0.0f;
     if (P.filter_algo == D3GS_FILTER_NONE) {
-        for (int y = rminy; y < rmaxy; ++y)
-            for (int x = rminx; x < rmaxx; ++x) { f(x, y); ++count; }
-        return count;
+        w.bminx = w.rminx;
+        w.bminy = w.rminy;
+        w.bw = w.rmaxx - w.rminx;
+        w.bh = w.rmaxy - w.rminy;
+        return w;
     }
     // half extents of the exact alpha >= alpha_eps ellipse (gs3d.py:710-742)
     float bound = 2.0f * det_logf(P.alpha_eps / g.opacity);
@@ -215,15 +233,17 @@ __device__ __forceinline__ int tile_walk(const d3gs_params& P, const TileWalkIn&
     by = vy > 0.0f ? by : 0.0f;
     bx = fabsf(bx);
     by = fabsf(by);
-    int bminx = tile_coord((g.u - bx) / 16.0f, TX);
-    int bminy = tile_coord((g.v - by) / 16.0f, TY);
+    w.bx = bx;
+    w.by = by;
+    w.bminx = tile_coord((g.u - bx) / 16.0f, TX);
+    w.bminy = tile_coord((g.v - by) / 16.0f, TY);
     int bmaxx = tile_coord(ceilf((g.u + bx) / 16.0f), TX);
     int bmaxy = tile_coord(ceilf((g.v + by) / 16.0f), TY);
-    float uo = g.u - (float)bminx * 16.0f;
-    float vo = g.v - (float)bminy * 16.0f;
-    float ow = 0.0f, oh = 0.0f, os = 0.0f, oc = 0.0f;
-    const bool use_obb = P.filter_algo == D3GS_FILTER_OBB || P.filter_algo == D3GS_FILTER_OBB_DFVT;
-    if (use_obb) {
+    w.bw = max(bmaxx - w.bminx, 0);
+    w.bh = max(bmaxy - w.bminy, 0);
+    w.uo = g.u - (float)w.bminx * 16.0f;
+    w.vo = g.v - (float)w.bminy * 16.0f;
+    if (P.filter_algo == D3GS_FILTER_OBB || P.filter_algo == D3GS_FILTER_OBB_DFVT) {
         // oriented bounding box of the ellipse x^T Q x = 1, Q = -conic / bound (gs3d.py:761-791, 981-987)
         float eA = (-g.conic0) / bound, eC = (-g.conic2) / bound, eB = (-g.conic1) / bound;
         float det = eA * eC - eB * eB;
@@ -237,30 +257,138 @@ __device__ __forceinline__ int tile_walk(const d3gs_params& P, const TileWalkIn&
         v2y = v2y / len;
         float minor = 1.0f / sqrtf(e1 * s1);
         float major = 1.0f / sqrtf(e2 * s2);
-        ow = major * 2.0f;
-        oh = minor * 2.0f;
-        os = v2y;
-        oc = v2x;
+        w.ow = major * 2.0f;
+        w.oh = minor * 2.0f;
+        w.os = v2y;
+        w.oc = v2x;
     }
-    for (int y = bminy; y < bmaxy; ++y) {
-        float py0 = (float)((y - bminy) * 16);
-        float py1 = py0 + 16.0f;
-        for (int x = bminx; x < bmaxx; ++x) {
-            float px0 = (float)((x - bminx) * 16);
-            float px1 = px0 + 16.0f;
-            bool keep;
-            if (!use_obb) {
-                bool xo = (uo - bx) <= px1 && (uo + bx) >= px0;
-                bool yo = (vo - by) <= py1 && (vo + by) >= py0;
-                keep = xo && yo;
-            } else {
-                keep = obb_overlaps_box(px0, py0, px1, py1, ow, oh, os, oc, uo, vo);
-            }
-            keep = keep && x >= rminx && x < rmaxx && y >= rminy && y < rmaxy;
-            if (keep) { f(x, y); ++count; }
+    return w;
+}
+
+// Is candidate tile (lx, ly) — coordinates relative to the candidate rect origin — kept?
+__device__ __forceinline__ bool tile_keep(const int filter_algo, const TileWalk& w, int lx, int ly) {
+    if (filter_algo == D3GS_FILTER_NONE) return true;
+    const float px0 = (float)(lx * 16), py0 = (float)(ly * 16);
+    const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
+    bool keep;
+    if (filter_algo == D3GS_FILTER_AABB) {
+        const bool xo = (w.uo - w.bx) <= px1 && (w.uo + w.bx) >= px0;
+        const bool yo = (w.vo - w.by) <= py1 && (w.vo + w.by) >= py0;
+        keep = xo && yo;
+    } else {
+        keep = obb_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
+    }
+    const int x = lx + w.bminx, y = ly + w.bminy;
+    return keep && x >= w.rminx && x < w.rmaxx && y >= w.rminy && y < w.rmaxy;
+}
+
+__device__ __forceinline__ int bcast_i(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
+__device__ __forceinline__ float bcast_f(float v, int src) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+}
+__device__ __forceinline__ TileWalk bcast_walk(const TileWalk& w, int src) {
+    TileWalk r;
+    r.rminx = bcast_i(w.rminx, src); r.rminy = bcast_i(w.rminy, src);
+    r.rmaxx = bcast_i(w.rmaxx, src); r.rmaxy = bcast_i(w.rmaxy, src);
+    r.bminx = bcast_i(w.bminx, src); r.bminy = bcast_i(w.bminy, src);
+    r.bw = bcast_i(w.bw, src); r.bh = bcast_i(w.bh, src);
+    r.uo = bcast_f(w.uo, src); r.vo = bcast_f(w.vo, src);
+    r.bx = bcast_f(w.bx, src); r.by = bcast_f(w.by, src);
+    r.ow = bcast_f(w.ow, src); r.oh = bcast_f(w.oh, src);
+    r.os = bcast_f(w.os, src); r.oc = bcast_f(w.oc, src);
+    return r;
+}
+
+constexpr int kSmallWalk = 16;  // candidate tiles a lane walks alone before the wavefront takes over
+
+// Number of kept tiles of this lane's gaussian.  Must be called by all 64 lanes of a wavefront
+// (lanes without a gaussian pass active = false).
+__device__ __forceinline__ int wave_tile_count(const int filter_algo, bool active, const TileWalk& w) {
+    const int area = active ? w.bw * w.bh : 0;
+    if (filter_algo == D3GS_FILTER_NONE) return area;
+    int count = 0;
+    const bool big = area > kSmallWalk;
+    if (!big) {
+        for (int t = 0; t < area; ++t) {
+            const int ly = t / w.bw;
+            count += tile_keep(filter_algo, w, t - ly * w.bw, ly) ? 1 : 0;
         }
     }
+    const int lane = threadIdx.x & 63;
+    unsigned long long todo = __ballot(big);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const TileWalk ws = bcast_walk(w, src);
+        const int a = ws.bw * ws.bh;
+        int c = 0;
+        for (int base = 0; base < a; base += 64) {
+            const int t = base + lane;
+            bool k = false;
+            if (t < a) {
+                const int ly = t / ws.bw;
+                k = tile_keep(filter_algo, ws, t - ly * ws.bw, ly);
+            }
+            c += __popcll(__ballot(k));
+        }
+        if (lane == src) count = c;
+    }
     return count;
+}
+
+// Emits (key, value) of every kept tile of this lane's gaussian at [off, end) in row-major tile
+// order.  Must be called by all 64 lanes of a wavefront.
+__device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool active, const TileWalk& w, int tiles_x,
+                                               uint32_t depth_bits, int value, long long off, long long end,
+                                               uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+    const int area = active ? w.bw * w.bh : 0;
+    const bool big = area > kSmallWalk;
+    if (!big) {
+        for (int t = 0; t < area; ++t) {
+            const int ly = t / w.bw, lx = t - ly * w.bw;
+            if (tile_keep(filter_algo, w, lx, ly)) {
+                if (off < end) {
+                    const uint64_t tile = (uint64_t)(uint32_t)((ly + w.bminy) * tiles_x + lx + w.bminx);
+                    keys[off] = (tile << 32) | depth_bits;
+                    vals[off] = value;
+                }
+                ++off;
+            }
+        }
+    }
+    const int lane = threadIdx.x & 63;
+    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    unsigned long long todo = __ballot(big);
+    while (todo) {
+        const int src = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const TileWalk ws = bcast_walk(w, src);
+        const uint32_t dbits = (uint32_t)bcast_i((int)depth_bits, src);
+        const int val = bcast_i(value, src);
+        long long o = ((long long)bcast_i((int)(off >> 32), src) << 32) | (uint32_t)bcast_i((int)off, src);
+        const long long e = ((long long)bcast_i((int)(end >> 32), src) << 32) | (uint32_t)bcast_i((int)end, src);
+        const int a = ws.bw * ws.bh;
+        for (int base = 0; base < a; base += 64) {
+            const int t = base + lane;
+            bool k = false;
+            int lx = 0, ly = 0;
+            if (t < a) {
+                ly = t / ws.bw;
+                lx = t - ly * ws.bw;
+                k = tile_keep(filter_algo, ws, lx, ly);
+            }
+            const unsigned long long b = __ballot(k);
+            if (k) {
+                const long long pos = o + __popcll(b & lt_mask);
+                if (pos < e) {
+                    const uint64_t tile = (uint64_t)(uint32_t)((ly + ws.bminy) * tiles_x + lx + ws.bminx);
+                    keys[pos] = (tile << 32) | dbits;
+                    vals[pos] = val;
+                }
+            }
+            o += __popcll(b);
+        }
+    }
 }
 
 constexpr float kShC0 = 0.28209479177387814f;

@@ -42,8 +42,10 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
     const float* __restrict__ sh_base, float* __restrict__ depths, int32_t* __restrict__ radii,
     float* __restrict__ uvs, float* __restrict__ conic_opacity, int32_t* __restrict__ tiles_touched,
     float* __restrict__ rgb_out, float* __restrict__ cov2d_out, uint8_t* __restrict__ ne0_out) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= P.n) return;
+    // no early return: every lane of the wavefront takes part in the cooperative tile count
+    const int i_raw = blockIdx.x * kBlock + threadIdx.x;
+    const bool in_range = i_raw < P.n;
+    const int i = in_range ? i_raw : P.n - 1;
 
     bool valid = true;
     float z = 0.0f, u = 0.0f, v = 0.0f, con0 = 0.0f, con1 = 0.0f, con2 = 0.0f, op = 0.0f;
@@ -55,7 +57,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
     float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
     float pc[3] = {dot3(P.w2c + 0, d), dot3(P.w2c + 3, d), dot3(P.w2c + 6, d)};
     z = pc[2];
-    valid = (z >= P.z_near && z <= P.z_far);
+    valid = in_range && (z >= P.z_near && z <= P.z_far);
     if (valid) {
         u = ((pc[0] / z) * P.fx + P.cx) - 0.5f;
         v = ((pc[1] / z) * P.fy + P.cy) - 0.5f;
@@ -101,10 +103,13 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
         int area = (rmaxx - rminx) * (rmaxy - rminy);
         valid = (det > 0.0f) && area != 0 && (op > P.alpha_eps);
     }
-    if (valid) {
+    {
         TileWalkIn g{u, v, radius, con0, con1, con2, op};
-        count = tile_walk(P, g, [](int, int) {});
-
+        TileWalk walk = {};
+        if (valid) walk = tile_walk_setup(P, g);
+        count = wave_tile_count(P.filter_algo, valid, walk);
+    }
+    if (valid) {
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
         float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
         const float* shp = sh + (size_t)i * P.sh_stride * 3;
@@ -118,6 +123,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
     } else {
         z = u = v = con0 = con1 = con2 = op = a = b = c = radius = 0.0f;
     }
+    if (!in_range) return;
 
     depths[i] = z;
     radii[i] = (int)radius;
