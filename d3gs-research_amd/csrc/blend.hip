@@ -57,6 +57,57 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// ---------------------------------------------------------------------------
+// Sum of nine per-lane values over the wavefront, as a transposing reduction:
+// every step exchanges halves so that the number of live registers halves with
+// the group size (9 -> 5 -> 3 -> 2 -> 1), ~25 VALU operations instead of nine
+// independent 64-lane butterflies.  Cross-half / cross-row exchanges use the
+// gfx950 v_permlane32_swap / v_permlane16_swap, the rest DPP.  On return lane
+// slot_lane(k) holds the total of value k; reduce9_slot() tells each lane which
+// value (or none) it holds.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float swap_add32(float a, float b) {
+    // lanes 0..31 <- a[l] + a[l+32]; lanes 32..63 <- b[l-32] + b[l]
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float swap_add16(float a, float b) {
+    // rows 0,2 <- a[row] + a[row+1]; rows 1,3 <- b[row-1] + b[row]   (row = 16 lanes)
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int kCtrl>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xF, 0xF, false));
+}
+
+__device__ __forceinline__ int reduce9_slot(int lane) {
+    if (lane & 3) return -1;
+    const int r = lane >> 4, h = (lane >> 3) & 1, k = (lane >> 2) & 1;
+    if (k) return (r == 0 && h == 0) ? 8 : -1;
+    const int rowmap = (r == 0) ? 0 : (r == 1) ? 2 : (r == 2) ? 1 : 3;
+    return rowmap + 4 * h;
+}
+
+__device__ __forceinline__ float wave_reduce9(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                                              float v7, float v8, bool hi8, bool hi4) {
+    // 64 -> 32: lower half keeps the first value of each pair, upper half the second
+    const float s01 = swap_add32(v0, v1), s23 = swap_add32(v2, v3), s45 = swap_add32(v4, v5),
+                s67 = swap_add32(v6, v7), s8 = swap_add32(v8, 0.0f);
+    // 32 -> 16: rows (0,2) keep the first register of each pair, rows (1,3) the second
+    const float q0 = swap_add16(s01, s23), q1 = swap_add16(s45, s67);
+    float q2 = swap_add16(s8, 0.0f);
+    // 16 -> 8: lanes 0-7 of a row keep q0, lanes 8-15 keep q1 (row_ror:8 pairs lane i with i^8)
+    float x = (hi8 ? q1 : q0) + dpp_f<0x128>(hi8 ? q0 : q1);
+    q2 = q2 + dpp_f<0x128>(q2);
+    // 8 -> 4: lanes with bit 2 clear keep x, the others q2 (row_half_mirror pairs lane i with 7 - i)
+    float y = (hi4 ? q2 : x) + dpp_f<0x141>(hi4 ? x : q2);
+    // 4 -> 1 inside each quad
+    y = y + dpp_f<0x4E>(y);
+    y = y + dpp_f<0xB1>(y);
+    return y;
+}
+
 __device__ __forceinline__ int wave_max_i32(int v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
@@ -264,6 +315,8 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         dr2 = drgb[3 * pid + 2];
     }
     const float dT_term = (-dT_val) * render_T;
+    const int slot = reduce9_slot(lane);
+    const bool hi8 = (lane & 8) != 0, hi4 = (lane & 4) != 0;
     const int wave_todo = wave_max_i32(contributor);
     if (lane == 0) s_wmax[wave] = wave_todo;
     __syncthreads();
@@ -330,26 +383,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
                 }
             }
             if (!__any(valid)) continue;
-            g0 = wave_sum(g0);
-            g1 = wave_sum(g1);
-            g2 = wave_sum(g2);
-            g3 = wave_sum(g3);
-            g4 = wave_sum(g4);
-            g5 = wave_sum(g5);
-            g6 = wave_sum(g6);
-            g7 = wave_sum(g7);
-            g8 = wave_sum(g8);
-            if (lane == 0) {
-                atomicAdd(&s_grad[0][j], g0);
-                atomicAdd(&s_grad[1][j], g1);
-                atomicAdd(&s_grad[2][j], g2);
-                atomicAdd(&s_grad[3][j], g3);
-                atomicAdd(&s_grad[4][j], g4);
-                atomicAdd(&s_grad[5][j], g5);
-                atomicAdd(&s_grad[6][j], g6);
-                atomicAdd(&s_grad[7][j], g7);
-                atomicAdd(&s_grad[8][j], g8);
-            }
+            // nine wave totals land in nine different lanes: one LDS atomic instruction adds them all
+            const float total = wave_reduce9(g0, g1, g2, g3, g4, g5, g6, g7, g8, hi8, hi4);
+            if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }
         __syncthreads();
