@@ -1,6 +1,7 @@
 // Tile binning: prefix scan of per-gaussian tile counts, (tile, depth) key
 // expansion, stable LSD radix sort of (u64 key, i32 value) pairs, and tile-range
-// extraction.  All stages are HBM-bandwidth-bound integer work.
+// extraction (the radix sort itself lives in radix_sort.hip).  All stages are
+// HBM-bandwidth-bound integer work.
 //
 // Reference: d3sim/algos/d3gs/render.py:694-695 (cumsum), 739-840 (keys),
 // 845-887 + d3sim/csrc/devsort.py:38-149 (CUB radix sort), 896-939 (ranges).
@@ -111,96 +112,6 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     TileWalk walk = {};
     if (active) walk = tile_walk_setup(P, g);
     wave_tile_emit(P.filter_algo, active, walk, P.tiles_x, dbits, i, off, end, keys, vals);
-}
-
-// ---------------------------------------------------------------------------
-// Radix sort, 8-bit digits, per pass: block histograms -> scan -> stable scatter.
-// A block owns a contiguous run of kSortTile keys; wave w of the block owns the
-// w-th quarter, processed 64 keys at a time, so (wave, round, lane) order equals
-// input order and ranks computed from it are stable.
-// ---------------------------------------------------------------------------
-constexpr int kSortItems = 16;
-constexpr int kSortTile = kBlock * kSortItems;  // 4096 keys per block
-constexpr int kRadix = 256;
-
-__global__ __launch_bounds__(kBlock) void sort_hist_kernel(const uint64_t* __restrict__ keys, long long m, int shift,
-                                                            uint32_t mask, int nblocks,
-                                                            int32_t* __restrict__ hist /* [kRadix][nblocks] */) {
-    __shared__ int h[kRadix];
-    h[threadIdx.x] = 0;
-    __syncthreads();
-    const long long base = (long long)blockIdx.x * kSortTile;
-#pragma unroll 4
-    for (int k = 0; k < kSortItems; ++k) {
-        long long idx = base + k * kBlock + threadIdx.x;
-        if (idx < m) {
-            uint32_t d = (uint32_t)(keys[idx] >> shift) & mask;
-            atomicAdd(&h[d], 1);
-        }
-    }
-    __syncthreads();
-    hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = h[threadIdx.x];
-}
-
-__global__ __launch_bounds__(kBlock) void sort_scatter_kernel(const uint64_t* __restrict__ keys_in,
-                                                               const int32_t* __restrict__ vals_in,
-                                                               uint64_t* __restrict__ keys_out,
-                                                               int32_t* __restrict__ vals_out, long long m, int shift,
-                                                               uint32_t mask, int nblocks,
-                                                               const int32_t* __restrict__ offsets /* scanned hist */) {
-    __shared__ int wave_cnt[4][kRadix];   // running / final per-wave digit counts
-    __shared__ int digit_base[kRadix];    // global output offset of this block's first key of each digit
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int k = threadIdx.x; k < 4 * kRadix; k += kBlock) (&wave_cnt[0][0])[k] = 0;
-    __syncthreads();
-
-    const long long base = (long long)blockIdx.x * kSortTile + wave * (kSortTile / 4);
-    uint64_t key[kSortItems];
-    int rank[kSortItems];
-    const uint64_t lt_mask = (1ull << lane) - 1ull;
-#pragma unroll
-    for (int k = 0; k < kSortItems; ++k) {
-        const long long idx = base + k * 64 + lane;
-        const bool in = idx < m;
-        key[k] = in ? keys_in[idx] : ~0ull;
-        const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
-        // lanes holding the same digit
-        uint64_t peers = __ballot(in);
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const uint64_t bal = __ballot((d >> b) & 1u);
-            peers &= ((d >> b) & 1u) ? bal : ~bal;
-        }
-        int before = 0;
-        if (in) before = wave_cnt[wave][d];
-        __builtin_amdgcn_wave_barrier();
-        if (in && (peers & lt_mask) == 0) wave_cnt[wave][d] = before + __popcll(peers);
-        __builtin_amdgcn_wave_barrier();
-        rank[k] = before + __popcll(peers & lt_mask);
-    }
-    __syncthreads();
-    {
-        // thread t owns digit t: exclusive prefix over waves + the block's global base
-        const int d = threadIdx.x;
-        int c0 = wave_cnt[0][d], c1 = wave_cnt[1][d], c2 = wave_cnt[2][d], c3 = wave_cnt[3][d];
-        // `offsets` is the inclusive scan of the (digit-major) block histograms
-        digit_base[d] = offsets[(size_t)d * nblocks + blockIdx.x] - (c0 + c1 + c2 + c3);
-        wave_cnt[0][d] = 0;
-        wave_cnt[1][d] = c0;
-        wave_cnt[2][d] = c0 + c1;
-        wave_cnt[3][d] = c0 + c1 + c2;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int k = 0; k < kSortItems; ++k) {
-        const long long idx = base + k * 64 + lane;
-        if (idx < m) {
-            const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
-            const long long pos = (long long)digit_base[d] + wave_cnt[wave][d] + rank[k];
-            keys_out[pos] = key[k];
-            vals_out[pos] = vals_in[idx];
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------
@@ -317,73 +228,6 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
                        radii, uvs, conic_opacity, depths, offsets, keys, gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
-    return D3GS_OK;
-}
-
-static int sort_blocks(int64_t m) { return (int)((m + kSortTile - 1) / kSortTile); }
-
-extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* bytes_out_host) {
-    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !bytes_out_host) {
-        set_error("d3gs_sort_workspace_bytes: bad argument");
-        return D3GS_ERR_INVALID_ARGUMENT;
-    }
-    const size_t hist_elems = (size_t)kRadix * std::max(1, sort_blocks(m));
-    *bytes_out_host = align_up(hist_elems * sizeof(int32_t), 256) + scan_ws_bytes((long long)hist_elems);
-    return D3GS_OK;
-}
-
-extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                               size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
-                               d3gs_stream_t stream) {
-    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !result_in_b_host) {
-        set_error("d3gs_sort_pairs: bad argument (m=%lld bits=[%d,%d))", (long long)m, begin_bit, end_bit);
-        return D3GS_ERR_INVALID_ARGUMENT;
-    }
-    if (m >= (1ll << 31)) { set_error("d3gs_sort_pairs: m >= 2^31 is not supported"); return D3GS_ERR_UNSUPPORTED; }
-    *result_in_b_host = 0;
-    if (m == 0 || begin_bit == end_bit) return D3GS_OK;
-    if (!keys_a || !keys_b || !vals_a || !vals_b || !workspace) {
-        set_error("d3gs_sort_pairs: NULL buffer");
-        return D3GS_ERR_INVALID_ARGUMENT;
-    }
-    size_t need = 0;
-    d3gs_sort_workspace_bytes(m, begin_bit, end_bit, &need);
-    if (workspace_bytes < need) {
-        set_error("d3gs_sort_pairs: workspace %zu < required %zu", workspace_bytes, need);
-        return D3GS_ERR_WORKSPACE_TOO_SMALL;
-    }
-    hipStream_t s = (hipStream_t)stream;
-    const int nblocks = sort_blocks(m);
-    const size_t hist_elems = (size_t)kRadix * nblocks;
-    int32_t* hist = (int32_t*)workspace;
-    void* scan_ws = (char*)workspace + align_up(hist_elems * sizeof(int32_t), 256);
-    uint64_t* kin = keys_a;
-    uint64_t* kout = keys_b;
-    int32_t* vin = vals_a;
-    int32_t* vout = vals_b;
-    int in_b = 0;
-    for (int bit = begin_bit; bit < end_bit; bit += 8) {
-        const int nb = std::min(8, end_bit - bit);
-        const uint32_t mask = (1u << nb) - 1u;
-        hipLaunchKernelGGL(sort_hist_kernel, dim3(nblocks), dim3(kBlock), 0, s, kin, (long long)m, bit, mask, nblocks, hist);
-        // inclusive scan of the digit-major histogram table, in place; the scatter kernel
-        // subtracts its own count to get the exclusive offset
-        {
-            const int nchunks = scan_chunks((long long)hist_elems);
-            int32_t* sums = (int32_t*)scan_ws;
-            hipLaunchKernelGGL(scan_chunk_sums_kernel, dim3(nchunks), dim3(kBlock), 0, s, hist, (int)hist_elems, sums);
-            hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, sums, nchunks, (int64_t*)nullptr);
-            hipLaunchKernelGGL(scan_apply_kernel, dim3(nchunks), dim3(kBlock), 0, s, hist, (int)hist_elems, sums);
-        }
-        hipLaunchKernelGGL(sort_scatter_kernel, dim3(nblocks), dim3(kBlock), 0, s, kin, vin, kout, vout, (long long)m, bit,
-                           mask, nblocks, hist);
-        std::swap(kin, kout);
-        std::swap(vin, vout);
-        in_b ^= 1;
-    }
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("d3gs_sort_pairs: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
-    *result_in_b_host = in_b;
     return D3GS_OK;
 }
 

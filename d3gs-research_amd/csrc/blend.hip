@@ -207,8 +207,10 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-            s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+            if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read
+                bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
+                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+            }
         }
         publish_masks(bits, wave, lane, s_mask);
         __syncthreads();
@@ -330,9 +332,11 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            s_id[tid] = g;
-            bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-            s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+            if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read or write
+                s_id[tid] = g;
+                bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
+                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+            }
         }
         publish_masks(bits, wave, lane, s_mask);
 #pragma unroll

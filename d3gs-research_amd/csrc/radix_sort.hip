@@ -1,0 +1,343 @@
+// Stable LSD radix sort of (u64 key, i32 value) pairs on a bit range — the gfx950
+// replacement of the reference's CUB DeviceRadixSort wrapper
+// (d3sim/csrc/devsort.py:38-129, call site d3sim/algos/d3gs/render.py:846-887).
+//
+// Single-sweep design: one kernel histograms every digit of every pass in one
+// read of the keys; then each 8-bit pass is ONE kernel that reads a pair once
+// and writes it once (24 B per pair per pass).  A workgroup owns 4096
+// consecutive keys, ranks them in LDS, and learns where its digits start in the
+// output from the workgroups before it through a decoupled look-back over
+// per-(tile, digit) status words instead of a separate scan kernel.
+//
+// Stability: wave w of a workgroup owns the w-th eighth of the tile and walks it
+// 64 keys at a time, so (wave, step, lane) order is input order; the rank of a
+// key among equal digits is (keys of earlier waves) + (earlier steps of this
+// wave) + (lower lanes of this step, by ballot matching).
+//
+// Coalescing: ranked pairs are first placed at their tile-local sorted position
+// in LDS, then written out by consecutive threads, so equal-digit runs leave as
+// contiguous segments.
+//
+// Look-back protocol: tiles are claimed from an atomic ticket, so a workgroup
+// only ever waits on tiles that started before it.  A status word carries a
+// 30-bit count and two flag bits (aggregate of this tile / inclusive prefix up
+// to this tile); words are read and written with relaxed device-scope atomics.
+// Polling is bounded: past the limit the workgroup raises an error flag and
+// stops waiting, so the grid always drains.
+#include "device_math.h"
+
+namespace d3gs {
+
+constexpr int kOsThreads = 512;
+constexpr int kOsWaves = kOsThreads / 64;
+constexpr int kOsItems = 8;
+constexpr int kOsTile = kOsThreads * kOsItems;  // 4096 pairs per workgroup
+constexpr int kOsRadix = 256;
+constexpr uint32_t kFlagAggregate = 1u << 30;
+constexpr uint32_t kFlagPrefix = 2u << 30;
+constexpr uint32_t kValueMask = (1u << 30) - 1u;
+constexpr int kSpinLimit = 1 << 22;
+constexpr int kLookWindow = 16;  // predecessor tiles polled per look-back step
+
+struct SortWorkspace {
+    uint32_t* hist;     // [passes][256] digit totals of the whole input
+    uint32_t* tickets;  // [passes] next tile to hand out
+    uint32_t* error;    // [1] set when a look-back gave up
+    uint32_t* status;   // [passes][ntiles][256]
+};
+
+__device__ __forceinline__ int os_wave_incl_scan(int v, int lane) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int t = __shfl_up(v, off, 64);
+        if (lane >= off) v += t;
+    }
+    return v;
+}
+
+// exclusive scan of one int per thread over a workgroup of kWaves wavefronts
+template <int kWaves>
+__device__ __forceinline__ int os_block_excl_scan(int v, int* smem /* kWaves ints */) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int incl = os_wave_incl_scan(v, lane);
+    if (lane == 63) smem[wave] = incl;
+    __syncthreads();
+    int base = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) base += (w < wave) ? smem[w] : 0;
+    __syncthreads();
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kBlock) void os_clear_kernel(uint32_t* __restrict__ p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) p[i] = 0u;
+}
+
+// All passes' digit histograms in one read of the keys.  Few, large workgroups: every workgroup
+// ends with one global atomic per (pass, digit), and atomics to one address from the whole chip
+// serialise, so their number (workgroups x passes x 256) is what has to stay small.  Inside a
+// workgroup each group of 8 lanes adds into its own LDS copy of the table, which divides the
+// same-address conflicts of skewed digits (the exponent byte of a depth takes a handful of values).
+constexpr int kHistThreads = 1024;
+constexpr int kHistCopies = 8;
+__global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const uint64_t* __restrict__ keys, long long m,
+                                                                int begin_bit, int end_bit, int passes,
+                                                                uint32_t* __restrict__ hist) {
+    extern __shared__ uint32_t h[];  // [kHistCopies][passes][256]
+    const int table = passes * kOsRadix;
+    for (int k = threadIdx.x; k < kHistCopies * table; k += kHistThreads) h[k] = 0u;
+    __syncthreads();
+    uint32_t* mine = h + (threadIdx.x & (kHistCopies - 1)) * table;
+    const long long stride = (long long)gridDim.x * kHistThreads;
+    for (long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x; i < m; i += stride) {
+        const uint64_t key = keys[i];
+        for (int p = 0; p < passes; ++p) {
+            const int bit = begin_bit + 8 * p;
+            const int nb = min(8, end_bit - bit);
+            atomicAdd(&mine[p * kOsRadix + ((uint32_t)(key >> bit) & ((1u << nb) - 1u))], 1u);
+        }
+    }
+    __syncthreads();
+    for (int k = threadIdx.x; k < table; k += kHistThreads) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int q = 0; q < kHistCopies; ++q) c += h[q * table + k];
+        if (c) atomicAdd(&hist[k], c);
+    }
+}
+
+__global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const uint64_t* __restrict__ keys_in,
+                                                              const int32_t* __restrict__ vals_in,
+                                                              uint64_t* __restrict__ keys_out,
+                                                              int32_t* __restrict__ vals_out, long long m, int shift,
+                                                              uint32_t mask, int ntiles,
+                                                              const uint32_t* __restrict__ hist /* this pass, [256] */,
+                                                              uint32_t* __restrict__ ticket,
+                                                              uint32_t* __restrict__ status,
+                                                              uint32_t* __restrict__ error) {
+    __shared__ int wave_cnt[kOsWaves][kOsRadix];  // running, then exclusive-over-waves, per-wave digit counts
+    __shared__ int digit_out[kOsRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
+    __shared__ uint64_t s_keys[kOsTile];
+    __shared__ uint16_t s_src[kOsTile];  // tile-local input index of the pair at each sorted position
+    __shared__ int s_scan[kOsWaves];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int k = tid; k < kOsWaves * kOsRadix; k += kOsThreads) (&wave_cnt[0][0])[k] = 0;
+    __syncthreads();
+    // Tile = workgroup id.  Workgroups of a 1-D grid are dispatched in id order (per XCD, which gets
+    // every 8th id), so every tile this one waits on has been dispatched before it; an atomic ticket
+    // would add one chip-wide same-address atomic per workgroup to the start of every pass.
+    const int tile = blockIdx.x;
+    if (tile >= ntiles) return;
+
+    const long long tile_begin = (long long)tile * kOsTile;
+    const int wave_begin = wave * (kOsTile / kOsWaves);
+    uint64_t key[kOsItems];
+    int rank[kOsItems];
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const long long idx = tile_begin + wave_begin + k * 64 + lane;
+        const bool in = idx < m;
+        key[k] = in ? keys_in[idx] : ~0ull;
+    }
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const bool in = tile_begin + wave_begin + k * 64 + lane < m;
+        const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
+        uint64_t peers = __ballot(in);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const uint64_t bal = __ballot((d >> b) & 1u);
+            peers &= ((d >> b) & 1u) ? bal : ~bal;
+        }
+        int before = 0;
+        if (in) before = wave_cnt[wave][d];
+        __builtin_amdgcn_wave_barrier();
+        if (in && (peers & lt_mask) == 0) wave_cnt[wave][d] = before + __popcll(peers);
+        __builtin_amdgcn_wave_barrier();
+        rank[k] = before + __popcll(peers & lt_mask);
+    }
+    __syncthreads();
+
+    // threads 0..255 each own one digit
+    const bool owner = tid < kOsRadix;
+    int c[kOsWaves];
+    uint32_t total = 0;
+    uint32_t* my_status = status + (size_t)tile * kOsRadix + (owner ? tid : 0);
+    if (owner) {
+#pragma unroll
+        for (int w = 0; w < kOsWaves; ++w) {
+            c[w] = wave_cnt[w][tid];
+            total += (uint32_t)c[w];
+        }
+        if (tile > 0) __hip_atomic_store(my_status, kFlagAggregate | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // where each digit starts in the whole output, and inside this tile
+    const int excl_global = os_block_excl_scan<kOsWaves>(owner ? (int)hist[tid] : 0, s_scan);
+    const int excl_local = os_block_excl_scan<kOsWaves>((int)total, s_scan);
+    if (owner) {
+        // digits of earlier tiles: walk back until a tile that already knows its inclusive prefix.
+        // kLookWindow predecessors are polled per step with independent loads, so the serial depth of
+        // the walk is a fraction of the tiles in flight.
+        uint32_t prev = 0;
+        if (tile > 0) {
+            int t = tile - 1;
+            int spins = 0;
+            bool finished = false;
+            while (!finished) {
+                uint32_t s[kLookWindow];
+#pragma unroll
+                for (int i = 0; i < kLookWindow; ++i) {
+                    const int tt = t - i;
+                    s[i] = tt >= 0 ? __hip_atomic_load(status + (size_t)tt * kOsRadix + tid, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT)
+                                   : kFlagPrefix;  // before the first tile: an empty inclusive prefix
+                }
+                int consumed = kLookWindow;
+#pragma unroll
+                for (int i = 0; i < kLookWindow; ++i) {
+                    if (consumed != kLookWindow) continue;
+                    const uint32_t flag = s[i] & ~kValueMask;
+                    if (flag == 0u) {
+                        consumed = i;  // not published yet: poll again from this tile
+                    } else {
+                        prev += s[i] & kValueMask;
+                        if (flag == kFlagPrefix) {
+                            finished = true;
+                            consumed = i + 1;
+                        }
+                    }
+                }
+                t -= consumed;
+                if (!finished && consumed < kLookWindow) {
+                    if (++spins > kSpinLimit) {
+                        atomicOr(error, 1u);
+                        finished = true;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+        }
+        __hip_atomic_store(my_status, kFlagPrefix | ((prev + total) & kValueMask), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        digit_out[tid] = excl_global + (int)prev - excl_local;
+        int running = excl_local;
+#pragma unroll
+        for (int w = 0; w < kOsWaves; ++w) {
+            wave_cnt[w][tid] = running;
+            running += c[w];
+        }
+    }
+    __syncthreads();
+
+    // place every pair at its tile-local sorted position
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const int local = wave_begin + k * 64 + lane;
+        if (tile_begin + local < m) {
+            const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
+            const int pos = wave_cnt[wave][d] + rank[k];
+            s_keys[pos] = key[k];
+            s_src[pos] = (uint16_t)local;
+        }
+    }
+    __syncthreads();
+    // consecutive threads write consecutive sorted positions: equal-digit runs leave as contiguous segments
+    const int count = (int)min((long long)kOsTile, m - tile_begin);
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const int i = k * kOsThreads + tid;
+        if (i < count) {
+            const uint64_t kk = s_keys[i];
+            const uint32_t d = (uint32_t)(kk >> shift) & mask;
+            const long long pos = (long long)digit_out[d] + i;
+            keys_out[pos] = kk;
+            vals_out[pos] = vals_in[tile_begin + s_src[i]];
+        }
+    }
+}
+
+static inline size_t os_align(size_t v) { return (v + 255) / 256 * 256; }
+static inline int os_tiles(int64_t m) { return (int)((m + kOsTile - 1) / kOsTile); }
+static inline int os_passes(int begin_bit, int end_bit) { return (end_bit - begin_bit + 7) / 8; }
+
+static size_t os_layout(int64_t m, int passes, SortWorkspace* ws, void* base) {
+    const int ntiles = os_tiles(m) > 0 ? os_tiles(m) : 1;
+    size_t off = 0;
+    char* b = (char*)base;
+    if (ws) ws->hist = (uint32_t*)(b + off);
+    off += os_align((size_t)passes * kOsRadix * 4);
+    if (ws) ws->tickets = (uint32_t*)(b + off);
+    off += os_align((size_t)passes * 4);
+    if (ws) ws->error = (uint32_t*)(b + off);
+    off += 256;
+    if (ws) ws->status = (uint32_t*)(b + off);
+    off += os_align((size_t)passes * ntiles * kOsRadix * 4);
+    return off;
+}
+
+}  // namespace d3gs
+
+using namespace d3gs;
+
+extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* bytes_out_host) {
+    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !bytes_out_host) {
+        set_error("d3gs_sort_workspace_bytes: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const int passes = os_passes(begin_bit, end_bit) > 0 ? os_passes(begin_bit, end_bit) : 1;
+    *bytes_out_host = os_layout(m, passes, nullptr, nullptr);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                               size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                               d3gs_stream_t stream) {
+    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !result_in_b_host) {
+        set_error("d3gs_sort_pairs: bad argument (m=%lld bits=[%d,%d))", (long long)m, begin_bit, end_bit);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (m >= (1ll << 30)) { set_error("d3gs_sort_pairs: m >= 2^30 is not supported"); return D3GS_ERR_UNSUPPORTED; }
+    *result_in_b_host = 0;
+    if (m == 0 || begin_bit == end_bit) return D3GS_OK;
+    if (!keys_a || !keys_b || !vals_a || !vals_b || !workspace) {
+        set_error("d3gs_sort_pairs: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const int passes = os_passes(begin_bit, end_bit);
+    SortWorkspace ws;
+    const size_t need = os_layout(m, passes, &ws, workspace);
+    if (workspace_bytes < need) {
+        set_error("d3gs_sort_pairs: workspace %zu < required %zu", workspace_bytes, need);
+        return D3GS_ERR_WORKSPACE_TOO_SMALL;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const int ntiles = os_tiles(m);
+    // a fill kernel, not a memset node, so the call can be captured in a graph
+    hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
+    const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
+    hipLaunchKernelGGL(os_hist_kernel, dim3(hist_blocks), dim3(kHistThreads),
+                       (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m, begin_bit,
+                       end_bit, passes, ws.hist);
+    uint64_t* kin = keys_a;
+    uint64_t* kout = keys_b;
+    int32_t* vin = vals_a;
+    int32_t* vout = vals_b;
+    int in_b = 0;
+    for (int p = 0; p < passes; ++p) {
+        const int bit = begin_bit + 8 * p;
+        const int nb = std::min(8, end_bit - bit);
+        const uint32_t mask = (1u << nb) - 1u;
+        hipLaunchKernelGGL(os_pass_kernel, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m, bit,
+                           mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
+                           ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
+        std::swap(kin, kout);
+        std::swap(vin, vout);
+        in_b ^= 1;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_sort_pairs: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    *result_in_b_host = in_b;
+    return D3GS_OK;
+}
