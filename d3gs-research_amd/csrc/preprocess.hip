@@ -144,18 +144,19 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
 // ---------------------------------------------------------------------------
 // Preprocess backward.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
-    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
-    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
-    const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ duv, const float* __restrict__ dconic, const float* dopacity_in /* may alias dopacity_out */,
+// One gaussian of the preprocess backward.  `shrow` is this gaussian's SH row staged in LDS: it holds
+// the coefficients on entry and receives their gradients (each channel's coefficients are read into
+// registers before that channel's gradients overwrite them).
+__device__ __forceinline__ void preprocess_bwd_one(
+    const d3gs_params& P, const int i, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const float* __restrict__ scale, const float* __restrict__ opacity, const int32_t* __restrict__ radii,
+    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0, const float* __restrict__ duv,
+    const float* __restrict__ dconic, const float* dopacity_in /* may alias dopacity_out */,
     const float* __restrict__ dcolor, const float* __restrict__ dz_in, const int sh_mask_compat,
-    float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale,
-    float* dopacity_out, float* __restrict__ dsh, float* __restrict__ dsh_base) {
-    const int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i >= P.n) return;
+    float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
+    float* shrow, float* __restrict__ dsh_base) {
     const int K = P.sh_stride;
-    float* dshp = dsh + (size_t)i * K * 3;
+    float* dshp = shrow;
 
     if (radii[i] == 0) {
         dxyz[3 * i] = dxyz[3 * i + 1] = dxyz[3 * i + 2] = 0.0f;
@@ -284,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
         cg[1] = dcolor[3 * i + 1] * ((m & 2) ? 0.0f : 1.0f);
         cg[2] = dcolor[3 * i + 2] * ((m & 1) ? 0.0f : 1.0f);
     }
-    const float* shp = sh + (size_t)i * K * 3;
+    const float* shp = shrow;
     const float* rest = P.has_sh_base ? shp : shp + 3;
     float* drest = P.has_sh_base ? dshp : dshp + 3;
     float* dbase = P.has_sh_base ? dsh_base + 3 * i : dshp;
@@ -300,15 +301,18 @@ __global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
 #pragma unroll
     for (int ch = 0; ch < 3; ++ch) {
         float gch = cg[ch];
+        float sv[15];
+#pragma unroll
+        for (int k = 0; k < 15; ++k) sv[k] = k < used ? rest[k * 3 + ch] : 0.0f;
         dbase[ch] = kShC0 * gch;
         float dx_ = 0.0f, dy_ = 0.0f, dz_ = 0.0f;
         if (deg > 0) {
             drest[0 * 3 + ch] = (-kShC1 * y) * gch;
             drest[1 * 3 + ch] = (kShC1 * zd) * gch;
             drest[2 * 3 + ch] = (-kShC1 * x) * gch;
-            dx_ = -kShC1 * rest[2 * 3 + ch];
-            dy_ = -kShC1 * rest[0 * 3 + ch];
-            dz_ = kShC1 * rest[1 * 3 + ch];
+            dx_ = -kShC1 * sv[2];
+            dy_ = -kShC1 * sv[0];
+            dz_ = kShC1 * sv[1];
             if (deg > 1) {
                 float xx = x * x, yy = y * y, zz2 = zd * zd, xy = x * y, yz = y * zd, xz = x * zd;
                 drest[3 * 3 + ch] = (kShC2[0] * xy) * gch;
@@ -316,8 +320,8 @@ __global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
                 drest[5 * 3 + ch] = (kShC2[2] * ((2.0f * zz2 - xx) - yy)) * gch;
                 drest[6 * 3 + ch] = (kShC2[3] * xz) * gch;
                 drest[7 * 3 + ch] = (kShC2[4] * (xx - yy)) * gch;
-                float s3 = rest[3 * 3 + ch], s4 = rest[4 * 3 + ch], s5 = rest[5 * 3 + ch], s6 = rest[6 * 3 + ch],
-                      s7 = rest[7 * 3 + ch];
+                float s3 = sv[3], s4 = sv[4], s5 = sv[5], s6 = sv[6],
+                      s7 = sv[7];
                 dx_ += kShC2[0] * y * s3 + kShC2[2] * 2.0f * (-x) * s5 + kShC2[3] * zd * s6 + kShC2[4] * 2.0f * x * s7;
                 dy_ += kShC2[0] * x * s3 + kShC2[1] * zd * s4 + kShC2[2] * 2.0f * (-y) * s5 + kShC2[4] * 2.0f * (-y) * s7;
                 dz_ += kShC2[1] * y * s4 + kShC2[2] * 2.0f * 2.0f * zd * s5 + kShC2[3] * x * s6;
@@ -329,9 +333,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
                     drest[12 * 3 + ch] = ((kShC3[4] * x) * ((4.0f * zz2 - xx) - yy)) * gch;
                     drest[13 * 3 + ch] = ((kShC3[5] * zd) * (xx - yy)) * gch;
                     drest[14 * 3 + ch] = ((kShC3[6] * x) * (xx - 3.0f * yy)) * gch;
-                    float s8 = rest[8 * 3 + ch], s9 = rest[9 * 3 + ch], s10 = rest[10 * 3 + ch],
-                          s11 = rest[11 * 3 + ch], s12 = rest[12 * 3 + ch], s13 = rest[13 * 3 + ch],
-                          s14 = rest[14 * 3 + ch];
+                    float s8 = sv[8], s9 = sv[9], s10 = sv[10],
+                          s11 = sv[11], s12 = sv[12], s13 = sv[13],
+                          s14 = sv[14];
                     dx_ += kShC3[0] * s8 * 3.0f * 2.0f * xy + kShC3[1] * s9 * yz + kShC3[2] * s10 * (-2.0f) * xy +
                            kShC3[3] * s11 * (-3.0f) * 2.0f * xz + kShC3[4] * s12 * ((-3.0f) * xx + 4.0f * zz2 - yy) +
                            kShC3[5] * s13 * 2.0f * xz + kShC3[6] * s14 * 3.0f * (xx - yy);
@@ -354,6 +358,81 @@ __global__ __launch_bounds__(kBlock) void preprocess_bwd_kernel(
     dxyz[3 * i + 0] = gx[0] + (ddir[0] - dirv[0] * dd) / dn;
     dxyz[3 * i + 1] = gx[1] + (ddir[1] - dirv[1] * dd) / dn;
     dxyz[3 * i + 2] = gx[2] + (ddir[2] - dirv[2] * dd) / dn;
+}
+
+constexpr int kBwdBlock = 128;  // gaussians (= threads) per workgroup of the backward kernel
+
+// Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
+// consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
+// different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
+__device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
+                                                   int stride) {
+    const int total = nrows * rowlen;
+    const float inv = 1.0f / (float)rowlen;
+    const bool vec = ((uintptr_t)src & 15u) == 0;
+    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kBwdBlock * 4) {
+        float v[4];
+        if (vec && e4 + 3 < total) {
+            const float4 t = *reinterpret_cast<const float4*>(src + e4);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = e4 + c < total ? src[e4 + c] : 0.0f;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int e = e4 + c;
+            if (e < total) {
+                const int g = (int)(((float)e + 0.5f) * inv);
+                lds[g * stride + (e - g * rowlen)] = v[c];
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, const float* lds, int nrows, int rowlen,
+                                                   int stride) {
+    const int total = nrows * rowlen;
+    const float inv = 1.0f / (float)rowlen;
+    const bool vec = ((uintptr_t)dst & 15u) == 0;
+    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kBwdBlock * 4) {
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int e = min(e4 + c, total - 1);
+            const int g = (int)(((float)e + 0.5f) * inv);
+            v[c] = lds[g * stride + (e - g * rowlen)];
+        }
+        if (vec && e4 + 3 < total) {
+            *reinterpret_cast<float4*>(dst + e4) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (e4 + c < total) dst[e4 + c] = v[c];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
+    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
+    const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
+    const float* __restrict__ duv, const float* __restrict__ dconic, const float* dopacity_in,
+    const float* __restrict__ dcolor, const float* __restrict__ dz_in, const int sh_mask_compat,
+    float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
+    float* __restrict__ dsh, float* __restrict__ dsh_base) {
+    extern __shared__ float s_rows[];
+    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    const int first = blockIdx.x * kBwdBlock;
+    const int nrows = min(kBwdBlock, P.n - first);
+    rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
+    __syncthreads();
+    if ((int)threadIdx.x < nrows)
+        preprocess_bwd_one(P, first + threadIdx.x, xyz, quat, scale, opacity, radii, cov2d, ne0, duv, dconic,
+                           dopacity_in, dcolor, dz_in, sh_mask_compat, dxyz, dquat, dscale, dopacity_out,
+                           s_rows + threadIdx.x * stride, dsh_base);
+    __syncthreads();
+    rows_lds_to_global(dsh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
 }
 
 int check_params(const d3gs_params* p, const char* who) {
@@ -429,10 +508,12 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
-    hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
-                       opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, duv, dconic, dopacity_in, dcolor, dz,
-                       (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
+    dim3 grid((p->n + kBwdBlock - 1) / kBwdBlock), block(kBwdBlock);
+    const size_t lds_bytes = (size_t)kBwdBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
+                       scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, duv, dconic, dopacity_in, dcolor,
+                       dz, (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
+                       dcolor_sh_base);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
