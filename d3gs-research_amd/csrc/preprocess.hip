@@ -1,7 +1,8 @@
 // Per-gaussian kernels: preprocess forward (projection, EWA covariance, conic,
 // radius, tile count, SH colour) and preprocess backward (chain rule back to the
-// raw model tensors).  One thread per gaussian, 256-thread blocks; both are
-// single streaming passes bound by HBM bandwidth.
+// raw model tensors).  One thread per gaussian, 128-thread workgroups whose SH rows
+// (and SH gradient rows) pass through LDS so that global traffic is coalesced; both
+// are single streaming passes bound by HBM bandwidth.
 //
 // Reference: d3sim/algos/d3gs/render.py:421-476, 569-619 (forward) and
 // 3217-3356 (backward); math in d3sim/csrc/gs3d.py and d3sim/csrc/camera.py.
@@ -36,14 +37,75 @@ __device__ __forceinline__ float sh_channel(int degree, float x, float y, float 
     return r + 0.5f;
 }
 
-__global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
+constexpr int kPrepBlock = 128;  // gaussians (= threads) per workgroup of the per-gaussian kernels
+
+// Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
+// consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
+// different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
+__device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
+                                                   int stride) {
+    const int total = nrows * rowlen;
+    const float inv = 1.0f / (float)rowlen;
+    const bool vec = ((uintptr_t)src & 15u) == 0;
+    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
+        float v[4];
+        if (vec && e4 + 3 < total) {
+            const float4 t = *reinterpret_cast<const float4*>(src + e4);
+            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = e4 + c < total ? src[e4 + c] : 0.0f;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int e = e4 + c;
+            if (e < total) {
+                const int g = (int)(((float)e + 0.5f) * inv);
+                lds[g * stride + (e - g * rowlen)] = v[c];
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, const float* lds, int nrows, int rowlen,
+                                                   int stride) {
+    const int total = nrows * rowlen;
+    const float inv = 1.0f / (float)rowlen;
+    const bool vec = ((uintptr_t)dst & 15u) == 0;
+    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
+        float v[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int e = min(e4 + c, total - 1);
+            const int g = (int)(((float)e + 0.5f) * inv);
+            v[c] = lds[g * stride + (e - g * rowlen)];
+        }
+        if (vec && e4 + 3 < total) {
+            *reinterpret_cast<float4*>(dst + e4) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (e4 + c < total) dst[e4 + c] = v[c];
+        }
+    }
+}
+
+__global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const float* __restrict__ sh_base, float* __restrict__ depths, int32_t* __restrict__ radii,
     float* __restrict__ uvs, float* __restrict__ conic_opacity, int32_t* __restrict__ tiles_touched,
     float* __restrict__ rgb_out, float* __restrict__ cov2d_out, uint8_t* __restrict__ ne0_out) {
+    // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
+    extern __shared__ float s_rows[];
+    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    {
+        const int first = blockIdx.x * kPrepBlock;
+        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P.n - first), rowlen, stride);
+    }
+    __syncthreads();
     // no early return: every lane of the wavefront takes part in the cooperative tile count
-    const int i_raw = blockIdx.x * kBlock + threadIdx.x;
+    const int i_raw = blockIdx.x * kPrepBlock + threadIdx.x;
     const bool in_range = i_raw < P.n;
     const int i = in_range ? i_raw : P.n - 1;
 
@@ -112,7 +174,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_fwd_kernel(
     if (valid) {
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
         float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
-        const float* shp = sh + (size_t)i * P.sh_stride * 3;
+        const float* shp = s_rows + threadIdx.x * stride;
         const float* base = P.has_sh_base ? sh_base + 3 * i : shp;
         const float* rest = P.has_sh_base ? shp : shp + 3;
 #pragma unroll
@@ -360,60 +422,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
     dxyz[3 * i + 2] = gx[2] + (ddir[2] - dirv[2] * dd) / dn;
 }
 
-constexpr int kBwdBlock = 128;  // gaussians (= threads) per workgroup of the backward kernel
-
-// Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
-// consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
-// different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
-__device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
-                                                   int stride) {
-    const int total = nrows * rowlen;
-    const float inv = 1.0f / (float)rowlen;
-    const bool vec = ((uintptr_t)src & 15u) == 0;
-    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kBwdBlock * 4) {
-        float v[4];
-        if (vec && e4 + 3 < total) {
-            const float4 t = *reinterpret_cast<const float4*>(src + e4);
-            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) v[c] = e4 + c < total ? src[e4 + c] : 0.0f;
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int e = e4 + c;
-            if (e < total) {
-                const int g = (int)(((float)e + 0.5f) * inv);
-                lds[g * stride + (e - g * rowlen)] = v[c];
-            }
-        }
-    }
-}
-
-__device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, const float* lds, int nrows, int rowlen,
-                                                   int stride) {
-    const int total = nrows * rowlen;
-    const float inv = 1.0f / (float)rowlen;
-    const bool vec = ((uintptr_t)dst & 15u) == 0;
-    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kBwdBlock * 4) {
-        float v[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int e = min(e4 + c, total - 1);
-            const int g = (int)(((float)e + 0.5f) * inv);
-            v[c] = lds[g * stride + (e - g * rowlen)];
-        }
-        if (vec && e4 + 3 < total) {
-            *reinterpret_cast<float4*>(dst + e4) = make_float4(v[0], v[1], v[2], v[3]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                if (e4 + c < total) dst[e4 + c] = v[c];
-        }
-    }
-}
-
-__global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
+__global__ __launch_bounds__(kPrepBlock) void preprocess_bwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
@@ -423,8 +432,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     extern __shared__ float s_rows[];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
-    const int first = blockIdx.x * kBwdBlock;
-    const int nrows = min(kBwdBlock, P.n - first);
+    const int first = blockIdx.x * kPrepBlock;
+    const int nrows = min(kPrepBlock, P.n - first);
     rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
     __syncthreads();
     if ((int)threadIdx.x < nrows)
@@ -483,8 +492,9 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
-    hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
+    dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
+    const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
                        opacity, color_sh, color_sh_base, depths, radii, uvs, conic_opacity, tiles_touched,
                        rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0);
     hipError_t e = hipGetLastError();
@@ -508,8 +518,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    dim3 grid((p->n + kBwdBlock - 1) / kBwdBlock), block(kBwdBlock);
-    const size_t lds_bytes = (size_t)kBwdBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
+    const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
     hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
                        scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, duv, dconic, dopacity_in, dcolor,
                        dz, (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
