@@ -28,8 +28,20 @@ namespace d3gs {
 
 struct __attribute__((aligned(16))) StagedGaussian {
     float x, y, thr, pad;   // pixel-space centre, cull threshold
-    float a, b, c, o;       // conic (a, b, c) and opacity
+    float ha, nb, hc, o;    // pre-scaled conic (-a/2, -b, -c/2) and opacity
 };
+
+// power = -1/2 (a dx^2 + c dy^2) - b dx dy (render.py:1765-1767) as a fixed sequence of three
+// multiplies and two fused multiply-adds; a CPU evaluating the same sequence gets the same bits.
+__device__ __forceinline__ float blend_power(const StagedGaussian& g, float dx, float dy) {
+    return __builtin_fmaf(g.nb * dx, dy, __builtin_fmaf(g.hc * dy, dy, (g.ha * dx) * dx));
+}
+
+// exp for an argument that already passed `x >= thr` (so x > -86 and x is not NaN)
+__device__ __forceinline__ float blend_expf(float x) {
+    const float e = det_expf_inrange(x);
+    return x > 88.0f ? __builtin_inff() : e;
+}
 
 // Tile index for a workgroup.  Tile list lengths are heavily skewed (dense screen regions hold
 // lists 20x the median), so the launch order matters more than L2 locality: with `tile_order`
@@ -126,9 +138,9 @@ __device__ __forceinline__ uint32_t stage_gaussian(const d3gs_params& P, int g, 
     s.y = xy.y;
     s.thr = __logf(P.alpha_eps / co.w) - 1.0e-3f;
     s.pad = 0.0f;
-    s.a = co.x;
-    s.b = co.y;
-    s.c = co.z;
+    s.ha = -0.5f * co.x;  // exact scalings: power = (ha dx) dx + (hc dy) dy + (nb dx) dy
+    s.nb = -co.y;
+    s.hc = -0.5f * co.z;
     s.o = co.w;
     *dst = s;
     // Level set {power >= thr}: a dx^2 + 2 b dx dy + c dy^2 <= R with R = -2 thr.  A pixel of this tile
@@ -223,9 +235,9 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 m &= m - 1;
                 const StagedGaussian sg = s_g[j];
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
-                const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
+                const float power = blend_power(sg, dx, dy);
                 if (!done && power >= sg.thr) {
-                    const float G = det_expf(power);
+                    const float G = blend_expf(power);
                     const float alpha = fminf(0.99f, sg.o * G);
                     if (alpha >= P.alpha_eps) {
                         const float nextT = T * (1.0f - alpha);
@@ -237,9 +249,9 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                             T = nextT;
                             contributor = round * kBlock + j;
                             const float4 c = s_rgb[j];
-                            acc0 = acc0 + w * c.x;
-                            acc1 = acc1 + w * c.y;
-                            acc2 = acc2 + w * c.z;
+                            acc0 = __builtin_fmaf(w, c.x, acc0);
+                            acc1 = __builtin_fmaf(w, c.y, acc1);
+                            acc2 = __builtin_fmaf(w, c.z, acc2);
                         }
                     }
                 }
@@ -351,35 +363,43 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             m &= m - 1;
             const StagedGaussian sg = s_g[j];
             const float dx = sg.x - pxf, dy = sg.y - pyf;
-            const float power = (-0.5f * ((sg.a * dx) * dx + (sg.c * dy) * dy)) - (sg.b * dx) * dy;
+            const float power = blend_power(sg, dx, dy);
             const bool cand = (round * kBlock + j < contributor) && power >= sg.thr && power <= 0.0f;
             if (!__any(cand)) continue;
             float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, g3 = 0.0f, g4 = 0.0f, g5 = 0.0f, g6 = 0.0f, g7 = 0.0f, g8 = 0.0f;
             bool valid = false;
             if (cand) {
-                const float G = det_expf(power);
+                // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
+                // gaussian contributed to.  The per-pixel terms below also follow one fixed sequence of
+                // fused multiply-adds (the colour still behind, T c - rr, cancels heavily, so a different
+                // rounding would already move a term by ~1e-4): only the order of the sums over pixels
+                // differs from a sequential evaluation.
+                const float G = blend_expf(power);
                 const float alpha = fminf(0.99f, sg.o * G);
                 if (alpha >= P.alpha_eps) {
                     valid = true;
-                    const float nextT = T * (1.0f - alpha);
+                    const float one_m = 1.0f - alpha;
                     const float w = alpha * T;
-                    T = nextT;
+                    T = T * one_m;
                     const float4 c = s_rgb[j];
-                    rr0 = rr0 - w * c.x;
-                    rr1 = rr1 - w * c.y;
-                    rr2 = rr2 - w * c.z;
-                    float dl = ((dr0 * (T * c.x - rr0) + dr1 * (T * c.y - rr1)) + dr2 * (T * c.z - rr2));
-                    dl = dl + dT_term;
-                    const float dL_dalpha = dl / (1.0f - alpha);
+                    rr0 = __builtin_fmaf(-w, c.x, rr0);
+                    rr1 = __builtin_fmaf(-w, c.y, rr1);
+                    rr2 = __builtin_fmaf(-w, c.z, rr2);
+                    float dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dT_term);
+                    dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
+                    dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
+                    const float dL_dalpha = dl / one_m;
                     const float dL_dG = sg.o * dL_dalpha;
                     const float gdx = G * dx, gdy = G * dy;
-                    const float dG_du = (-gdx) * sg.a - gdy * sg.b;
-                    const float dG_dv = (-gdy) * sg.c - gdx * sg.b;
+                    // dG/du = -gdx a - gdy b and dG/dv = -gdy c - gdx b, with a = -2 ha, b = -nb, c = -2 hc
+                    const float dG_du = __builtin_fmaf(gdy, sg.nb, (2.0f * gdx) * sg.ha);
+                    const float dG_dv = __builtin_fmaf(gdx, sg.nb, (2.0f * gdy) * sg.hc);
+                    const float half = -0.5f * dL_dG;
                     g0 = dL_dG * dG_du;
                     g1 = dL_dG * dG_dv;
-                    g2 = ((-0.5f) * gdx) * dx * dL_dG;
-                    g3 = ((-gdx) * dy) * dL_dG;
-                    g4 = ((-0.5f) * gdy) * dy * dL_dG;
+                    g2 = (half * gdx) * dx;
+                    g3 = ((-dL_dG) * gdx) * dy;
+                    g4 = (half * gdy) * dy;
                     g5 = dL_dalpha * G;
                     g6 = w * dr0;
                     g7 = w * dr1;

