@@ -25,6 +25,10 @@ CASES = [
     (2, 100000, (640, 360), AABB),
     (3, 100000, (480, 270), OBB),
     (4, 30000, (960, 540), AABB),
+    # BASELINE.json's full sizes (the CPU oracle renders these in a few seconds on the box's host cores)
+    (2, None, None, DFVT),
+    (3, None, None, AABB),
+    (4, None, None, DFVT),
 ]
 
 
@@ -86,7 +90,8 @@ def test_inference_path(oracle, cfg_id, n, wh, filt):
 
 @pytest.mark.parametrize("cfg_id,n,wh,filt", [(0, None, None, AABB), (0, None, None, NONE), (1, None, None, AABB),
                                               (1, 20000, (250, 190), OBB), (2, 100000, (640, 360), AABB),
-                                              (4, 30000, (960, 540), AABB)])
+                                              (4, 30000, (960, 540), AABB), (2, None, None, DFVT),
+                                              (4, None, None, AABB)])
 def test_backward_parity(oracle, cfg_id, n, wh, filt):
     import torch
     from d3gs_research_amd.render import GaussianSplatGradients
