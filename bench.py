@@ -25,7 +25,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
 # algorithmic HBM bytes per stage: N gaussians, M (tile, gaussian) pairs, P pixels, T tiles
 STAGE_BYTES = {
     "preprocess": lambda N, M, P, T, passes: 297 * N,
-    "scan": lambda N, M, P, T, passes: 8 * N,
+    "depth_order": lambda N, M, P, T, passes: (4 + 12) * N + (8 + 24 * 4) * N,
+    "scan": lambda N, M, P, T, passes: (12 + 8) * N,
     "make_keys": lambda N, M, P, T, passes: 36 * N + 12 * M,
     "sort": lambda N, M, P, T, passes: (8 + 24 * passes) * M,
     "tile_ranges": lambda N, M, P, T, passes: 8 * M + 8 * T,

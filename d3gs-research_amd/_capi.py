@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Params(C.Structure):
@@ -42,7 +42,9 @@ _SIGNATURES = {
     "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 14 + [_VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
-    "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 7 + [C.c_int64, _VP]),
+    "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 8 + [C.c_int64, _VP]),
+    "d3gs_depth_keys": (C.c_int, [_VP, C.c_int32, _VP, _VP, _VP]),
+    "d3gs_gather_i32": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP]),
     "d3gs_sort_workspace_bytes": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
     "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
                                   C.POINTER(C.c_int), _VP]),

@@ -94,17 +94,23 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             const float* __restrict__ conic_opacity,
                                                             const float* __restrict__ depths,
                                                             const int32_t* __restrict__ offsets,
+                                                            const int32_t* __restrict__ order,
                                                             uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
     // no early return: every lane takes part in the cooperative emission of large gaussians
-    const int i_raw = blockIdx.x * kBlock + threadIdx.x;
-    const bool in_range = i_raw < P.n;
-    const int i = in_range ? i_raw : P.n - 1;
+    const int j_raw = blockIdx.x * kBlock + threadIdx.x;
+    const bool in_range = j_raw < P.n;
+    const int j = in_range ? j_raw : P.n - 1;
+    // slot j of the emission order holds gaussian order[j] (identity without an order table);
+    // `offsets` is the inclusive scan of the tile counts taken in that same order
+    int i = order ? order[j] : j;
+    const bool sane = (unsigned)i < (unsigned)P.n;
+    i = sane ? i : 0;
     const int r = radii[i];
-    long long off = i == 0 ? 0 : offsets[i - 1];
-    const long long end = offsets[i];
+    long long off = j == 0 ? 0 : offsets[j - 1];
+    const long long end = offsets[j];
     // a caller that passed a smaller buffer than the scan total must never be written past
-    const bool active = in_range && r > 0 && end <= m;
+    const bool active = in_range && sane && r > 0 && end <= m;
     const uint32_t dbits = __float_as_uint(depths[i]);
     const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
     const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
@@ -112,6 +118,25 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     TileWalk walk = {};
     if (active) walk = tile_walk_setup(P, g);
     wave_tile_emit(P.filter_algo, active, walk, P.tiles_x, dbits, i, off, end, keys, vals);
+}
+
+// Sort keys of the gaussians themselves: the float bits of the depth (positive floats order like
+// their bit patterns), value = gaussian index.
+__global__ __launch_bounds__(kBlock) void depth_keys_kernel(const float* __restrict__ depths, int n,
+                                                             uint64_t* __restrict__ keys, int32_t* __restrict__ idx) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    keys[i] = (uint64_t)__float_as_uint(depths[i]);
+    idx[i] = i;
+}
+
+__global__ __launch_bounds__(kBlock) void gather_i32_kernel(const int32_t* __restrict__ src,
+                                                             const int32_t* __restrict__ index, int n, int src_n,
+                                                             int32_t* __restrict__ dst) {
+    const int j = blockIdx.x * kBlock + threadIdx.x;
+    if (j >= n) return;
+    const int i = index[j];
+    dst[j] = (unsigned)i < (unsigned)src_n ? src[i] : 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -214,8 +239,8 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
 }
 
 extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
-                              const float* depths, const int32_t* offsets, uint64_t* keys, int32_t* gaussian_idx,
-                              int64_t m, d3gs_stream_t stream) {
+                              const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                              uint64_t* keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
@@ -225,9 +250,33 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     hipLaunchKernelGGL(make_keys_kernel, dim3((p->n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                       radii, uvs, conic_opacity, depths, offsets, keys, gaussian_idx, (long long)m);
+                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, keys, gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_depth_keys(const float* depths, int32_t n, uint64_t* keys, int32_t* gaussian_idx,
+                               d3gs_stream_t stream) {
+    if (n < 0) { set_error("d3gs_depth_keys: n < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (n == 0) return D3GS_OK;
+    if (!depths || !keys || !gaussian_idx) { set_error("d3gs_depth_keys: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
+    hipLaunchKernelGGL(depth_keys_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, depths,
+                       (int)n, keys, gaussian_idx);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_depth_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* dst,
+                               d3gs_stream_t stream) {
+    if (n < 0 || src_n < 0) { set_error("d3gs_gather_i32: bad size"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (n == 0) return D3GS_OK;
+    if (!src || !index || !dst) { set_error("d3gs_gather_i32: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
+    hipLaunchKernelGGL(gather_i32_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, src,
+                       index, (int)n, (int)src_n, dst);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_gather_i32: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 2
+#define D3GS_ABI_VERSION 3
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -99,10 +99,27 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
                     d3gs_stream_t stream);
 
 /* K3 — replaces kernel_1d("prepare_sort_data_...") at render.py:739-840.
- * offsets = the inclusive scan from d3gs_scan_tiles; m = its total. */
+ * Without gaussian_order (NULL) this is the reference's call: offsets = the inclusive
+ * scan of tiles_touched from d3gs_scan_tiles, m = its total, pairs are emitted in
+ * gaussian-index order.  With gaussian_order (a permutation of 0..n-1), slot j emits
+ * gaussian gaussian_order[j] and offsets must be the inclusive scan of the tile counts
+ * taken in that order (see d3gs_depth_keys). */
 int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
-                   const float* depths, const int32_t* offsets, uint64_t* keys, int32_t* gaussian_idx, int64_t m,
-                   d3gs_stream_t stream);
+                   const float* depths, const int32_t* offsets, const int32_t* gaussian_order, uint64_t* keys,
+                   int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
+
+/* Depth-first factorisation of the pair sort (no counterpart in the reference, which
+ * radix-sorts all M pairs on the full (tile, depth) key; the result is bit-identical).
+ * An LSD radix sort is a chain of stable sorts from the least significant digit up, and
+ * the depth digits only depend on the gaussian, so: sort the N gaussians by depth bits
+ * (d3gs_depth_keys + d3gs_sort_pairs on bits [0, 32)), emit the pairs in that order
+ * (d3gs_gather_i32 of the tile counts, d3gs_scan_tiles, d3gs_make_keys with
+ * gaussian_order) and run only the tile digits, bits [32, end_bit), over the M pairs.
+ *   d3gs_depth_keys: keys[i] = float bits of depths[i] (zero-extended), gaussian_idx[i] = i
+ *   d3gs_gather_i32: dst[j] = src[index[j]] (0 for an index outside [0, src_n)) */
+int d3gs_depth_keys(const float* depths, int32_t n, uint64_t* keys, int32_t* gaussian_idx, d3gs_stream_t stream);
+int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* dst,
+                    d3gs_stream_t stream);
 
 /* K4 — replaces DeviceSort.get_sort_workspace_size / do_radix_sort_with_bit_range
  * (devsort.py:38-129; call site render.py:846-887).  Stable LSD radix sort of
