@@ -51,24 +51,6 @@ __device__ __forceinline__ int tile_for_block(int bid, const int32_t* __restrict
     return tile_order ? tile_order[bid] : bid;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-    // butterfly inside each row of 16 lanes with DPP, then add the 4 row sums
-    int x = __float_as_int(v);
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
-    x = __float_as_int(v);
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
-    x = __float_as_int(v);
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x141, 0xF, 0xF, false));  // row_half_mirror
-    x = __float_as_int(v);
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x140, 0xF, 0xF, false));  // row_mirror
-    x = __float_as_int(v);
-    float r0 = __int_as_float(__builtin_amdgcn_readlane(x, 0));
-    float r1 = __int_as_float(__builtin_amdgcn_readlane(x, 16));
-    float r2 = __int_as_float(__builtin_amdgcn_readlane(x, 32));
-    float r3 = __int_as_float(__builtin_amdgcn_readlane(x, 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
 // ---------------------------------------------------------------------------
 // Sum of nine per-lane values over the wavefront, as a transposing reduction:
 // every step exchanges halves so that the number of live registers halves with
