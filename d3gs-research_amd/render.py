@@ -367,10 +367,12 @@ class GaussianSplatOp:
         drgb = grad.drgb
         assert drgb.is_contiguous(), "drgb must be contiguous"
         assert grad.dT.is_contiguous(), "dT must be contiguous"
-        duv = torch.zeros((n, 2), dtype=torch.float32, device=dev)
-        dconic = torch.zeros((n, 3), dtype=torch.float32, device=dev)
-        dopacity = torch.zeros(n, dtype=torch.float32, device=dev)
-        dcolor = torch.zeros((n, 3), dtype=torch.float32, device=dev)
+        # the four accumulators are contiguous slices of one buffer: one zero-fill launch instead of four
+        acc = torch.zeros(9 * n, dtype=torch.float32, device=dev)
+        duv = acc[0:2 * n].view(n, 2)
+        dconic = acc[2 * n:5 * n].view(n, 3)
+        dopacity = acc[5 * n:6 * n]
+        dcolor = acc[6 * n:9 * n].view(n, 3)
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
             _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order), _capi.ptr(out.T),

@@ -1,0 +1,49 @@
+"""The operator used the way the reference's trainer uses it (d3sim/algos/d3gs/train.py:162-177):
+rasterize_gaussians(model, cam, op, training=True, uv_grad_holder=h) -> loss -> loss.backward()
+-> optimizer step.  A perturbed copy of a scene must move back towards the image of the original."""
+import numpy as np
+import pytest
+
+from helpers import gen_scene, op_config, torch_model
+
+pytestmark = pytest.mark.gpu
+
+
+def test_adam_steps_reduce_the_image_loss():
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp, rasterize_gaussians
+
+    scene = gen_scene(1, n=20000, wh=(256, 256))
+    cam = scene.camera()
+    op = GaussianSplatOp(op_config(scene, 4))          # the reference's default filter (OBB_DFVT)
+    target_model = torch_model(scene)
+    with torch.no_grad():
+        target = rasterize_gaussians(target_model, cam, op, training=True).color.clone()
+
+    model = torch_model(scene)
+    model.act_applied = False
+    g = torch.Generator(device="cuda").manual_seed(3)
+    with torch.no_grad():
+        model.xyz += 0.01 * torch.randn(model.xyz.shape, generator=g, device="cuda")
+        model.scale += 0.1 * torch.randn(model.scale.shape, generator=g, device="cuda")
+        model.opacity += 0.3 * torch.randn(model.opacity.shape, generator=g, device="cuda")
+        model.color_sh += 0.05 * torch.randn(model.color_sh.shape, generator=g, device="cuda")
+    model.set_requires_grad(True)
+    params = [model.xyz, model.scale, model.quaternion_xyzw, model.opacity, model.color_sh]
+    opt = torch.optim.Adam([{"params": [model.xyz], "lr": 2e-4}, {"params": [model.scale], "lr": 5e-3},
+                            {"params": [model.quaternion_xyzw], "lr": 1e-3}, {"params": [model.opacity], "lr": 2e-2},
+                            {"params": [model.color_sh], "lr": 2.5e-3}])
+    losses = []
+    for step in range(40):
+        holder = torch.zeros((1, scene.n, 2), device="cuda", requires_grad=True)
+        out = rasterize_gaussians(model, cam, op, training=True, uv_grad_holder=holder)
+        loss = (out.color - target).abs().mean()
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        assert all(p.grad is not None and bool(torch.isfinite(p.grad).all()) for p in params)
+        assert holder.grad is not None and holder.grad.shape == (1, scene.n, 2)   # the densification signal
+        opt.step()
+        losses.append(float(loss))
+    print("L1 loss: first %.5f  last %.5f" % (losses[0], losses[-1]), flush=True)
+    assert losses[-1] < 0.6 * losses[0]
+    assert np.isfinite(losses).all()
