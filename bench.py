@@ -18,7 +18,6 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
 
@@ -83,16 +82,15 @@ def main():
         print(json.dumps({"calibration": "torch.mul(x, 1.0, out=y)", "read_bytes": x.numel() * 4,
                           "write_bytes": y.numel() * 4, "launches": 5}))
         return
-    from helpers import op_config, oracle_params, torch_model
     from d3gs_research_amd.config_def import EarlyFilterAlgo
     from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
-    from d3gs_research_amd.synthetic import gen_scene
+    from d3gs_research_amd.synthetic import gen_scene, scene_config, scene_model
 
     filt = EarlyFilterAlgo[args.filter]
     scene = gen_scene(args.config)
     cam = scene.camera()
-    op = GaussianSplatOp(op_config(scene, filt))
-    model = torch_model(scene, "cuda:0")
+    op = GaussianSplatOp(scene_config(scene, filt))
+    model = scene_model(scene, "cuda:0")
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
 
     def step():
@@ -135,7 +133,7 @@ def main():
         from oracle import d3gs_oracle as O
         O.build()
         cs = scene if args.cpu_n in (0, scene.n) else gen_scene(args.config, n=args.cpu_n)
-        Pc = oracle_params(O, cs, int(filt))
+        Pc = O.params_for_scene(cs, int(filt))
         # repeat whole views until ~10 s of CPU work has been spent (at most 12 views); report the median
         fwd_ms, bwd_ms = [], []
         t_start = time.perf_counter()

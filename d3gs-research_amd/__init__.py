@@ -5,7 +5,7 @@ HIP kernels in ``csrc/`` (C ABI in ``include/d3gs_hip.h``).
 """
 from .config_def import EarlyFilterAlgo, GaussianSplatConfig, RasterizeBackwardAlgo  # noqa: F401
 from .camera import BasicPinholeCamera, Pose  # noqa: F401
-from .model import GaussianModelOriginBase, GaussianModelOriginFused  # noqa: F401
+from .model import GaussianModelOrigin, GaussianModelOriginBase, GaussianModelOriginFused  # noqa: F401
 
 
 def __getattr__(name):

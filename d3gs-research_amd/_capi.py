@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Params(C.Structure):
@@ -30,7 +30,7 @@ class Params(C.Structure):
         ("z_near", C.c_float), ("z_far", C.c_float), ("eps", C.c_float),
         ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
-        ("scale_global", C.c_float), ("bg", C.c_float * 3),
+        ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
     ]
 
 
@@ -39,7 +39,7 @@ _SIGNATURES = {
     "d3gs_abi_version": (C.c_int, []),
     "d3gs_last_error_string": (C.c_char_p, []),
     "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
-    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 14 + [_VP]),
+    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
     "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 8 + [C.c_int64, _VP]),

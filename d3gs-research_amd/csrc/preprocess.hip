@@ -93,9 +93,10 @@ __device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, cons
 __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
-    const float* __restrict__ sh_base, float* __restrict__ depths, int32_t* __restrict__ radii,
-    float* __restrict__ uvs, float* __restrict__ conic_opacity, int32_t* __restrict__ tiles_touched,
-    float* __restrict__ rgb_out, float* __restrict__ cov2d_out, uint8_t* __restrict__ ne0_out) {
+    const float* __restrict__ sh_base, const uint8_t* __restrict__ invalid_mask, float* __restrict__ depths,
+    int32_t* __restrict__ radii, float* __restrict__ uvs, float* __restrict__ conic_opacity,
+    int32_t* __restrict__ tiles_touched, float* __restrict__ rgb_out, float* __restrict__ cov2d_out,
+    uint8_t* __restrict__ ne0_out) {
     // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
     extern __shared__ float s_rows[];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
@@ -119,15 +120,19 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
     float pc[3] = {dot3(P.w2c + 0, d), dot3(P.w2c + 3, d), dot3(P.w2c + 6, d)};
     z = pc[2];
-    valid = in_range && (z >= P.z_near && z <= P.z_far);
+    valid = in_range && (z >= P.z_near && z <= P.z_far) && !(invalid_mask && invalid_mask[i]);
     if (valid) {
         u = ((pc[0] / z) * P.fx + P.cx) - 0.5f;
         v = ((pc[1] / z) * P.fy + P.cy) - 0.5f;
 
         const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
-        float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
-        float q[4] = {qr.x / qn, qr.y / qn, qr.z / qn, qr.w / qn};
-        float s[3] = {det_expf(scale[3 * i]), det_expf(scale[3 * i + 1]), det_expf(scale[3 * i + 2])};
+        float q[4] = {qr.x, qr.y, qr.z, qr.w};
+        float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+        if (P.fused_activation) {
+            float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
+            q[0] = qr.x / qn; q[1] = qr.y / qn; q[2] = qr.z / qn; q[3] = qr.w / qn;
+            s[0] = det_expf(s[0]); s[1] = det_expf(s[1]); s[2] = det_expf(s[2]);
+        }
         if (!P.training) {
             s[0] = s[0] * P.scale_global;
             s[1] = s[1] * P.scale_global;
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         con0 = c * det_inv;
         con1 = (-b) * det_inv;
         con2 = a * det_inv;
-        op = det_sigmoid(opacity[i]);
+        op = P.fused_activation ? det_sigmoid(opacity[i]) : opacity[i];
 
         float mid = 0.5f * (a + c);
         float sq = sqrtf(fmaxf(P.radii_eigen_eps, mid * mid - det));
@@ -250,9 +255,14 @@ __device__ __forceinline__ void preprocess_bwd_one(
     float dc = k2 * ((((-a) * a) * g2 + (a * b) * g1) + (det - a * c) * g0);
 
     const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
-    float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
-    float q[4] = {qr.x / qn, qr.y / qn, qr.z / qn, qr.w / qn};
-    float s[3] = {det_expf(scale[3 * i]), det_expf(scale[3 * i + 1]), det_expf(scale[3 * i + 2])};
+    float qn = 1.0f;
+    float q[4] = {qr.x, qr.y, qr.z, qr.w};
+    float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+    if (P.fused_activation) {
+        qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
+        q[0] = qr.x / qn; q[1] = qr.y / qn; q[2] = qr.z / qn; q[3] = qr.w / qn;
+        s[0] = det_expf(s[0]); s[1] = det_expf(s[1]); s[2] = det_expf(s[2]);
+    }
     float R[9], c6[6];
     quat_to_rot(q, R);
     cov3d_from_scale_rot(s, R, c6);
@@ -324,14 +334,23 @@ __device__ __forceinline__ void preprocess_bwd_one(
     dq[2] = 2.0f * (((qx * (dR[2] + dR[6]) + qy * (dR[5] + dR[7])) - (2.0f * qz) * (dR[0] + dR[4])) + qw * (dR[3] - dR[1]));
     dq[3] = 2.0f * ((qz * (dR[3] - dR[1]) + qy * (dR[2] - dR[6])) + qx * (dR[7] - dR[5]));
     // activation backward: exp, normalize, sigmoid (origin/model.py:332-383)
-    dscale[3 * i + 0] = ds[0] * s[0];
-    dscale[3 * i + 1] = ds[1] * s[1];
-    dscale[3 * i + 2] = ds[2] * s[2];
-    float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
-    *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
-                                                            (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
-    float o = det_sigmoid(opacity[i]);
-    dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+    if (P.fused_activation) {
+        dscale[3 * i + 0] = ds[0] * s[0];
+        dscale[3 * i + 1] = ds[1] * s[1];
+        dscale[3 * i + 2] = ds[2] * s[2];
+        float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
+        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
+                                                                (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
+        float o = det_sigmoid(opacity[i]);
+        dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+    } else {
+        // inputs were activated by the caller: gradients w.r.t. the activated values
+        dscale[3 * i + 0] = ds[0];
+        dscale[3 * i + 1] = ds[1];
+        dscale[3 * i + 2] = ds[2];
+        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(dq[0], dq[1], dq[2], dq[3]);
+        dopacity_out[i] = dopacity_in[i];
+    }
 
     // SH backward (gs3d.py:262-364)
     float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
@@ -481,9 +500,10 @@ using namespace d3gs;
 
 extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
-                                   const float* color_sh_base, float* depths, int32_t* radii, float* uvs,
-                                   float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
-                                   float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+                                   const float* color_sh_base, const uint8_t* invalid_mask, float* depths,
+                                   int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
+                                   float* rgb_gaussian, float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0,
+                                   d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_fwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -495,7 +515,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
     hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
-                       opacity, color_sh, color_sh_base, depths, radii, uvs, conic_opacity, tiles_touched,
+                       opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity, tiles_touched,
                        rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

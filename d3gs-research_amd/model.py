@@ -3,7 +3,9 @@
 ``GaussianModelOriginFused`` mirrors d3sim/algos/d3gs/origin/model.py:34-48 and
 435-465: raw (pre-activation) tensors whose activations — exp for scale,
 normalize for the quaternion, sigmoid for opacity — are applied inside the
-preprocess kernel.  Quaternions are stored (x, y, z, w).
+preprocess kernel.  ``GaussianModelOrigin`` (origin/model.py:249-270) applies the
+same activations with torch before the operator runs, so autograd differentiates
+them and the kernels see activated values.  Quaternions are stored (x, y, z, w).
 """
 from __future__ import annotations
 
@@ -52,10 +54,29 @@ class GaussianModelOriginBase:
         for t in self.get_proxy_field_dict().values():
             t.grad = None
 
+    # activated views (origin/model.py:50-84); the base class has identity activations
+    @property
+    def xyz_act(self) -> torch.Tensor:
+        return self.xyz
+
+    @property
+    def quaternion_xyzw_act(self) -> torch.Tensor:
+        return self.quaternion_xyzw
+
+    @property
+    def scale_act(self) -> torch.Tensor:
+        return self.scale
+
+    @property
+    def opacity_act(self) -> torch.Tensor:
+        return self.opacity
+
     def create_model_with_act(self):
+        """origin/model.py:144-156."""
         if self.act_applied:
             return dataclasses.replace(self)
-        return dataclasses.replace(self, act_applied=True)
+        return dataclasses.replace(self, xyz=self.xyz_act, quaternion_xyzw=self.quaternion_xyzw_act,
+                                   scale=self.scale_act, opacity=self.opacity_act, act_applied=True)
 
     def to_device(self, device):
         kw = {k: v.to(device) for k, v in self.get_proxy_field_dict().items()}
@@ -77,3 +98,29 @@ class GaussianModelOriginFused(GaussianModelOriginBase):
     @property
     def fused_opacity_act_op(self):
         return ("sigmoid", "sigmoid_grad_out")
+
+
+@dataclasses.dataclass(kw_only=True)
+class GaussianModelOrigin(GaussianModelOriginBase):
+    """Activations applied by torch ahead of the operator (origin/model.py:249-270)."""
+
+    @property
+    def quaternion_xyzw_act(self) -> torch.Tensor:
+        if self.act_applied:
+            return self.quaternion_xyzw
+        return torch.nn.functional.normalize(self.quaternion_xyzw, p=2, dim=-1)
+
+    @property
+    def scale_act(self) -> torch.Tensor:
+        if self.act_applied:
+            return self.scale
+        return torch.exp(self.scale)
+
+    def inverse_scale_act(self, scale_act: torch.Tensor) -> torch.Tensor:
+        return torch.log(scale_act)
+
+    @property
+    def opacity_act(self) -> torch.Tensor:
+        if self.act_applied:
+            return self.opacity
+        return torch.sigmoid(self.opacity)

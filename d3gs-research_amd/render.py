@@ -210,6 +210,8 @@ class GaussianSplatOp:
         P.transmittance_eps = float(c.transmittance_eps)
         P.scale_global = float(c.scale_global)
         P.bg[:] = [float(v) for v in np.asarray(c.bg_color, np.float32).reshape(3)]
+        # a fused model hands over raw tensors; any other family has applied its activations in torch
+        P.fused_activation = int(isinstance(model, GaussianModelOriginFused))
         return P
 
     @staticmethod
@@ -233,11 +235,15 @@ class GaussianSplatOp:
                 custom_features=None, mask=None, prep_user_inputs=None):
         """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
         assert model.act_applied, "model must be activated before render"
-        if instance2world_T is not None or custom_features is not None or mask is not None or prep_user_inputs:
-            raise NotImplementedError("instance2world_T / custom_features / mask / prep_user_inputs are not supported")
-        if not isinstance(model, GaussianModelOriginFused):
-            raise NotImplementedError("only GaussianModelOriginFused (in-kernel activations) is supported")
+        if instance2world_T is not None or custom_features is not None or prep_user_inputs:
+            raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
         self._check_model(model)
+        if mask is not None:
+            # True rejects the gaussian (render.py:306-308)
+            assert mask.is_cuda and mask.dtype in (torch.bool, torch.uint8) and mask.numel() == len(model) \
+                and mask.is_contiguous(), "mask must be a contiguous bool/uint8 cuda tensor with one entry per gaussian"
+            if mask.dtype == torch.bool:
+                mask = mask.view(torch.uint8)
         L = self._lib
         P = self.make_params(model, cameras, training)
         n, dev = P.n, model.xyz.device
@@ -258,7 +264,7 @@ class GaussianSplatOp:
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
-                _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                 _capi.ptr(tiles_touched), _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs), _capi.ptr(ne0), s),
                 "d3gs_preprocess_fwd")
 
@@ -423,12 +429,12 @@ class _RasterizeGaussians(torch.autograd.Function):
     """render.py:3376-3587, with saved tensors addressed by name."""
 
     @staticmethod
-    def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, model_cls, cameras,
-                training, op: GaussianSplatOp, uv_grad_holder=None):
+    def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, mask, model_cls,
+                cameras, training, op: GaussianSplatOp, uv_grad_holder=None):
         model = model_cls(xyz=xyz, color_sh=color_sh, color_sh_base=color_sh_base, scale=scale,
                           quaternion_xyzw=quaternion_xyzw, opacity=opacity, cur_sh_degree=cur_sh_degree,
                           act_applied=True)
-        out, fwd_ctx = op.forward(model, cameras, training)
+        out, fwd_ctx = op.forward(model, cameras, training, mask=mask)
         ctx.has_ctx = fwd_ctx is not None
         if fwd_ctx is not None:
             ctx.fwd_ctx = fwd_ctx
@@ -444,7 +450,7 @@ class _RasterizeGaussians(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, drgb, dT, dn_contrib, dradii):
         if not ctx.has_ctx:
-            return (None,) * 12
+            return (None,) * 13
         if drgb is None:
             drgb = torch.zeros_like(ctx.out.color)
         if dT is None:
@@ -453,18 +459,18 @@ class _RasterizeGaussians(torch.autograd.Function):
         gm, duv, _ = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
                                      return_uv_grad=ctx.return_uv_grad)
         return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, None, None,
-                None, None, duv)
+                None, None, None, duv)
 
 
 def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSplatOp, training=False,
                         uv_grad_holder: torch.Tensor | None = None, instance2world_T=None, custom_features=None,
                         mask=None) -> GaussianSplatOutput:
     """render.py:3783-3838."""
-    if instance2world_T is not None or custom_features is not None or mask is not None:
-        raise NotImplementedError("instance2world_T / custom_features / mask are not supported")
-    model = model.create_model_with_act()
+    if instance2world_T is not None or custom_features is not None:
+        raise NotImplementedError("instance2world_T / custom_features are not supported")
+    model = model.create_model_with_act()   # torch-side activations for the non-fused families
     res = _RasterizeGaussians.apply(model.xyz, model.color_sh, model.color_sh_base, model.scale,
-                                    model.quaternion_xyzw, model.opacity, model.cur_sh_degree, type(model), cameras,
-                                    training, op, uv_grad_holder)
+                                    model.quaternion_xyzw, model.opacity, model.cur_sh_degree, mask, type(model),
+                                    cameras, training, op, uv_grad_holder)
     return GaussianSplatOutput(color=res[0], depth=None, custom_features=None, T=res[1], n_contrib=res[2],
                                radii=res[3])

@@ -12,6 +12,7 @@ import dataclasses
 import numpy as np
 
 from .camera import BasicPinholeCamera
+from .config_def import EarlyFilterAlgo, GaussianSplatConfig
 
 
 @dataclasses.dataclass
@@ -141,3 +142,21 @@ def gen_scene(config_id: int, n: int | None = None, wh: tuple[int, int] | None =
     return Scene(config_id=config_id, name=spec["name"], xyz=xyz, quaternion_xyzw=q, scale=scale, opacity=opacity,
                  color_sh=sh, sh_degree=deg, width=W, height=H, fx=float(f), fy=float(f), cx=float(cx), cy=float(cy),
                  to_world=to_world, near=spec["near"], far=spec["far"], drgb=drgb, dT=dT)
+
+
+def scene_config(scene: Scene, filter_algo: int = int(EarlyFilterAlgo.OBB_DFVT), **over) -> GaussianSplatConfig:
+    """Rasterizer configuration for a synthetic scene: reference defaults with the scene's near / far planes."""
+    cfg = GaussianSplatConfig(near=scene.near, far=scene.far, early_filter_algo=EarlyFilterAlgo(int(filter_algo)))
+    for k, v in over.items():
+        setattr(cfg, k, v)
+    return cfg
+
+
+def scene_model(scene: Scene, device="cuda"):
+    """The scene's gaussians as a fused-activation model on ``device``."""
+    import torch
+    from .model import GaussianModelOriginFused
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
+    return GaussianModelOriginFused(xyz=t(scene.xyz), quaternion_xyzw=t(scene.quaternion_xyzw), scale=t(scene.scale),
+                                    opacity=t(scene.opacity), color_sh=t(scene.color_sh), color_sh_base=None,
+                                    cur_sh_degree=scene.sh_degree, act_applied=True)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 3
+#define D3GS_ABI_VERSION 4
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -73,6 +73,10 @@ typedef struct d3gs_params {
     float transmittance_eps;
     float scale_global;
     float bg[3];
+    int32_t fused_activation; /* 1: scale/quaternion/opacity are raw and the kernels apply exp / normalize /
+                                 sigmoid (GaussianModelOriginFused, origin/model.py:435-465); 0: they are already
+                                 activated (GaussianModelOrigin, origin/model.py:249-270) and gradients are
+                                 returned w.r.t. the activated values */
 } d3gs_params;
 
 int d3gs_abi_version(void);
@@ -85,9 +89,11 @@ int d3gs_higher_msb(uint32_t n);
  * 421-476, 569-619).  One pass over the gaussians: fused activations, projection,
  * EWA covariance, conic, radius, tile rect, validity, tile count under the chosen
  * early filter, SH colour.  Outputs of rejected gaussians are written as zeros.
- * cov2d_vecs and sh_to_rgb_ne_0 may be NULL (inference). sh_base may be NULL. */
+ * cov2d_vecs and sh_to_rgb_ne_0 may be NULL (inference). sh_base may be NULL.
+ * invalid_mask (uint8[N], may be NULL): non-zero rejects the gaussian (render.py:306-308). */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
-                        const float* opacity, const float* color_sh, const float* color_sh_base, float* depths,
+                        const float* opacity, const float* color_sh, const float* color_sh_base,
+                        const uint8_t* invalid_mask, float* depths,
                         int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
                         float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
 

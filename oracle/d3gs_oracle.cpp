@@ -80,6 +80,7 @@ struct orc_params {
     float transmittance_eps;
     float scale_global;
     float bg[3];
+    int32_t fused_activation;  // 1: raw tensors, activations applied here; 0: already activated
 };
 
 // ---------------------------------------------------------------------------
@@ -355,7 +356,8 @@ static inline int tile_walk(const orc_params* P, const TileWalkIn& g, F&& f) {
 // uninitialised).
 // ---------------------------------------------------------------------------
 ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const float* quat, const float* scale,
-                       const float* opacity, const float* sh, const float* sh_base, float* depths, int32_t* radii,
+                       const float* opacity, const float* sh, const float* sh_base, const uint8_t* invalid_mask,
+                       float* depths, int32_t* radii,
                        float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_out, float* cov2d_out,
                        uint8_t* ne0_out) {
     if (P->filter_algo == ORC_FILTER_ELLIPSE) return -1;
@@ -376,14 +378,20 @@ ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const floa
         float pc[3] = {dot3(P->w2c + 0, d), dot3(P->w2c + 3, d), dot3(P->w2c + 6, d)};
         float z = pc[2];
         if (!(z >= P->z_near && z <= P->z_far)) continue;
+        if (invalid_mask && invalid_mask[i]) continue;  // render.py:306-308
         float u = ((pc[0] / z) * P->fx + P->cx) - 0.5f;
         float v = ((pc[1] / z) * P->fy + P->cy) - 0.5f;
 
         // fused activations (origin/model.py:281-295, 452-462)
         const float* qr = quat + 4 * i;
-        float qn = sqrtf(((qr[0] * qr[0] + qr[1] * qr[1]) + qr[2] * qr[2]) + qr[3] * qr[3]);
-        float q[4] = {qr[0] / qn, qr[1] / qn, qr[2] / qn, qr[3] / qn};
-        float s[3] = {orc_expf(scale[3 * i]), orc_expf(scale[3 * i + 1]), orc_expf(scale[3 * i + 2])};
+        float qn = 1.0f;
+        float q[4] = {qr[0], qr[1], qr[2], qr[3]};
+        float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+        if (P->fused_activation) {
+            qn = sqrtf(((qr[0] * qr[0] + qr[1] * qr[1]) + qr[2] * qr[2]) + qr[3] * qr[3]);
+            for (int k = 0; k < 4; ++k) q[k] = qr[k] / qn;
+            for (int k = 0; k < 3; ++k) s[k] = orc_expf(s[k]);
+        }
         if (!P->training) {
             s[0] = s[0] * P->scale_global;
             s[1] = s[1] * P->scale_global;
@@ -405,7 +413,7 @@ ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const floa
         float det = a * c - b * b;
         float det_inv = 1.0f / (det + P->eps);
         float con0 = c * det_inv, con1 = (-b) * det_inv, con2 = a * det_inv;
-        float op = sigmoidf_det(opacity[i]);
+        float op = P->fused_activation ? sigmoidf_det(opacity[i]) : opacity[i];
 
         float mid = 0.5f * (a + c);
         float sq = sqrtf(fmaxf(P->radii_eigen_eps, mid * mid - det));
@@ -747,9 +755,14 @@ ORC_API void orc_preprocess_bwd(const orc_params* P, const float* xyz, const flo
 
         // recompute activations and cov3d
         const float* qr = quat + 4 * i;
-        float qn = sqrtf(((qr[0] * qr[0] + qr[1] * qr[1]) + qr[2] * qr[2]) + qr[3] * qr[3]);
-        float q[4] = {qr[0] / qn, qr[1] / qn, qr[2] / qn, qr[3] / qn};
-        float s[3] = {orc_expf(scale[3 * i]), orc_expf(scale[3 * i + 1]), orc_expf(scale[3 * i + 2])};
+        float qn = 1.0f;
+        float q[4] = {qr[0], qr[1], qr[2], qr[3]};
+        float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+        if (P->fused_activation) {
+            qn = sqrtf(((qr[0] * qr[0] + qr[1] * qr[1]) + qr[2] * qr[2]) + qr[3] * qr[3]);
+            for (int k = 0; k < 4; ++k) q[k] = qr[k] / qn;
+            for (int k = 0; k < 3; ++k) s[k] = orc_expf(s[k]);
+        }
         float R[9], c6[6];
         quat_to_rot(q, R);
         cov3d_from_scale_rot(s, R, c6);
@@ -809,11 +822,17 @@ ORC_API void orc_preprocess_bwd(const orc_params* P, const float* xyz, const flo
         dq[2] = 2.0f * (((qx * (dR[2] + dR[6]) + qy * (dR[5] + dR[7])) - (2.0f * qz) * (dR[0] + dR[4])) + qw * (dR[3] - dR[1]));
         dq[3] = 2.0f * ((qz * (dR[3] - dR[1]) + qy * (dR[2] - dR[6])) + qx * (dR[7] - dR[5]));
         // activation backward: exp, normalize, sigmoid (origin/model.py:332-383)
-        for (int k = 0; k < 3; ++k) dscale[3 * i + k] = ds[k] * s[k];
-        float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
-        for (int k = 0; k < 4; ++k) dquat[4 * i + k] = (dq[k] - q[k] * qd) / qn;
-        float o = sigmoidf_det(opacity[i]);
-        dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+        if (P->fused_activation) {
+            for (int k = 0; k < 3; ++k) dscale[3 * i + k] = ds[k] * s[k];
+            float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
+            for (int k = 0; k < 4; ++k) dquat[4 * i + k] = (dq[k] - q[k] * qd) / qn;
+            float o = sigmoidf_det(opacity[i]);
+            dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+        } else {
+            for (int k = 0; k < 3; ++k) dscale[3 * i + k] = ds[k];
+            for (int k = 0; k < 4; ++k) dquat[4 * i + k] = dq[k];
+            dopacity_out[i] = dopacity_in[i];
+        }
 
         // SH backward (gs3d.py:262-364)
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);

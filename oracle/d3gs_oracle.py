@@ -31,7 +31,7 @@ class OracleParams(C.Structure):
         ("z_near", C.c_float), ("z_far", C.c_float), ("eps", C.c_float),
         ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
-        ("scale_global", C.c_float), ("bg", C.c_float * 3),
+        ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
     ]
 
 
@@ -72,7 +72,7 @@ def _p(a):
 def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_degree, sh_stride,
                 has_sh_base=False, filter_algo=FILTER_NONE, training=True, near=0.2, far=10000.0, eps=1e-6,
                 radii_eigen_eps=0.1, clamp_factor=1.3, std_sigma=3.0, lowpass=0.3, alpha_eps=1.0 / 255.0,
-                transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0)) -> OracleParams:
+                transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0), fused_activation=True) -> OracleParams:
     """cam2world_T is the 4x3 matrix ``to_world[:3].T`` (render.py:205-206)."""
     P = OracleParams()
     P.n, P.width, P.height = int(n), int(width), int(height)
@@ -93,7 +93,19 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
     P.lowpass, P.alpha_eps, P.transmittance_eps = float(lowpass), float(alpha_eps), float(transmittance_eps)
     P.scale_global = float(scale_global)
     P.bg[:] = [float(v) for v in bg]
+    P.fused_activation = int(bool(fused_activation))
     return P
+
+
+def params_for_scene(scene, filter_algo, training=True, **over) -> OracleParams:
+    """Oracle parameters for a synthetic scene object (fields n, width, height, fx, fy, cx, cy,
+    cam2world_T, sh_degree, color_sh, near, far)."""
+    kw = dict(n=scene.n, width=scene.width, height=scene.height, focal_xy=(scene.fx, scene.fy),
+              principal_point=(scene.cx, scene.cy), cam2world_T=scene.cam2world_T, sh_degree=scene.sh_degree,
+              sh_stride=scene.color_sh.shape[1], has_sh_base=False, filter_algo=int(filter_algo), training=training,
+              near=scene.near, far=scene.far)
+    kw.update(over)
+    return make_params(**kw)
 
 
 def expf(x):
@@ -122,7 +134,7 @@ def _f32(a):
     return None if a is None else np.ascontiguousarray(a, np.float32)
 
 
-def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None):
+def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
     n = P.n
     out = dict(
         depths=np.empty(n, np.float32), radii=np.empty(n, np.int32), uvs=np.empty((n, 2), np.float32),
@@ -130,7 +142,8 @@ def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None):
         rgb_gaussian=np.empty((n, 3), np.float32), cov2d_vecs=np.empty((n, 3), np.float32),
         sh_to_rgb_ne_0=np.empty(n, np.uint8))
     xyz, quat, scale, opacity, sh, sh_base = map(_f32, (xyz, quat, scale, opacity, sh, sh_base))
-    rc = lib().orc_preprocess_fwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(sh_base),
+    mask = None if invalid_mask is None else np.ascontiguousarray(invalid_mask, np.uint8)
+    rc = lib().orc_preprocess_fwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(sh_base), _p(mask),
                                   _p(out["depths"]), _p(out["radii"]), _p(out["uvs"]), _p(out["conic_opacity"]),
                                   _p(out["tiles_touched"]), _p(out["rgb_gaussian"]), _p(out["cov2d_vecs"]),
                                   _p(out["sh_to_rgb_ne_0"]))
@@ -208,9 +221,9 @@ def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dco
     return out
 
 
-def forward(P, xyz, quat, scale, opacity, sh, sh_base=None):
+def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
     """Whole forward: K1 .. K6.  Returns every intermediate the op context holds."""
-    pre = preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base)
+    pre = preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base, invalid_mask)
     offsets, m = scan(pre["tiles_touched"])
     num_tiles = P.tiles_x * P.tiles_y
     keys, vals = make_keys(P, pre["radii"], pre["uvs"], pre["conic_opacity"], pre["depths"], offsets, m)

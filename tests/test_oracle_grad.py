@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from f64_reference import C0, C1, C2, C3
-from helpers import gen_scene, oracle_forward
+from helpers import oracle_params, gen_scene, oracle_forward
 
 torch.set_num_threads(4)
 
@@ -100,16 +100,8 @@ def _setup(seed_cfg=0, n=96, wh=(48, 32), filt=0, sh_cfg=None):
     return scene
 
 
-@pytest.mark.parametrize("sh3", [False, True])
-def test_backward_matches_float64_autograd(oracle, sh3):
-    scene = _setup(sh_cfg=1 if sh3 else None)
-    P, ref = oracle_forward(oracle, scene, 0)
-    rng = np.random.default_rng(11)
-    drgb = rng.standard_normal((scene.height, scene.width, 3)).astype(np.float32)
-    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
-    g_ref, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
-                                drgb, dT)
-
+def _f64_grads(scene, ref, drgb, dT):
+    """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) w.r.t. the raw model tensors."""
     # global depth order (stable) and per-pixel tile-list membership from the oracle's binning
     valid = np.flatnonzero(ref["radii"] > 0)
     order = valid[np.argsort(ref["depths"][valid].view(np.uint32), kind="stable")]
@@ -129,18 +121,33 @@ def test_backward_matches_float64_autograd(oracle, sh3):
     assert np.abs(Tfin.detach().numpy() - ref["T"]).max() <= 1e-5
     loss = (col * torch.from_numpy(drgb).double()).sum() + (Tfin * torch.from_numpy(dT).double()).sum()
     loss.backward()
+    return [p.grad for p in params]
 
-    def close(got, want, name):
-        want = want.numpy()
-        scale = np.abs(want).max()
-        err = np.abs(got.astype(np.float64) - want).max()
-        assert err <= 2e-4 * scale + 1e-9, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
 
-    close(pb["dxyz"], params[0].grad, "dxyz")
-    close(pb["dquat"], params[1].grad, "dquat")
-    close(pb["dscale"], params[2].grad, "dscale")
-    close(pb["dopacity"], params[3].grad, "dopacity")
-    close(pb["dsh"], params[4].grad, "dsh")
+def _close(got, want, name):
+    want = want.numpy()
+    scale = np.abs(want).max()
+    err = np.abs(np.asarray(got, np.float64) - want).max()
+    assert err <= 2e-4 * scale + 1e-9, f"{name}: max err {err:.3e} vs scale {scale:.3e}"
+
+
+@pytest.mark.parametrize("sh3", [False, True])
+def test_backward_matches_float64_autograd(oracle, sh3):
+    scene = _setup(sh_cfg=1 if sh3 else None)
+    P, ref = oracle_forward(oracle, scene, 0)
+    rng = np.random.default_rng(11)
+    drgb = rng.standard_normal((scene.height, scene.width, 3)).astype(np.float32)
+    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    g_ref, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                                drgb, dT)
+
+    grads = _f64_grads(scene, ref, drgb, dT)
+
+    _close(pb["dxyz"], grads[0], "dxyz")
+    _close(pb["dquat"], grads[1], "dquat")
+    _close(pb["dscale"], grads[2], "dscale")
+    _close(pb["dopacity"], grads[3], "dopacity")
+    _close(pb["dsh"], grads[4], "dsh")
 
 
 def test_blend_backward_finite_differences(oracle):
@@ -199,3 +206,36 @@ def test_sh_mask_bit_order_switch(oracle):
                                 drgb, dT, sh_mask_compat=True)
     assert not ok["dsh"][:, 0, 0].any() and ok["dsh"][:, 0, 2].any()           # red masked, blue flows
     assert compat["dsh"][:, 0, 0].any() and not compat["dsh"][:, 0, 2].any()   # reversed: blue masked instead
+
+
+def test_activated_inputs_chain_to_the_raw_gradients(oracle):
+    """fused_activation = 0 (GaussianModelOrigin, origin/model.py:249-270): the oracle takes activated
+    scale / quaternion / opacity and returns gradients w.r.t. them.  Pushed through the float64
+    Jacobians of exp / normalize / sigmoid they must equal the float64 autograd gradients of the raw
+    tensors, and the image must be the fused path's image."""
+    scene = _setup()
+    P, ref = oracle_forward(oracle, scene, 0)
+    q64 = torch.tensor(scene.quaternion_xyzw, dtype=torch.float64, requires_grad=True)
+    s64 = torch.tensor(scene.scale, dtype=torch.float64, requires_grad=True)
+    o64 = torch.tensor(scene.opacity, dtype=torch.float64, requires_grad=True)
+    q_act, s_act, o_act = q64 / q64.norm(dim=1, keepdim=True), torch.exp(s64), torch.sigmoid(o64)
+    act = [t.detach().numpy().astype(np.float32) for t in (q_act, s_act, o_act)]
+
+    P0 = oracle_params(oracle, scene, 0)
+    P0.fused_activation = 0
+    ref0 = oracle.forward(P0, scene.xyz, act[0], act[1], act[2], scene.color_sh)
+    assert np.abs(ref0["color"] - ref["color"]).max() <= 1e-5
+    assert np.abs(ref0["T"] - ref["T"]).max() <= 1e-5
+
+    rng = np.random.default_rng(11)
+    drgb = rng.standard_normal((scene.height, scene.width, 3)).astype(np.float32)
+    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    _, pb = oracle.backward(P0, ref0, scene.xyz, act[0], act[1], act[2], scene.color_sh, drgb, dT)
+    torch.autograd.backward([q_act, s_act, o_act],
+                            [torch.from_numpy(pb[k]).double() for k in ("dquat", "dscale", "dopacity")])
+    grads = _f64_grads(scene, ref, drgb, dT)
+    _close(pb["dxyz"], grads[0], "dxyz")
+    _close(q64.grad.numpy(), grads[1], "dquat")
+    _close(s64.grad.numpy(), grads[2], "dscale")
+    _close(o64.grad.numpy(), grads[3], "dopacity")
+    _close(pb["dsh"], grads[4], "dsh")

@@ -124,3 +124,24 @@ def test_notebook_eigen_radius_value(oracle):
     got = oracle.preprocess_fwd(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
     np.testing.assert_allclose(got["cov2d_vecs"][0], [a, b, c], rtol=1e-4)
     assert got["radii"][0] == int(np.ceil(3 * np.sqrt(lam)))
+
+
+def test_invalid_mask_equals_rendering_the_kept_subset(oracle):
+    """render.py:306-308: mask[i] true rejects gaussian i.  The masked render must be the render of
+    the scene with those gaussians removed, and the rejected records must be the zero records."""
+    scene = gen_scene(0)
+    rng = np.random.default_rng(5)
+    mask = rng.random(scene.n) < 0.3
+    P = oracle_params(oracle, scene, 0)
+    got = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                         invalid_mask=mask)
+    keep = np.flatnonzero(~mask)
+    Pk = oracle_params(oracle, scene, 0)
+    Pk.n = len(keep)
+    want = oracle.forward(Pk, scene.xyz[keep], scene.quaternion_xyzw[keep], scene.scale[keep], scene.opacity[keep],
+                          scene.color_sh[keep])
+    assert (got["radii"][mask] == 0).all() and (got["tiles_touched"][mask] == 0).all()
+    assert np.array_equal(got["radii"][keep], want["radii"])
+    assert np.array_equal(got["color"], want["color"]) and np.array_equal(got["T"], want["T"])
+    assert np.array_equal(got["n_contrib"], want["n_contrib"])
+    assert np.array_equal(keep[want["gaussian_idx_sorted"]], got["gaussian_idx_sorted"])
