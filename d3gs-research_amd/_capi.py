@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class Params(C.Structure):
@@ -31,6 +31,8 @@ class Params(C.Structure):
         ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
+        ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
+        ("enable_anti_aliasing", C.c_int32),
     ]
 
 
@@ -49,8 +51,8 @@ _SIGNATURES = {
     "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
                                   C.POINTER(C.c_int), _VP]),
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
-    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [_VP]),
-    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
+    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP]),
+    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 19 + [_VP]),
     "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 13 + [C.c_int32] + [_VP] * 6 + [_VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

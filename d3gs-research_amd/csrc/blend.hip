@@ -52,13 +52,14 @@ __device__ __forceinline__ int tile_for_block(int bid, const int32_t* __restrict
 }
 
 // ---------------------------------------------------------------------------
-// Sum of nine per-lane values over the wavefront, as a transposing reduction:
+// Sum of ten per-lane values over the wavefront, as a transposing reduction:
 // every step exchanges halves so that the number of live registers halves with
-// the group size (9 -> 5 -> 3 -> 2 -> 1), ~25 VALU operations instead of nine
+// the group size (10 -> 5 -> 3 -> 2 -> 1), ~25 VALU operations instead of ten
 // independent 64-lane butterflies.  Cross-half / cross-row exchanges use the
-// gfx950 v_permlane32_swap / v_permlane16_swap, the rest DPP.  On return lane
-// slot_lane(k) holds the total of value k; reduce9_slot() tells each lane which
-// value (or none) it holds.
+// gfx950 v_permlane32_swap / v_permlane16_swap, the rest DPP.  On return ten
+// lanes hold one total each; reduce_slot() tells each lane which value (or none)
+// it holds.  The tenth value (the depth gradient) shares the exchange of the
+// ninth, so it costs nothing when it is the constant zero.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float swap_add32(float a, float b) {
     // lanes 0..31 <- a[l] + a[l+32]; lanes 32..63 <- b[l-32] + b[l]
@@ -75,19 +76,19 @@ __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xF, 0xF, false));
 }
 
-__device__ __forceinline__ int reduce9_slot(int lane) {
+__device__ __forceinline__ int reduce_slot(int lane) {
     if (lane & 3) return -1;
     const int r = lane >> 4, h = (lane >> 3) & 1, k = (lane >> 2) & 1;
-    if (k) return (r == 0 && h == 0) ? 8 : -1;
+    if (k) return (h == 0 && r == 0) ? 8 : (h == 0 && r == 2) ? 9 : -1;
     const int rowmap = (r == 0) ? 0 : (r == 1) ? 2 : (r == 2) ? 1 : 3;
     return rowmap + 4 * h;
 }
 
-__device__ __forceinline__ float wave_reduce9(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
-                                              float v7, float v8, bool hi8, bool hi4) {
+__device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
+                                               float v7, float v8, float v9, bool hi8, bool hi4) {
     // 64 -> 32: lower half keeps the first value of each pair, upper half the second
     const float s01 = swap_add32(v0, v1), s23 = swap_add32(v2, v3), s45 = swap_add32(v4, v5),
-                s67 = swap_add32(v6, v7), s8 = swap_add32(v8, 0.0f);
+                s67 = swap_add32(v6, v7), s8 = swap_add32(v8, v9);
     // 32 -> 16: rows (0,2) keep the first register of each pair, rows (1,3) the second
     const float q0 = swap_add16(s01, s23), q1 = swap_add16(s45, s67);
     float q2 = swap_add16(s8, 0.0f);
@@ -163,17 +164,28 @@ __device__ __forceinline__ unsigned long long uniform_u64(unsigned long long v) 
     return ((unsigned long long)hi << 32) | lo;
 }
 
+// Index of channel ch of pixel pid in the colour image: [H,W,C] or, with use_nchw, [C,H,W].
+__device__ __forceinline__ size_t color_index(const d3gs_params& P, size_t pid, int ch, int channels) {
+    return P.use_nchw ? (size_t)ch * P.width * P.height + pid : pid * channels + ch;
+}
+
+// kDepth: blend the camera-space depth as one more channel (render.py:1532-1539, 1915-1919).
+// kRgba: fourth colour channel, the sum of the blend weights (render.py:1899-1906).
+template <bool kDepth, bool kRgba>
 __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, const int32_t* __restrict__ ranges,
                                                             const int32_t* __restrict__ idx_sorted,
                                                             const float* __restrict__ uvs,
                                                             const float* __restrict__ conic_opacity,
                                                             const float* __restrict__ rgb_g,
+                                                            const float* __restrict__ depths,
                                                             const int32_t* __restrict__ tile_order,
                                                             float* __restrict__ color, float* __restrict__ final_T,
-                                                            int32_t* __restrict__ n_contrib) {
+                                                            int32_t* __restrict__ n_contrib,
+                                                            float* __restrict__ final_depth) {
     __shared__ StagedGaussian s_g[kBlock];
-    __shared__ float4 s_rgb[kBlock];
+    __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
+    constexpr int kChannels = kRgba ? 4 : 3;
 
     const int ntiles = P.tiles_x * P.tiles_y;
     const int tile = tile_for_block(blockIdx.x, tile_order);
@@ -192,7 +204,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
 
     bool done = !inside;
     float T = 1.0f;
-    float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f;
+    float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f, depth_accum = 0.0f;
     int contributor = 0;
 
     for (int round = 0; round < rounds; ++round) {
@@ -203,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
             const int g = idx_sorted[src];
             if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read
                 bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
             }
         }
         publish_masks(bits, wave, lane, s_mask);
@@ -234,6 +246,8 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                             acc0 = __builtin_fmaf(w, c.x, acc0);
                             acc1 = __builtin_fmaf(w, c.y, acc1);
                             acc2 = __builtin_fmaf(w, c.z, acc2);
+                            if constexpr (kRgba) acc3 = acc3 + w;
+                            if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
                         }
                     }
                 }
@@ -249,34 +263,40 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         const size_t pid = (size_t)py * P.width + px;
         final_T[pid] = T;
         n_contrib[pid] = contributor;
-        if (P.training) {
-            color[3 * pid + 0] = acc0;
-            color[3 * pid + 1] = acc1;
-            color[3 * pid + 2] = acc2;
-        } else {
-            color[3 * pid + 0] = fminf(fmaxf(acc0 + T * P.bg[0], 0.0f), 1.0f);
-            color[3 * pid + 1] = fminf(fmaxf(acc1 + T * P.bg[1], 0.0f), 1.0f);
-            color[3 * pid + 2] = fminf(fmaxf(acc2 + T * P.bg[2], 0.0f), 1.0f);
+        if constexpr (kDepth)  // inference normalises by the opacity (render.py:2244-2254)
+            final_depth[pid] = P.training ? depth_accum : depth_accum / ((1e-10f + 1.0f) - T);
+        const float acc[4] = {acc0, acc1, acc2, acc3};
+#pragma unroll
+        for (int ch = 0; ch < kChannels; ++ch) {
+            float v = acc[ch];
+            // the alpha channel has no background (render.py:2227-2229)
+            if (!P.training) v = fminf(fmaxf(v + T * (ch < 3 ? P.bg[ch] : 0.0f), 0.0f), 1.0f);
+            color[color_index(P, pid, ch, kChannels)] = v;
         }
     }
 }
 
 // ---------------------------------------------------------------------------
-// Backward: front-to-back recompute; per gaussian the nine partial derivatives
-// are summed over the wavefront, then over the tile's four wavefronts in LDS,
-// and only then added to global memory: one atomic per value per (tile, gaussian).
+// Backward: front-to-back recompute; per gaussian the partial derivatives
+// (nine, ten with depth) are summed over the wavefront, then over the tile's
+// four wavefronts in LDS, and only then added to global memory: one atomic per
+// value per (tile, gaussian).
 // ---------------------------------------------------------------------------
+template <bool kDepth, bool kRgba>
 __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
     const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
-    const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
-    const int32_t* __restrict__ n_contrib, const float* __restrict__ color,
-    const float* __restrict__ drgb, const float* __restrict__ dT, float* __restrict__ duv, float* __restrict__ dconic,
-    float* __restrict__ dopacity, float* __restrict__ dcolor) {
+    const float* __restrict__ depths, const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
+    const int32_t* __restrict__ n_contrib, const float* __restrict__ color, const float* __restrict__ final_depth,
+    const float* __restrict__ drgb, const float* __restrict__ dT, const float* __restrict__ ddepth,
+    float* __restrict__ duv, float* __restrict__ dconic, float* __restrict__ dopacity, float* __restrict__ dcolor,
+    float* __restrict__ dz) {
+    constexpr int kValues = kDepth ? 10 : 9;
+    constexpr int kChannels = kRgba ? 4 : 3;
     __shared__ StagedGaussian s_g[kBlock];
-    __shared__ float4 s_rgb[kBlock];
+    __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ int s_id[kBlock];
-    __shared__ float s_grad[9][kBlock];
+    __shared__ float s_grad[kValues][kBlock];
     __shared__ int s_wmax[4];
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 
@@ -298,20 +318,30 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
 
     int contributor = 0;
     float render_T = 0.0f, dT_val = 0.0f;
-    float rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f, dr0 = 0.0f, dr1 = 0.0f, dr2 = 0.0f;
+    float rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f, rr3 = 0.0f, dr0 = 0.0f, dr1 = 0.0f, dr2 = 0.0f, dr3 = 0.0f;
+    float rdep = 0.0f, ddep = 0.0f;
     if (inside) {
         contributor = min(n_contrib[pid] + 1, len);
         render_T = final_T[pid];
         dT_val = dT[pid];
-        rr0 = color[3 * pid + 0];
-        rr1 = color[3 * pid + 1];
-        rr2 = color[3 * pid + 2];
-        dr0 = drgb[3 * pid + 0];
-        dr1 = drgb[3 * pid + 1];
-        dr2 = drgb[3 * pid + 2];
+        rr0 = color[color_index(P, pid, 0, kChannels)];
+        rr1 = color[color_index(P, pid, 1, kChannels)];
+        rr2 = color[color_index(P, pid, 2, kChannels)];
+        dr0 = drgb[color_index(P, pid, 0, kChannels)];
+        dr1 = drgb[color_index(P, pid, 1, kChannels)];
+        dr2 = drgb[color_index(P, pid, 2, kChannels)];
+        if constexpr (kRgba) {
+            rr3 = color[color_index(P, pid, 3, kChannels)];
+            dr3 = drgb[color_index(P, pid, 3, kChannels)];
+        }
+        if constexpr (kDepth) {
+            rdep = final_depth[pid];
+            ddep = ddepth[pid];
+        }
     }
     const float dT_term = (-dT_val) * render_T;
-    const int slot = reduce9_slot(lane);
+    int slot = reduce_slot(lane);
+    if (slot >= kValues) slot = -1;
     const bool hi8 = (lane & 8) != 0, hi4 = (lane & 4) != 0;
     const int wave_todo = wave_max_i32(contributor);
     if (lane == 0) s_wmax[wave] = wave_todo;
@@ -329,12 +359,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read or write
                 s_id[tid] = g;
                 bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], 0.0f);
+                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
             }
         }
         publish_masks(bits, wave, lane, s_mask);
 #pragma unroll
-        for (int k = 0; k < 9; ++k) s_grad[k][tid] = 0.0f;
+        for (int k = 0; k < kValues; ++k) s_grad[k][tid] = 0.0f;
         __syncthreads();
         const int cnt = min(kBlock, wave_todo - round * kBlock);
         for (int chunk = 0; chunk < 4 && chunk * 64 < cnt; ++chunk) {
@@ -348,7 +378,8 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float power = blend_power(sg, dx, dy);
             const bool cand = (round * kBlock + j < contributor) && power >= sg.thr && power <= 0.0f;
             if (!__any(cand)) continue;
-            float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, g3 = 0.0f, g4 = 0.0f, g5 = 0.0f, g6 = 0.0f, g7 = 0.0f, g8 = 0.0f;
+            float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, g3 = 0.0f, g4 = 0.0f, g5 = 0.0f, g6 = 0.0f, g7 = 0.0f, g8 = 0.0f,
+                  g9 = 0.0f;
             bool valid = false;
             if (cand) {
                 // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
@@ -367,7 +398,17 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
                     rr0 = __builtin_fmaf(-w, c.x, rr0);
                     rr1 = __builtin_fmaf(-w, c.y, rr1);
                     rr2 = __builtin_fmaf(-w, c.z, rr2);
-                    float dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dT_term);
+                    float dl = dT_term;
+                    if constexpr (kDepth) {  // render.py:1887-1890, 1948-1950
+                        rdep = __builtin_fmaf(-w, c.w, rdep);
+                        dl = __builtin_fmaf(ddep, __builtin_fmaf(T, c.w, -rdep), dl);
+                        g9 = w * ddep;       // render.py:1964-1967
+                    }
+                    if constexpr (kRgba) {   // the alpha channel blends the constant 1 (render.py:1871-1874, 1926-1931)
+                        rr3 = rr3 - w;
+                        dl = __builtin_fmaf(dr3, T - rr3, dl);
+                    }
+                    dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dl);
                     dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
                     dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
                     const float dL_dalpha = dl / one_m;
@@ -389,17 +430,17 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
                 }
             }
             if (!__any(valid)) continue;
-            // nine wave totals land in nine different lanes: one LDS atomic instruction adds them all
-            const float total = wave_reduce9(g0, g1, g2, g3, g4, g5, g6, g7, g8, hi8, hi4);
+            // the wave totals land in different lanes: one LDS atomic instruction adds them all
+            const float total = wave_reduce10(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9, hi8, hi4);
             if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }
         __syncthreads();
         if (round * kBlock + tid < len) {
-            float v[9];
+            float v[kValues];
             bool any = false;
 #pragma unroll
-            for (int k = 0; k < 9; ++k) {
+            for (int k = 0; k < kValues; ++k) {
                 v[k] = s_grad[k][tid];
                 any = any || v[k] != 0.0f;
             }
@@ -414,6 +455,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
                 unsafeAtomicAdd(dcolor + 3 * g + 0, v[6]);
                 unsafeAtomicAdd(dcolor + 3 * g + 1, v[7]);
                 unsafeAtomicAdd(dcolor + 3 * g + 2, v[8]);
+                if constexpr (kDepth) unsafeAtomicAdd(dz + g, v[kValues - 1]);
             }
         }
     }
@@ -425,39 +467,53 @@ using namespace d3gs;
 
 static int blend_grid(const d3gs_params* p) { return p->tiles_x * p->tiles_y; }
 
+static int finish_launch(const char* who) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
 extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                               const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                              const int32_t* tile_order, float* color, float* final_T, int32_t* n_contrib,
-                              d3gs_stream_t stream) {
+                              const float* depths, const int32_t* tile_order, float* color, float* final_T,
+                              int32_t* n_contrib, float* final_depth, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_fwd");
     if (rc) return rc;
-    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib) {
+    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib ||
+        (p->render_depth && (!depths || !final_depth))) {
         set_error("d3gs_blend_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    hipLaunchKernelGGL(blend_fwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
-                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, color, final_T, n_contrib);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("d3gs_blend_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
-    return D3GS_OK;
+#define D3GS_LAUNCH_FWD(D, A)                                                                                       \
+    hipLaunchKernelGGL((blend_fwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
+                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
+                       color, final_T, n_contrib, final_depth)
+    if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true); else D3GS_LAUNCH_FWD(true, false); }
+    else                 { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true); else D3GS_LAUNCH_FWD(false, false); }
+#undef D3GS_LAUNCH_FWD
+    return finish_launch("d3gs_blend_fwd");
 }
 
 extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                               const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                              const int32_t* tile_order, const float* final_T, const int32_t* n_contrib,
-                              const float* color, const float* drgb, const float* dT, float* duv, float* dconic,
-                              float* dopacity, float* dcolor, d3gs_stream_t stream) {
+                              const float* depths, const int32_t* tile_order, const float* final_T,
+                              const int32_t* n_contrib, const float* color, const float* final_depth,
+                              const float* drgb, const float* dT, const float* ddepth, float* duv, float* dconic,
+                              float* dopacity, float* dcolor, float* dz, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_bwd");
     if (rc) return rc;
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb ||
-        !dT || !duv || !dconic || !dopacity || !dcolor) {
+        !dT || !duv || !dconic || !dopacity || !dcolor ||
+        (p->render_depth && (!depths || !final_depth || !ddepth || !dz))) {
         set_error("d3gs_blend_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    hipLaunchKernelGGL(blend_bwd_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p, workload_ranges,
-                       gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, final_T, n_contrib, color,
-                       drgb, dT, duv, dconic, dopacity, dcolor);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("d3gs_blend_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
-    return D3GS_OK;
+#define D3GS_LAUNCH_BWD(D, A)                                                                                       \
+    hipLaunchKernelGGL((blend_bwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
+                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
+                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, duv, dconic, dopacity, dcolor, dz)
+    if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_BWD(true, true); else D3GS_LAUNCH_BWD(true, false); }
+    else                 { if (p->render_rgba) D3GS_LAUNCH_BWD(false, true); else D3GS_LAUNCH_BWD(false, false); }
+#undef D3GS_LAUNCH_BWD
+    return finish_launch("d3gs_blend_bwd");
 }

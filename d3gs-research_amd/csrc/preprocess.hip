@@ -151,12 +151,27 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         b = dot3(t0, v1);
         c = dot3(t1, v1) + P.lowpass;
 
-        float det = a * c - b * b;
-        float det_inv = 1.0f / (det + P.eps);
-        con0 = c * det_inv;
-        con1 = (-b) * det_inv;
-        con2 = a * det_inv;
+        float det;
         op = P.fused_activation ? det_sigmoid(opacity[i]) : opacity[i];
+        if (P.enable_anti_aliasing) {
+            // gs3d.py:592-617: exact inverse of the low-passed covariance; the determinant handed on to
+            // the radius and the det > 0 test is the one without the low-pass term (render.py:466-476);
+            // opacity scaled by sqrt(max(0.000025, det / det_lowpass)) (render.py:393, 404-407)
+            const float a0 = a - P.lowpass, c0 = c - P.lowpass;
+            const float det_lp = a * c - b * b;
+            det = a0 * c0 - b * b;
+            const float inv = 1.0f / det_lp;
+            con0 = c * inv;
+            con1 = (-b) * inv;
+            con2 = a * inv;
+            op = op * sqrtf(fmaxf(0.000025f, det / det_lp));
+        } else {
+            det = a * c - b * b;
+            const float det_inv = 1.0f / (det + P.eps);
+            con0 = c * det_inv;
+            con1 = (-b) * det_inv;
+            con2 = a * det_inv;
+        }
 
         float mid = 0.5f * (a + c);
         float sq = sqrtf(fmaxf(P.radii_eigen_eps, mid * mid - det));
@@ -253,6 +268,23 @@ __device__ __forceinline__ void preprocess_bwd_one(
     float da = k2 * ((((-c) * c) * g0 + (b * c) * g1) + (det - a * c) * g2);
     float db = (k2 * 2.0f) * (((b * c) * g0 - (det / 2.0f + b * b) * g1) + (a * b) * g2);
     float dc = k2 * ((((-a) * a) * g2 + (a * b) * g1) + (det - a * c) * g0);
+    float dop_in = dopacity_in[i];
+    if (P.enable_anti_aliasing) {
+        // render.py:3293-3306; gs3d.py:671-679: dop_in is the gradient of opacity * comp with
+        // comp = sqrt(max(0.000025, ratio)), ratio = det_without_lowpass / det
+        const float lf = P.lowpass;
+        const float a0 = a - lf, c0 = c - lf;
+        const float ratio = (a0 * c0 - b * b) / det;
+        const float comp = sqrtf(fmaxf(0.000025f, ratio));
+        const float op_act = P.fused_activation ? det_sigmoid(opacity[i]) : opacity[i];
+        const float dcomp = dop_in * op_act;
+        const float dratio = ratio <= 0.000025f ? 0.0f : (dcomp * 0.5f) / comp;
+        const float gm = dratio * k2;
+        da += (lf * ((c * c + b * b) - c * lf)) * gm;
+        db += ((-2.0f * b) * lf) * ((a + c) - lf) * gm;
+        dc += (lf * ((a * a + b * b) - a * lf)) * gm;
+        dop_in = dop_in * comp;
+    }
 
     const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
     float qn = 1.0f;
@@ -342,14 +374,14 @@ __device__ __forceinline__ void preprocess_bwd_one(
         *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
                                                                 (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
         float o = det_sigmoid(opacity[i]);
-        dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+        dopacity_out[i] = dop_in * (o * (1.0f - o));
     } else {
         // inputs were activated by the caller: gradients w.r.t. the activated values
         dscale[3 * i + 0] = ds[0];
         dscale[3 * i + 1] = ds[1];
         dscale[3 * i + 2] = ds[2];
         *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(dq[0], dq[1], dq[2], dq[3]);
-        dopacity_out[i] = dopacity_in[i];
+        dopacity_out[i] = dop_in;
     }
 
     // SH backward (gs3d.py:262-364)

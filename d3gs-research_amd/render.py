@@ -129,9 +129,10 @@ class GaussianSplatOp:
         c = self._cfg
         unsupported = {
             "tile_size != (16, 16)": tuple(c.tile_size) != (16, 16),
-            "enable_32bit_sort": c.enable_32bit_sort, "render_depth": c.render_depth,
-            "render_inv_depth": c.render_inv_depth, "enable_anti_aliasing": c.enable_anti_aliasing,
-            "use_nchw": c.use_nchw, "render_rgba": c.render_rgba,
+            "enable_32bit_sort": c.enable_32bit_sort,
+            # the reference stores 1/z in the buffer it also sorts by (render.py:582, 773), which blends
+            # back to front: not reproduced
+            "render_inv_depth": c.render_inv_depth,
             "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
             "disable_builtin_rgb": c.disable_builtin_rgb,
             "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
@@ -212,6 +213,8 @@ class GaussianSplatOp:
         P.bg[:] = [float(v) for v in np.asarray(c.bg_color, np.float32).reshape(3)]
         # a fused model hands over raw tensors; any other family has applied its activations in torch
         P.fused_activation = int(isinstance(model, GaussianModelOriginFused))
+        P.render_depth, P.render_rgba = int(c.render_depth), int(c.render_rgba)
+        P.use_nchw, P.enable_anti_aliasing = int(c.use_nchw), int(c.enable_anti_aliasing)
         return P
 
     @staticmethod
@@ -306,19 +309,26 @@ class GaussianSplatOp:
 
         final_T = torch.empty((1, height, width), dtype=f32, device=dev)
         n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
-        out_color = torch.empty((1, height, width, 3), dtype=f32, device=dev)
-        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=None, n_contrib=n_contrib,
-                                  radii=radii)
+        channels = self._cfg.num_channels
+        color_shape = (1, channels, height, width) if self._cfg.use_nchw else (1, height, width, channels)
+        out_color = torch.empty(color_shape, dtype=f32, device=dev)
+        out_depth = torch.empty((1, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
+        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=out_depth,
+                                  n_contrib=n_contrib, radii=radii)
         if num_rendered == 0:
             # the reference returns uninitialised buffers here (render.py:706-729); fill with the
             # values an empty scene renders to instead
             final_T.fill_(1.0)
             n_contrib.zero_()
-            if training:
-                out_color.zero_()
-            else:
+            out_color.zero_()
+            if out_depth is not None:
+                out_depth.zero_()
+            if not training:
                 bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=dev).clamp(0, 1)
-                out_color[:] = bg
+                if self._cfg.use_nchw:
+                    out_color[:, :3] = bg.view(1, 3, 1, 1)
+                else:
+                    out_color[..., :3] = bg
             return out, None
 
         with self._stage("make_keys"):
@@ -345,7 +355,8 @@ class GaussianSplatOp:
             tile_order=tile_order)
         self._last_keys_sorted = keys_sorted  # kept for parity tests (sorted key order)
         with self._stage("blend_fwd"):
-            self.rasterize_forward_backward(model, ctx, out, training=training, _params=P)
+            self.rasterize_forward_backward(model, ctx, out, training=training, render_depth=self._cfg.render_depth,
+                                            _params=P)
         if not training:
             ctx = None
         return out, ctx
@@ -355,8 +366,9 @@ class GaussianSplatOp:
                                    grad: GaussianSplatGradients | None = None, training: bool = False,
                                    render_depth: bool = False, custom_features=None, _params=None, _cameras=None):
         """render.py:1329-2316: blend forward when ``grad`` is None, else blend backward."""
-        if render_depth or custom_features is not None:
-            raise NotImplementedError("render_depth / custom_features are not supported")
+        if custom_features is not None:
+            raise NotImplementedError("custom_features are not supported")
+        assert bool(render_depth) == bool(self._cfg.render_depth), "render_depth must match the op's config"
         L = self._lib
         P = _params
         if P is None:
@@ -367,24 +379,32 @@ class GaussianSplatOp:
         if grad is None:
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order),
-                _capi.ptr(out.color), _capi.ptr(out.T), _capi.ptr(out.n_contrib), s), "d3gs_blend_fwd")
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
+                _capi.ptr(ctx.tile_order), _capi.ptr(out.color), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
+                _capi.ptr(out.depth), s), "d3gs_blend_fwd")
             return None
         drgb = grad.drgb
         assert drgb.is_contiguous(), "drgb must be contiguous"
+        assert drgb.shape == out.color.shape, "drgb must have the shape of the colour image"
         assert grad.dT.is_contiguous(), "dT must be contiguous"
-        # the four accumulators are contiguous slices of one buffer: one zero-fill launch instead of four
-        acc = torch.zeros(9 * n, dtype=torch.float32, device=dev)
+        ddepth = None
+        if render_depth:
+            ddepth = grad.ddepth if grad.ddepth is not None else torch.zeros_like(out.depth)
+            assert ddepth.is_contiguous() and ddepth.shape == out.depth.shape, "ddepth must be contiguous [1,H,W]"
+        # the accumulators are contiguous slices of one buffer: one zero-fill launch instead of four
+        acc = torch.zeros((10 if render_depth else 9) * n, dtype=torch.float32, device=dev)
         duv = acc[0:2 * n].view(n, 2)
         dconic = acc[2 * n:5 * n].view(n, 3)
         dopacity = acc[5 * n:6 * n]
         dcolor = acc[6 * n:9 * n].view(n, 3)
+        dz = acc[9 * n:10 * n] if render_depth else None
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
-            _capi.ptr(out.n_contrib), _capi.ptr(out.color), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(duv),
-            _capi.ptr(dconic), _capi.ptr(dopacity), _capi.ptr(dcolor), s), "d3gs_blend_bwd")
-        return RasterizeGradientOutput(duv=duv, dconic=dconic, dopacity=dopacity, dcolor=dcolor)
+            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
+            _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(out.color),
+            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(duv),
+            _capi.ptr(dconic), _capi.ptr(dopacity), _capi.ptr(dcolor), _capi.ptr(dz), s), "d3gs_blend_bwd")
+        return RasterizeGradientOutput(duv=duv, dconic=dconic, dopacity=dopacity, dcolor=dcolor, dz=dz)
 
     # --------------------------------------------------------------- backward
     def backward(self, model: GaussianModelOriginBase, cameras, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
@@ -394,14 +414,15 @@ class GaussianSplatOp:
         is a model-shaped dataclass holding the gradients of the raw tensors."""
         if instance2world_T is not None or custom_features is not None or prep_user_inputs:
             raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
-        if grad.ddepth is not None or grad.dcustom_features is not None:
-            raise NotImplementedError("depth / custom feature gradients are not supported")
+        if grad.dcustom_features is not None:
+            raise NotImplementedError("custom feature gradients are not supported")
         L = self._lib
         P = self.make_params(model, cameras, True)
         s = self._stream()
         n, dev = P.n, model.xyz.device
         with self._stage("blend_bwd"):
-            g = self.rasterize_forward_backward(model, ctx, out, grad, training=True, _params=P)
+            g = self.rasterize_forward_backward(model, ctx, out, grad, training=True,
+                                                render_depth=self._cfg.render_depth, _params=P)
         with self._stage("preprocess_bwd"):
             dxyz = torch.empty_like(model.xyz)
             dquat = torch.empty_like(model.quaternion_xyzw)
@@ -414,7 +435,7 @@ class GaussianSplatOp:
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
                 _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.duv), _capi.ptr(g.dconic), _capi.ptr(g.dopacity),
-                _capi.ptr(g.dcolor), None, int(self._cfg.compat_ref_sh_mask_bitorder), _capi.ptr(dxyz),
+                _capi.ptr(g.dcolor), _capi.ptr(g.dz), int(self._cfg.compat_ref_sh_mask_bitorder), _capi.ptr(dxyz),
                 _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(g.dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), s),
                 "d3gs_preprocess_bwd")
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=g.dopacity,
@@ -444,18 +465,21 @@ class _RasterizeGaussians(torch.autograd.Function):
         ctx.cameras = cameras
         ctx.return_uv_grad = uv_grad_holder is not None
         ctx.mark_non_differentiable(out.n_contrib, out.radii)
-        return out.color, out.T, out.n_contrib, out.radii
+        # same tuple as the reference (render.py:3493-3499); custom features are not supported
+        return out.color, out.depth, None, out.T, out.n_contrib, out.radii
 
     @staticmethod
     @torch.autograd.function.once_differentiable
-    def backward(ctx, drgb, dT, dn_contrib, dradii):
+    def backward(ctx, drgb, ddepth, dcustom_features, dT, dn_contrib, dradii):
         if not ctx.has_ctx:
             return (None,) * 13
         if drgb is None:
             drgb = torch.zeros_like(ctx.out.color)
         if dT is None:
             dT = torch.zeros_like(ctx.out.T)
-        grads = GaussianSplatGradients(drgb=drgb.contiguous(), dT=dT.contiguous())
+        if ddepth is not None:
+            ddepth = ddepth.contiguous()
+        grads = GaussianSplatGradients(drgb=drgb.contiguous(), dT=dT.contiguous(), ddepth=ddepth)
         gm, duv, _ = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
                                      return_uv_grad=ctx.return_uv_grad)
         return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, None, None,
@@ -472,5 +496,5 @@ def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSpl
     res = _RasterizeGaussians.apply(model.xyz, model.color_sh, model.color_sh_base, model.scale,
                                     model.quaternion_xyzw, model.opacity, model.cur_sh_degree, mask, type(model),
                                     cameras, training, op, uv_grad_holder)
-    return GaussianSplatOutput(color=res[0], depth=None, custom_features=None, T=res[1], n_contrib=res[2],
-                               radii=res[3])
+    return GaussianSplatOutput(color=res[0], depth=res[1], custom_features=res[2], T=res[3], n_contrib=res[4],
+                               radii=res[5])

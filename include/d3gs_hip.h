@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 4
+#define D3GS_ABI_VERSION 5
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -77,6 +77,10 @@ typedef struct d3gs_params {
                                  sigmoid (GaussianModelOriginFused, origin/model.py:435-465); 0: they are already
                                  activated (GaussianModelOrigin, origin/model.py:249-270) and gradients are
                                  returned w.r.t. the activated values */
+    int32_t render_depth;         /* blend camera-space depth as one more channel (render.py:1532-1539, 1915-1919) */
+    int32_t render_rgba;          /* colour has a fourth channel, the sum of the blend weights (render.py:1899-1906) */
+    int32_t use_nchw;             /* colour / drgb stored [C,H,W] instead of [H,W,C] (render.py:702, 2272-2294) */
+    int32_t enable_anti_aliasing; /* conic without eps and opacity *= sqrt(det / det_lowpass) (render.py:391-407) */
 } d3gs_params;
 
 int d3gs_abi_version(void);
@@ -146,22 +150,27 @@ int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_r
                      int32_t* tile_order, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
- * color [H,W,3], final_T [H,W], n_contrib [H,W]. */
+ * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].
+ * depths [N] (K1's output) and final_depth [H,W] are read / written only when p->render_depth and may be
+ * NULL otherwise.  In inference the depth is divided by the accumulated opacity, which makes it NaN (0/0)
+ * for a pixel nothing reached, as in the reference (render.py:2244-2250). */
 int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
-                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
                    const int32_t* tile_order /* from d3gs_tile_ranges, or NULL for raster order */, float* color,
-                   float* final_T, int32_t* n_contrib, d3gs_stream_t stream);
+                   float* final_T, int32_t* n_contrib, float* final_depth, d3gs_stream_t stream);
 
 /* K7 — replaces kernel_raw("rasterize_True_...") (same generator, grad != None,
  * render.py:1341, 1589-1676, 1774-2210).  Produces the complete gradient (the
  * reference's backward_reduction_balanced_factor <= 0 branch, render.py:2024-2050,
- * 2182-2210).  duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3] are
- * accumulated with atomics: zero-fill them first. */
+ * 2182-2210).  duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3] and, with
+ * p->render_depth, dz [N] are accumulated with atomics: zero-fill them first.
+ * drgb has the layout of color; final_depth / ddepth [H,W] and dz may be NULL
+ * without p->render_depth. */
 int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
-                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                   const int32_t* tile_order /* or NULL */, const float* final_T, const int32_t* n_contrib,
-                   const float* color, const float* drgb, const float* dT, float* duv, float* dconic,
-                   float* dopacity, float* dcolor, d3gs_stream_t stream);
+                   const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
+                   const int32_t* tile_order, const float* final_T, const int32_t* n_contrib, const float* color,
+                   const float* final_depth, const float* drgb, const float* dT, const float* ddepth, float* duv,
+                   float* dconic, float* dopacity, float* dcolor, float* dz, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from (duv, dconic, dopacity, dcolor[, dz]) to

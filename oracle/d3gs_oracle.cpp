@@ -81,6 +81,10 @@ struct orc_params {
     float scale_global;
     float bg[3];
     int32_t fused_activation;  // 1: raw tensors, activations applied here; 0: already activated
+    int32_t render_depth;          // blend the camera-space depth as one more channel (render.py:1532-1539)
+    int32_t render_rgba;           // fourth colour channel = sum of blend weights (render.py:1899-1906)
+    int32_t use_nchw;              // colour image stored [C,H,W] instead of [H,W,C] (render.py:702)
+    int32_t enable_anti_aliasing;  // opacity scaled by sqrt(det / det_lowpass) (render.py:391-407)
 };
 
 // ---------------------------------------------------------------------------
@@ -410,10 +414,24 @@ ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const floa
         float b = dot3(t0, v1);
         float c = dot3(t1, v1) + P->lowpass;
 
-        float det = a * c - b * b;
-        float det_inv = 1.0f / (det + P->eps);
-        float con0 = c * det_inv, con1 = (-b) * det_inv, con2 = a * det_inv;
+        float det, con0, con1, con2;
         float op = P->fused_activation ? sigmoidf_det(opacity[i]) : opacity[i];
+        if (P->enable_anti_aliasing) {
+            // gs3d.py:592-617: the conic is the exact inverse of the low-passed covariance (no eps), the
+            // returned determinant is the one WITHOUT the low-pass term (it feeds the radius and the
+            // det > 0 test below, render.py:466-476), and the opacity is scaled by
+            // sqrt(max(0.000025, det / det_lowpass)) (render.py:393, 404-407).
+            const float a0 = a - P->lowpass, c0 = c - P->lowpass;
+            const float det_lp = a * c - b * b;
+            det = a0 * c0 - b * b;
+            const float inv = 1.0f / det_lp;
+            con0 = c * inv, con1 = (-b) * inv, con2 = a * inv;
+            op = op * sqrtf(fmaxf(0.000025f, det / det_lp));
+        } else {
+            det = a * c - b * b;
+            const float det_inv = 1.0f / (det + P->eps);
+            con0 = c * det_inv, con1 = (-b) * det_inv, con2 = a * det_inv;
+        }
 
         float mid = 0.5f * (a + c);
         float sq = sqrtf(fmaxf(P->radii_eigen_eps, mid * mid - det));
@@ -549,12 +567,20 @@ static inline float blend_power(const float* co, float dx, float dy) {
 
 // ---------------------------------------------------------------------------
 // K6 blend forward (render.py:1541-1570, 1677-1923, 2222-2271)
-// color[H,W,3], final_T[H,W], n_contrib[H,W]
+// color[H,W,C] (or [C,H,W] with use_nchw), C = 3 + render_rgba; final_T[H,W], n_contrib[H,W],
+// final_depth[H,W] when render_depth.
 // ---------------------------------------------------------------------------
+static inline size_t color_index(const orc_params* P, size_t pid, int ch) {
+    const int C = 3 + (P->render_rgba ? 1 : 0);
+    return P->use_nchw ? (size_t)ch * P->width * P->height + pid : pid * C + ch;
+}
+
 ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int32_t* idx_sorted, const float* uvs,
-                   const float* conic_opacity, const float* rgb_g, float* color, float* final_T, int32_t* n_contrib) {
+                   const float* conic_opacity, const float* rgb_g, const float* depths, float* color, float* final_T,
+                   int32_t* n_contrib, float* final_depth) {
     const int W = P->width, H = P->height;
     const int ntiles = P->tiles_x * P->tiles_y;
+    const int C = 3 + (P->render_rgba ? 1 : 0);
 #pragma omp parallel for schedule(dynamic, 1)
     for (int t = 0; t < ntiles; ++t) {
         int tx = t % P->tiles_x, ty = t / P->tiles_x;
@@ -565,7 +591,8 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
                 if (px >= W || py >= H) continue;
                 float pxf = (float)px, pyf = (float)py;
                 float T = 1.0f;
-                float acc[3] = {0, 0, 0};
+                float acc[4] = {0, 0, 0, 0};
+                float depth_accum = 0.0f;
                 int contributor = 0;
                 for (int k = r0; k < r1; ++k) {
                     int g = idx_sorted[k];
@@ -587,16 +614,20 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
                     acc[0] = fmaf(w, rgb_g[3 * g + 0], acc[0]);
                     acc[1] = fmaf(w, rgb_g[3 * g + 1], acc[1]);
                     acc[2] = fmaf(w, rgb_g[3 * g + 2], acc[2]);
+                    if (P->render_rgba) acc[3] = acc[3] + w;                               // render.py:1899-1906
+                    if (P->render_depth) depth_accum = fmaf(w, depths[g], depth_accum);   // render.py:1915-1919
                 }
                 size_t pid = (size_t)py * W + px;
                 final_T[pid] = T;
                 n_contrib[pid] = contributor;
+                if (P->render_depth)  // render.py:2244-2254
+                    final_depth[pid] = P->training ? depth_accum : depth_accum / ((1e-10f + 1.0f) - T);
                 if (P->training) {
-                    for (int ch = 0; ch < 3; ++ch) color[3 * pid + ch] = acc[ch];
+                    for (int ch = 0; ch < C; ++ch) color[color_index(P, pid, ch)] = acc[ch];
                 } else {
-                    for (int ch = 0; ch < 3; ++ch) {
-                        float vv = acc[ch] + T * P->bg[ch];
-                        color[3 * pid + ch] = fminf(fmaxf(vv, 0.0f), 1.0f);
+                    for (int ch = 0; ch < C; ++ch) {
+                        float vv = acc[ch] + T * (ch < 3 ? P->bg[ch] : 0.0f);   // alpha has no background (render.py:2227-2229)
+                        color[color_index(P, pid, ch)] = fminf(fmaxf(vv, 0.0f), 1.0f);
                     }
                 }
             }
@@ -608,21 +639,25 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
 // gradient (reference semantics with backward_reduction_balanced_factor = 0;
 // the default balanced branch drops dcolor for sparse warps, render.py:2125-2148).
 // Per-pixel terms in float32, accumulation over pixels in float64.
+// Ten values per gaussian: duv(2), dconic(3), dopacity, dcolor(3), dz.
 // ---------------------------------------------------------------------------
 ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int32_t* idx_sorted, const float* uvs,
-                   const float* conic_opacity, const float* rgb_g, const float* final_T, const int32_t* n_contrib,
-                   const float* color, const float* drgb, const float* dT, double* duv, double* dconic,
-                   double* dopacity, double* dcolor, double* absmass /* [N,9] sum of |terms|, may be NULL */) {
+                   const float* conic_opacity, const float* rgb_g, const float* depths, const float* final_T,
+                   const int32_t* n_contrib, const float* color, const float* final_depth, const float* drgb,
+                   const float* dT, const float* ddepth, double* duv, double* dconic, double* dopacity,
+                   double* dcolor, double* dz /* [N], used when render_depth */,
+                   double* absmass /* [N,10] sum of |terms|, may be NULL */) {
     const int W = P->width, H = P->height;
     const int ntiles = P->tiles_x * P->tiles_y;
+    const int NV = 10;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int t = 0; t < ntiles; ++t) {
         int tx = t % P->tiles_x, ty = t / P->tiles_x;
         int r0 = ranges[2 * t], r1 = ranges[2 * t + 1];
         int len = r1 - r0;
         if (len <= 0) continue;
-        std::vector<double> acc((size_t)len * 9, 0.0);
-        std::vector<double> mass((size_t)len * 9, 0.0);
+        std::vector<double> acc((size_t)len * NV, 0.0);
+        std::vector<double> mass((size_t)len * NV, 0.0);
         for (int ly = 0; ly < 16; ++ly)
             for (int lx = 0; lx < 16; ++lx) {
                 int px = tx * 16 + lx, py = ty * 16 + ly;
@@ -632,8 +667,13 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                 int contributor = n_contrib[pid] + 1;
                 float render_T = final_T[pid];
                 float dT_val = dT[pid];
-                float rr[3] = {color[3 * pid], color[3 * pid + 1], color[3 * pid + 2]};
-                float dr[3] = {drgb[3 * pid], drgb[3 * pid + 1], drgb[3 * pid + 2]};
+                float rr[4] = {0, 0, 0, 0}, dr[4] = {0, 0, 0, 0};
+                for (int ch = 0; ch < 3 + (P->render_rgba ? 1 : 0); ++ch) {
+                    rr[ch] = color[color_index(P, pid, ch)];
+                    dr[ch] = drgb[color_index(P, pid, ch)];
+                }
+                float rdep = P->render_depth ? final_depth[pid] : 0.0f;
+                float ddep = P->render_depth ? ddepth[pid] : 0.0f;
                 float T = 1.0f;
                 int lim = std::min(contributor, len);
                 for (int j = 0; j < lim; ++j) {
@@ -655,7 +695,17 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     rr[0] = fmaf(-w, cg[0], rr[0]);
                     rr[1] = fmaf(-w, cg[1], rr[1]);
                     rr[2] = fmaf(-w, cg[2], rr[2]);
-                    float dl = fmaf(dr[2], fmaf(T, cg[2], -rr[2]), (-dT_val) * render_T);
+                    float dl = (-dT_val) * render_T;
+                    if (P->render_depth) {   // render.py:1887-1890, 1948-1950
+                        const float dg = depths[g];
+                        rdep = fmaf(-w, dg, rdep);
+                        dl = fmaf(ddep, fmaf(T, dg, -rdep), dl);
+                    }
+                    if (P->render_rgba) {    // render.py:1871-1874, 1926-1931: the alpha channel blends the constant 1
+                        rr[3] = rr[3] - w;
+                        dl = fmaf(dr[3], T - rr[3], dl);
+                    }
+                    dl = fmaf(dr[2], fmaf(T, cg[2], -rr[2]), dl);
                     dl = fmaf(dr[1], fmaf(T, cg[1], -rr[1]), dl);
                     dl = fmaf(dr[0], fmaf(T, cg[0], -rr[0]), dl);
                     float dL_dalpha = dl / one_m;
@@ -665,12 +715,13 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     float dG_du = fmaf(gdy, nb, (2.0f * gdx) * ha);
                     float dG_dv = fmaf(gdx, nb, (2.0f * gdy) * hc);
                     const float half = -0.5f * dL_dG;
-                    double* a9 = acc.data() + (size_t)j * 9;
-                    double* m9 = mass.data() + (size_t)j * 9;
+                    double* a9 = acc.data() + (size_t)j * NV;
+                    double* m9 = mass.data() + (size_t)j * NV;
                     // dconic = dL/dG * (-1/2 G dx^2, -G dx dy, -1/2 G dy^2): no 1/2 on the off-diagonal (render.py:2013-2017)
-                    const float term[9] = {dL_dG * dG_du, dL_dG * dG_dv, (half * gdx) * dx, ((-dL_dG) * gdx) * dy,
-                                           (half * gdy) * dy, dL_dalpha * G, w * dr[0], w * dr[1], w * dr[2]};
-                    for (int k = 0; k < 9; ++k) {
+                    const float term[NV] = {dL_dG * dG_du, dL_dG * dG_dv, (half * gdx) * dx, ((-dL_dG) * gdx) * dy,
+                                            (half * gdy) * dy, dL_dalpha * G, w * dr[0], w * dr[1], w * dr[2],
+                                            w * ddep /* render.py:1964-1967 */};
+                    for (int k = 0; k < NV; ++k) {
                         a9[k] += (double)term[k];
                         m9[k] += fabs((double)term[k]);
                     }
@@ -678,33 +729,22 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
             }
         for (int j = 0; j < len; ++j) {
             int g = idx_sorted[r0 + j];
-            const double* a9 = acc.data() + (size_t)j * 9;
+            const double* a9 = acc.data() + (size_t)j * NV;
             bool any = false;
-            for (int k = 0; k < 9; ++k) any = any || a9[k] != 0.0;
+            for (int k = 0; k < NV; ++k) any = any || a9[k] != 0.0;
             if (!any) continue;
+            double* dst[NV] = {duv + 2 * g, duv + 2 * g + 1, dconic + 3 * g, dconic + 3 * g + 1, dconic + 3 * g + 2,
+                               dopacity + g, dcolor + 3 * g, dcolor + 3 * g + 1, dcolor + 3 * g + 2,
+                               P->render_depth ? dz + g : nullptr};
+            for (int k = 0; k < NV; ++k) {
+                if (!dst[k]) continue;
 #pragma omp atomic
-            duv[2 * g] += a9[0];
+                *dst[k] += a9[k];
+                if (absmass) {
 #pragma omp atomic
-            duv[2 * g + 1] += a9[1];
-#pragma omp atomic
-            dconic[3 * g] += a9[2];
-#pragma omp atomic
-            dconic[3 * g + 1] += a9[3];
-#pragma omp atomic
-            dconic[3 * g + 2] += a9[4];
-#pragma omp atomic
-            dopacity[g] += a9[5];
-#pragma omp atomic
-            dcolor[3 * g] += a9[6];
-#pragma omp atomic
-            dcolor[3 * g + 1] += a9[7];
-#pragma omp atomic
-            dcolor[3 * g + 2] += a9[8];
-            if (absmass)
-                for (int k = 0; k < 9; ++k) {
-#pragma omp atomic
-                    absmass[9 * (size_t)g + k] += mass[(size_t)j * 9 + k];
+                    absmass[NV * (size_t)g + k] += mass[(size_t)j * NV + k];
                 }
+            }
         }
     }
 }
@@ -752,6 +792,23 @@ ORC_API void orc_preprocess_bwd(const orc_params* P, const float* xyz, const flo
         float da = k2 * ((((-c) * c) * g0 + (b * c) * g1) + (det - a * c) * g2);
         float db = (k2 * 2.0f) * (((b * c) * g0 - (det / 2.0f + b * b) * g1) + (a * b) * g2);
         float dc = k2 * ((((-a) * a) * g2 + (a * b) * g1) + (det - a * c) * g0);
+        float dop_in = dopacity_in[i];
+        if (P->enable_anti_aliasing) {
+            // render.py:3293-3306; gs3d.py:671-679.  dop_in is the gradient of opacity * comp with
+            // comp = sqrt(max(0.000025, ratio)), ratio = det_without_lowpass / det.
+            const float lf = P->lowpass;
+            const float a0 = a - lf, c0 = c - lf;
+            const float ratio = (a0 * c0 - b * b) / det;
+            const float comp = sqrtf(fmaxf(0.000025f, ratio));
+            const float op_act = P->fused_activation ? sigmoidf_det(opacity[i]) : opacity[i];
+            const float dcomp = dop_in * op_act;
+            const float dratio = ratio <= 0.000025f ? 0.0f : (dcomp * 0.5f) / comp;
+            const float gm = dratio * k2;
+            da += (lf * ((c * c + b * b) - c * lf)) * gm;
+            db += ((-2.0f * b) * lf) * ((a + c) - lf) * gm;
+            dc += (lf * ((a * a + b * b) - a * lf)) * gm;
+            dop_in = dop_in * comp;
+        }
 
         // recompute activations and cov3d
         const float* qr = quat + 4 * i;
@@ -827,11 +884,11 @@ ORC_API void orc_preprocess_bwd(const orc_params* P, const float* xyz, const flo
             float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
             for (int k = 0; k < 4; ++k) dquat[4 * i + k] = (dq[k] - q[k] * qd) / qn;
             float o = sigmoidf_det(opacity[i]);
-            dopacity_out[i] = dopacity_in[i] * (o * (1.0f - o));
+            dopacity_out[i] = dop_in * (o * (1.0f - o));
         } else {
             for (int k = 0; k < 3; ++k) dscale[3 * i + k] = ds[k];
             for (int k = 0; k < 4; ++k) dquat[4 * i + k] = dq[k];
-            dopacity_out[i] = dopacity_in[i];
+            dopacity_out[i] = dop_in;
         }
 
         // SH backward (gs3d.py:262-364)

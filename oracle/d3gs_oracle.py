@@ -32,6 +32,8 @@ class OracleParams(C.Structure):
         ("radii_eigen_eps", C.c_float), ("clamp_factor", C.c_float), ("std_sigma", C.c_float),
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
+        ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
+        ("enable_anti_aliasing", C.c_int32),
     ]
 
 
@@ -72,7 +74,8 @@ def _p(a):
 def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_degree, sh_stride,
                 has_sh_base=False, filter_algo=FILTER_NONE, training=True, near=0.2, far=10000.0, eps=1e-6,
                 radii_eigen_eps=0.1, clamp_factor=1.3, std_sigma=3.0, lowpass=0.3, alpha_eps=1.0 / 255.0,
-                transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0), fused_activation=True) -> OracleParams:
+                transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0), fused_activation=True,
+                render_depth=False, render_rgba=False, use_nchw=False, enable_anti_aliasing=False) -> OracleParams:
     """cam2world_T is the 4x3 matrix ``to_world[:3].T`` (render.py:205-206)."""
     P = OracleParams()
     P.n, P.width, P.height = int(n), int(width), int(height)
@@ -94,6 +97,8 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
     P.scale_global = float(scale_global)
     P.bg[:] = [float(v) for v in bg]
     P.fused_activation = int(bool(fused_activation))
+    P.render_depth, P.render_rgba = int(bool(render_depth)), int(bool(render_rgba))
+    P.use_nchw, P.enable_anti_aliasing = int(bool(use_nchw)), int(bool(enable_anti_aliasing))
     return P
 
 
@@ -180,29 +185,42 @@ def tile_ranges(keys_sorted, num_tiles):
     return r
 
 
-def blend_fwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb):
+def _color_shape(P):
+    ch = 3 + int(bool(P.render_rgba))
+    return (ch, P.height, P.width) if P.use_nchw else (P.height, P.width, ch)
+
+
+def blend_fwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, depths=None):
+    """Returns (color, T, n_contrib, depth); depth is None unless P.render_depth."""
     H, W = P.height, P.width
-    color = np.zeros((H, W, 3), np.float32)
+    color = np.zeros(_color_shape(P), np.float32)
     T = np.zeros((H, W), np.float32)
     nc = np.zeros((H, W), np.int32)
-    lib().orc_blend_fwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(color), _p(T),
-                        _p(nc))
-    return color, T, nc
+    depth = np.zeros((H, W), np.float32) if P.render_depth else None
+    assert not P.render_depth or depths is not None
+    lib().orc_blend_fwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(depths),
+                        _p(color), _p(T), _p(nc), _p(depth))
+    return color, T, nc, depth
 
 
-def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib, color, drgb, dT):
+def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib, color, drgb, dT, depths=None,
+              final_depth=None, ddepth=None):
     n = P.n
     duv = np.zeros((n, 2), np.float64)
     dconic = np.zeros((n, 3), np.float64)
     dop = np.zeros(n, np.float64)
     dcol = np.zeros((n, 3), np.float64)
-    mass = np.zeros((n, 9), np.float64)
-    drgb, dT = _f32(drgb), _f32(dT)
-    lib().orc_blend_bwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(final_T),
-                        _p(n_contrib), _p(color), _p(drgb), _p(dT), _p(duv), _p(dconic), _p(dop), _p(dcol), _p(mass))
-    # absmass[:, k]: sum of |per-pixel terms| behind each of the nine gradient values (the scale that
-    # bounds reordering error): columns duv(2), dconic(3), dopacity(1), dcolor(3)
-    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol, absmass=mass)
+    dz = np.zeros(n, np.float64) if P.render_depth else None
+    mass = np.zeros((n, 10), np.float64)
+    drgb, dT, ddepth = _f32(drgb), _f32(dT), _f32(ddepth)
+    assert drgb.shape == _color_shape(P)
+    assert not P.render_depth or (depths is not None and final_depth is not None and ddepth is not None)
+    lib().orc_blend_bwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(depths),
+                        _p(final_T), _p(n_contrib), _p(color), _p(final_depth), _p(drgb), _p(dT), _p(ddepth),
+                        _p(duv), _p(dconic), _p(dop), _p(dcol), _p(dz), _p(mass))
+    # absmass[:, k]: sum of |per-pixel terms| behind each of the ten gradient values (the scale that
+    # bounds reordering error): columns duv(2), dconic(3), dopacity(1), dcolor(3), dz(1)
+    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol, dz=dz, absmass=mass)
 
 
 def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dconic, dopacity, dcolor, dz=None,
@@ -230,20 +248,21 @@ def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
     end_bit = 32 + higher_msb(num_tiles)
     ks, vs = sort_pairs(keys, vals, 0, end_bit)
     ranges = tile_ranges(ks, num_tiles)
-    color, T, nc = blend_fwd(P, ranges, vs, pre["uvs"], pre["conic_opacity"], pre["rgb_gaussian"])
+    color, T, nc, depth = blend_fwd(P, ranges, vs, pre["uvs"], pre["conic_opacity"], pre["rgb_gaussian"], pre["depths"])
     out = dict(pre)
     out.update(offsets=offsets, num_rendered=m, keys=keys, vals=vals, keys_sorted=ks, gaussian_idx_sorted=vs,
-               workload_ranges=ranges, color=color, T=T, n_contrib=nc, end_bit=end_bit)
+               workload_ranges=ranges, color=color, T=T, n_contrib=nc, depth=depth, end_bit=end_bit)
     return out
 
 
-def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False):
+def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False, ddepth=None):
     """Whole backward: K7 + K9 from the dict ``forward`` returned."""
     g = blend_bwd(P, fwd["workload_ranges"], fwd["gaussian_idx_sorted"], fwd["uvs"], fwd["conic_opacity"],
-                  fwd["rgb_gaussian"], fwd["T"], fwd["n_contrib"], fwd["color"], drgb, dT)
+                  fwd["rgb_gaussian"], fwd["T"], fwd["n_contrib"], fwd["color"], drgb, dT, fwd["depths"],
+                  fwd["depth"], ddepth)
     sh_in = sh
     pb = preprocess_bwd(P, xyz, quat, scale, opacity, sh_in, fwd["radii"], fwd["cov2d_vecs"], fwd["sh_to_rgb_ne_0"],
                         g["duv"].astype(np.float32), g["dconic"].astype(np.float32),
                         g["dopacity"].astype(np.float32), g["dcolor"].astype(np.float32),
-                        sh_mask_compat=sh_mask_compat)
+                        dz=None if g["dz"] is None else g["dz"].astype(np.float32), sh_mask_compat=sh_mask_compat)
     return g, pb

@@ -25,14 +25,14 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_params_struct_matches_header_layout():
     from d3gs_research_amd import _capi
-    # 10 int32 + 6 float + 9 + 3 + 10 float + 3 float + 1 int32
-    assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3 + 1)
+    # 10 int32 + 6 float + 9 + 3 + 10 float + 3 float + 5 int32
+    assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3 + 5)
 
 
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 4
+    assert L.d3gs_abi_version() == 5
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
 
@@ -42,7 +42,7 @@ def test_error_codes_without_compute():
     L = _capi.lib()
     P = _capi.Params()
     P.n, P.width, P.height, P.tiles_x, P.tiles_y, P.sh_stride = 4, 32, 32, 3, 2, 1   # wrong tile counts
-    nul = [None] * 10
+    nul = [None] * 12
     rc = L.d3gs_blend_fwd(C.byref(P), *nul)
     assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
     P.tiles_x = 2

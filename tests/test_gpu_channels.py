@@ -1,0 +1,127 @@
+"""GPU parity for the output channels and layouts beyond plain RGB: render_depth
+(render.py:1532-1539, 1915-1919, 1948-1950, 1964-1967), render_rgba (1899-1906, 1926-1931),
+use_nchw (702, 2272-2294) and enable_anti_aliasing (391-407, 3293-3306), forward bit-exact and
+backward to the same bars as the plain path, all through the C ABI."""
+import numpy as np
+import pytest
+
+from helpers import gen_scene, grad_close, op_config, oracle_params, torch_model
+
+pytestmark = pytest.mark.gpu
+
+AABB, DFVT = 1, 4
+
+# (config id, n, (w, h), filter, anti-aliasing, depth, rgba, nchw)
+CASES = [
+    (0, None, None, AABB, False, True, False, False),
+    (0, None, None, AABB, False, False, True, False),
+    (0, None, None, AABB, True, False, False, False),
+    (0, None, None, AABB, False, False, False, True),
+    (1, 20000, (250, 190), DFVT, True, True, True, True),
+    (2, 100000, (640, 360), DFVT, True, True, True, False),
+]
+
+
+def _setup(oracle, cfg_id, n, wh, filt, aa, depth, rgba, nchw, training=True, **over):
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    P = oracle_params(oracle, scene, filt, training, **over)
+    P.enable_anti_aliasing, P.render_depth, P.render_rgba, P.use_nchw = int(aa), int(depth), int(rgba), int(nchw)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    cfg = op_config(scene, filt, enable_anti_aliasing=aa, render_depth=depth, render_rgba=rgba, use_nchw=nchw)
+    return scene, P, ref, cfg
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt,aa,depth,rgba,nchw", CASES)
+def test_forward_and_backward(oracle, cfg_id, n, wh, filt, aa, depth, rgba, nchw):
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene, P, ref, cfg = _setup(oracle, cfg_id, n, wh, filt, aa, depth, rgba, nchw)
+    print(f"channels case cfg={cfg_id} n={scene.n} aa={aa} depth={depth} rgba={rgba} nchw={nchw}", flush=True)
+    op = GaussianSplatOp(cfg)
+    assert op.is_nchw == nchw and op.is_rgba == rgba
+    model = torch_model(scene)
+    out, ctx = op.forward(model, scene.camera(), training=True)
+    torch.cuda.synchronize()
+    cpu = lambda t: t.detach().cpu().numpy()
+    ch = 4 if rgba else 3
+    assert tuple(out.color.shape) == ((1, ch, scene.height, scene.width) if nchw else (1, scene.height, scene.width, ch))
+    assert np.array_equal(cpu(ctx.radii), ref["radii"])
+    assert np.array_equal(_bits(cpu(ctx.conic_opacity)), _bits(ref["conic_opacity"]))
+    assert np.array_equal(cpu(ctx.gaussian_idx_sorted), ref["gaussian_idx_sorted"])
+    assert np.array_equal(cpu(out.n_contrib)[0], ref["n_contrib"])
+    assert np.array_equal(_bits(cpu(out.color)[0]), _bits(ref["color"]))
+    assert np.array_equal(_bits(cpu(out.T)[0]), _bits(ref["T"]))
+    if depth:
+        assert np.array_equal(_bits(cpu(out.depth)[0]), _bits(ref["depth"]))
+    else:
+        assert out.depth is None
+
+    rng = np.random.default_rng(21)
+    drgb = rng.standard_normal(ref["color"].shape).astype(np.float32)
+    dT = rng.standard_normal(ref["T"].shape).astype(np.float32)
+    ddepth = rng.standard_normal(ref["T"].shape).astype(np.float32) if depth else None
+    g_ref, pb_ref = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                    scene.color_sh, drgb, dT, ddepth=ddepth)
+    t = lambda a: None if a is None else torch.from_numpy(a[None]).cuda()
+    gm, _, _ = op.backward(model, scene.camera(), ctx, out, GaussianSplatGradients(drgb=t(drgb), dT=t(dT), ddepth=t(ddepth)))
+    torch.cuda.synchronize()
+    g = op.last_raster_grads
+    mass = g_ref["absmass"]
+    checks = [("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)), ("dcolor", g.dcolor, slice(6, 9))]
+    if depth:
+        checks.append(("dz", g.dz, slice(9, 10)))
+    for name, got, cols in checks:
+        a, b = cpu(got).astype(np.float64).reshape(scene.n, -1), g_ref[name].reshape(scene.n, -1)
+        excess = np.abs(a - b) - (1e-4 * mass[:, cols] + 1e-30)
+        assert (excess <= 0).all(), f"{name}: {int((excess > 0).sum())} values beyond 1e-4 * sum|terms|"
+        ok, worst, nbad = grad_close(a, b)
+        assert ok, f"{name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+    for name, got in (("dxyz", gm.xyz), ("dquat", gm.quaternion_xyzw), ("dscale", gm.scale),
+                      ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
+        a = cpu(got).astype(np.float64).reshape(scene.n, -1)
+        b = pb_ref[name].astype(np.float64).reshape(scene.n, -1)
+        rn = np.linalg.norm(b, axis=1)
+        e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
+        med, p99 = np.quantile(e, [0.5, 0.99])
+        assert med <= 1e-4 and p99 <= 5e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
+
+
+@pytest.mark.parametrize("nchw", [False, True])
+def test_inference_all_channels(oracle, nchw):
+    """Inference: background on RGB only, alpha clamped, depth divided by the opacity (NaN where
+    nothing was hit, as the reference's 0 / 0)."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    bg = (0.2, 0.5, 0.7)
+    scene, P, ref, cfg = _setup(oracle, 1, 20000, (250, 190), AABB, True, True, True, nchw, training=False, bg=bg)
+    cfg.bg_color = np.array(bg, np.float32)
+    out, ctx = GaussianSplatOp(cfg).forward(torch_model(scene), scene.camera(), training=False)
+    assert ctx is None
+    assert np.array_equal(_bits(out.color.cpu().numpy()[0]), _bits(ref["color"]))
+    assert np.array_equal(_bits(out.depth.cpu().numpy()[0]), _bits(ref["depth"]))
+
+
+def test_depth_through_autograd_entry_point(oracle):
+    """rasterize_gaussians returns the depth image and routes its gradient (render.py:3493-3499)."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp, rasterize_gaussians
+    scene, P, ref, cfg = _setup(oracle, 0, None, None, AABB, False, True, False, False)
+    op = GaussianSplatOp(cfg)
+    model = torch_model(scene)
+    model.act_applied = False
+    model.set_requires_grad(True)
+    out = rasterize_gaussians(model, scene.camera(), op, training=True)
+    ddepth = np.random.default_rng(4).standard_normal(ref["T"].shape).astype(np.float32)
+    (out.depth * torch.from_numpy(ddepth[None]).cuda()).sum().backward()
+    zeros = np.zeros_like(ref["color"])
+    _, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                            zeros, np.zeros_like(ref["T"]), ddepth=ddepth)
+    for name, tns in (("dxyz", model.xyz), ("dscale", model.scale), ("dquat", model.quaternion_xyzw),
+                      ("dopacity", model.opacity)):
+        ok, worst, nbad = grad_close(tns.grad.cpu().numpy(), pb[name], rel=1e-3, abs_frac=1e-4)
+        assert ok, f"{name}: {nbad} bad (worst {worst:.2f}x)"
+    assert float(model.color_sh.grad.abs().max()) == 0.0

@@ -60,3 +60,41 @@ def test_inference_background_and_clamp(oracle):
     want = np.clip(tr["color"].astype(np.float64) + tr["T"][..., None] * np.array(bg, np.float32).astype(np.float64), 0, 1)
     assert np.abs(inf["color"] - want).max() <= 1e-6
     assert np.array_equal(inf["T"], tr["T"])
+
+
+def test_extra_channels_layouts_and_inference_depth(oracle):
+    """render_rgba: alpha = sum of weights = 1 - T in exact arithmetic and no background in inference
+    (render.py:1899-1906, 2227-2229); use_nchw is the same image transposed (render.py:702, 2272-2294);
+    render_depth in inference is normalised by the opacity (render.py:2244-2250)."""
+    from helpers import oracle_params
+    scene = gen_scene(1, n=30000, wh=(200, 136))
+    args = (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    base = oracle.forward(oracle_params(oracle, scene, 1), *args)
+
+    P = oracle_params(oracle, scene, 1)
+    P.render_rgba, P.render_depth = 1, 1
+    full = oracle.forward(P, *args)
+    assert np.array_equal(full["color"][..., :3], base["color"]) and np.array_equal(full["T"], base["T"])
+    assert np.abs(full["color"][..., 3] + full["T"] - 1.0).max() <= 2e-6
+    # depth is a convex-ish combination of the member depths: bounded by alpha * max depth
+    assert (full["depth"] >= 0).all()
+    assert (full["depth"] <= full["color"][..., 3] * full["depths"].max() * (1 + 1e-5) + 1e-6).all()
+
+    P.use_nchw = 1
+    nchw = oracle.forward(P, *args)
+    assert nchw["color"].shape == (4, scene.height, scene.width)
+    assert np.array_equal(nchw["color"].transpose(1, 2, 0), full["color"])
+    assert np.array_equal(nchw["depth"], full["depth"])
+
+    bg = (0.3, 0.6, 0.1)
+    Pi = oracle_params(oracle, scene, 1, training=False, bg=bg)
+    Pi.render_rgba, Pi.render_depth = 1, 1
+    inf = oracle.forward(Pi, *args)
+    assert np.array_equal(inf["T"], full["T"])
+    want_rgb = np.clip(full["color"][..., :3] + full["T"][..., None] * np.array(bg, np.float32), 0, 1)
+    assert np.abs(inf["color"][..., :3] - want_rgb).max() <= 1e-6
+    assert np.abs(inf["color"][..., 3] - np.clip(full["color"][..., 3], 0, 1)).max() == 0
+    want_depth = full["depth"] / (np.float32(1.0) - full["T"])
+    seen = full["T"] < 1
+    assert np.allclose(inf["depth"][seen], want_depth[seen], rtol=1e-6, atol=0)
+    assert (inf["depth"][~seen] == 0).all() or np.isnan(inf["depth"][~seen]).all()

@@ -39,8 +39,9 @@ def _quat_to_R(q):
         torch.stack([2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)], -1)], -2)
 
 
-def _render_f64(scene, params, member, order):
-    """Dense float64 forward: `member[p, j]` says gaussian order[j] is in pixel p's tile list."""
+def _render_f64(scene, params, member, order, anti_aliasing=False):
+    """Dense float64 forward: `member[p, j]` says gaussian order[j] is in pixel p's tile list.
+    Returns colour, T, blended depth and blended alpha (the sum of the weights)."""
     xyz, quat, scale, opac, sh = params
     tw = torch.tensor(scene.to_world, dtype=torch.float64)
     W, c = tw[:3, :3].T, tw[:3, 3]
@@ -62,8 +63,15 @@ def _render_f64(scene, params, member, order):
     S2 = T @ S3 @ T.transpose(1, 2)
     a, b, cc = S2[:, 0, 0] + 0.3, S2[:, 0, 1], S2[:, 1, 1] + 0.3
     det = a * cc - b * b
-    ca, cb, ccn = cc / (det + 1e-6), -b / (det + 1e-6), a / (det + 1e-6)
     o = torch.sigmoid(opac)
+    if anti_aliasing:
+        # mip-splatting style compensation: exact inverse of the low-passed covariance, opacity scaled by
+        # sqrt(det(cov) / det(cov + 0.3 I)) (clamped below at 0.000025)
+        ca, cb, ccn = cc / det, -b / det, a / det
+        ratio = ((a - 0.3) * (cc - 0.3) - b * b) / det
+        o = o * torch.sqrt(torch.clamp_min(ratio, 0.000025))
+    else:
+        ca, cb, ccn = cc / (det + 1e-6), -b / (det + 1e-6), a / (det + 1e-6)
     d = xyz - c
     rgb = torch.clamp_min(_sh_torch(scene.sh_degree, sh, d / d.norm(dim=1, keepdim=True)), 0.0)
 
@@ -72,6 +80,8 @@ def _render_f64(scene, params, member, order):
     px, py = xs.reshape(-1), ys.reshape(-1)
     Tcur = torch.ones(H * Wd, dtype=torch.float64)
     col = torch.zeros(H * Wd, 3, dtype=torch.float64)
+    dep = torch.zeros(H * Wd, dtype=torch.float64)
+    asum = torch.zeros(H * Wd, dtype=torch.float64)
     done = torch.zeros(H * Wd, dtype=torch.bool)
     for j, g in enumerate(order):
         dx, dy = uv[g, 0] - px, uv[g, 1] - py
@@ -85,8 +95,10 @@ def _render_f64(scene, params, member, order):
         use = live & ~stop & (power.detach() <= 0)
         w = torch.where(use, alpha * Tcur, torch.zeros_like(Tcur))
         col = col + w[:, None] * rgb[g]
+        dep = dep + w * z[g]
+        asum = asum + w
         Tcur = torch.where(use, nT, Tcur)
-    return col.reshape(H, Wd, 3), Tcur.reshape(H, Wd)
+    return col.reshape(H, Wd, 3), Tcur.reshape(H, Wd), dep.reshape(H, Wd), asum.reshape(H, Wd)
 
 
 def _setup(seed_cfg=0, n=96, wh=(48, 32), filt=0, sh_cfg=None):
@@ -100,8 +112,9 @@ def _setup(seed_cfg=0, n=96, wh=(48, 32), filt=0, sh_cfg=None):
     return scene
 
 
-def _f64_grads(scene, ref, drgb, dT):
-    """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) w.r.t. the raw model tensors."""
+def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False):
+    """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) (+ sum(depth*ddepth)) w.r.t. the raw
+    model tensors.  A four-channel drgb also weights the blended alpha."""
     # global depth order (stable) and per-pixel tile-list membership from the oracle's binning
     valid = np.flatnonzero(ref["radii"] > 0)
     order = valid[np.argsort(ref["depths"][valid].view(np.uint32), kind="stable")]
@@ -115,11 +128,18 @@ def _f64_grads(scene, ref, drgb, dT):
 
     params = [torch.tensor(a, dtype=torch.float64, requires_grad=True)
               for a in (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)]
-    col, Tfin = _render_f64(scene, params, torch.from_numpy(member), order.tolist())
+    col, Tfin, dep, asum = _render_f64(scene, params, torch.from_numpy(member), order.tolist(), anti_aliasing)
     # the float64 forward agrees with the oracle's float32 forward (no threshold flips on this scene)
-    assert np.abs(col.detach().numpy() - ref["color"]).max() <= 2e-5
+    assert np.abs(col.detach().numpy() - ref["color"][..., :3]).max() <= 2e-5
     assert np.abs(Tfin.detach().numpy() - ref["T"]).max() <= 1e-5
-    loss = (col * torch.from_numpy(drgb).double()).sum() + (Tfin * torch.from_numpy(dT).double()).sum()
+    d64 = torch.from_numpy(drgb).double()
+    loss = (col * d64[..., :3]).sum() + (Tfin * torch.from_numpy(dT).double()).sum()
+    if drgb.shape[-1] == 4:
+        assert np.abs(asum.detach().numpy() - ref["color"][..., 3]).max() <= 2e-5
+        loss = loss + (asum * d64[..., 3]).sum()
+    if ddepth is not None:
+        assert np.abs(dep.detach().numpy() - ref["depth"]).max() <= 1e-4
+        loss = loss + (dep * torch.from_numpy(ddepth).double()).sum()
     loss.backward()
     return [p.grad for p in params]
 
@@ -239,3 +259,25 @@ def test_activated_inputs_chain_to_the_raw_gradients(oracle):
     _close(s64.grad.numpy(), grads[2], "dscale")
     _close(o64.grad.numpy(), grads[3], "dopacity")
     _close(pb["dsh"], grads[4], "dsh")
+
+
+@pytest.mark.parametrize("aa,depth,rgba", [(True, False, False), (False, True, False), (False, False, True),
+                                           (True, True, True)])
+def test_channels_and_anti_aliasing_match_float64_autograd(oracle, aa, depth, rgba):
+    """render_depth (render.py:1915-1919, 1948-1950, 1964-1967 and dz into the pinhole backward,
+    render.py:3283-3292), render_rgba (1899-1906, 1926-1931) and enable_anti_aliasing (391-407,
+    3293-3306; gs3d.py:592-679) against float64 autograd over the dense restatement."""
+    scene = _setup()
+    P = oracle_params(oracle, scene, 0)
+    P.enable_anti_aliasing, P.render_depth, P.render_rgba = int(aa), int(depth), int(rgba)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    rng = np.random.default_rng(12)
+    drgb = rng.standard_normal((scene.height, scene.width, 4 if rgba else 3)).astype(np.float32)
+    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    ddepth = rng.standard_normal((scene.height, scene.width)).astype(np.float32) if depth else None
+    g, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                            drgb, dT, ddepth=ddepth)
+    assert (g["dz"] is not None) == depth
+    grads = _f64_grads(scene, ref, drgb, dT, ddepth, aa)
+    for i, name in enumerate(["dxyz", "dquat", "dscale", "dopacity", "dsh"]):
+        _close(pb[name], grads[i], name)
