@@ -185,7 +185,7 @@ struct TileWalk {
     int rminx, rminy, rmaxx, rmaxy;  // 3-sigma tile rect
     int bminx, bminy, bw, bh;        // candidate rect (origin, size); the 3-sigma rect when no filter
     float uo, vo, bx, by;            // centre relative to the candidate rect origin, AABB half extents
-    float ow, oh, os, oc;            // oriented box: width, height, sin, cos
+    float ow, oh, os, oc;            // oriented box: width, height, sin, cos; ELLIPSE: conic a, b, c and the bound
 };
 
 __device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1, float by1, float w, float h, float s,
@@ -205,6 +205,38 @@ __device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1
     r1 = l1x * fabsf(-s); r2 = l1y * fabsf(c); r3 = l2x * fabsf(c * (-s) + s * c); r4 = l2y * fabsf((-s) * (-s) + c * c);
     if (((r1 + r2) + r3) + r4 <= fabsf(lx * (-s) + ly * c)) return false;
     return true;
+}
+
+// Where the level set {conic form = -bound} crosses a horizontal (axis = 1) or vertical (axis = 0)
+// line (gs3d.py:1149-1178, 1210-1240; coordinates relative to the centre).  lo = hi = -1 on a miss.
+struct EllipseCut { float lo, hi; };
+__device__ __forceinline__ EllipseCut ellipse_cut(int axis, float line, float cu, float cv, float cx, float cy,
+                                                  float cz, float bound) {
+    const float own = axis ? cv : cu, other = axis ? cu : cv, lead = axis ? cx : cz;
+    const float t = line - own;
+    const float val = (((-bound) * lead) - ((cx * cz) * t) * t) + ((cy * cy) * t) * t;
+    EllipseCut r{-1.0f, -1.0f};
+    if (val >= 0.0f) {
+        const float sq = sqrtf(fmaxf(0.0f, val));
+        r.lo = other + ((-cy) * t - sq) / lead;
+        r.hi = other + ((-cy) * t + sq) / lead;
+    }
+    return r;
+}
+
+// gs3d.py:1078-1117: an edge line cuts the ellipse inside the edge, or the ellipse covers the box,
+// or its centre lies in the box.
+__device__ __forceinline__ bool ellipse_overlaps_box(float bx0, float by0, float bx1, float by1, float cx, float cy,
+                                                     float cz, float bound, float cu, float cv) {
+    const EllipseCut x0 = ellipse_cut(0, bx0, cu, cv, cx, cy, cz, bound), x1 = ellipse_cut(0, bx1, cu, cv, cx, cy, cz, bound);
+    const EllipseCut y0 = ellipse_cut(1, by0, cu, cv, cx, cy, cz, bound), y1 = ellipse_cut(1, by1, cu, cv, cx, cy, cz, bound);
+    auto in = [](float v, float lo, float hi) { return v >= lo && v <= hi; };
+    const bool valid = in(x0.lo, by0, by1) || in(x0.hi, by0, by1) || in(x1.lo, by0, by1) || in(x1.hi, by0, by1) ||
+                       in(y0.lo, bx0, bx1) || in(y0.hi, bx0, bx1) || in(y1.lo, bx0, bx1) || in(y1.hi, bx0, bx1);
+    const bool cover = x0.lo <= by0 && x0.hi >= by1 && x1.lo <= by0 && x1.hi >= by1 && y0.lo <= bx0 && y0.hi >= bx1 &&
+                       y1.lo <= bx0 && y1.hi >= bx1;
+    const bool centre = bx0 <= cu && bx1 >= cu && by0 <= cv && by1 >= cv;
+    return valid || cover || centre;
 }
 
 __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const TileWalkIn& g) {
@@ -261,6 +293,11 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
         w.oh = minor * 2.0f;
         w.os = v2y;
         w.oc = v2x;
+    } else if (P.filter_algo == D3GS_FILTER_ELLIPSE) {
+        w.ow = g.conic0;
+        w.oh = g.conic1;
+        w.os = g.conic2;
+        w.oc = bound;
     }
     return w;
 }
@@ -275,6 +312,8 @@ __device__ __forceinline__ bool tile_keep(const int filter_algo, const TileWalk&
         const bool xo = (w.uo - w.bx) <= px1 && (w.uo + w.bx) >= px0;
         const bool yo = (w.vo - w.by) <= py1 && (w.vo + w.by) >= py0;
         keep = xo && yo;
+    } else if (filter_algo == D3GS_FILTER_ELLIPSE) {
+        keep = ellipse_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
     } else {
         keep = obb_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
     }

@@ -515,10 +515,6 @@ int check_params(const d3gs_params* p, const char* who) {
                   p->sh_degree, need);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    if (p->filter_algo == D3GS_FILTER_ELLIPSE) {
-        set_error("%s: early_filter_algo ELLIPSE is not implemented", who);
-        return D3GS_ERR_UNSUPPORTED;
-    }
     if (p->filter_algo < 0 || p->filter_algo > 4) {
         set_error("%s: unknown early_filter_algo %d", who, p->filter_algo);
         return D3GS_ERR_INVALID_ARGUMENT;

@@ -138,7 +138,6 @@ class GaussianSplatOp:
             "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
             "use_int64_tile_touched": c.use_int64_tile_touched,
             "rasterize_backward_algo=PER_GAUSSIAN": c.rasterize_backward_algo != RasterizeBackwardAlgo.DEFAULT,
-            "early_filter_algo=ELLIPSE": c.early_filter_algo == EarlyFilterAlgo.ELLIPSE,
         }
         bad = [k for k, v in unsupported.items() if v]
         if bad:

@@ -42,7 +42,7 @@ extern "C" {
 /* EarlyFilterAlgo, d3sim/algos/d3gs/config_def.py:59-70 */
 #define D3GS_FILTER_NONE 0
 #define D3GS_FILTER_AABB 1
-#define D3GS_FILTER_ELLIPSE 2 /* not implemented: returns D3GS_ERR_UNSUPPORTED */
+#define D3GS_FILTER_ELLIPSE 2 /* exact ellipse / tile test, render.py:1277-1297; gs3d.py:1078-1240 */
 #define D3GS_FILTER_OBB 3
 #define D3GS_FILTER_OBB_DFVT 4 /* computed as the OBB tile set */
 

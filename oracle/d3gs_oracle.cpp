@@ -281,6 +281,37 @@ static inline bool obb_overlaps_box(float bx0, float by0, float bx1, float by1, 
     return true;
 }
 
+// Where the level set {conic form = -bound} crosses a horizontal (axis = 1) or vertical (axis = 0)
+// line, gs3d.py:1149-1178 / 1210-1240 ("_v2": coordinates relative to the centre).  lo = hi = -1 when
+// the line misses the ellipse.
+struct EllipseCut { float lo, hi; };
+static inline EllipseCut ellipse_cut(int axis, float line, float cu, float cv, const float conic[3], float bound) {
+    const float cx = conic[0], cy = conic[1], cz = conic[2];
+    const float own = axis ? cv : cu;      // centre coordinate along the line's normal
+    const float other = axis ? cu : cv;    // centre coordinate along the line
+    const float lead = axis ? cx : cz;     // coefficient of the unknown squared
+    const float t = line - own;
+    const float val = (((-bound) * lead) - ((cx * cz) * t) * t) + ((cy * cy) * t) * t;
+    if (!(val >= 0.0f)) return {-1.0f, -1.0f};
+    const float sq = sqrtf(fmaxf(0.0f, val));
+    return {other + ((-cy) * t - sq) / lead, other + ((-cy) * t + sq) / lead};
+}
+
+// gs3d.py:1078-1117: the ellipse touches the box when an edge line cuts it inside the edge, when it
+// covers the whole box, or when its centre lies in the box.
+static inline bool ellipse_overlaps_box(float bx0, float by0, float bx1, float by1, const float conic[3], float bound,
+                                        float cu, float cv) {
+    const EllipseCut x0 = ellipse_cut(0, bx0, cu, cv, conic, bound), x1 = ellipse_cut(0, bx1, cu, cv, conic, bound);
+    const EllipseCut y0 = ellipse_cut(1, by0, cu, cv, conic, bound), y1 = ellipse_cut(1, by1, cu, cv, conic, bound);
+    auto in = [](float v, float lo, float hi) { return v >= lo && v <= hi; };
+    bool valid = in(x0.lo, by0, by1) || in(x0.hi, by0, by1) || in(x1.lo, by0, by1) || in(x1.hi, by0, by1) ||
+                 in(y0.lo, bx0, bx1) || in(y0.hi, bx0, bx1) || in(y1.lo, bx0, bx1) || in(y1.hi, bx0, bx1);
+    bool cover = x0.lo <= by0 && x0.hi >= by1 && x1.lo <= by0 && x1.hi >= by1 && y0.lo <= bx0 && y0.hi >= bx1 &&
+                 y1.lo <= bx0 && y1.hi >= bx1;
+    bool centre = bx0 <= cu && bx1 >= cu && by0 <= cv && by1 >= cv;
+    return valid || cover || centre;
+}
+
 template <class F>
 static inline int tile_walk(const orc_params* P, const TileWalkIn& g, F&& f) {
     const int TX = P->tiles_x, TY = P->tiles_y;
@@ -344,6 +375,8 @@ static inline int tile_walk(const orc_params* P, const TileWalkIn& g, F&& f) {
                 bool xo = (uo - bx) <= px1 && (uo + bx) >= px0;
                 bool yo = (vo - by) <= py1 && (vo + by) >= py0;
                 keep = xo && yo;
+            } else if (P->filter_algo == ORC_FILTER_ELLIPSE) {
+                keep = ellipse_overlaps_box(px0, py0, px1, py1, g.conic, bound, uo, vo);
             } else {
                 keep = obb_overlaps_box(px0, py0, px1, py1, whsc, uo, vo);
             }
@@ -364,7 +397,6 @@ ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const floa
                        float* depths, int32_t* radii,
                        float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_out, float* cov2d_out,
                        uint8_t* ne0_out) {
-    if (P->filter_algo == ORC_FILTER_ELLIPSE) return -1;
     const int n = P->n;
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int i = 0; i < n; ++i) {

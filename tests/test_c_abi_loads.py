@@ -46,8 +46,8 @@ def test_error_codes_without_compute():
     rc = L.d3gs_blend_fwd(C.byref(P), *nul)
     assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
     P.tiles_x = 2
-    P.filter_algo = 2   # ELLIPSE: declared, not implemented
-    assert L.d3gs_blend_fwd(C.byref(P), *nul) == -2
+    P.filter_algo = 7
+    assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"early_filter_algo" in L.d3gs_last_error_string()
     P.filter_algo = 1
     assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"NULL" in L.d3gs_last_error_string()
     P.sh_degree, P.sh_stride = 3, 4
@@ -56,6 +56,7 @@ def test_error_codes_without_compute():
     assert L.d3gs_sort_workspace_bytes(1000, 0, 65, C.byref(n)) == -1
     assert L.d3gs_sort_workspace_bytes(1000, 0, 45, C.byref(n)) == 0 and n.value > 0
     in_b = C.c_int(7)
+    assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 1 << 30, 0, 45, C.byref(in_b), None) == -2   # unsupported size
     assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 0, 0, 45, C.byref(in_b), None) == 0 and in_b.value == 0
 
 

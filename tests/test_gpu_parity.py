@@ -12,7 +12,7 @@ from helpers import gen_scene, grad_close, op_config, oracle_forward, torch_mode
 
 pytestmark = pytest.mark.gpu
 
-NONE, AABB, OBB, DFVT = 0, 1, 3, 4
+NONE, AABB, ELLIPSE, OBB, DFVT = 0, 1, 2, 3, 4
 
 CASES = [
     # (config id, n override, (w,h) override, filter)
@@ -25,6 +25,9 @@ CASES = [
     (2, 100000, (640, 360), AABB),
     (3, 100000, (480, 270), OBB),
     (4, 30000, (960, 540), AABB),
+    (0, None, None, ELLIPSE),
+    (2, 100000, (640, 360), ELLIPSE),
+    (4, 30000, (960, 540), ELLIPSE),
     # BASELINE.json's full sizes (the CPU oracle renders these in a few seconds on the box's host cores)
     (2, None, None, DFVT),
     (3, None, None, AABB),

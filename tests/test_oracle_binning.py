@@ -7,7 +7,7 @@ import pytest
 from f64_reference import preprocess_f64
 from helpers import gen_scene, oracle_forward
 
-NONE, AABB, OBB, DFVT = 0, 1, 3, 4
+NONE, AABB, ELLIPSE, OBB, DFVT = 0, 1, 2, 3, 4
 
 
 def _tile_sets(ref, n):
@@ -23,7 +23,7 @@ def test_filters_are_lossless_and_nested(oracle, make):
     """config_def.py:136-141: AABB / OBB only drop tiles in which no pixel reaches alpha >= 1/255;
     OBB tiles are a subset of AABB tiles, which are a subset of the 3-sigma rect (NONE)."""
     scene = make()
-    refs = {f: oracle_forward(oracle, scene, f)[1] for f in (NONE, AABB, OBB, DFVT)}
+    refs = {f: oracle_forward(oracle, scene, f)[1] for f in (NONE, AABB, ELLIPSE, OBB, DFVT)}
     sets = {f: _tile_sets(refs[f], scene.n) for f in refs}
     pre = refs[NONE]
     tiles_x = (scene.width + 15) // 16
@@ -31,10 +31,11 @@ def test_filters_are_lossless_and_nested(oracle, make):
     co = pre["conic_opacity"].astype(np.float64)
     dropped_checked = 0
     for g in range(scene.n):
-        s_none, s_aabb, s_obb = sets[NONE][g], sets[AABB][g], sets[OBB][g]
+        s_none, s_aabb, s_obb, s_ell = sets[NONE][g], sets[AABB][g], sets[OBB][g], sets[ELLIPSE][g]
         assert s_obb <= s_aabb <= s_none
+        assert s_ell <= s_aabb                             # the ellipse lies inside its bounding boxes
         assert sets[DFVT][g] == s_obb                      # the author's invariant, render.py:1051-1072
-        for t in s_none - s_obb:
+        for t in s_none - (s_obb & s_ell):
             tx, ty = t % tiles_x, t // tiles_x
             xs = np.arange(tx * 16, min(tx * 16 + 16, scene.width), dtype=np.float64)
             ys = np.arange(ty * 16, min(ty * 16 + 16, scene.height), dtype=np.float64)
@@ -46,7 +47,7 @@ def test_filters_are_lossless_and_nested(oracle, make):
             dropped_checked += 1
     assert dropped_checked > 100          # the test did examine dropped tiles
     # a lossless filter cannot change the image
-    for f in (AABB, OBB, DFVT):
+    for f in (AABB, ELLIPSE, OBB, DFVT):
         assert np.array_equal(refs[f]["color"], refs[NONE]["color"])
         assert np.array_equal(refs[f]["T"], refs[NONE]["T"])
 
@@ -118,3 +119,50 @@ def test_sort_bit_range_and_stability(oracle):
         masked = (keys >> np.uint64(b)) & np.uint64((1 << (e - b)) - 1)
         order = np.argsort(masked, kind="stable")
         assert np.array_equal(vo, vals[order]) and np.array_equal(ko, keys[order])
+
+
+def _min_form_over_box(a, b, c, u, v, x0, y0, x1, y1):
+    """Exact minimum of q(p) = a (px-u)^2 + 2 b (px-u)(py-v) + c (py-v)^2 over the closed box (float64):
+    zero if the centre is inside, else the minimum over the four edges (a convex quadratic on a segment)."""
+    if x0 <= u <= x1 and y0 <= v <= y1:
+        return 0.0
+    best = np.inf
+    for y in (y0, y1):                      # horizontal edges: minimise over px
+        dy = y - v
+        px = np.clip(u - b * dy / a, x0, x1)
+        dx = px - u
+        best = min(best, a * dx * dx + 2 * b * dx * dy + c * dy * dy)
+    for x in (x0, x1):                      # vertical edges: minimise over py
+        dx = x - u
+        py = np.clip(v - b * dx / c, y0, y1)
+        dy = py - v
+        best = min(best, a * dx * dx + 2 * b * dx * dy + c * dy * dy)
+    return best
+
+
+@pytest.mark.parametrize("make", [lambda: gen_scene(0, n=1500), lambda: gen_scene(4, n=3000, wh=(480, 270))])
+def test_ellipse_filter_is_the_exact_ellipse_box_test(oracle, make):
+    """render.py:1277-1297; gs3d.py:1078-1240.  Inside the AABB candidate rect and the 3-sigma rect the
+    ELLIPSE filter keeps exactly the tiles whose closed box [16x, 16x+16] x [16y, 16y+16] meets the
+    level set {alpha >= alpha_eps}: checked against the float64 minimum of the quadratic form over the
+    box, skipping tiles within 1e-3 relative of the boundary."""
+    scene = make()
+    ref_a = oracle_forward(oracle, scene, AABB)[1]
+    ref_e = oracle_forward(oracle, scene, ELLIPSE)[1]
+    s_aabb, s_ell = _tile_sets(ref_a, scene.n), _tile_sets(ref_e, scene.n)
+    tiles_x = (scene.width + 15) // 16
+    uv = ref_a["uvs"].astype(np.float64)
+    co = ref_a["conic_opacity"].astype(np.float64)
+    decided = dropped = 0
+    for g in np.flatnonzero(ref_a["radii"] > 0):
+        a, b, c, o = co[g]
+        level = -2.0 * np.log((1 / 255.0) / o)              # q(p) <= level  <=>  alpha >= 1/255
+        for t in s_aabb[g]:
+            tx, ty = t % tiles_x, t // tiles_x
+            q = _min_form_over_box(a, b, c, uv[g, 0], uv[g, 1], tx * 16.0, ty * 16.0, tx * 16.0 + 16, ty * 16.0 + 16)
+            if abs(q - level) <= 1e-3 * level:
+                continue
+            assert (t in s_ell[g]) == (q < level), (g, t, q, level)
+            decided += 1
+            dropped += t not in s_ell[g]
+    assert decided > 1000 and dropped > 50
