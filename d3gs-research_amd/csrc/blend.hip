@@ -289,14 +289,15 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const float* __restrict__ depths, const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
     const int32_t* __restrict__ n_contrib, const float* __restrict__ color, const float* __restrict__ final_depth,
     const float* __restrict__ drgb, const float* __restrict__ dT, const float* __restrict__ ddepth,
-    float* __restrict__ duv, float* __restrict__ dconic, float* __restrict__ dopacity, float* __restrict__ dcolor,
-    float* __restrict__ dz) {
+    float* __restrict__ grad_records) {
     constexpr int kValues = kDepth ? 10 : 9;
     constexpr int kChannels = kRgba ? 4 : 3;
     __shared__ StagedGaussian s_g[kBlock];
     __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ int s_id[kBlock];
-    __shared__ float s_grad[kValues][kBlock];
+    // one row per value; the odd row stride puts the (up to ten) lanes of one LDS atomic instruction,
+    // which address the same gaussian in consecutive rows, into different banks
+    __shared__ float s_grad[kValues][kBlock + 1];
     __shared__ int s_wmax[4];
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 
@@ -343,7 +344,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     int slot = reduce_slot(lane);
     if (slot >= kValues) slot = -1;
     const bool hi8 = (lane & 8) != 0, hi4 = (lane & 4) != 0;
-    const int wave_todo = wave_max_i32(contributor);
+    // wave-uniform by construction; readfirstlane tells the compiler, which keeps the gaussian
+    // bit masks and loop bounds below in scalar registers
+    const int wave_todo = __builtin_amdgcn_readfirstlane(wave_max_i32(contributor));
     if (lane == 0) s_wmax[wave] = wave_todo;
     __syncthreads();
     const int block_todo = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
@@ -370,92 +373,91 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         for (int chunk = 0; chunk < 4 && chunk * 64 < cnt; ++chunk) {
           unsigned long long m = uniform_u64(s_mask[wave][chunk]);
           if (cnt - chunk * 64 < 64) m &= (1ull << (cnt - chunk * 64)) - 1ull;
+          if (!m) continue;
+          // the next gaussian's record is fetched from LDS while the current one is evaluated
+          int j_next = chunk * 64 + __builtin_ctzll(m);
+          StagedGaussian sg_next = s_g[j_next];
+          float4 c_next = s_rgb[j_next];
           while (m) {
-            const int j = chunk * 64 + __builtin_ctzll(m);
+            const int j = j_next;
+            const StagedGaussian sg = sg_next;
+            const float4 c = c_next;
             m &= m - 1;
-            const StagedGaussian sg = s_g[j];
+            if (m) {
+                j_next = chunk * 64 + __builtin_ctzll(m);
+                sg_next = s_g[j_next];
+                c_next = s_rgb[j_next];
+            }
             const float dx = sg.x - pxf, dy = sg.y - pyf;
             const float power = blend_power(sg, dx, dy);
             const bool cand = (round * kBlock + j < contributor) && power >= sg.thr && power <= 0.0f;
             if (!__any(cand)) continue;
-            float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, g3 = 0.0f, g4 = 0.0f, g5 = 0.0f, g6 = 0.0f, g7 = 0.0f, g8 = 0.0f,
-                  g9 = 0.0f;
-            bool valid = false;
-            if (cand) {
-                // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
-                // gaussian contributed to.  The per-pixel terms below also follow one fixed sequence of
-                // fused multiply-adds (the colour still behind, T c - rr, cancels heavily, so a different
-                // rounding would already move a term by ~1e-4): only the order of the sums over pixels
-                // differs from a sequential evaluation.
-                const float G = blend_expf(power);
-                const float alpha = fminf(0.99f, sg.o * G);
-                if (alpha >= P.alpha_eps) {
-                    valid = true;
-                    const float one_m = 1.0f - alpha;
-                    const float w = alpha * T;
-                    T = T * one_m;
-                    const float4 c = s_rgb[j];
-                    rr0 = __builtin_fmaf(-w, c.x, rr0);
-                    rr1 = __builtin_fmaf(-w, c.y, rr1);
-                    rr2 = __builtin_fmaf(-w, c.z, rr2);
-                    float dl = dT_term;
-                    if constexpr (kDepth) {  // render.py:1887-1890, 1948-1950
-                        rdep = __builtin_fmaf(-w, c.w, rdep);
-                        dl = __builtin_fmaf(ddep, __builtin_fmaf(T, c.w, -rdep), dl);
-                        g9 = w * ddep;       // render.py:1964-1967
-                    }
-                    if constexpr (kRgba) {   // the alpha channel blends the constant 1 (render.py:1871-1874, 1926-1931)
-                        rr3 = rr3 - w;
-                        dl = __builtin_fmaf(dr3, T - rr3, dl);
-                    }
-                    dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dl);
-                    dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
-                    dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
-                    const float dL_dalpha = dl / one_m;
-                    const float dL_dG = sg.o * dL_dalpha;
-                    const float gdx = G * dx, gdy = G * dy;
-                    // dG/du = -gdx a - gdy b and dG/dv = -gdy c - gdx b, with a = -2 ha, b = -nb, c = -2 hc
-                    const float dG_du = __builtin_fmaf(gdy, sg.nb, (2.0f * gdx) * sg.ha);
-                    const float dG_dv = __builtin_fmaf(gdx, sg.nb, (2.0f * gdy) * sg.hc);
-                    const float half = -0.5f * dL_dG;
-                    g0 = dL_dG * dG_du;
-                    g1 = dL_dG * dG_dv;
-                    g2 = (half * gdx) * dx;
-                    g3 = ((-dL_dG) * gdx) * dy;
-                    g4 = (half * gdy) * dy;
-                    g5 = dL_dalpha * G;
-                    g6 = w * dr0;
-                    g7 = w * dr1;
-                    g8 = w * dr2;
-                }
-            }
+            // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
+            // gaussian contributed to.  From here on every lane runs the same instructions: a lane the
+            // gaussian did not contribute to carries G = alpha = 0, which leaves its running state
+            // (T, colour behind) untouched and makes all of its terms exact zeros, so no lane masking
+            // or zero-filling is needed.  (exp of a non-candidate lane's power may be garbage; it is
+            // discarded by the select.)
+            const float G0 = det_expf_inrange(power);   // candidates have power in [thr, 0]
+            const float alpha0 = fminf(0.99f, sg.o * G0);
+            const bool valid = cand && alpha0 >= P.alpha_eps;
             if (!__any(valid)) continue;
+            const float G = valid ? G0 : 0.0f;
+            const float alpha = valid ? alpha0 : 0.0f;
+            // The per-pixel terms follow one fixed sequence of fused multiply-adds (the colour still
+            // behind, T c - rr, cancels heavily, so a different rounding would already move a term by
+            // ~1e-4): only the order of the sums over pixels differs from a sequential evaluation.
+            const float one_m = 1.0f - alpha;
+            const float w = alpha * T;
+            T = T * one_m;
+            rr0 = __builtin_fmaf(-w, c.x, rr0);
+            rr1 = __builtin_fmaf(-w, c.y, rr1);
+            rr2 = __builtin_fmaf(-w, c.z, rr2);
+            float dl = dT_term;
+            float g9 = 0.0f;
+            if constexpr (kDepth) {  // render.py:1887-1890, 1948-1950
+                rdep = __builtin_fmaf(-w, c.w, rdep);
+                dl = __builtin_fmaf(ddep, __builtin_fmaf(T, c.w, -rdep), dl);
+                g9 = w * ddep;       // render.py:1964-1967
+            }
+            if constexpr (kRgba) {   // the alpha channel blends the constant 1 (render.py:1871-1874, 1926-1931)
+                rr3 = rr3 - w;
+                dl = __builtin_fmaf(dr3, T - rr3, dl);
+            }
+            dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dl);
+            dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
+            dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
+            const float dL_dalpha = dl / one_m;
+            const float dL_dG = sg.o * dL_dalpha;
+            const float gdx = G * dx, gdy = G * dy;
+            // dG/du = -gdx a - gdy b and dG/dv = -gdy c - gdx b, with a = -2 ha, b = -nb, c = -2 hc
+            const float dG_du = __builtin_fmaf(gdy, sg.nb, (2.0f * gdx) * sg.ha);
+            const float dG_dv = __builtin_fmaf(gdx, sg.nb, (2.0f * gdy) * sg.hc);
+            const float half = -0.5f * dL_dG;
+            const float g0 = dL_dG * dG_du;
+            const float g1 = dL_dG * dG_dv;
+            const float g2 = (half * gdx) * dx;
+            const float g3 = ((-dL_dG) * gdx) * dy;
+            const float g4 = (half * gdy) * dy;
+            const float g5 = dL_dalpha * G;
+            const float g6 = w * dr0;
+            const float g7 = w * dr1;
+            const float g8 = w * dr2;
             // the wave totals land in different lanes: one LDS atomic instruction adds them all
             const float total = wave_reduce10(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9, hi8, hi4);
             if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }
         __syncthreads();
-        if (round * kBlock + tid < len) {
-            float v[kValues];
-            bool any = false;
-#pragma unroll
-            for (int k = 0; k < kValues; ++k) {
-                v[k] = s_grad[k][tid];
-                any = any || v[k] != 0.0f;
-            }
-            if (any) {
-                const int g = s_id[tid];
-                unsafeAtomicAdd(duv + 2 * g + 0, v[0]);
-                unsafeAtomicAdd(duv + 2 * g + 1, v[1]);
-                unsafeAtomicAdd(dconic + 3 * g + 0, v[2]);
-                unsafeAtomicAdd(dconic + 3 * g + 1, v[3]);
-                unsafeAtomicAdd(dconic + 3 * g + 2, v[4]);
-                unsafeAtomicAdd(dopacity + g, v[5]);
-                unsafeAtomicAdd(dcolor + 3 * g + 0, v[6]);
-                unsafeAtomicAdd(dcolor + 3 * g + 1, v[7]);
-                unsafeAtomicAdd(dcolor + 3 * g + 2, v[8]);
-                if constexpr (kDepth) unsafeAtomicAdd(dz + g, v[kValues - 1]);
+        // Flush: sixteen lanes add one gaussian's record (one 64-byte line) at a time, so the memory
+        // side sees one line-wide atomic request per (tile, gaussian) instead of one per value.
+        const int flush_cnt = min(kBlock, block_todo - round * kBlock);
+        const int slot_k = tid & 15;
+        for (int gl = tid >> 4; gl < flush_cnt; gl += kBlock / 16) {
+            if (slot_k < kValues) {
+                const float v = s_grad[slot_k][gl];
+                if (v != 0.0f)
+                    unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * s_id[gl] + slot_k, v);
             }
         }
     }
@@ -498,20 +500,19 @@ extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_rang
                               const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
                               const float* depths, const int32_t* tile_order, const float* final_T,
                               const int32_t* n_contrib, const float* color, const float* final_depth,
-                              const float* drgb, const float* dT, const float* ddepth, float* duv, float* dconic,
-                              float* dopacity, float* dcolor, float* dz, d3gs_stream_t stream) {
+                              const float* drgb, const float* dT, const float* ddepth, float* grad_records,
+                              d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_bwd");
     if (rc) return rc;
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb ||
-        !dT || !duv || !dconic || !dopacity || !dcolor ||
-        (p->render_depth && (!depths || !final_depth || !ddepth || !dz))) {
+        !dT || !grad_records || (p->render_depth && (!depths || !final_depth || !ddepth))) {
         set_error("d3gs_blend_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
 #define D3GS_LAUNCH_BWD(D, A)                                                                                       \
     hipLaunchKernelGGL((blend_bwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
                        workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
-                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, duv, dconic, dopacity, dcolor, dz)
+                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, grad_records)
     if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_BWD(true, true); else D3GS_LAUNCH_BWD(true, false); }
     else                 { if (p->render_rgba) D3GS_LAUNCH_BWD(false, true); else D3GS_LAUNCH_BWD(false, false); }
 #undef D3GS_LAUNCH_BWD

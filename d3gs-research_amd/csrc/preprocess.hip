@@ -232,9 +232,8 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
 __device__ __forceinline__ void preprocess_bwd_one(
     const d3gs_params& P, const int i, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const int32_t* __restrict__ radii,
-    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0, const float* __restrict__ duv,
-    const float* __restrict__ dconic, const float* dopacity_in /* may alias dopacity_out */,
-    const float* __restrict__ dcolor, const float* __restrict__ dz_in, const int sh_mask_compat,
+    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0, const float* __restrict__ grad_records,
+    const int sh_mask_compat,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* shrow, float* __restrict__ dsh_base) {
     const int K = P.sh_stride;
@@ -250,25 +249,28 @@ __device__ __forceinline__ void preprocess_bwd_one(
         return;
     }
 
+    // the blend backward's record of this gaussian: duv(2) dconic(3) dopacity dcolor(3) dz
+    const float4* rec4 = reinterpret_cast<const float4*>(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * i);
+    const float4 ra = rec4[0], rb = rec4[1], rc = rec4[2];
     const float* W = P.w2c;
     float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
     float pc[3] = {dot3(W + 0, d), dot3(W + 3, d), dot3(W + 6, d)};
     float z = pc[2];
     // pinhole backward (camera.py:357-369)
-    float gu = duv[2 * i] * P.fx, gv = duv[2 * i + 1] * P.fy;
+    float gu = ra.x * P.fx, gv = ra.y * P.fy;
     float zi = 1.0f / z, zi2 = 1.0f / (z * z);
-    float dzin = dz_in ? dz_in[i] : 0.0f;
+    float dzin = P.render_depth ? rc.y : 0.0f;
     float dpc[3] = {gu * zi, gv * zi, (dzin + ((-gu) * pc[0]) * zi2) + ((-gv) * pc[1]) * zi2};
 
     // conic -> cov2d backward (gs3d.py:571-586)
     float a = cov2d[3 * i], b = cov2d[3 * i + 1], c = cov2d[3 * i + 2];
-    float g0 = dconic[3 * i], g1 = dconic[3 * i + 1], g2 = dconic[3 * i + 2];
+    float g0 = ra.z, g1 = ra.w, g2 = rb.x;
     float det = a * c - b * b;
     float k2 = 1.0f / (det * det + 1e-8f);
     float da = k2 * ((((-c) * c) * g0 + (b * c) * g1) + (det - a * c) * g2);
     float db = (k2 * 2.0f) * (((b * c) * g0 - (det / 2.0f + b * b) * g1) + (a * b) * g2);
     float dc = k2 * ((((-a) * a) * g2 + (a * b) * g1) + (det - a * c) * g0);
-    float dop_in = dopacity_in[i];
+    float dop_in = rb.y;
     if (P.enable_anti_aliasing) {
         // render.py:3293-3306; gs3d.py:671-679: dop_in is the gradient of opacity * comp with
         // comp = sqrt(max(0.000025, ratio)), ratio = det_without_lowpass / det
@@ -390,13 +392,13 @@ __device__ __forceinline__ void preprocess_bwd_one(
     uint32_t m = ne0[i];
     float cg[3];
     if (sh_mask_compat) {
-        cg[0] = dcolor[3 * i + 0] * ((m & 1) ? 0.0f : 1.0f);
-        cg[1] = dcolor[3 * i + 1] * ((m & 2) ? 0.0f : 1.0f);
-        cg[2] = dcolor[3 * i + 2] * ((m & 4) ? 0.0f : 1.0f);
+        cg[0] = rb.z * ((m & 1) ? 0.0f : 1.0f);
+        cg[1] = rb.w * ((m & 2) ? 0.0f : 1.0f);
+        cg[2] = rc.x * ((m & 4) ? 0.0f : 1.0f);
     } else {
-        cg[0] = dcolor[3 * i + 0] * ((m & 4) ? 0.0f : 1.0f);
-        cg[1] = dcolor[3 * i + 1] * ((m & 2) ? 0.0f : 1.0f);
-        cg[2] = dcolor[3 * i + 2] * ((m & 1) ? 0.0f : 1.0f);
+        cg[0] = rb.z * ((m & 4) ? 0.0f : 1.0f);
+        cg[1] = rb.w * ((m & 2) ? 0.0f : 1.0f);
+        cg[2] = rc.x * ((m & 1) ? 0.0f : 1.0f);
     }
     const float* shp = shrow;
     const float* rest = P.has_sh_base ? shp : shp + 3;
@@ -477,8 +479,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_bwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ duv, const float* __restrict__ dconic, const float* dopacity_in,
-    const float* __restrict__ dcolor, const float* __restrict__ dz_in, const int sh_mask_compat,
+    const float* __restrict__ grad_records, const int sh_mask_compat,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     extern __shared__ float s_rows[];
@@ -488,9 +489,9 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_bwd_kernel(
     rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
     __syncthreads();
     if ((int)threadIdx.x < nrows)
-        preprocess_bwd_one(P, first + threadIdx.x, xyz, quat, scale, opacity, radii, cov2d, ne0, duv, dconic,
-                           dopacity_in, dcolor, dz_in, sh_mask_compat, dxyz, dquat, dscale, dopacity_out,
-                           s_rows + threadIdx.x * stride, dsh_base);
+        preprocess_bwd_one(P, first + threadIdx.x, xyz, quat, scale, opacity, radii, cov2d, ne0, grad_records,
+                           sh_mask_compat, dxyz, dquat, dscale, dopacity_out, s_rows + threadIdx.x * stride,
+                           dsh_base);
     __syncthreads();
     rows_lds_to_global(dsh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
 }
@@ -553,15 +554,14 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
 extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
                                    const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
-                                   const float* duv, const float* dconic, const float* dopacity_in,
-                                   const float* dcolor, const float* dz, int32_t sh_mask_compat, float* dxyz,
+                                   const float* grad_records, int32_t sh_mask_compat, float* dxyz,
                                    float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
                                    float* dcolor_sh_base, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_bwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
     if (!xyz || !quaternion_xyzw || !scale || !opacity || !color_sh || !radii || !cov2d_vecs || !sh_to_rgb_ne_0 ||
-        !duv || !dconic || !dopacity_in || !dcolor || !dxyz || !dquaternion_xyzw || !dscale || !dopacity_out ||
+        !grad_records || !dxyz || !dquaternion_xyzw || !dscale || !dopacity_out ||
         !dcolor_sh || (p->has_sh_base && !dcolor_sh_base)) {
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -569,8 +569,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
     dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
     hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
-                       scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, duv, dconic, dopacity_in, dcolor,
-                       dz, (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
+                       scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,
+                       (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
                        dcolor_sh_base);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

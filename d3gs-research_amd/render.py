@@ -82,6 +82,8 @@ class RasterizeGradientOutput:
     dcolor: torch.Tensor | None
     dcustom_features: torch.Tensor | None = None
     dz: torch.Tensor | None = None
+    # not in the reference: the [N, 16] buffer the tensors above are strided views of
+    records: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -390,20 +392,18 @@ class GaussianSplatOp:
         if render_depth:
             ddepth = grad.ddepth if grad.ddepth is not None else torch.zeros_like(out.depth)
             assert ddepth.is_contiguous() and ddepth.shape == out.depth.shape, "ddepth must be contiguous [1,H,W]"
-        # the accumulators are contiguous slices of one buffer: one zero-fill launch instead of four
-        acc = torch.zeros((10 if render_depth else 9) * n, dtype=torch.float32, device=dev)
-        duv = acc[0:2 * n].view(n, 2)
-        dconic = acc[2 * n:5 * n].view(n, 3)
-        dopacity = acc[5 * n:6 * n]
-        dcolor = acc[6 * n:9 * n].view(n, 3)
-        dz = acc[9 * n:10 * n] if render_depth else None
+        # one 64-byte record per gaussian (see D3GS_GRAD_RECORD_FLOATS); the reference's four tensors
+        # and dz are strided views of it
+        rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
             _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
             _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(out.color),
-            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(duv),
-            _capi.ptr(dconic), _capi.ptr(dopacity), _capi.ptr(dcolor), _capi.ptr(dz), s), "d3gs_blend_bwd")
-        return RasterizeGradientOutput(duv=duv, dconic=dconic, dopacity=dopacity, dcolor=dcolor, dz=dz)
+            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec), s),
+            "d3gs_blend_bwd")
+        res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
+                                      dz=rec[:, 9] if render_depth else None, records=rec)
+        return res
 
     # --------------------------------------------------------------- backward
     def backward(self, model: GaussianModelOriginBase, cameras, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
@@ -428,20 +428,19 @@ class GaussianSplatOp:
             dscale = torch.empty_like(model.scale)
             dsh = torch.empty_like(model.color_sh)
             dsh_base = torch.empty_like(model.color_sh_base) if model.color_sh_base is not None else None
-            # opacity gradient is finished in place in the buffer the blend accumulated into
-            # (render.py:2918 external_tensors={"opacity": dopacity})
+            dopacity = torch.empty_like(model.opacity)
             _capi.check(L.d3gs_preprocess_bwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.duv), _capi.ptr(g.dconic), _capi.ptr(g.dopacity),
-                _capi.ptr(g.dcolor), _capi.ptr(g.dz), int(self._cfg.compat_ref_sh_mask_bitorder), _capi.ptr(dxyz),
-                _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(g.dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), s),
+                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), int(self._cfg.compat_ref_sh_mask_bitorder),
+                _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh),
+                _capi.ptr(dsh_base), s),
                 "d3gs_preprocess_bwd")
-        grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=g.dopacity,
+        grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,
                                          color_sh=dsh, color_sh_base=dsh_base)
         self.last_raster_grads = g
         if return_uv_grad:
-            return grad_model, g.duv.view(1, -1, 2), None
+            return grad_model, g.duv.unsqueeze(0), None
         return grad_model, None, None
 
 

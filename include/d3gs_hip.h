@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 5
+#define D3GS_ABI_VERSION 6
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -159,29 +159,38 @@ int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const i
                    const int32_t* tile_order /* from d3gs_tile_ranges, or NULL for raster order */, float* color,
                    float* final_T, int32_t* n_contrib, float* final_depth, d3gs_stream_t stream);
 
+/* Per-gaussian gradient record written by K7 and read by K9: one 64-byte line per gaussian so that
+ * the sixteen lanes flushing one gaussian issue a single line-wide atomic request.  The reference keeps
+ * four separate tensors (duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3], render.py:1388-1411) and dz;
+ * they are the strided slices below of this buffer. */
+#define D3GS_GRAD_RECORD_FLOATS 16
+#define D3GS_GRAD_DUV 0      /* 2 floats */
+#define D3GS_GRAD_DCONIC 2   /* 3 floats */
+#define D3GS_GRAD_DOPACITY 5 /* 1 float  */
+#define D3GS_GRAD_DCOLOR 6   /* 3 floats */
+#define D3GS_GRAD_DZ 9       /* 1 float, written with p->render_depth */
+
 /* K7 — replaces kernel_raw("rasterize_True_...") (same generator, grad != None,
  * render.py:1341, 1589-1676, 1774-2210).  Produces the complete gradient (the
  * reference's backward_reduction_balanced_factor <= 0 branch, render.py:2024-2050,
- * 2182-2210).  duv [N,2], dconic [N,3], dopacity [N], dcolor [N,3] and, with
- * p->render_depth, dz [N] are accumulated with atomics: zero-fill them first.
- * drgb has the layout of color; final_depth / ddepth [H,W] and dz may be NULL
- * without p->render_depth. */
+ * 2182-2210).  grad_records [N][D3GS_GRAD_RECORD_FLOATS] is accumulated with
+ * atomics: zero-fill it first.  drgb has the layout of color; final_depth /
+ * ddepth [H,W] may be NULL without p->render_depth. */
 int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                    const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
                    const int32_t* tile_order, const float* final_T, const int32_t* n_contrib, const float* color,
-                   const float* final_depth, const float* drgb, const float* dT, const float* ddepth, float* duv,
-                   float* dconic, float* dopacity, float* dcolor, float* dz, d3gs_stream_t stream);
+                   const float* final_depth, const float* drgb, const float* dT, const float* ddepth,
+                   float* grad_records, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
- * (body 3217-3356).  Chain rule from (duv, dconic, dopacity, dcolor[, dz]) to
- * the raw model tensors, including the fused activation gradients.  Gradients
- * of gaussians with radii == 0 are written as zeros.  dz and the *_base
+ * (body 3217-3356).  Chain rule from K7's records (duv, dconic, dopacity, dcolor
+ * [, dz]) to the raw model tensors, including the fused activation gradients.
+ * Gradients of gaussians with radii == 0 are written as zeros.  The *_base
  * pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
  * reference's reversed bit order (render.py:3344-3350). */
 int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
-                        const uint8_t* sh_to_rgb_ne_0, const float* duv, const float* dconic,
-                        const float* dopacity_in, const float* dcolor, const float* dz, int32_t sh_mask_compat,
+                        const uint8_t* sh_to_rgb_ne_0, const float* grad_records, int32_t sh_mask_compat,
                         float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
                         float* dcolor_sh_base, d3gs_stream_t stream);
 

@@ -71,7 +71,8 @@ def test_forward_and_backward(oracle, cfg_id, n, wh, filt, aa, depth, rgba, nchw
     torch.cuda.synchronize()
     g = op.last_raster_grads
     mass = g_ref["absmass"]
-    checks = [("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)), ("dcolor", g.dcolor, slice(6, 9))]
+    checks = [("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)), ("dopacity", g.dopacity, slice(5, 6)),
+              ("dcolor", g.dcolor, slice(6, 9))]
     if depth:
         checks.append(("dz", g.dz, slice(9, 10)))
     for name, got, cols in checks:

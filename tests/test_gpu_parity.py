@@ -113,11 +113,11 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
     cpu = lambda t: t.detach().cpu().numpy()
     # blend backward: a float32 sum of n terms in any order is within ~n*eps*sum|terms| of the exact
     # sum, so each value is judged against the oracle's sum of absolute terms ("absmass"); on top of
-    # that the plain elementwise 1e-4 relative check.  dopacity was finished in place by preprocess
-    # backward, so it is compared below through the isolated call.
+    # that the plain elementwise 1e-4 relative check.
     mass = g_ref["absmass"]
-    for name, got, cols in (("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)), ("dcolor", g.dcolor, slice(6, 9))):
-        a, b = cpu(got).astype(np.float64), g_ref[name]
+    for name, got, cols in (("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)),
+                            ("dopacity", g.dopacity, slice(5, 6)), ("dcolor", g.dcolor, slice(6, 9))):
+        a, b = cpu(got).astype(np.float64).reshape(scene.n, -1), g_ref[name].reshape(scene.n, -1)
         excess = np.abs(a - b) - (1e-4 * mass[:, cols] + 1e-30)
         assert (excess <= 0).all(), f"{name}: {int((excess > 0).sum())} values beyond 1e-4 * sum|terms|"
         ok, worst, nbad = grad_close(a, b)
@@ -142,16 +142,17 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
     from d3gs_research_amd import _capi
     L = _capi.lib()
     Pg = op.make_params(model, scene.camera(), True)
-    dop_io = f32(g_ref["dopacity"])
-    in_duv, in_dconic, in_dcolor = f32(g_ref["duv"]), f32(g_ref["dconic"]), f32(g_ref["dcolor"])  # keep alive
+    rec_np = np.zeros((scene.n, _capi.GRAD_RECORD_FLOATS), np.float32)
+    rec_np[:, 0:2], rec_np[:, 2:5], rec_np[:, 5], rec_np[:, 6:9] = g_ref["duv"], g_ref["dconic"], g_ref["dopacity"], g_ref["dcolor"]
+    rec = f32(rec_np)
+    dop_io = torch.empty_like(model.opacity)
     o_xyz, o_q, o_s = torch.empty_like(model.xyz), torch.empty_like(model.quaternion_xyzw), torch.empty_like(model.scale)
     o_sh = torch.empty_like(model.color_sh)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     _capi.check(L.d3gs_preprocess_bwd(
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(in_duv), _capi.ptr(in_dconic),
-        _capi.ptr(dop_io), _capi.ptr(in_dcolor), None, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
         _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, stream), "d3gs_preprocess_bwd")
     torch.cuda.synchronize()
     for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", dop_io), ("dsh", o_sh)):
