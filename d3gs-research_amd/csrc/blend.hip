@@ -230,28 +230,30 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 const StagedGaussian sg = s_g[j];
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
                 const float power = blend_power(sg, dx, dy);
-                if (!done && power >= sg.thr) {
-                    const float G = blend_expf(power);
-                    const float alpha = fminf(0.99f, sg.o * G);
-                    if (alpha >= P.alpha_eps) {
-                        const float nextT = T * (1.0f - alpha);
-                        const bool should_done = nextT < P.transmittance_eps;
-                        if (power > 0.0f || should_done) {
-                            done = should_done;
-                        } else {
-                            const float w = alpha * T;
-                            T = nextT;
-                            contributor = round * kBlock + j;
-                            const float4 c = s_rgb[j];
-                            acc0 = __builtin_fmaf(w, c.x, acc0);
-                            acc1 = __builtin_fmaf(w, c.y, acc1);
-                            acc2 = __builtin_fmaf(w, c.z, acc2);
-                            if constexpr (kRgba) acc3 = acc3 + w;
-                            if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
-                        }
-                    }
-                }
-                if (__all(done)) {
+                const bool live = !done && power >= sg.thr;
+                if (!__any(live)) continue;
+                // From here on every lane runs the same instructions and the outcome is applied with
+                // selects (w = 0 leaves the accumulators untouched): far fewer scalar mask operations
+                // than nested per-lane branches.  exp of a lane that is not live may be garbage; it is
+                // never selected.
+                const float G = blend_expf(power);
+                const float alpha = fminf(0.99f, sg.o * G);
+                const bool hit = live && alpha >= P.alpha_eps;
+                const float nextT = T * (1.0f - alpha);
+                const bool should_done = nextT < P.transmittance_eps;
+                const bool stop = hit && should_done;                      // render.py:1781-1792
+                const bool use = hit && !should_done && !(power > 0.0f);
+                const float w = use ? alpha * T : 0.0f;
+                T = use ? nextT : T;
+                contributor = use ? round * kBlock + j : contributor;
+                const float4 c = s_rgb[j];
+                acc0 = __builtin_fmaf(w, c.x, acc0);
+                acc1 = __builtin_fmaf(w, c.y, acc1);
+                acc2 = __builtin_fmaf(w, c.z, acc2);
+                if constexpr (kRgba) acc3 = acc3 + w;
+                if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
+                done = done || stop;
+                if (__any(stop) && __all(done)) {
                     wave_done = true;
                     break;
                 }
@@ -428,18 +430,18 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
             dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
             const float dL_dalpha = dl / one_m;
-            const float dL_dG = sg.o * dL_dalpha;
-            const float gdx = G * dx, gdy = G * dy;
-            // dG/du = -gdx a - gdy b and dG/dv = -gdy c - gdx b, with a = -2 ha, b = -nb, c = -2 hc
-            const float dG_du = __builtin_fmaf(gdy, sg.nb, (2.0f * gdx) * sg.ha);
-            const float dG_dv = __builtin_fmaf(gdx, sg.nb, (2.0f * gdy) * sg.hc);
-            const float half = -0.5f * dL_dG;
-            const float g0 = dL_dG * dG_du;
-            const float g1 = dL_dG * dG_dv;
-            const float g2 = (half * gdx) * dx;
-            const float g3 = ((-dL_dG) * gdx) * dy;
-            const float g4 = (half * gdy) * dy;
+            // With q = dL/dG * G the screen-space gradients are linear in five moments of q:
+            // dL/du = -(a S1 + b S2), dL/dv = -(c S2 + b S1), dL/dconic = (-S3/2, -S4, -S5/2), where
+            // S1 = sum q dx, S2 = sum q dy, S3 = sum q dx^2, S4 = sum q dx dy, S5 = sum q dy^2
+            // (render.py:1996-2017 evaluates the products per pixel).  The lanes only form the
+            // moments; the per-gaussian map is applied once per (tile, gaussian) before the flush.
             const float g5 = dL_dalpha * G;
+            const float q = sg.o * g5;
+            const float g0 = q * dx;
+            const float g1 = q * dy;
+            const float g2 = g0 * dx;
+            const float g3 = g0 * dy;
+            const float g4 = g1 * dy;
             const float g6 = w * dr0;
             const float g7 = w * dr1;
             const float g8 = w * dr2;
@@ -449,9 +451,19 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
           }
         }
         __syncthreads();
+        const int flush_cnt = min(kBlock, block_todo - round * kBlock);
+        if (tid < flush_cnt) {  // moments -> (duv, dconic) of gaussian tid, with a = -2 ha, b = -nb, c = -2 hc
+            const StagedGaussian sg = s_g[tid];
+            const float S1 = s_grad[0][tid], S2 = s_grad[1][tid];
+            s_grad[0][tid] = __builtin_fmaf(sg.nb, S2, (2.0f * sg.ha) * S1);
+            s_grad[1][tid] = __builtin_fmaf(sg.nb, S1, (2.0f * sg.hc) * S2);
+            s_grad[2][tid] = -0.5f * s_grad[2][tid];
+            s_grad[3][tid] = -s_grad[3][tid];
+            s_grad[4][tid] = -0.5f * s_grad[4][tid];
+        }
+        __syncthreads();
         // Flush: sixteen lanes add one gaussian's record (one 64-byte line) at a time, so the memory
         // side sees one line-wide atomic request per (tile, gaussian) instead of one per value.
-        const int flush_cnt = min(kBlock, block_todo - round * kBlock);
         const int slot_k = tid & 15;
         for (int gl = tid >> 4; gl < flush_cnt; gl += kBlock / 16) {
             if (slot_k < kValues) {

@@ -719,7 +719,6 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     if (!valid) continue;
                     // fixed operation sequence (shared with the HIP kernel) so that the per-pixel terms
                     // agree bit for bit and only the order of the sums differs
-                    const float ha = -0.5f * co[0], nb = -co[1], hc = -0.5f * co[2];
                     const float one_m = 1.0f - alpha;
                     float w = alpha * T;
                     T = T * one_m;
@@ -741,17 +740,17 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     dl = fmaf(dr[1], fmaf(T, cg[1], -rr[1]), dl);
                     dl = fmaf(dr[0], fmaf(T, cg[0], -rr[0]), dl);
                     float dL_dalpha = dl / one_m;
-                    float dL_dG = co[3] * dL_dalpha;
-                    float gdx = G * dx, gdy = G * dy;
-                    // dG/du = -gdx a - gdy b, dG/dv = -gdy c - gdx b  (a = -2 ha, b = -nb, c = -2 hc)
-                    float dG_du = fmaf(gdy, nb, (2.0f * gdx) * ha);
-                    float dG_dv = fmaf(gdx, nb, (2.0f * gdy) * hc);
-                    const float half = -0.5f * dL_dG;
+                    // With q = dL/dG * G, the screen-space gradients are linear in five moments of q
+                    // (render.py:1996-2017 per pixel):  dL/du = -(a S1 + b S2), dL/dv = -(c S2 + b S1),
+                    // dL/dconic = (-S3 / 2, -S4, -S5 / 2) with S1 = sum q dx, S2 = sum q dy, S3 = sum q dx^2,
+                    // S4 = sum q dx dy, S5 = sum q dy^2.  The moments are accumulated per pixel and the
+                    // per-gaussian linear map is applied once per (tile, gaussian), as the kernel does.
+                    const float gop = dL_dalpha * G;       // dL/dopacity term
+                    const float q = co[3] * gop;
+                    const float qx = q * dx, qy = q * dy;
                     double* a9 = acc.data() + (size_t)j * NV;
                     double* m9 = mass.data() + (size_t)j * NV;
-                    // dconic = dL/dG * (-1/2 G dx^2, -G dx dy, -1/2 G dy^2): no 1/2 on the off-diagonal (render.py:2013-2017)
-                    const float term[NV] = {dL_dG * dG_du, dL_dG * dG_dv, (half * gdx) * dx, ((-dL_dG) * gdx) * dy,
-                                            (half * gdy) * dy, dL_dalpha * G, w * dr[0], w * dr[1], w * dr[2],
+                    const float term[NV] = {qx, qy, qx * dx, qx * dy, qy * dy, gop, w * dr[0], w * dr[1], w * dr[2],
                                             w * ddep /* render.py:1964-1967 */};
                     for (int k = 0; k < NV; ++k) {
                         a9[k] += (double)term[k];
@@ -759,6 +758,23 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     }
                 }
             }
+        // moments -> (duv, dconic) per (tile, gaussian); the magnitudes follow the same map with absolute values
+        for (int j = 0; j < len; ++j) {
+            const float* co = conic_opacity + 4 * idx_sorted[r0 + j];
+            const double a = co[0], b = co[1], c = co[2];
+            double* S = acc.data() + (size_t)j * NV;
+            double* Ms = mass.data() + (size_t)j * NV;
+            const double S1 = S[0], S2 = S[1], M1 = Ms[0], M2 = Ms[1];
+            S[0] = -(a * S1 + b * S2);
+            S[1] = -(c * S2 + b * S1);
+            S[2] = -0.5 * S[2];
+            S[3] = -S[3];
+            S[4] = -0.5 * S[4];
+            Ms[0] = fabs(a) * M1 + fabs(b) * M2;
+            Ms[1] = fabs(c) * M2 + fabs(b) * M1;
+            Ms[2] = 0.5 * Ms[2];
+            Ms[4] = 0.5 * Ms[4];
+        }
         for (int j = 0; j < len; ++j) {
             int g = idx_sorted[r0 + j];
             const double* a9 = acc.data() + (size_t)j * NV;
