@@ -95,6 +95,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             const float* __restrict__ depths,
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ order,
+                                                            const unsigned long long* __restrict__ tile_masks,
                                                             uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
     // no early return: every lane takes part in the cooperative emission of large gaussians
@@ -112,12 +113,24 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     // a caller that passed a smaller buffer than the scan total must never be written past
     const bool active = in_range && sane && r > 0 && end <= m;
     const uint32_t dbits = __float_as_uint(depths[i]);
-    const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
-    const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
-    TileWalkIn g{uv.x, uv.y, (float)r, co.x, co.y, co.z, co.w};
+    // the preprocess kernel's record of the kept tiles, when it was asked to write one
+    bool walk_again = active;
+    if (tile_masks && active) {
+        const unsigned long long meta = tile_masks[2 * (size_t)i + 1];
+        if (meta & kTileMaskHas) {
+            mask_tile_emit(tile_masks[2 * (size_t)i], meta, P.tiles_x, dbits, i, off, end, keys, vals);
+            walk_again = false;
+        }
+    }
+    if (!__any(walk_again)) return;   // wave-uniform
     TileWalk walk = {};
-    if (active) walk = tile_walk_setup(P, g);
-    wave_tile_emit(P.filter_algo, active, walk, P.tiles_x, dbits, i, off, end, keys, vals);
+    if (walk_again) {
+        const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
+        const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
+        TileWalkIn g{uv.x, uv.y, (float)r, co.x, co.y, co.z, co.w};
+        walk = tile_walk_setup(P, g);
+    }
+    wave_tile_emit(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
 }
 
 // Sort keys of the gaussians themselves: the float bits of the depth (positive floats order like
@@ -240,7 +253,8 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
 
 extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                               const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                              uint64_t* keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
+                              const uint64_t* tile_masks, uint64_t* keys, int32_t* gaussian_idx, int64_t m,
+                              d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
@@ -250,7 +264,8 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     hipLaunchKernelGGL(make_keys_kernel, dim3((p->n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, keys, gaussian_idx, (long long)m);
+                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, (const unsigned long long*)tile_masks, keys,
+                       gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

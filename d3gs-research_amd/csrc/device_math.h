@@ -185,25 +185,34 @@ struct TileWalk {
     int rminx, rminy, rmaxx, rmaxy;  // 3-sigma tile rect
     int bminx, bminy, bw, bh;        // candidate rect (origin, size); the 3-sigma rect when no filter
     float uo, vo, bx, by;            // centre relative to the candidate rect origin, AABB half extents
-    float ow, oh, os, oc;            // oriented box: width, height, sin, cos; ELLIPSE: conic a, b, c and the bound
+    float ow, oh, os, oc;            // OBB: axis radii r1, r2 (ow, oh) and sin, cos; ELLIPSE: conic a, b, c and the bound
+    float or3, or4;                  // OBB: axis radii r3, r4
 };
 
-__device__ __forceinline__ bool obb_overlaps_box(float bx0, float by0, float bx1, float by1, float w, float h, float s,
-                                                 float c, float cu, float cv) {
-    // 4-axis separating-axis test (gs3d.py:1254-1322).  With NaN sin/cos every
-    // "<=" below is false, so the tile is kept.
-    float l1x = (bx1 - bx0) / 2.0f, l1y = (by1 - by0) / 2.0f;
-    float l2x = w / 2.0f, l2y = h / 2.0f;
-    float lx = (bx1 + bx0) / 2.0f - cu, ly = (by1 + by0) / 2.0f - cv;
-    float r1, r2, r3, r4;
-    r1 = l1x * 1.0f; r2 = l1y * 0.0f; r3 = l2x * fabsf(c); r4 = l2y * fabsf(-s);
-    if (((r1 + r2) + r3) + r4 <= fabsf(lx)) return false;
-    r1 = l1x * 0.0f; r2 = l1y * 1.0f; r3 = l2x * fabsf(s); r4 = l2y * fabsf(c);
-    if (((r1 + r2) + r3) + r4 <= fabsf(ly)) return false;
-    r1 = l1x * fabsf(c); r2 = l1y * fabsf(s); r3 = l2x * fabsf(c * c + s * s); r4 = l2y * fabsf((-s) * c + c * s);
-    if (((r1 + r2) + r3) + r4 <= fabsf(lx * c + ly * s)) return false;
-    r1 = l1x * fabsf(-s); r2 = l1y * fabsf(c); r3 = l2x * fabsf(c * (-s) + s * c); r4 = l2y * fabsf((-s) * (-s) + c * c);
-    if (((r1 + r2) + r3) + r4 <= fabsf(lx * (-s) + ly * c)) return false;
+// Separating-axis test of a 16x16 tile box against the oriented box of a gaussian
+// (gs3d.py:1254-1322).  With l1 = (8, 8) the tile half extents, l2 = (w/2, h/2) the box half
+// extents and (c, s) the box direction, the four projected-radius sums do not depend on the tile:
+// they are formed once per gaussian, in the operation order of the reference's expression
+// ((r1 + r2) + r3) + r4, and the per-tile work is the projection of the centre offset on each
+// axis.  With NaN sin/cos every "<=" is false, so the tile is kept.
+struct ObbAxes { float r1, r2, r3, r4, s, c; };
+__device__ __forceinline__ ObbAxes obb_axes(float w, float h, float s, float c) {
+    const float l1x = 8.0f, l1y = 8.0f, l2x = w / 2.0f, l2y = h / 2.0f;
+    ObbAxes a;
+    a.r1 = ((l1x * 1.0f + l1y * 0.0f) + l2x * fabsf(c)) + l2y * fabsf(-s);
+    a.r2 = ((l1x * 0.0f + l1y * 1.0f) + l2x * fabsf(s)) + l2y * fabsf(c);
+    a.r3 = ((l1x * fabsf(c) + l1y * fabsf(s)) + l2x * fabsf(c * c + s * s)) + l2y * fabsf((-s) * c + c * s);
+    a.r4 = ((l1x * fabsf(-s) + l1y * fabsf(c)) + l2x * fabsf(c * (-s) + s * c)) + l2y * fabsf((-s) * (-s) + c * c);
+    a.s = s;
+    a.c = c;
+    return a;
+}
+__device__ __forceinline__ bool obb_overlaps_tile(float bx0, float by0, const ObbAxes& a, float cu, float cv) {
+    const float lx = (bx0 + 8.0f) - cu, ly = (by0 + 8.0f) - cv;   // (bx1 + bx0) / 2 is exactly bx0 + 8
+    if (a.r1 <= fabsf(lx)) return false;
+    if (a.r2 <= fabsf(ly)) return false;
+    if (a.r3 <= fabsf(lx * a.c + ly * a.s)) return false;
+    if (a.r4 <= fabsf(lx * (-a.s) + ly * a.c)) return false;
     return true;
 }
 
@@ -246,7 +255,7 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
     w.rminy = tile_coord((g.v - g.radius) / 16.0f, TY);
     w.rmaxx = tile_coord((((g.u + g.radius) + 16.0f) - 1.0f) / 16.0f, TX);
     w.rmaxy = tile_coord((((g.v + g.radius) + 16.0f) - 1.0f) / 16.0f, TY);
-    w.uo = w.vo = w.bx = w.by = w.ow = w.oh = w.os = w.oc = 0.0f;
+    w.uo = w.vo = w.bx = w.by = w.ow = w.oh = w.os = w.oc = w.or3 = w.or4 = 0.0f;
     if (P.filter_algo == D3GS_FILTER_NONE) {
         w.bminx = w.rminx;
         w.bminy = w.rminy;
@@ -289,8 +298,11 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
         v2y = v2y / len;
         float minor = 1.0f / sqrtf(e1 * s1);
         float major = 1.0f / sqrtf(e2 * s2);
-        w.ow = major * 2.0f;
-        w.oh = minor * 2.0f;
+        const ObbAxes ax = obb_axes(major * 2.0f, minor * 2.0f, v2y, v2x);
+        w.ow = ax.r1;
+        w.oh = ax.r2;
+        w.or3 = ax.r3;
+        w.or4 = ax.r4;
         w.os = v2y;
         w.oc = v2x;
     } else if (P.filter_algo == D3GS_FILTER_ELLIPSE) {
@@ -315,7 +327,8 @@ __device__ __forceinline__ bool tile_keep(const int filter_algo, const TileWalk&
     } else if (filter_algo == D3GS_FILTER_ELLIPSE) {
         keep = ellipse_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
     } else {
-        keep = obb_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
+        const ObbAxes ax{w.ow, w.oh, w.or3, w.or4, w.os, w.oc};
+        keep = obb_overlaps_tile(px0, py0, ax, w.uo, w.vo);
     }
     const int x = lx + w.bminx, y = ly + w.bminy;
     return keep && x >= w.rminx && x < w.rmaxx && y >= w.rminy && y < w.rmaxy;
@@ -335,22 +348,42 @@ __device__ __forceinline__ TileWalk bcast_walk(const TileWalk& w, int src) {
     r.bx = bcast_f(w.bx, src); r.by = bcast_f(w.by, src);
     r.ow = bcast_f(w.ow, src); r.oh = bcast_f(w.oh, src);
     r.os = bcast_f(w.os, src); r.oc = bcast_f(w.oc, src);
+    r.or3 = bcast_f(w.or3, src); r.or4 = bcast_f(w.or4, src);
     return r;
 }
 
 constexpr int kSmallWalk = 16;  // candidate tiles a lane walks alone before the wavefront takes over
 
+// Compact record of a gaussian's kept tiles, written by the preprocess kernel so that key
+// expansion does not repeat the per-tile tests: word 0 is a bit mask over the candidate rect in
+// row-major order (bit ly * bw + lx), word 1 packs the rect origin and width.  Gaussians whose
+// candidate rect has more than 64 tiles carry no mask (kTileMaskNone) and are walked again.
+constexpr unsigned long long kTileMaskHas = 1ull << 40;
+__device__ __forceinline__ unsigned long long tile_mask_meta(const TileWalk& w, bool has_mask) {
+    return (unsigned long long)(uint32_t)w.bminx | ((unsigned long long)(uint32_t)w.bminy << 16) |
+           ((unsigned long long)(uint32_t)w.bw << 32) | (has_mask ? kTileMaskHas : 0ull);
+}
+
 // Number of kept tiles of this lane's gaussian.  Must be called by all 64 lanes of a wavefront
-// (lanes without a gaussian pass active = false).
-__device__ __forceinline__ int wave_tile_count(const int filter_algo, bool active, const TileWalk& w) {
+// (lanes without a gaussian pass active = false).  `mask` receives the kept-tile bit mask when the
+// candidate rect has at most 64 tiles (`has_mask`).
+__device__ __forceinline__ int wave_tile_count(const int filter_algo, bool active, const TileWalk& w,
+                                               unsigned long long& mask, bool& has_mask) {
     const int area = active ? w.bw * w.bh : 0;
-    if (filter_algo == D3GS_FILTER_NONE) return area;
+    has_mask = active && area <= 64 && w.bw <= 64;
+    mask = 0ull;
+    if (filter_algo == D3GS_FILTER_NONE) {
+        if (has_mask) mask = area == 64 ? ~0ull : (1ull << area) - 1ull;
+        return area;
+    }
     int count = 0;
     const bool big = area > kSmallWalk;
     if (!big) {
         for (int t = 0; t < area; ++t) {
             const int ly = t / w.bw;
-            count += tile_keep(filter_algo, w, t - ly * w.bw, ly) ? 1 : 0;
+            const bool k = tile_keep(filter_algo, w, t - ly * w.bw, ly);
+            count += k ? 1 : 0;
+            mask |= k ? (1ull << t) : 0ull;
         }
     }
     const int lane = threadIdx.x & 63;
@@ -361,6 +394,7 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
         const TileWalk ws = bcast_walk(w, src);
         const int a = ws.bw * ws.bh;
         int c = 0;
+        unsigned long long first = 0ull;
         for (int base = 0; base < a; base += 64) {
             const int t = base + lane;
             bool k = false;
@@ -368,11 +402,35 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
                 const int ly = t / ws.bw;
                 k = tile_keep(filter_algo, ws, t - ly * ws.bw, ly);
             }
-            c += __popcll(__ballot(k));
+            const unsigned long long b = __ballot(k);
+            if (base == 0) first = b;
+            c += __popcll(b);
         }
-        if (lane == src) count = c;
+        if (lane == src) {
+            count = c;
+            mask = first;   // the whole rect when it has at most 64 tiles
+        }
     }
     return count;
+}
+
+// Emits the tiles named by a kept-tile mask.  Per lane; consecutive lanes write consecutive runs.
+__device__ __forceinline__ void mask_tile_emit(unsigned long long mask, unsigned long long meta, int tiles_x,
+                                               uint32_t depth_bits, int value, long long off, long long end,
+                                               uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+    const int bminx = (int)(meta & 0xFFFFu), bminy = (int)((meta >> 16) & 0xFFFFu), bw = (int)((meta >> 32) & 0xFFu);
+    const uint32_t recip = bw > 0 ? (65536u + (uint32_t)bw - 1u) / (uint32_t)bw : 0u;  // exact t / bw for t < 64
+    while (mask) {
+        const int t = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        const int ly = (int)(((uint32_t)t * recip) >> 16), lx = t - ly * bw;
+        if (off < end) {
+            const uint64_t tile = (uint64_t)(uint32_t)((ly + bminy) * tiles_x + lx + bminx);
+            keys[off] = (tile << 32) | depth_bits;
+            vals[off] = value;
+        }
+        ++off;
+    }
 }
 
 // Emits (key, value) of every kept tile of this lane's gaussian at [off, end) in row-major tile

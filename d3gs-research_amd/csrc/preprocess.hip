@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const float* __restrict__ sh_base, const uint8_t* __restrict__ invalid_mask, float* __restrict__ depths,
     int32_t* __restrict__ radii, float* __restrict__ uvs, float* __restrict__ conic_opacity,
     int32_t* __restrict__ tiles_touched, float* __restrict__ rgb_out, float* __restrict__ cov2d_out,
-    uint8_t* __restrict__ ne0_out) {
+    uint8_t* __restrict__ ne0_out, unsigned long long* __restrict__ tile_masks) {
     // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
     extern __shared__ float s_rows[];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
@@ -114,6 +114,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     float z = 0.0f, u = 0.0f, v = 0.0f, con0 = 0.0f, con1 = 0.0f, con2 = 0.0f, op = 0.0f;
     float a = 0.0f, b = 0.0f, c = 0.0f, radius = 0.0f;
     int count = 0;
+    unsigned long long kept_mask = 0ull, kept_meta = 0ull;
     float rgb[3] = {0.0f, 0.0f, 0.0f};
     uint32_t ne0 = 0;
 
@@ -189,7 +190,9 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         TileWalkIn g{u, v, radius, con0, con1, con2, op};
         TileWalk walk = {};
         if (valid) walk = tile_walk_setup(P, g);
-        count = wave_tile_count(P.filter_algo, valid, walk);
+        bool has_mask;
+        count = wave_tile_count(P.filter_algo, valid, walk, kept_mask, has_mask);
+        kept_meta = tile_mask_meta(walk, has_mask);
     }
     if (valid) {
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
@@ -212,6 +215,10 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     *reinterpret_cast<float2*>(uvs + 2 * i) = make_float2(u, v);
     *reinterpret_cast<float4*>(conic_opacity + 4 * i) = make_float4(con0, con1, con2, op);
     tiles_touched[i] = count;
+    if (tile_masks) {
+        tile_masks[2 * (size_t)i] = kept_mask;
+        tile_masks[2 * (size_t)i + 1] = kept_meta;
+    }
     rgb_out[3 * i + 0] = rgb[0];
     rgb_out[3 * i + 1] = rgb[1];
     rgb_out[3 * i + 2] = rgb[2];
@@ -532,7 +539,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
                                    const float* color_sh_base, const uint8_t* invalid_mask, float* depths,
                                    int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
                                    float* rgb_gaussian, float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0,
-                                   d3gs_stream_t stream) {
+                                   uint64_t* tile_masks, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_fwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -545,7 +552,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
     hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
                        opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity, tiles_touched,
-                       rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0);
+                       rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

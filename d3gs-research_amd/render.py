@@ -265,11 +265,14 @@ class GaussianSplatOp:
             rgb_gaussian = torch.empty((n, 3), dtype=f32, device=dev)
             cov2d_vecs = torch.empty((n, 3), dtype=f32, device=dev) if training else None
             ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
+            # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
+            tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                _capi.ptr(tiles_touched), _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs), _capi.ptr(ne0), s),
+                _capi.ptr(tiles_touched), _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs), _capi.ptr(ne0),
+                _capi.ptr(tile_masks), s),
                 "d3gs_preprocess_fwd")
 
         def _sort(keys_a, vals_a, count, begin_bit, end_bit):
@@ -337,7 +340,8 @@ class GaussianSplatOp:
             gaussian_idx = torch.empty(num_rendered, dtype=i32, device=dev)
             _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                                          _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                         _capi.ptr(keys), _capi.ptr(gaussian_idx), num_rendered, s), "d3gs_make_keys")
+                                         _capi.ptr(tile_masks), _capi.ptr(keys), _capi.ptr(gaussian_idx),
+                                         num_rendered, s), "d3gs_make_keys")
 
         with self._stage("sort"):
             end_bit = 32 + L.d3gs_higher_msb(num_tiles)

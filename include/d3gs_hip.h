@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 6
+#define D3GS_ABI_VERSION 7
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -94,12 +94,15 @@ int d3gs_higher_msb(uint32_t n);
  * EWA covariance, conic, radius, tile rect, validity, tile count under the chosen
  * early filter, SH colour.  Outputs of rejected gaussians are written as zeros.
  * cov2d_vecs and sh_to_rgb_ne_0 may be NULL (inference). sh_base may be NULL.
- * invalid_mask (uint8[N], may be NULL): non-zero rejects the gaussian (render.py:306-308). */
+ * invalid_mask (uint8[N], may be NULL): non-zero rejects the gaussian (render.py:306-308).
+ * tile_masks (uint64[N][2], may be NULL; no counterpart in the reference): a record of the tiles the
+ * early filter kept for each gaussian (word 0: bit mask over its candidate rect, word 1: the rect), which
+ * d3gs_make_keys expands instead of repeating the per-tile tests. */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const float* color_sh_base,
                         const uint8_t* invalid_mask, float* depths,
                         int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
-                        float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
+                        float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, uint64_t* tile_masks, d3gs_stream_t stream);
 
 /* K2 — replaces `tiles_touched.cumsum_(0)` + `.item()` at render.py:694-695.
  * In-place inclusive scan; the grand total is written to *total_dev (device
@@ -113,10 +116,11 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
  * scan of tiles_touched from d3gs_scan_tiles, m = its total, pairs are emitted in
  * gaussian-index order.  With gaussian_order (a permutation of 0..n-1), slot j emits
  * gaussian gaussian_order[j] and offsets must be the inclusive scan of the tile counts
- * taken in that order (see d3gs_depth_keys). */
+ * taken in that order (see d3gs_depth_keys).  tile_masks (may be NULL) is the record
+ * d3gs_preprocess_fwd wrote with the same params; the pairs emitted are the same either way. */
 int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
-                   const float* depths, const int32_t* offsets, const int32_t* gaussian_order, uint64_t* keys,
-                   int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
+                   const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                   const uint64_t* tile_masks, uint64_t* keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
 
 /* Depth-first factorisation of the pair sort (no counterpart in the reference, which
  * radix-sorts all M pairs on the full (tile, depth) key; the result is bit-identical).

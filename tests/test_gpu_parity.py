@@ -197,7 +197,8 @@ def test_empty_scene_returns_background():
 
 
 @pytest.mark.parametrize("m,begin,end", [(1, 0, 45), (255, 0, 8), (4096, 0, 45), (4097, 3, 41), (100003, 0, 64),
-                                         (1 << 20, 0, 47), (300000, 32, 45)])
+                                         (1 << 20, 0, 47), (300000, 32, 45), ((1 << 21) + 1, 0, 45), (1 << 21, 32, 45),
+                                         (5_000_003, 30, 47)])
 def test_sort_pairs_c_abi(oracle, m, begin, end):
     """d3gs_sort_pairs against numpy's stable argsort on the masked key bits; many duplicate keys."""
     import torch
