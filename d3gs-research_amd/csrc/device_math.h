@@ -379,11 +379,12 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
     int count = 0;
     const bool big = area > kSmallWalk;
     if (!big) {
+        int lx = 0, ly = 0;
         for (int t = 0; t < area; ++t) {
-            const int ly = t / w.bw;
-            const bool k = tile_keep(filter_algo, w, t - ly * w.bw, ly);
+            const bool k = tile_keep(filter_algo, w, lx, ly);
             count += k ? 1 : 0;
             mask |= k ? (1ull << t) : 0ull;
+            if (++lx == w.bw) { lx = 0; ++ly; }
         }
     }
     const int lane = threadIdx.x & 63;
@@ -395,11 +396,12 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
         const int a = ws.bw * ws.bh;
         int c = 0;
         unsigned long long first = 0ull;
+        const float inv_bw = 1.0f / (float)ws.bw;   // row of candidate t: exact for the rect sizes a screen can hold
         for (int base = 0; base < a; base += 64) {
             const int t = base + lane;
             bool k = false;
             if (t < a) {
-                const int ly = t / ws.bw;
+                const int ly = (int)(((float)t + 0.5f) * inv_bw);
                 k = tile_keep(filter_algo, ws, t - ly * ws.bw, ly);
             }
             const unsigned long long b = __ballot(k);
@@ -441,8 +443,8 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
     const int area = active ? w.bw * w.bh : 0;
     const bool big = area > kSmallWalk;
     if (!big) {
-        for (int t = 0; t < area; ++t) {
-            const int ly = t / w.bw, lx = t - ly * w.bw;
+        int lx = 0, ly = 0;
+        for (int t = 0; t < area; ++t, lx = (lx + 1 == w.bw ? 0 : lx + 1), ly += (lx == 0)) {
             if (tile_keep(filter_algo, w, lx, ly)) {
                 if (off < end) {
                     const uint64_t tile = (uint64_t)(uint32_t)((ly + w.bminy) * tiles_x + lx + w.bminx);
@@ -465,12 +467,13 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
         long long o = ((long long)bcast_i((int)(off >> 32), src) << 32) | (uint32_t)bcast_i((int)off, src);
         const long long e = ((long long)bcast_i((int)(end >> 32), src) << 32) | (uint32_t)bcast_i((int)end, src);
         const int a = ws.bw * ws.bh;
+        const float inv_bw = 1.0f / (float)ws.bw;
         for (int base = 0; base < a; base += 64) {
             const int t = base + lane;
             bool k = false;
             int lx = 0, ly = 0;
             if (t < a) {
-                ly = t / ws.bw;
+                ly = (int)(((float)t + 0.5f) * inv_bw);
                 lx = t - ly * ws.bw;
                 k = tile_keep(filter_algo, ws, lx, ly);
             }
