@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -44,6 +44,7 @@ _SIGNATURES = {
     "d3gs_last_error_string": (C.c_char_p, []),
     "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
     "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
+    "d3gs_sh_colors": (C.c_int, [C.POINTER(Params)] + [_VP] * 6 + [_VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
     "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int64, _VP]),

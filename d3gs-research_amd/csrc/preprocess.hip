@@ -37,7 +37,8 @@ __device__ __forceinline__ float sh_channel(int degree, float x, float y, float 
     return r + 0.5f;
 }
 
-constexpr int kPrepBlock = 128;  // gaussians (= threads) per workgroup of the per-gaussian kernels
+constexpr int kPrepBlock = 128;   // gaussians (= threads) per workgroup of the per-gaussian kernels
+constexpr int kShColorBlocks = 512;   // two workgroups per CU for the SH colour kernel
 
 // Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
 // consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
@@ -90,6 +91,8 @@ __device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, cons
     }
 }
 
+// kWithSh = false leaves the SH colour to sh_colors_kernel: no LDS, twice the resident wavefronts.
+template <bool kWithSh>
 __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
@@ -100,11 +103,11 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
     extern __shared__ float s_rows[];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
-    {
+    if constexpr (kWithSh) {
         const int first = blockIdx.x * kPrepBlock;
         rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P.n - first), rowlen, stride);
+        __syncthreads();
     }
-    __syncthreads();
     // no early return: every lane of the wavefront takes part in the cooperative tile count
     const int i_raw = blockIdx.x * kPrepBlock + threadIdx.x;
     const bool in_range = i_raw < P.n;
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         count = wave_tile_count(P.filter_algo, valid, walk, kept_mask, has_mask);
         kept_meta = tile_mask_meta(walk, has_mask);
     }
-    if (valid) {
+    if (valid && kWithSh) {
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
         float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
         const float* shp = s_rows + threadIdx.x * stride;
@@ -205,9 +208,8 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         ne0 = ((rgb[0] < 0.0f) << 2) | ((rgb[1] < 0.0f) << 1) | (rgb[2] < 0.0f);
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch) rgb[ch] = fmaxf(rgb[ch], 0.0f);
-    } else {
-        z = u = v = con0 = con1 = con2 = op = a = b = c = radius = 0.0f;
     }
+    if (!valid) z = u = v = con0 = con1 = con2 = op = a = b = c = radius = 0.0f;
     if (!in_range) return;
 
     depths[i] = z;
@@ -219,15 +221,55 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         tile_masks[2 * (size_t)i] = kept_mask;
         tile_masks[2 * (size_t)i + 1] = kept_meta;
     }
-    rgb_out[3 * i + 0] = rgb[0];
-    rgb_out[3 * i + 1] = rgb[1];
-    rgb_out[3 * i + 2] = rgb[2];
     if (cov2d_out) {
         cov2d_out[3 * i + 0] = a;
         cov2d_out[3 * i + 1] = b;
         cov2d_out[3 * i + 2] = c;
     }
-    if (ne0_out) ne0_out[i] = (uint8_t)ne0;
+    if constexpr (kWithSh) {
+        rgb_out[3 * i + 0] = rgb[0];
+        rgb_out[3 * i + 1] = rgb[1];
+        rgb_out[3 * i + 2] = rgb[2];
+        if (ne0_out) ne0_out[i] = (uint8_t)ne0;
+    }
+}
+
+// SH colour of the gaussians the preprocess kernel accepted (radii > 0), the part of K1 that
+// streams the 192-byte SH rows: same operations as the fused kernel, zeros for rejected gaussians.
+__global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
+    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ sh,
+    const float* __restrict__ sh_base, const int32_t* __restrict__ radii, float* __restrict__ rgb_out,
+    uint8_t* __restrict__ ne0_out) {
+    extern __shared__ float s_rows[];
+    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    // grid-stride over 128-gaussian chunks: a small grid leaves most of every CU to the kernels this
+    // one runs beside
+    for (int first = blockIdx.x * kPrepBlock; first < P.n; first += gridDim.x * kPrepBlock) {
+        __syncthreads();   // the previous chunk's rows have been read
+        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P.n - first), rowlen, stride);
+        __syncthreads();
+        const int i = first + threadIdx.x;
+        if (i >= P.n) continue;
+        float rgb[3] = {0.0f, 0.0f, 0.0f};
+        uint32_t ne0 = 0;
+        if (radii[i] > 0) {
+            float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+            float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
+            float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
+            const float* shp = s_rows + threadIdx.x * stride;
+            const float* base = P.has_sh_base ? sh_base + 3 * i : shp;
+            const float* rest = P.has_sh_base ? shp : shp + 3;
+#pragma unroll
+            for (int ch = 0; ch < 3; ++ch) rgb[ch] = sh_channel(P.sh_degree, dx, dy, dz, base[ch], rest, ch);
+            ne0 = ((rgb[0] < 0.0f) << 2) | ((rgb[1] < 0.0f) << 1) | (rgb[2] < 0.0f);
+#pragma unroll
+            for (int ch = 0; ch < 3; ++ch) rgb[ch] = fmaxf(rgb[ch], 0.0f);
+        }
+        rgb_out[3 * i + 0] = rgb[0];
+        rgb_out[3 * i + 1] = rgb[1];
+        rgb_out[3 * i + 2] = rgb[2];
+        if (ne0_out) ne0_out[i] = (uint8_t)ne0;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -543,18 +585,45 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     int rc = check_params(p, "d3gs_preprocess_fwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
-    if (!xyz || !quaternion_xyzw || !scale || !opacity || !color_sh || !depths || !radii || !uvs || !conic_opacity ||
-        !tiles_touched || !rgb_gaussian || (p->has_sh_base && !color_sh_base)) {
+    const bool with_sh = rgb_gaussian != nullptr;
+    if (!xyz || !quaternion_xyzw || !scale || !opacity || !depths || !radii || !uvs || !conic_opacity ||
+        !tiles_touched || (with_sh && (!color_sh || (p->has_sh_base && !color_sh_base)))) {
         set_error("d3gs_preprocess_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
-    const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
-    hipLaunchKernelGGL(preprocess_fwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale,
-                       opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity, tiles_touched,
-                       rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks);
+    if (with_sh) {
+        const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+        hipLaunchKernelGGL(preprocess_fwd_kernel<true>, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz,
+                           quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs,
+                           conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,
+                           (unsigned long long*)tile_masks);
+    } else {
+        hipLaunchKernelGGL(preprocess_fwd_kernel<false>, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
+                           scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity,
+                           tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const float* color_sh, const float* color_sh_base,
+                              const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_sh_colors");
+    if (rc) return rc;
+    if (p->n == 0) return D3GS_OK;
+    if (!xyz || !color_sh || !radii || !rgb_gaussian || (p->has_sh_base && !color_sh_base)) {
+        set_error("d3gs_sh_colors: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const int chunks = (p->n + kPrepBlock - 1) / kPrepBlock;
+    dim3 grid(chunks < kShColorBlocks ? chunks : kShColorBlocks), block(kPrepBlock);
+    const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    hipLaunchKernelGGL(sh_colors_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, color_sh, color_sh_base,
+                       radii, rgb_gaussian, sh_to_rgb_ne_0);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_sh_colors: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 

@@ -125,6 +125,10 @@ class GaussianSplatOp:
         # optional per-stage timing: set to a dict to collect torch.cuda.Event pairs
         self.stage_events: dict[str, list] | None = None
         self.last_num_rendered = 0
+        # The SH colours are only read by the blend, so they are computed on a second stream beside the
+        # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
+        self.overlap_sh_colors = True
+        self._side_stream: torch.cuda.Stream | None = None
 
     # ------------------------------------------------------------------ utils
     def _check_supported(self):
@@ -267,13 +271,32 @@ class GaussianSplatOp:
             ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
             # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
             tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
+            overlap = bool(self.overlap_sh_colors)
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                _capi.ptr(tiles_touched), _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs), _capi.ptr(ne0),
-                _capi.ptr(tile_masks), s),
+                _capi.ptr(tiles_touched), None if overlap else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
+                None if overlap else _capi.ptr(ne0), _capi.ptr(tile_masks), s),
                 "d3gs_preprocess_fwd")
+        sh_done = None
+        if overlap:
+            if self._side_stream is None or self._side_stream.device != dev:
+                self._side_stream = torch.cuda.Stream(device=dev)   # default priority
+            main = torch.cuda.current_stream()
+            side = self._side_stream
+            side.wait_stream(main)          # radii (and the buffers' allocation) are ready
+            ta = torch.cuda.Event(enable_timing=True) if self.stage_events is not None else None
+            if ta is not None:
+                ta.record(side)
+            _capi.check(L.d3gs_sh_colors(
+                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
+                _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), C.c_void_p(side.cuda_stream)),
+                "d3gs_sh_colors")
+            sh_done = torch.cuda.Event(enable_timing=self.stage_events is not None)
+            sh_done.record(side)
+            if ta is not None:
+                self.stage_events.setdefault("sh_colors", []).append((ta, sh_done))
 
         def _sort(keys_a, vals_a, count, begin_bit, end_bit):
             keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
@@ -320,6 +343,8 @@ class GaussianSplatOp:
         out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=out_depth,
                                   n_contrib=n_contrib, radii=radii)
         if num_rendered == 0:
+            if sh_done is not None:
+                torch.cuda.current_stream().wait_event(sh_done)
             # the reference returns uninitialised buffers here (render.py:706-729); fill with the
             # values an empty scene renders to instead
             final_T.fill_(1.0)
@@ -359,6 +384,8 @@ class GaussianSplatOp:
             image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
             tile_order=tile_order)
         self._last_keys_sorted = keys_sorted  # kept for parity tests (sorted key order)
+        if sh_done is not None:
+            torch.cuda.current_stream().wait_event(sh_done)
         with self._stage("blend_fwd"):
             self.rasterize_forward_backward(model, ctx, out, training=training, render_depth=self._cfg.render_depth,
                                             _params=P)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 7
+#define D3GS_ABI_VERSION 8
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -97,12 +97,20 @@ int d3gs_higher_msb(uint32_t n);
  * invalid_mask (uint8[N], may be NULL): non-zero rejects the gaussian (render.py:306-308).
  * tile_masks (uint64[N][2], may be NULL; no counterpart in the reference): a record of the tiles the
  * early filter kept for each gaussian (word 0: bit mask over its candidate rect, word 1: the rect), which
- * d3gs_make_keys expands instead of repeating the per-tile tests. */
+ * d3gs_make_keys expands instead of repeating the per-tile tests.
+ * rgb_gaussian may be NULL: the SH colour (and sh_to_rgb_ne_0) is then left to d3gs_sh_colors, which a
+ * caller can run on a second stream beside the sort, the only consumer being the blend. */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const float* color_sh_base,
                         const uint8_t* invalid_mask, float* depths,
                         int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
                         float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, uint64_t* tile_masks, d3gs_stream_t stream);
+
+/* The SH-colour part of K1 on its own (render.py:569-613): rgb_gaussian [N,3] and, when not NULL, the
+ * clamp mask sh_to_rgb_ne_0 [N] of the gaussians with radii > 0, zeros for the rest.  Same values as the
+ * fused call. */
+int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const float* color_sh, const float* color_sh_base,
+                   const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
 
 /* K2 — replaces `tiles_touched.cumsum_(0)` + `.item()` at render.py:694-695.
  * In-place inclusive scan; the grand total is written to *total_dev (device
