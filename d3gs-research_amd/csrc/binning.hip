@@ -89,45 +89,76 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int32_t* __restrict_
 // Key expansion: one thread per gaussian, emits its (tile << 32 | depth bits)
 // keys at the offset the scan assigned (render.py:745-840).
 // ---------------------------------------------------------------------------
+constexpr int kKeyStage = 512;   // pairs a wavefront stages in LDS before writing them out coalesced
+
 __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, const int32_t* __restrict__ radii,
                                                             const float* __restrict__ uvs,
                                                             const float* __restrict__ conic_opacity,
                                                             const float* __restrict__ depths,
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ order,
+                                                            const uint64_t* __restrict__ ordered_depth_keys,
                                                             const unsigned long long* __restrict__ tile_masks,
                                                             uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
+    __shared__ uint64_t s_key[kBlock / 64][kKeyStage];
+    __shared__ int32_t s_val[kBlock / 64][kKeyStage];
     // no early return: every lane takes part in the cooperative emission of large gaussians
     const int j_raw = blockIdx.x * kBlock + threadIdx.x;
     const bool in_range = j_raw < P.n;
     const int j = in_range ? j_raw : P.n - 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // slot j of the emission order holds gaussian order[j] (identity without an order table);
     // `offsets` is the inclusive scan of the tile counts taken in that same order
     int i = order ? order[j] : j;
     const bool sane = (unsigned)i < (unsigned)P.n;
     i = sane ? i : 0;
-    const int r = radii[i];
-    long long off = j == 0 ? 0 : offsets[j - 1];
     const long long end = offsets[j];
-    // a caller that passed a smaller buffer than the scan total must never be written past
-    const bool active = in_range && sane && r > 0 && end <= m;
-    const uint32_t dbits = __float_as_uint(depths[i]);
+    long long off = !in_range ? end : (j == 0 ? 0 : offsets[j - 1]);   // lanes past the end: an empty range at the total
+    // a gaussian with no tiles has an empty slot range; a caller that passed a smaller buffer than
+    // the scan total must never be written past
+    const bool active = in_range && sane && end > off && end <= m;
+    const uint32_t dbits = ordered_depth_keys ? (uint32_t)ordered_depth_keys[j] : __float_as_uint(depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
-    bool walk_again = active;
+    unsigned long long kept = 0ull, meta = 0ull;
     if (tile_masks && active) {
-        const unsigned long long meta = tile_masks[2 * (size_t)i + 1];
-        if (meta & kTileMaskHas) {
-            mask_tile_emit(tile_masks[2 * (size_t)i], meta, P.tiles_x, dbits, i, off, end, keys, vals);
-            walk_again = false;
-        }
+        meta = tile_masks[2 * (size_t)i + 1];
+        if (meta & kTileMaskHas) kept = tile_masks[2 * (size_t)i];
     }
+    const bool has_mask = (meta & kTileMaskHas) != 0;
+    const bool walk_again = active && !has_mask;
+    // The slots of a wavefront's gaussians are consecutive.  When they all come from masks and fit the
+    // staging buffer they are assembled in LDS and leave as whole coalesced segments; otherwise each
+    // lane writes its own run.
+    const long long wave_base = __shfl(off, 0, 64);
+    const long long wave_end = __shfl(end, 63, 64);
+    const bool staged = !__any(walk_again) && !__any(in_range && !sane) && wave_end - wave_base <= kKeyStage &&
+                        wave_end <= m && wave_end >= wave_base;
+    if (staged) {
+        if (has_mask)
+            mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
+                s_key[wave][slot - wave_base] = key;
+                s_val[wave][slot - wave_base] = i;
+            });
+        __builtin_amdgcn_wave_barrier();
+        const int total = (int)(wave_end - wave_base);
+        for (int sidx = lane; sidx < total; sidx += 64) {
+            keys[wave_base + sidx] = s_key[wave][sidx];
+            vals[wave_base + sidx] = s_val[wave][sidx];
+        }
+        return;   // wave-uniform
+    }
+    if (has_mask)
+        mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
+            keys[slot] = key;
+            vals[slot] = i;
+        });
     if (!__any(walk_again)) return;   // wave-uniform
     TileWalk walk = {};
     if (walk_again) {
         const float2 uv = *reinterpret_cast<const float2*>(uvs + 2 * i);
         const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
-        TileWalkIn g{uv.x, uv.y, (float)r, co.x, co.y, co.z, co.w};
+        TileWalkIn g{uv.x, uv.y, (float)radii[i], co.x, co.y, co.z, co.w};
         walk = tile_walk_setup(P, g);
     }
     wave_tile_emit(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
@@ -253,8 +284,8 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
 
 extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                               const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                              const uint64_t* tile_masks, uint64_t* keys, int32_t* gaussian_idx, int64_t m,
-                              d3gs_stream_t stream) {
+                              const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                              int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
@@ -264,7 +295,8 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     hipLaunchKernelGGL(make_keys_kernel, dim3((p->n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, (const unsigned long long*)tile_masks, keys,
+                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, ordered_depth_keys,
+                       (const unsigned long long*)tile_masks, keys,
                        gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

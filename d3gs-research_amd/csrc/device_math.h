@@ -416,10 +416,10 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
     return count;
 }
 
-// Emits the tiles named by a kept-tile mask.  Per lane; consecutive lanes write consecutive runs.
+// Emits the tiles named by a kept-tile mask through `put(slot, key)`, slot counting from `off`.
+template <class Put>
 __device__ __forceinline__ void mask_tile_emit(unsigned long long mask, unsigned long long meta, int tiles_x,
-                                               uint32_t depth_bits, int value, long long off, long long end,
-                                               uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+                                               uint32_t depth_bits, long long off, long long end, Put&& put) {
     const int bminx = (int)(meta & 0xFFFFu), bminy = (int)((meta >> 16) & 0xFFFFu), bw = (int)((meta >> 32) & 0xFFu);
     const uint32_t recip = bw > 0 ? (65536u + (uint32_t)bw - 1u) / (uint32_t)bw : 0u;  // exact t / bw for t < 64
     while (mask) {
@@ -428,8 +428,7 @@ __device__ __forceinline__ void mask_tile_emit(unsigned long long mask, unsigned
         const int ly = (int)(((uint32_t)t * recip) >> 16), lx = t - ly * bw;
         if (off < end) {
             const uint64_t tile = (uint64_t)(uint32_t)((ly + bminy) * tiles_x + lx + bminx);
-            keys[off] = (tile << 32) | depth_bits;
-            vals[off] = value;
+            put(off, (tile << 32) | depth_bits);
         }
         ++off;
     }

@@ -319,7 +319,7 @@ class GaussianSplatOp:
             iota = torch.empty(n, dtype=i32, device=dev)
             _capi.check(L.d3gs_depth_keys(_capi.ptr(depths), n, _capi.ptr(depth_keys), _capi.ptr(iota), s),
                         "d3gs_depth_keys")
-            _, gaussian_order = _sort(depth_keys, iota, n, 0, 32)
+            depth_keys_sorted, gaussian_order = _sort(depth_keys, iota, n, 0, 32)
 
         with self._stage("scan"):
             counts_ordered = torch.empty(n, dtype=i32, device=dev)
@@ -365,7 +365,8 @@ class GaussianSplatOp:
             gaussian_idx = torch.empty(num_rendered, dtype=i32, device=dev)
             _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                                          _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                         _capi.ptr(tile_masks), _capi.ptr(keys), _capi.ptr(gaussian_idx),
+                                         _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), _capi.ptr(keys),
+                                         _capi.ptr(gaussian_idx),
                                          num_rendered, s), "d3gs_make_keys")
 
         with self._stage("sort"):

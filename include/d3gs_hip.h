@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 8
+#define D3GS_ABI_VERSION 9
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -124,11 +124,14 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
  * scan of tiles_touched from d3gs_scan_tiles, m = its total, pairs are emitted in
  * gaussian-index order.  With gaussian_order (a permutation of 0..n-1), slot j emits
  * gaussian gaussian_order[j] and offsets must be the inclusive scan of the tile counts
- * taken in that order (see d3gs_depth_keys).  tile_masks (may be NULL) is the record
- * d3gs_preprocess_fwd wrote with the same params; the pairs emitted are the same either way. */
+ * taken in that order (see d3gs_depth_keys).  Two optional inputs (may be NULL) save gathers
+ * without changing the pairs emitted: ordered_depth_keys[j], the sorted keys of the depth sort
+ * (low 32 bits = depth bits of gaussian gaussian_order[j]), read instead of depths[gaussian_order[j]];
+ * tile_masks, the record d3gs_preprocess_fwd wrote with the same params. */
 int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                    const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                   const uint64_t* tile_masks, uint64_t* keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
+                   const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                   int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
 
 /* Depth-first factorisation of the pair sort (no counterpart in the reference, which
  * radix-sorts all M pairs on the full (tile, depth) key; the result is bit-identical).
