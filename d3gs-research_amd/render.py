@@ -50,6 +50,15 @@ class GaussianSplatOpContext:
 
 
 @dataclasses.dataclass
+class GaussianSplatOpBatchContext:
+    """Context of a camera bundle with more than one camera: the cameras are rendered one after the
+    other, each keeping its own single-camera context (None where nothing was rendered)."""
+    per_camera: list
+    cameras: list
+    image_shape_wh: tuple[int, int]
+
+
+@dataclasses.dataclass
 class GaussianSplatOutput:
     """render.py:74-100"""
     custom_features: torch.Tensor | None
@@ -104,8 +113,15 @@ class CameraParamBundle:
 
 @dataclasses.dataclass
 class CameraBundle(CameraParamBundle):
-    """render.py:129-150; only bundles holding one camera are accepted here."""
+    """render.py:129-150."""
     cam2world_T: torch.Tensor = None
+
+    def __len__(self):
+        return int(self.cam2world_T.shape[0])
+
+    def select(self, b: int) -> "CameraBundle":
+        return CameraBundle(self.focal_xy_ppoint[b:b + 1], self.image_shape_wh,
+                            None if self.frame_ids is None else self.frame_ids[b:b + 1], self.cam2world_T[b:b + 1])
 
     @classmethod
     def from_pinhole_cams(cls, cams: list[BasicPinholeCamera], device="cuda"):
@@ -180,8 +196,7 @@ class GaussianSplatOp:
             pp = np.array([intrinsic[0, 2], intrinsic[1, 2]], np.float32)
             c2w_T = np.ascontiguousarray(np.asarray(cameras.pose.to_world)[:3].T).astype(np.float32)
         elif isinstance(cameras, CameraBundle):
-            if cameras.cam2world_T.shape[0] != 1:
-                raise NotImplementedError("camera bundles with more than one camera are not supported")
+            assert cameras.cam2world_T.shape[0] == 1, "one camera per kernel pass"
             fpp = cameras.focal_xy_ppoint[0].detach().cpu().numpy().astype(np.float32)
             focal, pp = fpp[:2], fpp[2:]
             c2w_T = cameras.cam2world_T[0].detach().cpu().numpy().astype(np.float32).reshape(4, 3)
@@ -243,6 +258,9 @@ class GaussianSplatOp:
                 custom_features=None, mask=None, prep_user_inputs=None):
         """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
         assert model.act_applied, "model must be activated before render"
+        if isinstance(cameras, CameraBundle) and len(cameras) != 1:
+            return self._forward_bundle(model, cameras, training, instance2world_T, custom_features, mask,
+                                        prep_user_inputs)
         if instance2world_T is not None or custom_features is not None or prep_user_inputs:
             raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
         self._check_model(model)
@@ -394,6 +412,37 @@ class GaussianSplatOp:
             ctx = None
         return out, ctx
 
+    def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
+                        prep_user_inputs):
+        """A bundle of B cameras (render.py:314-326, 787, 1515-1522 index one launch by batch): rendered
+        here as B single-camera passes over the shared model.  Outputs are stacked along the batch
+        axis; radii and the mask are flat [B * N] as in the reference."""
+        B, n = len(cameras), len(model)
+        assert B > 0, "empty camera bundle"
+        if mask is not None:
+            assert mask.numel() == B * n, "mask must have one entry per (camera, gaussian)"
+            mask = mask.reshape(B, n)
+        outs, ctxs, cams, rendered = [], [], [], 0
+        for b in range(B):
+            cam_b = cameras.select(b)
+            out_b, ctx_b = self.forward(model, cam_b, training, instance2world_T, custom_features,
+                                        None if mask is None else mask[b].contiguous(), prep_user_inputs)
+            outs.append(out_b)
+            ctxs.append(ctx_b)
+            cams.append(cam_b)
+            rendered += self.last_num_rendered
+        self.last_num_rendered = rendered
+        cat = lambda name: torch.cat([getattr(o, name) for o in outs], 0)
+        out = GaussianSplatOutput(custom_features=None, T=cat("T"), color=cat("color"),
+                                  depth=cat("depth") if outs[0].depth is not None else None,
+                                  n_contrib=cat("n_contrib"), radii=cat("radii"))
+        if not training:
+            return out, None
+        return out, GaussianSplatOpBatchContext(per_camera=ctxs, cameras=cams, image_shape_wh=cameras.image_shape_wh)
+
+    def _backward_bundle(self, model, ctx, out, grad, return_uv_grad):
+        return _backward_bundle_impl(self, model, ctx, out, grad, return_uv_grad)
+
     # ------------------------------------------------------- blend fwd / bwd
     def rasterize_forward_backward(self, model, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
                                    grad: GaussianSplatGradients | None = None, training: bool = False,
@@ -447,6 +496,8 @@ class GaussianSplatOp:
             raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
         if grad.dcustom_features is not None:
             raise NotImplementedError("custom feature gradients are not supported")
+        if isinstance(ctx, GaussianSplatOpBatchContext):
+            return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
         L = self._lib
         P = self.make_params(model, cameras, True)
         s = self._stream()
@@ -474,6 +525,31 @@ class GaussianSplatOp:
         if return_uv_grad:
             return grad_model, g.duv.unsqueeze(0), None
         return grad_model, None, None
+
+
+def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
+    """Per-camera backward passes; the model gradients add up over the cameras, duv stays per camera."""
+    total, duvs = None, []
+    n = len(model)
+    for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
+        if ctx_b is None:       # nothing was rendered for this camera: zero gradient
+            duvs.append(torch.zeros((1, n, 2), dtype=torch.float32, device=model.xyz.device))
+            continue
+        g_b = GaussianSplatGradients(drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
+                                     ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous())
+        gm, duv, _ = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True)
+        duvs.append(duv)
+        if total is None:
+            total = gm
+        else:
+            for name in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh", "color_sh_base"):
+                t = getattr(total, name)
+                if t is not None:
+                    t.add_(getattr(gm, name))
+    if total is None:
+        zeros = {k: torch.zeros_like(v) for k, v in model.get_proxy_field_dict().items()}
+        total = dataclasses.replace(model, **zeros)
+    return total, (torch.cat(duvs, 0) if return_uv_grad else None), None
 
 
 class _RasterizeGaussians(torch.autograd.Function):

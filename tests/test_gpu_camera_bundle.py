@@ -1,0 +1,114 @@
+"""Camera bundles (render.py:129-150, 314-326): B cameras over one model.  Each camera of the
+bundle must give exactly the single-camera result (itself checked against the oracle elsewhere),
+outputs stacked on the batch axis, radii / mask flat [B * N], model gradients summed over cameras."""
+import numpy as np
+import pytest
+from scipy.spatial.transform import Rotation
+
+from helpers import gen_scene, op_config, oracle_params, torch_model
+
+pytestmark = pytest.mark.gpu
+
+
+def _cameras(scene):
+    from d3gs_research_amd.camera import BasicPinholeCamera
+    cams = []
+    for k, (euler, shift) in enumerate([((0, 0, 0), (0, 0, 0)), ((0.1, -0.2, 0.3), (0.3, -0.1, -0.4)),
+                                        ((-0.15, 0.25, -0.1), (-0.2, 0.2, 0.3))]):
+        tw = np.array(scene.to_world, np.float64)
+        tw[:3, :3] = tw[:3, :3] @ Rotation.from_euler("xyz", euler).as_matrix()
+        tw[:3, 3] += shift
+        cams.append(BasicPinholeCamera.from_params(scene.fx * (1 + 0.1 * k), scene.fy * (1 + 0.1 * k), scene.cx + k,
+                                                   scene.cy - k, scene.width, scene.height, tw))
+    return cams
+
+
+@pytest.mark.parametrize("depth", [False, True])
+def test_bundle_equals_single_cameras(oracle, depth):
+    import torch
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    cams = _cameras(scene)
+    B, n = len(cams), scene.n
+    op = GaussianSplatOp(op_config(scene, 4, render_depth=depth))
+    model = torch_model(scene)
+    bundle = CameraBundle.from_pinhole_cams(cams)
+    assert len(bundle) == B
+    mask = torch.from_numpy(np.random.default_rng(8).random(B * n) < 0.2).cuda()
+
+    out, ctx = op.forward(model, bundle, training=True, mask=mask)
+    assert tuple(out.color.shape) == (B, scene.height, scene.width, 3) and tuple(out.T.shape) == (B, scene.height, scene.width)
+    assert tuple(out.radii.shape) == (B * n,) and (out.depth is not None) == depth
+    rng = np.random.default_rng(9)
+    drgb = torch.from_numpy(rng.standard_normal(out.color.shape).astype(np.float32)).cuda()
+    dT = torch.from_numpy(rng.standard_normal(out.T.shape).astype(np.float32)).cuda()
+    dd = torch.from_numpy(rng.standard_normal(out.T.shape).astype(np.float32)).cuda() if depth else None
+    gm, duv, _ = op.backward(model, bundle, ctx, out, GaussianSplatGradients(drgb=drgb, dT=dT, ddepth=dd), return_uv_grad=True)
+    assert tuple(duv.shape) == (B, n, 2)
+
+    want = {k: torch.zeros_like(v, dtype=torch.float64) for k, v in model.get_proxy_field_dict().items()}
+    for b, cam in enumerate(cams):
+        o1, c1 = op.forward(model, cam, training=True, mask=mask[b * n:(b + 1) * n].contiguous())
+        assert torch.equal(o1.color[0], out.color[b]) and torch.equal(o1.T[0], out.T[b])
+        assert torch.equal(o1.n_contrib[0], out.n_contrib[b]) and torch.equal(o1.radii, out.radii[b * n:(b + 1) * n])
+        assert not bool(o1.radii[mask[b * n:(b + 1) * n]].any())
+        if depth:
+            assert torch.equal(o1.depth[0], out.depth[b])
+        g1 = GaussianSplatGradients(drgb=drgb[b:b + 1].contiguous(), dT=dT[b:b + 1].contiguous(),
+                                    ddepth=None if dd is None else dd[b:b + 1].contiguous())
+        gm1, duv1, _ = op.backward(model, cam, c1, o1, g1, return_uv_grad=True)
+        # atomics order differs between two runs of the same backward: compare with a tolerance
+        scale_uv = float(duv1.abs().max())
+        assert float((duv1[0] - duv[b]).abs().max()) <= 1e-4 * scale_uv
+        for k in want:
+            want[k] += getattr(gm1, k).double()
+    for k, w in want.items():
+        got = getattr(gm, k).double()
+        assert float((got - w).abs().max()) <= 1e-4 * float(w.abs().max()), k
+
+    # one oracle check of the second camera, so that the per-camera parameters are known to be that camera's
+    cam = cams[1]
+    P = oracle_params(oracle, scene, 4)
+    P.fx, P.fy, P.cx, P.cy = [float(v) for v in (*cam.focal_length, *cam.principal_point)]
+    P.tan_fovx = float(np.float32(0.5) * np.float32(scene.width) / np.float32(P.fx))
+    P.tan_fovy = float(np.float32(0.5) * np.float32(scene.height) / np.float32(P.fy))
+    c2w_T = np.ascontiguousarray(np.asarray(cam.pose.to_world)[:3].T).astype(np.float32)
+    P.w2c[:] = [float(v) for v in c2w_T[:3].reshape(-1)]
+    P.cam_center[:] = [float(v) for v in c2w_T[3]]
+    P.render_depth = int(depth)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                         invalid_mask=mask[n:2 * n].cpu().numpy())
+    assert np.array_equal(out.color[1].cpu().numpy().view(np.uint32), ref["color"].view(np.uint32))
+    assert np.array_equal(out.n_contrib[1].cpu().numpy(), ref["n_contrib"])
+
+
+def test_bundle_through_autograd_entry_point():
+    import torch
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatOp, rasterize_gaussians
+    scene = gen_scene(0)
+    cams = _cameras(scene)
+    op = GaussianSplatOp(op_config(scene, 1))
+    bundle = CameraBundle.from_pinhole_cams(cams)
+
+    def grads(cameras):
+        model = torch_model(scene)
+        model.act_applied = False
+        model.set_requires_grad(True)
+        holder = torch.zeros((len(cams), scene.n, 2), device="cuda", requires_grad=True)
+        loss = 0.0
+        if isinstance(cameras, list):
+            for b, cam in enumerate(cameras):
+                h = torch.zeros((1, scene.n, 2), device="cuda", requires_grad=True)
+                o = rasterize_gaussians(model, cam, op, training=True, uv_grad_holder=h)
+                loss = loss + (o.color ** 2).sum() + o.T.sum()
+        else:
+            o = rasterize_gaussians(model, cameras, op, training=True, uv_grad_holder=holder)
+            loss = (o.color ** 2).sum() + o.T.sum()
+        loss.backward()
+        return {k: v.grad.double() for k, v in model.get_proxy_field_dict().items()}, holder.grad
+
+    g_bundle, duv = grads(bundle)
+    g_single, _ = grads(cams)
+    assert duv is not None and tuple(duv.shape) == (len(cams), scene.n, 2) and float(duv.abs().max()) > 0
+    for k in g_single:
+        assert float((g_bundle[k] - g_single[k]).abs().max()) <= 1e-4 * float(g_single[k].abs().max()), k
