@@ -1,0 +1,87 @@
+"""The Inria point-cloud file (d3sim/algos/d3gs/tools.py:20-62 reads what
+origin/data/scene/gaussian_model.py:177-208 writes): the test writes the file itself, property by
+property in the Inria order, so the loader's channel / quaternion reordering is checked against the
+layout and not against the package's own writer."""
+import numpy as np
+import pytest
+import torch
+
+from d3gs_research_amd import tools
+from d3gs_research_amd.model import GaussianModelOrigin, GaussianModelOriginFused
+
+NAMES = ["x", "y", "z", "nx", "ny", "nz"] + [f"f_dc_{i}" for i in range(3)] + [f"f_rest_{i}" for i in range(45)] + \
+        ["opacity"] + [f"scale_{i}" for i in range(3)] + [f"rot_{i}" for i in range(4)]
+
+
+def _write(path, table, fmt):
+    n = table.shape[0]
+    header = f"ply\nformat {fmt} 1.0\ncomment made by a test\nelement vertex {n}\n" + \
+             "".join(f"property float {name}\n" for name in NAMES) + "end_header\n"
+    with open(path, "wb") as f:
+        f.write(header.encode())
+        if fmt == "ascii":
+            for row in table:
+                f.write((" ".join(repr(float(v)) for v in row) + "\n").encode())
+        else:
+            f.write(table.astype("<f4" if fmt == "binary_little_endian" else ">f4").tobytes())
+
+
+@pytest.mark.parametrize("fmt", ["binary_little_endian", "binary_big_endian", "ascii"])
+@pytest.mark.parametrize("split,fused", [(True, True), (False, False)])
+def test_loader_follows_the_inria_layout(tmp_path, fmt, split, fused):
+    n = 37
+    table = np.random.default_rng(0).standard_normal((n, len(NAMES))).astype(np.float32)
+    col = {name: table[:, k] for k, name in enumerate(NAMES)}
+    path = str(tmp_path / "pc.ply")
+    _write(path, table, fmt)
+    m = tools.load_3dgs_origin_model(path, fused=fused, split=split, device="cpu")
+    assert isinstance(m, GaussianModelOriginFused if fused else GaussianModelOrigin)
+    assert m.cur_sh_degree == 3 and len(m) == n and not m.act_applied
+    assert np.array_equal(m.xyz.numpy(), np.stack([col["x"], col["y"], col["z"]], 1))
+    # rotation is stored w, x, y, z; the model keeps x, y, z, w
+    assert np.array_equal(m.quaternion_xyzw.numpy(), np.stack([col["rot_1"], col["rot_2"], col["rot_3"], col["rot_0"]], 1))
+    assert np.array_equal(m.scale.numpy(), np.stack([col[f"scale_{i}"] for i in range(3)], 1))   # raw log-scale
+    assert np.array_equal(m.opacity.numpy(), col["opacity"])                                      # raw logit
+    sh = m.color_sh.numpy()
+    base = m.color_sh_base.numpy() if split else sh[:, 0]
+    rest = sh if split else sh[:, 1:]
+    assert rest.shape == (n, 15, 3) and (m.color_sh_base is not None) == split
+    for c in range(3):
+        assert np.array_equal(base[:, c], col[f"f_dc_{c}"])
+        for k in range(15):          # f_rest is channel-major: index c * 15 + k holds coefficient k + 1 of channel c
+            assert np.array_equal(rest[:, k, c], col[f"f_rest_{c * 15 + k}"])
+
+
+def test_writer_round_trip_and_errors(tmp_path):
+    n = 11
+    g = torch.Generator().manual_seed(1)
+    m = GaussianModelOriginFused(xyz=torch.randn(n, 3, generator=g), quaternion_xyzw=torch.randn(n, 4, generator=g),
+                                 scale=torch.randn(n, 3, generator=g), opacity=torch.randn(n, generator=g),
+                                 color_sh=torch.randn(n, 15, 3, generator=g), color_sh_base=torch.randn(n, 3, generator=g),
+                                 cur_sh_degree=3)
+    path = str(tmp_path / "rt.ply")
+    tools.save_3dgs_origin_model(m, path)
+    back = tools.load_3dgs_origin_model(path, device="cpu")
+    for k, v in m.get_proxy_field_dict().items():
+        assert torch.equal(getattr(back, k), v), k
+    v = tools.read_ply_vertices(path)
+    assert list(v) == NAMES and not v["nx"].any()
+    bad = tmp_path / "bad.ply"
+    bad.write_bytes(b"plx\n")
+    with pytest.raises(ValueError):
+        tools.read_ply_vertices(str(bad))
+    trunc = tmp_path / "trunc.ply"
+    trunc.write_bytes(open(path, "rb").read()[:-8])
+    with pytest.raises(ValueError):
+        tools.read_ply_vertices(str(trunc))
+
+
+def test_learning_rate_schedule_closed_form():
+    """tools.py:92-126: log-linear between the end points, sine warm-up multiplier."""
+    f = tools.get_expon_lr_func(1.6e-4, 1.6e-6, lr_delay_mult=0.01, max_steps=30000)
+    assert f(0) == pytest.approx(1.6e-4) and f(30000) == pytest.approx(1.6e-6) and f(60000) == pytest.approx(1.6e-6)
+    assert f(15000) == pytest.approx(1.6e-5)                      # geometric mean at the half point
+    g = tools.get_expon_lr_func(1e-2, 1e-4, lr_delay_steps=100, lr_delay_mult=0.1, max_steps=1000)
+    assert g(0) == pytest.approx(1e-3) and g(-1) == 0.0
+    assert g(50) == pytest.approx((0.1 + 0.9 * np.sin(0.25 * np.pi)) * 10 ** (-2 - 0.1))
+    assert tools.get_expon_lr_func(0.0, 0.0)(5) == 0.0
