@@ -91,6 +91,9 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int32_t* __restrict_
 // ---------------------------------------------------------------------------
 constexpr int kKeyStage = 512;   // pairs a wavefront stages in LDS before writing them out coalesced
 
+// Key = uint64_t: the reference's (tile << 32) | depth bits.  Key = uint32_t: the tile id alone, all the
+// pair sort needs once the pairs are emitted in depth order.
+template <typename Key>
 __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, const int32_t* __restrict__ radii,
                                                             const float* __restrict__ uvs,
                                                             const float* __restrict__ conic_opacity,
@@ -99,9 +102,9 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             const int32_t* __restrict__ order,
                                                             const uint64_t* __restrict__ ordered_depth_keys,
                                                             const unsigned long long* __restrict__ tile_masks,
-                                                            uint64_t* __restrict__ keys, int32_t* __restrict__ vals,
+                                                            Key* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
-    __shared__ uint64_t s_key[kBlock / 64][kKeyStage];
+    __shared__ Key s_key[kBlock / 64][kKeyStage];
     __shared__ int32_t s_val[kBlock / 64][kKeyStage];
     // no early return: every lane takes part in the cooperative emission of large gaussians
     const int j_raw = blockIdx.x * kBlock + threadIdx.x;
@@ -137,7 +140,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     if (staged) {
         if (has_mask)
             mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
-                s_key[wave][slot - wave_base] = key;
+                s_key[wave][slot - wave_base] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
                 s_val[wave][slot - wave_base] = i;
             });
         __builtin_amdgcn_wave_barrier();
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     }
     if (has_mask)
         mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
-            keys[slot] = key;
+            keys[slot] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
             vals[slot] = i;
         });
     if (!__any(walk_again)) return;   // wave-uniform
@@ -161,7 +164,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
         TileWalkIn g{uv.x, uv.y, (float)radii[i], co.x, co.y, co.z, co.w};
         walk = tile_walk_setup(P, g);
     }
-    wave_tile_emit(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
+    wave_tile_emit<Key>(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
 }
 
 // Sort keys of the gaussians themselves: the float bits of the depth (positive floats order like
@@ -186,16 +189,23 @@ __global__ __launch_bounds__(kBlock) void gather_i32_kernel(const int32_t* __res
 // ---------------------------------------------------------------------------
 // Tile ranges (render.py:897-939)
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const uint64_t* __restrict__ keys, long long m,
+template <typename Key>
+__device__ __forceinline__ uint32_t key_tile(Key k) {
+    if constexpr (sizeof(Key) == 8) return (uint32_t)(k >> 32);
+    else return (uint32_t)k;
+}
+
+template <typename Key>
+__global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restrict__ keys, long long m,
                                                               int32_t* __restrict__ ranges, int num_tiles) {
     const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
     if (i >= m) return;
-    const uint32_t t = (uint32_t)(keys[i] >> 32);
+    const uint32_t t = key_tile<Key>(keys[i]);
     if (t >= (uint32_t)num_tiles) return;  // corrupt key: never write outside the table
     if (i == 0) {
         ranges[2 * t] = 0;
     } else {
-        const uint32_t tp = (uint32_t)(keys[i - 1] >> 32);
+        const uint32_t tp = key_tile<Key>(keys[i - 1]);
         if (t != tp) {
             if (tp < (uint32_t)num_tiles) ranges[2 * tp + 1] = (int32_t)i;
             ranges[2 * t] = (int32_t)i;
@@ -285,19 +295,25 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
 extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                               const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
                               const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
-                              int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
+                              uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
     if (p->n == 0 || m == 0) return D3GS_OK;
-    if (!radii || !uvs || !conic_opacity || !depths || !offsets || !keys || !gaussian_idx) {
-        set_error("d3gs_make_keys: NULL buffer");
+    if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
+        !gaussian_idx) {
+        set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    hipLaunchKernelGGL(make_keys_kernel, dim3((p->n + kBlock - 1) / kBlock), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                       radii, uvs, conic_opacity, depths, offsets, gaussian_order, ordered_depth_keys,
-                       (const unsigned long long*)tile_masks, keys,
-                       gaussian_idx, (long long)m);
+    const dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
+    if (keys)
+        hipLaunchKernelGGL(make_keys_kernel<uint64_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
+                           depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,
+                           keys, gaussian_idx, (long long)m);
+    else
+        hipLaunchKernelGGL(make_keys_kernel<uint32_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
+                           depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,
+                           tile_keys, gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
@@ -327,20 +343,32 @@ extern "C" int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t*
     return D3GS_OK;
 }
 
-extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
-                                int32_t* tile_order, d3gs_stream_t stream) {
-    if (m < 0 || num_tiles < 0) { set_error("d3gs_tile_ranges: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+template <typename Key>
+static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, int32_t* workload_ranges,
+                            int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
+    if (m < 0 || num_tiles < 0) { set_error("%s: bad argument", who); return D3GS_ERR_INVALID_ARGUMENT; }
     if ((m > 0 && !keys_sorted) || (num_tiles > 0 && !workload_ranges)) {
-        set_error("d3gs_tile_ranges: NULL buffer");
+        set_error("%s: NULL buffer", who);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     if (m > 0)
-        hipLaunchKernelGGL(tile_ranges_kernel, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+        hipLaunchKernelGGL(tile_ranges_kernel<Key>, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                            (hipStream_t)stream, keys_sorted, (long long)m, workload_ranges, (int)num_tiles);
     if (tile_order && num_tiles > 0)
         hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, workload_ranges,
                            (int)num_tiles, tile_order);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("d3gs_tile_ranges: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
+}
+
+extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
+                                int32_t* tile_order, d3gs_stream_t stream) {
+    return tile_ranges_impl<uint64_t>("d3gs_tile_ranges", keys_sorted, m, workload_ranges, num_tiles, tile_order, stream);
+}
+
+extern "C" int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, int32_t* workload_ranges,
+                                    int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
+    return tile_ranges_impl<uint32_t>("d3gs_tile_ranges_u32", tile_keys_sorted, m, workload_ranges, num_tiles, tile_order,
+                                      stream);
 }

@@ -436,9 +436,17 @@ __device__ __forceinline__ void mask_tile_emit(unsigned long long mask, unsigned
 
 // Emits (key, value) of every kept tile of this lane's gaussian at [off, end) in row-major tile
 // order.  Must be called by all 64 lanes of a wavefront.
+template <typename Key>
+__device__ __forceinline__ Key make_pair_key(uint64_t tile, uint32_t depth_bits) {
+    if constexpr (sizeof(Key) == 8) return (Key)((tile << 32) | depth_bits);
+    else return (Key)tile;
+}
+
+// Key: uint64_t for (tile << 32) | depth bits, uint32_t for the tile id alone.
+template <typename Key>
 __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool active, const TileWalk& w, int tiles_x,
                                                uint32_t depth_bits, int value, long long off, long long end,
-                                               uint64_t* __restrict__ keys, int32_t* __restrict__ vals) {
+                                               Key* __restrict__ keys, int32_t* __restrict__ vals) {
     const int area = active ? w.bw * w.bh : 0;
     const bool big = area > kSmallWalk;
     if (!big) {
@@ -447,7 +455,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
             if (tile_keep(filter_algo, w, lx, ly)) {
                 if (off < end) {
                     const uint64_t tile = (uint64_t)(uint32_t)((ly + w.bminy) * tiles_x + lx + w.bminx);
-                    keys[off] = (tile << 32) | depth_bits;
+                    keys[off] = make_pair_key<Key>(tile, depth_bits);
                     vals[off] = value;
                 }
                 ++off;
@@ -481,7 +489,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
                 const long long pos = o + __popcll(b & lt_mask);
                 if (pos < e) {
                     const uint64_t tile = (uint64_t)(uint32_t)((ly + ws.bminy) * tiles_x + lx + ws.bminx);
-                    keys[pos] = (tile << 32) | dbits;
+                    keys[pos] = make_pair_key<Key>(tile, dbits);
                     vals[pos] = val;
                 }
             }

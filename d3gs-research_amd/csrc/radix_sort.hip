@@ -80,7 +80,8 @@ __global__ __launch_bounds__(kBlock) void os_clear_kernel(uint32_t* __restrict__
 // same-address conflicts of skewed digits (the exponent byte of a depth takes a handful of values).
 constexpr int kHistThreads = 1024;
 constexpr int kHistCopies = 8;
-__global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const uint64_t* __restrict__ keys, long long m,
+template <typename Key>
+__global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __restrict__ keys, long long m,
                                                                 int begin_bit, int end_bit, int passes,
                                                                 uint32_t* __restrict__ hist) {
     extern __shared__ uint32_t h[];  // [kHistCopies][passes][256]
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const uint64_t* _
     uint32_t* mine = h + (threadIdx.x & (kHistCopies - 1)) * table;
     const long long stride = (long long)gridDim.x * kHistThreads;
     for (long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x; i < m; i += stride) {
-        const uint64_t key = keys[i];
+        const Key key = keys[i];
         for (int p = 0; p < passes; ++p) {
             const int bit = begin_bit + 8 * p;
             const int nb = min(8, end_bit - bit);
@@ -106,9 +107,10 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const uint64_t* _
     }
 }
 
-__global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const uint64_t* __restrict__ keys_in,
+template <typename Key>
+__global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restrict__ keys_in,
                                                               const int32_t* __restrict__ vals_in,
-                                                              uint64_t* __restrict__ keys_out,
+                                                              Key* __restrict__ keys_out,
                                                               int32_t* __restrict__ vals_out, long long m, int shift,
                                                               uint32_t mask, int ntiles,
                                                               const uint32_t* __restrict__ hist /* this pass, [256] */,
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const uint64_t* __r
                                                               uint32_t* __restrict__ error) {
     __shared__ int wave_cnt[kOsWaves][kOsRadix];  // running, then exclusive-over-waves, per-wave digit counts
     __shared__ int digit_out[kOsRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
-    __shared__ uint64_t s_keys[kOsTile];
+    __shared__ Key s_keys[kOsTile];
     __shared__ uint16_t s_src[kOsTile];  // tile-local input index of the pair at each sorted position
     __shared__ int s_scan[kOsWaves];
 
@@ -132,14 +134,14 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const uint64_t* __r
 
     const long long tile_begin = (long long)tile * kOsTile;
     const int wave_begin = wave * (kOsTile / kOsWaves);
-    uint64_t key[kOsItems];
+    Key key[kOsItems];
     int rank[kOsItems];
     const uint64_t lt_mask = (1ull << lane) - 1ull;
 #pragma unroll
     for (int k = 0; k < kOsItems; ++k) {
         const long long idx = tile_begin + wave_begin + k * 64 + lane;
         const bool in = idx < m;
-        key[k] = in ? keys_in[idx] : ~0ull;
+        key[k] = in ? keys_in[idx] : (Key)~(Key)0;
     }
 #pragma unroll
     for (int k = 0; k < kOsItems; ++k) {
@@ -249,7 +251,7 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const uint64_t* __r
     for (int k = 0; k < kOsItems; ++k) {
         const int i = k * kOsThreads + tid;
         if (i < count) {
-            const uint64_t kk = s_keys[i];
+            const Key kk = s_keys[i];
             const uint32_t d = (uint32_t)(kk >> shift) & mask;
             const long long pos = (long long)digit_out[d] + i;
             keys_out[pos] = kk;
@@ -291,25 +293,26 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
     return D3GS_OK;
 }
 
-extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                               size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
-                               d3gs_stream_t stream) {
-    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !result_in_b_host) {
-        set_error("d3gs_sort_pairs: bad argument (m=%lld bits=[%d,%d))", (long long)m, begin_bit, end_bit);
+template <typename Key>
+static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys_b, int32_t* vals_a, int32_t* vals_b,
+                           void* workspace, size_t workspace_bytes, int64_t m, int begin_bit, int end_bit,
+                           int* result_in_b_host, d3gs_stream_t stream) {
+    if (m < 0 || begin_bit < 0 || end_bit > key_bits || begin_bit > end_bit || !result_in_b_host) {
+        set_error("%s: bad argument (m=%lld bits=[%d,%d))", who, (long long)m, begin_bit, end_bit);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    if (m >= (1ll << 30)) { set_error("d3gs_sort_pairs: m >= 2^30 is not supported"); return D3GS_ERR_UNSUPPORTED; }
+    if (m >= (1ll << 30)) { set_error("%s: m >= 2^30 is not supported", who); return D3GS_ERR_UNSUPPORTED; }
     *result_in_b_host = 0;
     if (m == 0 || begin_bit == end_bit) return D3GS_OK;
     if (!keys_a || !keys_b || !vals_a || !vals_b || !workspace) {
-        set_error("d3gs_sort_pairs: NULL buffer");
+        set_error("%s: NULL buffer", who);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     const int passes = os_passes(begin_bit, end_bit);
     SortWorkspace ws;
     const size_t need = os_layout(m, passes, &ws, workspace);
     if (workspace_bytes < need) {
-        set_error("d3gs_sort_pairs: workspace %zu < required %zu", workspace_bytes, need);
+        set_error("%s: workspace %zu < required %zu", who, workspace_bytes, need);
         return D3GS_ERR_WORKSPACE_TOO_SMALL;
     }
     hipStream_t s = (hipStream_t)stream;
@@ -317,11 +320,11 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
     // a fill kernel, not a memset node, so the call can be captured in a graph
     hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
     const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
-    hipLaunchKernelGGL(os_hist_kernel, dim3(hist_blocks), dim3(kHistThreads),
+    hipLaunchKernelGGL(os_hist_kernel<Key>, dim3(hist_blocks), dim3(kHistThreads),
                        (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m, begin_bit,
                        end_bit, passes, ws.hist);
-    uint64_t* kin = keys_a;
-    uint64_t* kout = keys_b;
+    Key* kin = keys_a;
+    Key* kout = keys_b;
     int32_t* vin = vals_a;
     int32_t* vout = vals_b;
     int in_b = 0;
@@ -329,15 +332,29 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
         const int bit = begin_bit + 8 * p;
         const int nb = std::min(8, end_bit - bit);
         const uint32_t mask = (1u << nb) - 1u;
-        hipLaunchKernelGGL(os_pass_kernel, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m, bit,
-                           mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
+        hipLaunchKernelGGL(os_pass_kernel<Key>, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
+                           bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
                            ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
         std::swap(kin, kout);
         std::swap(vin, vout);
         in_b ^= 1;
     }
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { set_error("d3gs_sort_pairs: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     *result_in_b_host = in_b;
     return D3GS_OK;
+}
+
+extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                               size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                               d3gs_stream_t stream) {
+    return sort_pairs_impl<uint64_t>("d3gs_sort_pairs", 64, keys_a, keys_b, vals_a, vals_b, workspace, workspace_bytes, m,
+                                     begin_bit, end_bit, result_in_b_host, stream);
+}
+
+extern "C" int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                                   size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                                   d3gs_stream_t stream) {
+    return sort_pairs_impl<uint32_t>("d3gs_sort_pairs_u32", 32, keys_a, keys_b, vals_a, vals_b, workspace,
+                                     workspace_bytes, m, begin_bit, end_bit, result_in_b_host, stream);
 }

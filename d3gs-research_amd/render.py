@@ -166,6 +166,14 @@ class GaussianSplatOp:
             raise NotImplementedError("GaussianSplatOp (gfx950 build): unsupported config options: " + ", ".join(bad))
 
     @property
+    def _last_keys_sorted(self) -> torch.Tensor:
+        """The reference's sorted 64-bit keys, (tile << 32) | depth bits, rebuilt from the last forward's
+        sorted tile keys and gaussian indices (parity tests compare them with the oracle's)."""
+        tile_keys, idx, depths = self._last_sorted
+        bits = depths.view(torch.int32)[idx.long()].long() & 0xFFFFFFFF
+        return (tile_keys.long() << 32) | bits
+
+    @property
     def is_nchw(self):
         return self._cfg.use_nchw
 
@@ -323,8 +331,9 @@ class GaussianSplatOp:
                         "d3gs_sort_workspace_bytes")
             ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
             in_b = C.c_int(0)
-            _capi.check(L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                          _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s),
+            fn = L.d3gs_sort_pairs if keys_a.dtype == torch.int64 else L.d3gs_sort_pairs_u32
+            _capi.check(fn(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
+                           _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s),
                         "d3gs_sort_pairs")
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
 
@@ -378,31 +387,32 @@ class GaussianSplatOp:
                     out_color[..., :3] = bg
             return out, None
 
+        # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
         with self._stage("make_keys"):
-            keys = torch.empty(num_rendered, dtype=torch.int64, device=dev)
+            tile_keys = torch.empty(num_rendered, dtype=i32, device=dev)
             gaussian_idx = torch.empty(num_rendered, dtype=i32, device=dev)
             _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                                          _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                         _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), _capi.ptr(keys),
-                                         _capi.ptr(gaussian_idx),
-                                         num_rendered, s), "d3gs_make_keys")
+                                         _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
+                                         _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), num_rendered, s),
+                        "d3gs_make_keys")
 
         with self._stage("sort"):
-            end_bit = 32 + L.d3gs_higher_msb(num_tiles)
-            keys_sorted, gaussian_idx_sorted = _sort(keys, gaussian_idx, num_rendered, 32, end_bit)
+            tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, num_rendered, 0,
+                                                          L.d3gs_higher_msb(num_tiles))
 
         with self._stage("tile_ranges"):
             workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
             tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
-            _capi.check(L.d3gs_tile_ranges(_capi.ptr(keys_sorted), num_rendered, _capi.ptr(workload_ranges),
-                                           num_tiles, _capi.ptr(tile_order), s), "d3gs_tile_ranges")
+            _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), num_rendered, _capi.ptr(workload_ranges),
+                                               num_tiles, _capi.ptr(tile_order), s), "d3gs_tile_ranges_u32")
 
         ctx = GaussianSplatOpContext(
             conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
             gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
             image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
             tile_order=tile_order)
-        self._last_keys_sorted = keys_sorted  # kept for parity tests (sorted key order)
+        self._last_sorted = (tile_keys_sorted, gaussian_idx_sorted, depths)  # kept for parity tests
         if sh_done is not None:
             torch.cuda.current_stream().wait_event(sh_done)
         with self._stage("blend_fwd"):

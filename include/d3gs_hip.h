@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 9
+#define D3GS_ABI_VERSION 10
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -127,11 +127,14 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
  * taken in that order (see d3gs_depth_keys).  Two optional inputs (may be NULL) save gathers
  * without changing the pairs emitted: ordered_depth_keys[j], the sorted keys of the depth sort
  * (low 32 bits = depth bits of gaussian gaussian_order[j]), read instead of depths[gaussian_order[j]];
- * tile_masks, the record d3gs_preprocess_fwd wrote with the same params. */
+ * tile_masks, the record d3gs_preprocess_fwd wrote with the same params.
+ * Exactly one of keys / tile_keys is given.  tile_keys (uint32[m]) receives the tile id alone: with the
+ * pairs emitted in depth order the pair sort only needs the tile digits, so the 32-bit variants below
+ * (d3gs_sort_pairs_u32 on bits [0, d3gs_higher_msb(num_tiles)), d3gs_tile_ranges_u32) move a third less. */
 int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                    const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
                    const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
-                   int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
+                   uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
 
 /* Depth-first factorisation of the pair sort (no counterpart in the reference, which
  * radix-sorts all M pairs on the full (tile, depth) key; the result is bit-identical).
@@ -155,6 +158,10 @@ int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* byt
 int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
                     size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
                     d3gs_stream_t stream);
+/* the same over 32-bit keys (end_bit <= 32); the workspace size is that of d3gs_sort_workspace_bytes */
+int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                        size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
+                        d3gs_stream_t stream);
 
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
  * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],
@@ -163,6 +170,9 @@ int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t
  * reference, which launches tiles in raster order; it changes scheduling, not results). */
 int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
                      int32_t* tile_order, d3gs_stream_t stream);
+/* the same over 32-bit tile keys (see d3gs_make_keys) */
+int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
+                         int32_t* tile_order, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
  * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].

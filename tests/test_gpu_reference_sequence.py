@@ -51,7 +51,7 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
 
     keys, vals = torch.empty(M, dtype=torch.int64, device=dev), torch.empty(M, dtype=i32, device=dev)
     _capi.check(L.d3gs_make_keys(C.byref(P), p(radii), p(uvs), p(conic), p(depths), p(touched), None, None, None,
-                                 p(keys), p(vals), M, s), "make_keys")
+                                 p(keys), None, p(vals), M, s), "make_keys")
     assert np.array_equal(cpu(keys).view(np.uint64), ref["keys"])
     assert np.array_equal(cpu(vals), ref["vals"])
 
