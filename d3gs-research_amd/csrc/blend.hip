@@ -37,12 +37,6 @@ __device__ __forceinline__ float blend_power(const StagedGaussian& g, float dx, 
     return __builtin_fmaf(g.nb * dx, dy, __builtin_fmaf(g.hc * dy, dy, (g.ha * dx) * dx));
 }
 
-// exp for an argument that already passed `x >= thr` (so x > -86 and x is not NaN)
-__device__ __forceinline__ float blend_expf(float x) {
-    const float e = det_expf_inrange(x);
-    return x > 88.0f ? __builtin_inff() : e;
-}
-
 // Tile index for a workgroup.  Tile list lengths are heavily skewed (dense screen regions hold
 // lists 20x the median), so the launch order matters more than L2 locality: with `tile_order`
 // (tiles by descending list length) the long tiles start first and, because consecutive
@@ -236,7 +230,9 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 // selects (w = 0 leaves the accumulators untouched): far fewer scalar mask operations
                 // than nested per-lane branches.  exp of a lane that is not live may be garbage; it is
                 // never selected.
-                const float G = blend_expf(power);
+                // no overflow guard: beyond exp's range the product o * G is inf, huge or NaN, and
+                // fminf(0.99, .) gives 0.99 in every case, as it does for the guarded exp's inf
+                const float G = det_expf_inrange(power);
                 const float alpha = fminf(0.99f, sg.o * G);
                 const bool hit = live && alpha >= P.alpha_eps;
                 const float nextT = T * (1.0f - alpha);
@@ -429,7 +425,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dl);
             dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
             dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
-            const float dL_dalpha = dl / one_m;
+            // 1 - alpha lies in [0.01, 1): the hardware reciprocal (1 ulp) replaces the 11-instruction IEEE
+            // division; the quotient scales every term of this pixel alike, by at most 2 ulp
+            const float dL_dalpha = dl * __builtin_amdgcn_rcpf(one_m);
             // With q = dL/dG * G the screen-space gradients are linear in five moments of q:
             // dL/du = -(a S1 + b S2), dL/dv = -(c S2 + b S1), dL/dconic = (-S3/2, -S4, -S5/2), where
             // S1 = sum q dx, S2 = sum q dy, S3 = sum q dx^2, S4 = sum q dx dy, S5 = sum q dy^2

@@ -717,8 +717,9 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     float alpha = fminf(0.99f, co[3] * G);
                     bool valid = power <= 0.0f && alpha >= P->alpha_eps;
                     if (!valid) continue;
-                    // fixed operation sequence (shared with the HIP kernel) so that the per-pixel terms
-                    // agree bit for bit and only the order of the sums differs
+                    // fixed operation sequence shared with the HIP kernel: which pixels a gaussian touches,
+                    // T and the colour still behind agree bit for bit; the kernel forms dl / (1 - alpha) with
+                    // the hardware reciprocal (within 2 ulp of this division), and the order of the sums differs
                     const float one_m = 1.0f - alpha;
                     float w = alpha * T;
                     T = T * one_m;
