@@ -197,7 +197,9 @@ __device__ __forceinline__ uint32_t key_tile(Key k) {
 
 template <typename Key>
 __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restrict__ keys, long long m,
+                                                              const long long* __restrict__ m_device,
                                                               int32_t* __restrict__ ranges, int num_tiles) {
+    if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the key buffer
     const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
     if (i >= m) return;
     const uint32_t t = key_tile<Key>(keys[i]);
@@ -344,8 +346,8 @@ extern "C" int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t*
 }
 
 template <typename Key>
-static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, int32_t* workload_ranges,
-                            int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
+static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, const int64_t* m_device,
+                            int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
     if (m < 0 || num_tiles < 0) { set_error("%s: bad argument", who); return D3GS_ERR_INVALID_ARGUMENT; }
     if ((m > 0 && !keys_sorted) || (num_tiles > 0 && !workload_ranges)) {
         set_error("%s: NULL buffer", who);
@@ -353,7 +355,8 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
     }
     if (m > 0)
         hipLaunchKernelGGL(tile_ranges_kernel<Key>, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           (hipStream_t)stream, keys_sorted, (long long)m, workload_ranges, (int)num_tiles);
+                           (hipStream_t)stream, keys_sorted, (long long)m, (const long long*)m_device, workload_ranges,
+                           (int)num_tiles);
     if (tile_order && num_tiles > 0)
         hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, workload_ranges,
                            (int)num_tiles, tile_order);
@@ -364,11 +367,13 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
 
 extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
                                 int32_t* tile_order, d3gs_stream_t stream) {
-    return tile_ranges_impl<uint64_t>("d3gs_tile_ranges", keys_sorted, m, workload_ranges, num_tiles, tile_order, stream);
+    return tile_ranges_impl<uint64_t>("d3gs_tile_ranges", keys_sorted, m, nullptr, workload_ranges, num_tiles, tile_order,
+                                      stream);
 }
 
-extern "C" int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, int32_t* workload_ranges,
-                                    int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
-    return tile_ranges_impl<uint32_t>("d3gs_tile_ranges_u32", tile_keys_sorted, m, workload_ranges, num_tiles, tile_order,
-                                      stream);
+extern "C" int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
+                                    int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
+                                    d3gs_stream_t stream) {
+    return tile_ranges_impl<uint32_t>("d3gs_tile_ranges_u32", tile_keys_sorted, m, m_device, workload_ranges, num_tiles,
+                                      tile_order, stream);
 }

@@ -82,8 +82,10 @@ constexpr int kHistThreads = 1024;
 constexpr int kHistCopies = 8;
 template <typename Key>
 __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __restrict__ keys, long long m,
+                                                                const long long* __restrict__ m_device,
                                                                 int begin_bit, int end_bit, int passes,
                                                                 uint32_t* __restrict__ hist) {
+    if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the buffers
     extern __shared__ uint32_t h[];  // [kHistCopies][passes][256]
     const int table = passes * kOsRadix;
     for (int k = threadIdx.x; k < kHistCopies * table; k += kHistThreads) h[k] = 0u;
@@ -111,7 +113,8 @@ template <typename Key>
 __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restrict__ keys_in,
                                                               const int32_t* __restrict__ vals_in,
                                                               Key* __restrict__ keys_out,
-                                                              int32_t* __restrict__ vals_out, long long m, int shift,
+                                                              int32_t* __restrict__ vals_out, long long m,
+                                                              const long long* __restrict__ m_device, int shift,
                                                               uint32_t mask, int ntiles,
                                                               const uint32_t* __restrict__ hist /* this pass, [256] */,
                                                               uint32_t* __restrict__ ticket,
@@ -131,6 +134,10 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
     // would add one chip-wide same-address atomic per workgroup to the start of every pass.
     const int tile = blockIdx.x;
     if (tile >= ntiles) return;
+    // with a device-side count the grid covers the buffers' capacity: tiles past the count hold no pair,
+    // nobody looks back at them, and they leave at once
+    if (m_device) m = min(m, max(*m_device, 0ll));
+    if ((long long)tile * kOsTile >= m) return;
 
     const long long tile_begin = (long long)tile * kOsTile;
     const int wave_begin = wave * (kOsTile / kOsWaves);
@@ -295,8 +302,8 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
 
 template <typename Key>
 static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys_b, int32_t* vals_a, int32_t* vals_b,
-                           void* workspace, size_t workspace_bytes, int64_t m, int begin_bit, int end_bit,
-                           int* result_in_b_host, d3gs_stream_t stream) {
+                           void* workspace, size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit,
+                           int end_bit, int* result_in_b_host, d3gs_stream_t stream) {
     if (m < 0 || begin_bit < 0 || end_bit > key_bits || begin_bit > end_bit || !result_in_b_host) {
         set_error("%s: bad argument (m=%lld bits=[%d,%d))", who, (long long)m, begin_bit, end_bit);
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -321,8 +328,8 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
     hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
     const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
     hipLaunchKernelGGL(os_hist_kernel<Key>, dim3(hist_blocks), dim3(kHistThreads),
-                       (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m, begin_bit,
-                       end_bit, passes, ws.hist);
+                       (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m,
+                       (const long long*)m_device, begin_bit, end_bit, passes, ws.hist);
     Key* kin = keys_a;
     Key* kout = keys_b;
     int32_t* vin = vals_a;
@@ -333,7 +340,7 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         const int nb = std::min(8, end_bit - bit);
         const uint32_t mask = (1u << nb) - 1u;
         hipLaunchKernelGGL(os_pass_kernel<Key>, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
-                           bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
+                           (const long long*)m_device, bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
                            ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
         std::swap(kin, kout);
         std::swap(vin, vout);
@@ -349,12 +356,12 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
                                size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
                                d3gs_stream_t stream) {
     return sort_pairs_impl<uint64_t>("d3gs_sort_pairs", 64, keys_a, keys_b, vals_a, vals_b, workspace, workspace_bytes, m,
-                                     begin_bit, end_bit, result_in_b_host, stream);
+                                     nullptr, begin_bit, end_bit, result_in_b_host, stream);
 }
 
 extern "C" int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                                   size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
-                                   d3gs_stream_t stream) {
+                                   size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit, int end_bit,
+                                   int* result_in_b_host, d3gs_stream_t stream) {
     return sort_pairs_impl<uint32_t>("d3gs_sort_pairs_u32", 32, keys_a, keys_b, vals_a, vals_b, workspace,
-                                     workspace_bytes, m, begin_bit, end_bit, result_in_b_host, stream);
+                                     workspace_bytes, m, m_device, begin_bit, end_bit, result_in_b_host, stream);
 }

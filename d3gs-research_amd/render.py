@@ -144,6 +144,10 @@ class GaussianSplatOp:
         # The SH colours are only read by the blend, so they are computed on a second stream beside the
         # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
         self.overlap_sh_colors = True
+        # size the pair buffers from the previous view's count instead of waiting for this view's
+        self.speculative_pair_buffers = True
+        self._pair_capacity = 0
+        self._count_host: torch.Tensor | None = None
         self._side_stream: torch.cuda.Stream | None = None
 
     # ------------------------------------------------------------------ utils
@@ -324,17 +328,21 @@ class GaussianSplatOp:
             if ta is not None:
                 self.stage_events.setdefault("sh_colors", []).append((ta, sh_done))
 
-        def _sort(keys_a, vals_a, count, begin_bit, end_bit):
+        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None):
             keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
             nbytes = C.c_size_t(0)
             _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
                         "d3gs_sort_workspace_bytes")
             ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
             in_b = C.c_int(0)
-            fn = L.d3gs_sort_pairs if keys_a.dtype == torch.int64 else L.d3gs_sort_pairs_u32
-            _capi.check(fn(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                           _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s),
-                        "d3gs_sort_pairs")
+            if keys_a.dtype == torch.int64:
+                rc = L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
+                                       _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s)
+            else:
+                rc = L.d3gs_sort_pairs_u32(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
+                                           _capi.ptr(ws), nbytes.value, count, count_dev, begin_bit, end_bit,
+                                           C.byref(in_b), s)
+            _capi.check(rc, "d3gs_sort_pairs")
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
 
         # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
@@ -358,8 +366,13 @@ class GaussianSplatOp:
             total = torch.empty(1, dtype=torch.int64, device=dev)
             _capi.check(L.d3gs_scan_tiles(_capi.ptr(counts_ordered), n, _capi.ptr(scan_ws), ws_bytes.value,
                                           _capi.ptr(total), s), "d3gs_scan_tiles")
-            num_rendered = int(total.item())  # host sync: sizes the next allocations (render.py:695)
-        self.last_num_rendered = num_rendered
+            # the count travels to pinned host memory behind the scan; the host looks at it only after
+            # the rest of the forward pass has been enqueued
+            if self._count_host is None:
+                self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+            self._count_host.copy_(total, non_blocking=True)
+            count_ready = torch.cuda.Event()
+            count_ready.record()
 
         final_T = torch.empty((1, height, width), dtype=f32, device=dev)
         n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
@@ -369,7 +382,8 @@ class GaussianSplatOp:
         out_depth = torch.empty((1, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
         out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=out_depth,
                                   n_contrib=n_contrib, radii=radii)
-        if num_rendered == 0:
+
+        def _empty_result():
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             # the reference returns uninitialised buffers here (render.py:706-729); fill with the
@@ -387,37 +401,58 @@ class GaussianSplatOp:
                     out_color[..., :3] = bg
             return out, None
 
-        # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
-        with self._stage("make_keys"):
-            tile_keys = torch.empty(num_rendered, dtype=i32, device=dev)
-            gaussian_idx = torch.empty(num_rendered, dtype=i32, device=dev)
-            _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                                         _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                         _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
-                                         _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), num_rendered, s),
-                        "d3gs_make_keys")
+        def _bin_and_blend(capacity: int, count_on_device: bool):
+            """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
+            read the pair count from `total` on the device and nothing here waits for the host."""
+            m_dev = _capi.ptr(total) if count_on_device else None
+            # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
+            with self._stage("make_keys"):
+                tile_keys = torch.empty(capacity, dtype=i32, device=dev)
+                gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
+                _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                                             _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
+                                             _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
+                                             _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
+                            "d3gs_make_keys")
+            with self._stage("sort"):
+                tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0,
+                                                              L.d3gs_higher_msb(num_tiles), m_dev)
+            with self._stage("tile_ranges"):
+                workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+                tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
+                _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
+                                                   _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
+                            "d3gs_tile_ranges_u32")
+            ctx = GaussianSplatOpContext(
+                conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
+                gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
+                image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
+                tile_order=tile_order)
+            if sh_done is not None:
+                torch.cuda.current_stream().wait_event(sh_done)
+            with self._stage("blend_fwd"):
+                self.rasterize_forward_backward(model, ctx, out, training=training,
+                                                render_depth=self._cfg.render_depth, _params=P)
+            return ctx, tile_keys_sorted
 
-        with self._stage("sort"):
-            tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, num_rendered, 0,
-                                                          L.d3gs_higher_msb(num_tiles))
-
-        with self._stage("tile_ranges"):
-            workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
-            tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
-            _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), num_rendered, _capi.ptr(workload_ranges),
-                                               num_tiles, _capi.ptr(tile_order), s), "d3gs_tile_ranges_u32")
-
-        ctx = GaussianSplatOpContext(
-            conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
-            gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
-            image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
-            tile_order=tile_order)
-        self._last_sorted = (tile_keys_sorted, gaussian_idx_sorted, depths)  # kept for parity tests
-        if sh_done is not None:
-            torch.cuda.current_stream().wait_event(sh_done)
-        with self._stage("blend_fwd"):
-            self.rasterize_forward_backward(model, ctx, out, training=training, render_depth=self._cfg.render_depth,
-                                            _params=P)
+        # The reference reads the pair count back before it can size the key buffers (render.py:695),
+        # which idles the GPU for a host round trip.  From the second view on the buffers are sized from
+        # the previous count with head room, everything is enqueued at once and the count is read
+        # afterwards; a view that outgrows its buffers is binned again with exact sizes.
+        capacity = self._pair_capacity if self.speculative_pair_buffers else 0
+        ctx = None
+        if capacity > 0:
+            ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
+        count_ready.synchronize()
+        num_rendered = int(self._count_host[0])
+        self.last_num_rendered = num_rendered
+        self._pair_capacity = num_rendered + num_rendered // 4 + 4096
+        if num_rendered == 0:
+            return _empty_result()
+        if ctx is None or num_rendered > capacity:
+            ctx, tile_keys_sorted = _bin_and_blend(num_rendered, False)
+        ctx.gaussian_idx_sorted = ctx.gaussian_idx_sorted[:num_rendered]
+        self._last_sorted = (tile_keys_sorted[:num_rendered], ctx.gaussian_idx_sorted, depths)  # kept for parity tests
         if not training:
             ctx = None
         return out, ctx

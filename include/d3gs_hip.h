@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 10
+#define D3GS_ABI_VERSION 11
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -158,10 +158,13 @@ int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* byt
 int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
                     size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
                     d3gs_stream_t stream);
-/* the same over 32-bit keys (end_bit <= 32); the workspace size is that of d3gs_sort_workspace_bytes */
+/* The same over 32-bit keys (end_bit <= 32); the workspace size is that of d3gs_sort_workspace_bytes(m).
+ * m_device (device int64, may be NULL): when given, m is the capacity of the buffers and the number of
+ * pairs sorted is min(m, *m_device), read on the device - a caller that sized its buffers from an
+ * earlier view can enqueue the sort without waiting for the scan total to reach the host. */
 int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                        size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
-                        d3gs_stream_t stream);
+                        size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit, int end_bit,
+                        int* result_in_b_host, d3gs_stream_t stream);
 
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
  * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],
@@ -170,9 +173,9 @@ int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int
  * reference, which launches tiles in raster order; it changes scheduling, not results). */
 int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
                      int32_t* tile_order, d3gs_stream_t stream);
-/* the same over 32-bit tile keys (see d3gs_make_keys) */
-int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, int32_t* workload_ranges, int32_t num_tiles,
-                         int32_t* tile_order, d3gs_stream_t stream);
+/* the same over 32-bit tile keys (see d3gs_make_keys); m_device as in d3gs_sort_pairs_u32 */
+int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
+                         int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
  * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].

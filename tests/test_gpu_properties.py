@@ -99,3 +99,32 @@ def test_forward_is_deterministic_and_backward_is_linear():
         e = ((a + b - c).norm(dim=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = float(e.quantile(0.5)), float(torch.quantile(e[:: max(1, e.numel() // 1_000_000)], 0.99))
         assert med <= 1e-4 and p99 <= 1e-2, f"{name}: additivity per-gaussian median {med:.2e} p99 {p99:.2e}"
+
+
+def test_pair_buffers_sized_from_the_previous_view(oracle):
+    """The operator sizes the pair buffers of a view from the previous view's count (no host wait
+    before binning).  A view that fits, one that outgrows the buffers (binned again), an empty one and
+    the unspeculative path must all equal the oracle."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    from helpers import oracle_forward
+    small, big = gen_scene(1, n=5000, wh=(250, 190), with_grad=False), gen_scene(1, n=40000, wh=(250, 190), with_grad=False)
+    op = GaussianSplatOp(op_config(small, DFVT))
+    refs = {id(sc): oracle_forward(oracle, sc, DFVT)[1] for sc in (small, big)}
+    seq = [small, small, big, big, small]          # exact, fits, outgrown, fits, fits with large head room
+    for k, sc in enumerate(seq):
+        out, ctx = op.forward(torch_model(sc), sc.camera(), training=True)
+        ref = refs[id(sc)]
+        assert op.last_num_rendered == ref["num_rendered"], k
+        assert tuple(ctx.gaussian_idx_sorted.shape) == (ref["num_rendered"],)
+        assert np.array_equal(ctx.gaussian_idx_sorted.cpu().numpy(), ref["gaussian_idx_sorted"]), k
+        assert np.array_equal(ctx.workload_ranges.cpu().numpy(), ref["workload_ranges"]), k
+        assert np.array_equal(out.color.cpu().numpy()[0].view(np.uint32), ref["color"].view(np.uint32)), k
+        assert np.array_equal(out.n_contrib.cpu().numpy()[0], ref["n_contrib"]), k
+    hidden = gen_scene(0, n=64, with_grad=False)
+    hidden.xyz[:, 2] = -5.0
+    out, ctx = op.forward(torch_model(hidden), hidden.camera(), training=True)
+    assert ctx is None and float(out.T.min()) == 1.0 and float(out.color.abs().max()) == 0.0
+    op.speculative_pair_buffers = False
+    out, ctx = op.forward(torch_model(big), big.camera(), training=True)
+    assert np.array_equal(out.color.cpu().numpy()[0].view(np.uint32), refs[id(big)]["color"].view(np.uint32))
