@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -43,7 +43,7 @@ _SIGNATURES = {
     "d3gs_abi_version": (C.c_int, []),
     "d3gs_last_error_string": (C.c_char_p, []),
     "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
-    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
+    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [_VP]),
     "d3gs_sh_colors": (C.c_int, [C.POINTER(Params)] + [_VP] * 6 + [_VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
@@ -53,7 +53,7 @@ _SIGNATURES = {
     "d3gs_sort_workspace_bytes": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
     "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
                                   C.POINTER(C.c_int), _VP]),
-    "d3gs_sort_pairs_u32": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, _VP, C.c_int, C.c_int,
+    "d3gs_sort_pairs_u32": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, _VP, C.c_int, C.c_int, C.c_int,
                                       C.POINTER(C.c_int), _VP]),
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             const float* __restrict__ depths,
                                                             const int32_t* __restrict__ offsets,
                                                             const int32_t* __restrict__ order,
-                                                            const uint64_t* __restrict__ ordered_depth_keys,
+                                                            const uint32_t* __restrict__ ordered_depth_keys,
                                                             const unsigned long long* __restrict__ tile_masks,
                                                             Key* __restrict__ keys, int32_t* __restrict__ vals,
                                                             long long m) {
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     // a gaussian with no tiles has an empty slot range; a caller that passed a smaller buffer than
     // the scan total must never be written past
     const bool active = in_range && sane && end > off && end <= m;
-    const uint32_t dbits = ordered_depth_keys ? (uint32_t)ordered_depth_keys[j] : __float_as_uint(depths[i]);
+    const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : __float_as_uint(depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
     unsigned long long kept = 0ull, meta = 0ull;
     if (tile_masks && active) {
@@ -296,7 +296,7 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
 
 extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                               const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                              const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                              const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
                               uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;

@@ -99,7 +99,8 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const float* __restrict__ sh_base, const uint8_t* __restrict__ invalid_mask, float* __restrict__ depths,
     int32_t* __restrict__ radii, float* __restrict__ uvs, float* __restrict__ conic_opacity,
     int32_t* __restrict__ tiles_touched, float* __restrict__ rgb_out, float* __restrict__ cov2d_out,
-    uint8_t* __restrict__ ne0_out, unsigned long long* __restrict__ tile_masks) {
+    uint8_t* __restrict__ ne0_out, unsigned long long* __restrict__ tile_masks,
+    uint32_t* __restrict__ depth_sort_keys) {
     // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
     extern __shared__ float s_rows[];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
@@ -213,6 +214,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     if (!in_range) return;
 
     depths[i] = z;
+    if (depth_sort_keys) depth_sort_keys[i] = __float_as_uint(z);   // positive floats order like their bits
     radii[i] = (int)radius;
     *reinterpret_cast<float2*>(uvs + 2 * i) = make_float2(u, v);
     *reinterpret_cast<float4*>(conic_opacity + 4 * i) = make_float4(con0, con1, con2, op);
@@ -581,7 +583,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
                                    const float* color_sh_base, const uint8_t* invalid_mask, float* depths,
                                    int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
                                    float* rgb_gaussian, float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0,
-                                   uint64_t* tile_masks, d3gs_stream_t stream) {
+                                   uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_fwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -597,11 +599,12 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
         hipLaunchKernelGGL(preprocess_fwd_kernel<true>, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz,
                            quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs,
                            conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,
-                           (unsigned long long*)tile_masks);
+                           (unsigned long long*)tile_masks, depth_sort_keys);
     } else {
         hipLaunchKernelGGL(preprocess_fwd_kernel<false>, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
                            scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity,
-                           tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks);
+                           tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks,
+                           depth_sort_keys);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

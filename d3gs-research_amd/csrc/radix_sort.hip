@@ -262,7 +262,8 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
             const uint32_t d = (uint32_t)(kk >> shift) & mask;
             const long long pos = (long long)digit_out[d] + i;
             keys_out[pos] = kk;
-            vals_out[pos] = vals_in[tile_begin + s_src[i]];
+            // without an input value array the values are the pairs' own indices
+            vals_out[pos] = vals_in ? vals_in[tile_begin + s_src[i]] : (int32_t)(tile_begin + s_src[i]);
         }
     }
 }
@@ -302,8 +303,9 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
 
 template <typename Key>
 static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys_b, int32_t* vals_a, int32_t* vals_b,
-                           void* workspace, size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit,
-                           int end_bit, int* result_in_b_host, d3gs_stream_t stream) {
+                           void* workspace, size_t workspace_bytes, int64_t m, const int64_t* m_device,
+                           int values_are_indices, int begin_bit, int end_bit, int* result_in_b_host,
+                           d3gs_stream_t stream) {
     if (m < 0 || begin_bit < 0 || end_bit > key_bits || begin_bit > end_bit || !result_in_b_host) {
         set_error("%s: bad argument (m=%lld bits=[%d,%d))", who, (long long)m, begin_bit, end_bit);
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -332,7 +334,7 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
                        (const long long*)m_device, begin_bit, end_bit, passes, ws.hist);
     Key* kin = keys_a;
     Key* kout = keys_b;
-    int32_t* vin = vals_a;
+    const int32_t* vin = values_are_indices ? nullptr : vals_a;   // first pass only
     int32_t* vout = vals_b;
     int in_b = 0;
     for (int p = 0; p < passes; ++p) {
@@ -343,7 +345,8 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
                            (const long long*)m_device, bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
                            ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
         std::swap(kin, kout);
-        std::swap(vin, vout);
+        vin = vout;
+        vout = in_b ? vals_b : vals_a;
         in_b ^= 1;
     }
     hipError_t e = hipGetLastError();
@@ -356,12 +359,13 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
                                size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
                                d3gs_stream_t stream) {
     return sort_pairs_impl<uint64_t>("d3gs_sort_pairs", 64, keys_a, keys_b, vals_a, vals_b, workspace, workspace_bytes, m,
-                                     nullptr, begin_bit, end_bit, result_in_b_host, stream);
+                                     nullptr, 0, begin_bit, end_bit, result_in_b_host, stream);
 }
 
 extern "C" int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                                   size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit, int end_bit,
-                                   int* result_in_b_host, d3gs_stream_t stream) {
+                                   size_t workspace_bytes, int64_t m, const int64_t* m_device, int values_are_indices,
+                                   int begin_bit, int end_bit, int* result_in_b_host, d3gs_stream_t stream) {
     return sort_pairs_impl<uint32_t>("d3gs_sort_pairs_u32", 32, keys_a, keys_b, vals_a, vals_b, workspace,
-                                     workspace_bytes, m, m_device, begin_bit, end_bit, result_in_b_host, stream);
+                                     workspace_bytes, m, m_device, values_are_indices, begin_bit, end_bit,
+                                     result_in_b_host, stream);
 }

@@ -301,13 +301,14 @@ class GaussianSplatOp:
             ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
             # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
             tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
+            depth_keys = torch.empty(n, dtype=i32, device=dev)      # float bits of the depths: the depth sort's keys
             overlap = bool(self.overlap_sh_colors)
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                 _capi.ptr(tiles_touched), None if overlap else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
-                None if overlap else _capi.ptr(ne0), _capi.ptr(tile_masks), s),
+                None if overlap else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), s),
                 "d3gs_preprocess_fwd")
         sh_done = None
         if overlap:
@@ -328,7 +329,7 @@ class GaussianSplatOp:
             if ta is not None:
                 self.stage_events.setdefault("sh_colors", []).append((ta, sh_done))
 
-        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None):
+        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False):
             keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
             nbytes = C.c_size_t(0)
             _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
@@ -340,8 +341,8 @@ class GaussianSplatOp:
                                        _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s)
             else:
                 rc = L.d3gs_sort_pairs_u32(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                           _capi.ptr(ws), nbytes.value, count, count_dev, begin_bit, end_bit,
-                                           C.byref(in_b), s)
+                                           _capi.ptr(ws), nbytes.value, count, count_dev, int(values_are_indices),
+                                           begin_bit, end_bit, C.byref(in_b), s)
             _capi.check(rc, "d3gs_sort_pairs")
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
 
@@ -350,11 +351,8 @@ class GaussianSplatOp:
         # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
         # tile digits only: 2 passes over M pairs instead of 6.
         with self._stage("depth_order"):
-            depth_keys = torch.empty(n, dtype=torch.int64, device=dev)
-            iota = torch.empty(n, dtype=i32, device=dev)
-            _capi.check(L.d3gs_depth_keys(_capi.ptr(depths), n, _capi.ptr(depth_keys), _capi.ptr(iota), s),
-                        "d3gs_depth_keys")
-            depth_keys_sorted, gaussian_order = _sort(depth_keys, iota, n, 0, 32)
+            depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, 32,
+                                                      values_are_indices=True)
 
         with self._stage("scan"):
             counts_ordered = torch.empty(n, dtype=i32, device=dev)

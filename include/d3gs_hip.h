@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 11
+#define D3GS_ABI_VERSION 12
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -99,12 +99,15 @@ int d3gs_higher_msb(uint32_t n);
  * early filter kept for each gaussian (word 0: bit mask over its candidate rect, word 1: the rect), which
  * d3gs_make_keys expands instead of repeating the per-tile tests.
  * rgb_gaussian may be NULL: the SH colour (and sh_to_rgb_ne_0) is then left to d3gs_sh_colors, which a
- * caller can run on a second stream beside the sort, the only consumer being the blend. */
+ * caller can run on a second stream beside the sort, the only consumer being the blend.
+ * depth_sort_keys (uint32[N], may be NULL): the float bits of depths, the keys of the depth sort
+ * (saves the d3gs_depth_keys pass). */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const float* color_sh_base,
                         const uint8_t* invalid_mask, float* depths,
                         int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
-                        float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, uint64_t* tile_masks, d3gs_stream_t stream);
+                        float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, uint64_t* tile_masks, uint32_t* depth_sort_keys,
+                        d3gs_stream_t stream);
 
 /* The SH-colour part of K1 on its own (render.py:569-613): rgb_gaussian [N,3] and, when not NULL, the
  * clamp mask sh_to_rgb_ne_0 [N] of the gaussians with radii > 0, zeros for the rest.  Same values as the
@@ -125,15 +128,15 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
  * gaussian-index order.  With gaussian_order (a permutation of 0..n-1), slot j emits
  * gaussian gaussian_order[j] and offsets must be the inclusive scan of the tile counts
  * taken in that order (see d3gs_depth_keys).  Two optional inputs (may be NULL) save gathers
- * without changing the pairs emitted: ordered_depth_keys[j], the sorted keys of the depth sort
- * (low 32 bits = depth bits of gaussian gaussian_order[j]), read instead of depths[gaussian_order[j]];
+ * without changing the pairs emitted: ordered_depth_keys[j] (uint32), the sorted keys of the depth sort
+ * (= depth bits of gaussian gaussian_order[j]), read instead of depths[gaussian_order[j]];
  * tile_masks, the record d3gs_preprocess_fwd wrote with the same params.
  * Exactly one of keys / tile_keys is given.  tile_keys (uint32[m]) receives the tile id alone: with the
  * pairs emitted in depth order the pair sort only needs the tile digits, so the 32-bit variants below
  * (d3gs_sort_pairs_u32 on bits [0, d3gs_higher_msb(num_tiles)), d3gs_tile_ranges_u32) move a third less. */
 int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                    const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                   const uint64_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                   const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
                    uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
 
 /* Depth-first factorisation of the pair sort (no counterpart in the reference, which
@@ -161,10 +164,12 @@ int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t
 /* The same over 32-bit keys (end_bit <= 32); the workspace size is that of d3gs_sort_workspace_bytes(m).
  * m_device (device int64, may be NULL): when given, m is the capacity of the buffers and the number of
  * pairs sorted is min(m, *m_device), read on the device - a caller that sized its buffers from an
- * earlier view can enqueue the sort without waiting for the scan total to reach the host. */
+ * earlier view can enqueue the sort without waiting for the scan total to reach the host.
+ * values_are_indices != 0: the input values are taken to be 0..m-1 and vals_a is not read (it is still
+ * one of the two output buffers). */
 int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
-                        size_t workspace_bytes, int64_t m, const int64_t* m_device, int begin_bit, int end_bit,
-                        int* result_in_b_host, d3gs_stream_t stream);
+                        size_t workspace_bytes, int64_t m, const int64_t* m_device, int values_are_indices,
+                        int begin_bit, int end_bit, int* result_in_b_host, d3gs_stream_t stream);
 
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
  * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],

@@ -245,3 +245,37 @@ def test_scan_c_abi(n):
     _capi.check(L.d3gs_scan_tiles(_capi.ptr(t), n, _capi.ptr(ws), nbytes.value, _capi.ptr(total), stream), "scan")
     assert np.array_equal(t.cpu().numpy(), np.cumsum(x, dtype=np.int64).astype(np.int32))
     assert int(total.item()) == int(x.sum())
+
+
+@pytest.mark.parametrize("m,cap,begin,end,implicit", [(1000, 1000, 0, 13, False), (70001, 90000, 0, 32, True),
+                                                      (0, 5000, 0, 13, False), (3_000_000, 3_100_000, 2, 15, True),
+                                                      (9000, 5000, 0, 32, False)])
+def test_sort_pairs_u32_c_abi(m, cap, begin, end, implicit):
+    """32-bit keys, the pair count read on the device (buffers of `cap` pairs, min(cap, m) sorted), and
+    values that are implicitly the pairs' indices."""
+    import torch
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    rng = np.random.default_rng(m + cap)
+    keys = rng.integers(0, 1 << 32, size=cap, dtype=np.uint64).astype(np.uint32)
+    keys[rng.random(cap) < 0.5] &= np.uint32(0x00001F0F)
+    vals = rng.integers(0, 1 << 30, size=cap).astype(np.int32)
+    cnt = min(m, cap)
+    mask = np.uint32(((1 << (end - begin)) - 1) << begin)
+    order = np.argsort(keys[:cnt] & mask, kind="stable")
+    ka, va = torch.from_numpy(keys.view(np.int32)).cuda(), torch.from_numpy(vals).cuda()
+    kb, vb = torch.full_like(ka, -1), torch.full_like(va, -1)
+    nbytes = C.c_size_t(0)
+    _capi.check(L.d3gs_sort_workspace_bytes(cap, begin, end, C.byref(nbytes)), "ws")
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device="cuda")
+    m_dev = torch.tensor([m], dtype=torch.int64, device="cuda")
+    in_b = C.c_int(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _capi.check(L.d3gs_sort_pairs_u32(_capi.ptr(ka), _capi.ptr(kb), _capi.ptr(va), _capi.ptr(vb), _capi.ptr(ws),
+                                      nbytes.value, cap, _capi.ptr(m_dev), int(implicit), begin, end, C.byref(in_b),
+                                      stream), "sort")
+    torch.cuda.synchronize()
+    ks, vs = (kb, vb) if in_b.value else (ka, va)
+    want_vals = order.astype(np.int32) if implicit else vals[:cnt][order]
+    assert np.array_equal(ks.cpu().numpy().view(np.uint32)[:cnt], keys[:cnt][order])
+    assert np.array_equal(vs.cpu().numpy()[:cnt], want_vals)

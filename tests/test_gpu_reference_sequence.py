@@ -35,7 +35,7 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     cov2d, ne0 = torch.empty((N, 3), dtype=f32, device=dev), torch.empty(N, dtype=torch.uint8, device=dev)
     _capi.check(L.d3gs_preprocess_fwd(C.byref(P), p(model.xyz), p(model.quaternion_xyzw), p(model.scale), p(model.opacity),
                                       p(model.color_sh), None, None, p(depths), p(radii), p(uvs), p(conic), p(touched),
-                                      p(rgb), p(cov2d), p(ne0), None, s), "preprocess")
+                                      p(rgb), p(cov2d), p(ne0), None, None, s), "preprocess")
     cpu = lambda t: t.cpu().numpy()
     assert np.array_equal(cpu(touched), ref["tiles_touched"])
     assert np.array_equal(cpu(rgb).view(np.uint32), ref["rgb_gaussian"].view(np.uint32))
