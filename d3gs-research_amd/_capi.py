@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -53,7 +53,7 @@ _SIGNATURES = {
     "d3gs_sort_workspace_bytes": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
     "d3gs_sort_pairs": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, C.c_int, C.c_int,
                                   C.POINTER(C.c_int), _VP]),
-    "d3gs_sort_pairs_u32": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, _VP, C.c_int, C.c_int, C.c_int,
+    "d3gs_sort_pairs_u32": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, _VP, C.c_int, C.c_int, C.c_int, C.c_int,
                                       C.POINTER(C.c_int), _VP]),
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),

@@ -304,8 +304,8 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
 template <typename Key>
 static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys_b, int32_t* vals_a, int32_t* vals_b,
                            void* workspace, size_t workspace_bytes, int64_t m, const int64_t* m_device,
-                           int values_are_indices, int begin_bit, int end_bit, int* result_in_b_host,
-                           d3gs_stream_t stream) {
+                           int values_are_indices, int workspace_is_zero, int begin_bit, int end_bit,
+                           int* result_in_b_host, d3gs_stream_t stream) {
     if (m < 0 || begin_bit < 0 || end_bit > key_bits || begin_bit > end_bit || !result_in_b_host) {
         set_error("%s: bad argument (m=%lld bits=[%d,%d))", who, (long long)m, begin_bit, end_bit);
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -327,7 +327,8 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
     hipStream_t s = (hipStream_t)stream;
     const int ntiles = os_tiles(m);
     // a fill kernel, not a memset node, so the call can be captured in a graph
-    hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
+    if (!workspace_is_zero)
+        hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
     const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
     hipLaunchKernelGGL(os_hist_kernel<Key>, dim3(hist_blocks), dim3(kHistThreads),
                        (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m,
@@ -359,13 +360,14 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
                                size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,
                                d3gs_stream_t stream) {
     return sort_pairs_impl<uint64_t>("d3gs_sort_pairs", 64, keys_a, keys_b, vals_a, vals_b, workspace, workspace_bytes, m,
-                                     nullptr, 0, begin_bit, end_bit, result_in_b_host, stream);
+                                     nullptr, 0, 0, begin_bit, end_bit, result_in_b_host, stream);
 }
 
 extern "C" int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
                                    size_t workspace_bytes, int64_t m, const int64_t* m_device, int values_are_indices,
-                                   int begin_bit, int end_bit, int* result_in_b_host, d3gs_stream_t stream) {
+                                   int workspace_is_zero, int begin_bit, int end_bit, int* result_in_b_host,
+                                   d3gs_stream_t stream) {
     return sort_pairs_impl<uint32_t>("d3gs_sort_pairs_u32", 32, keys_a, keys_b, vals_a, vals_b, workspace,
-                                     workspace_bytes, m, m_device, values_are_indices, begin_bit, end_bit,
-                                     result_in_b_host, stream);
+                                     workspace_bytes, m, m_device, values_are_indices, workspace_is_zero, begin_bit,
+                                     end_bit, result_in_b_host, stream);
 }

@@ -47,6 +47,9 @@ class GaussianSplatOpContext:
     per_gaussian_snap: None = None
     # not in the reference: tile ids by descending list length, the blend kernels' launch order
     tile_order: torch.Tensor | None = None
+    # not in the reference: the backward's [N, 16] gradient records, zero-filled during the forward pass
+    # on the second stream (consumed by the first backward over this context)
+    grad_records: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -302,6 +305,9 @@ class GaussianSplatOp:
             # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
             tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
             depth_keys = torch.empty(n, dtype=i32, device=dev)      # float bits of the depths: the depth sort's keys
+            grad_records = None
+            if training and self.overlap_sh_colors:
+                grad_records = torch.empty((n, _capi.GRAD_RECORD_FLOATS), dtype=f32, device=dev)
             overlap = bool(self.overlap_sh_colors)
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
@@ -324,27 +330,49 @@ class GaussianSplatOp:
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), C.c_void_p(side.cuda_stream)),
                 "d3gs_sh_colors")
-            sh_done = torch.cuda.Event(enable_timing=self.stage_events is not None)
+            tb = torch.cuda.Event(enable_timing=True) if ta is not None else None
+            if tb is not None:
+                tb.record(side)
+                self.stage_events.setdefault("sh_colors", []).append((ta, tb))
+            if grad_records is not None:
+                with torch.cuda.stream(side):
+                    grad_records.zero_()      # the backward's accumulators, cleared while the sort runs
+            sh_done = torch.cuda.Event()
             sh_done.record(side)
-            if ta is not None:
-                self.stage_events.setdefault("sh_colors", []).append((ta, sh_done))
 
-        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False):
-            keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
+        def _sort_ws_bytes(count, begin_bit, end_bit):
             nbytes = C.c_size_t(0)
             _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
                         "d3gs_sort_workspace_bytes")
-            ws = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+            return nbytes.value
+
+        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None):
+            keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
+            nbytes = _sort_ws_bytes(count, begin_bit, end_bit)
+            ws = zero_ws if zero_ws is not None else torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            assert ws.numel() >= nbytes
             in_b = C.c_int(0)
             if keys_a.dtype == torch.int64:
                 rc = L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                       _capi.ptr(ws), nbytes.value, count, begin_bit, end_bit, C.byref(in_b), s)
+                                       _capi.ptr(ws), nbytes, count, begin_bit, end_bit, C.byref(in_b), s)
             else:
                 rc = L.d3gs_sort_pairs_u32(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                           _capi.ptr(ws), nbytes.value, count, count_dev, int(values_are_indices),
-                                           begin_bit, end_bit, C.byref(in_b), s)
+                                           _capi.ptr(ws), nbytes, count, count_dev, int(values_are_indices),
+                                           int(zero_ws is not None), begin_bit, end_bit, C.byref(in_b), s)
             _capi.check(rc, "d3gs_sort_pairs")
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
+
+        # every zero-initialised work buffer of the forward pass comes out of one fill: the two sorts'
+        # workspaces and the tile ranges
+        tile_bits = L.d3gs_higher_msb(num_tiles)
+        spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
+        align = lambda v: (v + 255) // 256 * 256
+        sizes = [align(_sort_ws_bytes(n, 0, 32)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
+                 align(num_tiles * 8)]
+        zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
+        zero_ws_n = zero_pool[:sizes[0]]
+        zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
+        zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
 
         # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
         # digits only depend on the gaussian, so the same stable order comes from sorting the N
@@ -352,7 +380,7 @@ class GaussianSplatOp:
         # tile digits only: 2 passes over M pairs instead of 6.
         with self._stage("depth_order"):
             depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, 32,
-                                                      values_are_indices=True)
+                                                      values_are_indices=True, zero_ws=zero_ws_n)
 
         with self._stage("scan"):
             counts_ordered = torch.empty(n, dtype=i32, device=dev)
@@ -399,6 +427,8 @@ class GaussianSplatOp:
                     out_color[..., :3] = bg
             return out, None
 
+        pooled_ranges_used = [False]
+
         def _bin_and_blend(capacity: int, count_on_device: bool):
             """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
             read the pair count from `total` on the device and nothing here waits for the host."""
@@ -413,10 +443,12 @@ class GaussianSplatOp:
                                              _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
                             "d3gs_make_keys")
             with self._stage("sort"):
-                tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0,
-                                                              L.d3gs_higher_msb(num_tiles), m_dev)
+                tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0, tile_bits, m_dev,
+                                                              zero_ws=zero_ws_m if count_on_device else None)
             with self._stage("tile_ranges"):
-                workload_ranges = torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+                # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
+                workload_ranges = zero_ranges if not pooled_ranges_used[0] else torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+                pooled_ranges_used[0] = True
                 tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
                 _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
                                                    _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
@@ -425,7 +457,7 @@ class GaussianSplatOp:
                 conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
-                tile_order=tile_order)
+                tile_order=tile_order, grad_records=grad_records)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
@@ -437,7 +469,7 @@ class GaussianSplatOp:
         # which idles the GPU for a host round trip.  From the second view on the buffers are sized from
         # the previous count with head room, everything is enqueued at once and the count is read
         # afterwards; a view that outgrows its buffers is binned again with exact sizes.
-        capacity = self._pair_capacity if self.speculative_pair_buffers else 0
+        capacity = spec_capacity
         ctx = None
         if capacity > 0:
             ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
@@ -518,7 +550,9 @@ class GaussianSplatOp:
             assert ddepth.is_contiguous() and ddepth.shape == out.depth.shape, "ddepth must be contiguous [1,H,W]"
         # one 64-byte record per gaussian (see D3GS_GRAD_RECORD_FLOATS); the reference's four tensors
         # and dz are strided views of it
-        rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
+        rec, ctx.grad_records = ctx.grad_records, None
+        if rec is None:
+            rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
             _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),

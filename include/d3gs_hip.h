@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 12
+#define D3GS_ABI_VERSION 13
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -166,10 +166,13 @@ int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t
  * pairs sorted is min(m, *m_device), read on the device - a caller that sized its buffers from an
  * earlier view can enqueue the sort without waiting for the scan total to reach the host.
  * values_are_indices != 0: the input values are taken to be 0..m-1 and vals_a is not read (it is still
- * one of the two output buffers). */
+ * one of the two output buffers).
+ * workspace_is_zero != 0: the caller has zero-filled the workspace (say, together with its other
+ * zero-initialised buffers in one fill) and the sort does not clear it again. */
 int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
                         size_t workspace_bytes, int64_t m, const int64_t* m_device, int values_are_indices,
-                        int begin_bit, int end_bit, int* result_in_b_host, d3gs_stream_t stream);
+                        int workspace_is_zero, int begin_bit, int end_bit, int* result_in_b_host,
+                        d3gs_stream_t stream);
 
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
  * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],

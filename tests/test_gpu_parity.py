@@ -272,7 +272,7 @@ def test_sort_pairs_u32_c_abi(m, cap, begin, end, implicit):
     in_b = C.c_int(0)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     _capi.check(L.d3gs_sort_pairs_u32(_capi.ptr(ka), _capi.ptr(kb), _capi.ptr(va), _capi.ptr(vb), _capi.ptr(ws),
-                                      nbytes.value, cap, _capi.ptr(m_dev), int(implicit), begin, end, C.byref(in_b),
+                                      nbytes.value, cap, _capi.ptr(m_dev), int(implicit), 0, begin, end, C.byref(in_b),
                                       stream), "sort")
     torch.cuda.synchronize()
     ks, vs = (kb, vb) if in_b.value else (ka, va)
