@@ -218,36 +218,45 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
 
 // Tile ids ordered by descending list length (counting sort over 256 length buckets, one
 // workgroup).  Order inside a bucket is arbitrary: the result only steers scheduling.
-__global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t* __restrict__ ranges, int num_tiles,
+__global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t* __restrict__ work, int num_tiles,
                                                           int32_t* __restrict__ order) {
     __shared__ int s_max;
     __shared__ int s_bin[256];
+    __shared__ int s_wave[4];
+    auto amount = [&](int t) { return work[2 * t + 1] - work[2 * t]; };
     if (threadIdx.x == 0) s_max = 0;
     if (threadIdx.x < 256) s_bin[threadIdx.x] = 0;
     __syncthreads();
     int mx = 0;
-    for (int t = threadIdx.x; t < num_tiles; t += 1024) mx = max(mx, ranges[2 * t + 1] - ranges[2 * t]);
+    for (int t = threadIdx.x; t < num_tiles; t += 1024) mx = max(mx, amount(t));
     atomicMax(&s_max, mx);
     __syncthreads();
     const long long denom = (long long)s_max + 1;
-    for (int t = threadIdx.x; t < num_tiles; t += 1024) {
-        const int len = ranges[2 * t + 1] - ranges[2 * t];
-        atomicAdd(&s_bin[255 - (int)((long long)len * 256 / denom)], 1);
-    }
+    for (int t = threadIdx.x; t < num_tiles; t += 1024)
+        atomicAdd(&s_bin[255 - (int)((long long)max(amount(t), 0) * 256 / denom)], 1);
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int acc = 0;
-        for (int b = 0; b < 256; ++b) {
-            const int c = s_bin[b];
-            s_bin[b] = acc;
-            acc += c;
+    // exclusive scan of the 256 bucket counts by the first four wavefronts
+    int c = 0, incl = 0;
+    if (threadIdx.x < 256) {
+        c = s_bin[threadIdx.x];
+        incl = c;
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
         }
+        if (lane == 63) s_wave[threadIdx.x >> 6] = incl;
     }
     __syncthreads();
-    for (int t = threadIdx.x; t < num_tiles; t += 1024) {
-        const int len = ranges[2 * t + 1] - ranges[2 * t];
-        order[atomicAdd(&s_bin[255 - (int)((long long)len * 256 / denom)], 1)] = t;
+    if (threadIdx.x < 256) {
+        int base = 0;
+        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) base += s_wave[w];
+        s_bin[threadIdx.x] = base + incl - c;
     }
+    __syncthreads();
+    for (int t = threadIdx.x; t < num_tiles; t += 1024)
+        order[atomicAdd(&s_bin[255 - (int)((long long)max(amount(t), 0) * 256 / denom)], 1)] = t;
 }
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
