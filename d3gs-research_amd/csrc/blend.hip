@@ -196,13 +196,15 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
     const int len = r1 - r0;
     const int rounds = (len + kBlock - 1) / kBlock;
 
-    bool done = !inside;
+    // "this pixel is finished" lives in a vector register as an integer: a loop-carried bool would be kept
+    // as a lane mask in scalar registers and merged with scalar instructions on every iteration
+    int done = inside ? 0 : 1;
     float T = 1.0f;
     float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f, depth_accum = 0.0f;
     int contributor = 0;
 
     for (int round = 0; round < rounds; ++round) {
-        if (__syncthreads_count(done) == kBlock) break;
+        if (__syncthreads_count(done != 0) == kBlock) break;
         const int src = r0 + round * kBlock + tid;
         uint32_t bits = 0;
         if (src < r1) {
@@ -214,9 +216,8 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         }
         publish_masks(bits, wave, lane, s_mask);
         __syncthreads();
-        if (__all(done)) continue;
-        bool wave_done = false;
-        for (int chunk = 0; chunk < 4 && !wave_done; ++chunk) {
+        if (__all(done != 0)) continue;
+        for (int chunk = 0; chunk < 4; ++chunk) {
             unsigned long long m = uniform_u64(s_mask[wave][chunk]);
             while (m) {
                 const int j = chunk * 64 + __builtin_ctzll(m);
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 const StagedGaussian sg = s_g[j];
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
                 const float power = blend_power(sg, dx, dy);
-                const bool live = !done && power >= sg.thr;
+                const bool live = done == 0 && power >= sg.thr;
                 if (!__any(live)) continue;
                 // From here on every lane runs the same instructions and the outcome is applied with
                 // selects (w = 0 leaves the accumulators untouched): far fewer scalar mask operations
@@ -248,13 +249,11 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 acc2 = __builtin_fmaf(w, c.z, acc2);
                 if constexpr (kRgba) acc3 = acc3 + w;
                 if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
-                done = done || stop;
-                if (__any(stop) && __all(done)) {
-                    wave_done = true;
-                    break;
-                }
+                done = stop ? 1 : done;
+                if (__any(stop) && __all(done != 0)) goto wave_finished;
             }
         }
+    wave_finished:;
     }
 
     if (inside) {
