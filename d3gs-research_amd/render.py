@@ -50,6 +50,8 @@ class GaussianSplatOpContext:
     # not in the reference: the backward's [N, 16] gradient records, zero-filled during the forward pass
     # on the second stream (consumed by the first backward over this context)
     grad_records: torch.Tensor | None = None
+    # custom feature channels of this view ([N, F]) kept for the backward pass
+    custom_features: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -276,9 +278,13 @@ class GaussianSplatOp:
         if isinstance(cameras, CameraBundle) and len(cameras) != 1:
             return self._forward_bundle(model, cameras, training, instance2world_T, custom_features, mask,
                                         prep_user_inputs)
-        if instance2world_T is not None or custom_features is not None or prep_user_inputs:
-            raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
+        if instance2world_T is not None or prep_user_inputs:
+            raise NotImplementedError("instance2world_T / prep_user_inputs are not supported")
         self._check_model(model)
+        if custom_features is not None:
+            assert not self.is_nchw, "custom feat don't support nchw, set use_nchw=False in config."   # render.py:246
+            assert custom_features.is_cuda and custom_features.dtype == torch.float32 and custom_features.ndim == 2 \
+                and custom_features.shape[0] == len(model), "custom_features must be a float32 cuda tensor [N, F]"
         if mask is not None:
             # True rejects the gaussian (render.py:306-308)
             assert mask.is_cuda and mask.dtype in (torch.bool, torch.uint8) and mask.numel() == len(model) \
@@ -410,6 +416,8 @@ class GaussianSplatOp:
                                   n_contrib=n_contrib, radii=radii)
 
         def _empty_result():
+            if custom_features is not None:
+                out.custom_features = torch.zeros((1, height, width, custom_features.shape[1]), dtype=f32, device=dev)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             # the reference returns uninitialised buffers here (render.py:706-729); fill with the
@@ -482,6 +490,9 @@ class GaussianSplatOp:
         if ctx is None or num_rendered > capacity:
             ctx, tile_keys_sorted = _bin_and_blend(num_rendered, False)
         ctx.gaussian_idx_sorted = ctx.gaussian_idx_sorted[:num_rendered]
+        if custom_features is not None:
+            out.custom_features = self._blend_custom_features(P, ctx, out, custom_features)
+            ctx.custom_features = custom_features
         self._last_sorted = (tile_keys_sorted[:num_rendered], ctx.gaussian_idx_sorted, depths)  # kept for parity tests
         if not training:
             ctx = None
@@ -508,7 +519,8 @@ class GaussianSplatOp:
             rendered += self.last_num_rendered
         self.last_num_rendered = rendered
         cat = lambda name: torch.cat([getattr(o, name) for o in outs], 0)
-        out = GaussianSplatOutput(custom_features=None, T=cat("T"), color=cat("color"),
+        out = GaussianSplatOutput(custom_features=cat("custom_features") if custom_features is not None else None,
+                                  T=cat("T"), color=cat("color"),
                                   depth=cat("depth") if outs[0].depth is not None else None,
                                   n_contrib=cat("n_contrib"), radii=cat("radii"))
         if not training:
@@ -518,13 +530,70 @@ class GaussianSplatOp:
     def _backward_bundle(self, model, ctx, out, grad, return_uv_grad):
         return _backward_bundle_impl(self, model, ctx, out, grad, return_uv_grad)
 
+    # ------------------------------------------------------- custom features
+    # The blend is linear in the per-gaussian channel values and every channel shares the weights
+    # alpha * T, so F custom feature channels (render.py:1536-1539, 1892-1923, 1952-1971) are blended by
+    # running the colour kernels again over three channels at a time; in the backward pass each such
+    # run adds its share of d(uv, conic, opacity) and yields the gradient of its three channels where a
+    # colour run yields dcolor.
+    @staticmethod
+    def _feature_params(P: _capi.Params) -> _capi.Params:
+        Q = _capi.Params.from_buffer_copy(P)
+        Q.training, Q.render_depth, Q.render_rgba, Q.use_nchw = 1, 0, 0, 0     # raw sums, [H, W, 3]
+        return Q
+
+    @staticmethod
+    def _feature_triples(feat: torch.Tensor):
+        n, F = feat.shape
+        for k in range(0, F, 3):
+            tri = torch.zeros((n, 3), dtype=torch.float32, device=feat.device)
+            tri[:, :min(3, F - k)] = feat[:, k:k + 3]
+            yield k, min(3, F - k), tri
+
+    def _blend_custom_features(self, P, ctx, out, feat):
+        L, s = self._lib, self._stream()
+        Q = self._feature_params(P)
+        H, W = out.T.shape[1], out.T.shape[2]
+        res = torch.empty((1, H, W, feat.shape[1]), dtype=torch.float32, device=feat.device)
+        T2, nc2 = torch.empty_like(out.T), torch.empty_like(out.n_contrib)
+        for k, w, tri in self._feature_triples(feat.detach()):
+            img = torch.empty((H, W, 3), dtype=torch.float32, device=feat.device)
+            _capi.check(L.d3gs_blend_fwd(
+                C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(tri), None, _capi.ptr(ctx.tile_order), _capi.ptr(img),
+                _capi.ptr(T2), _capi.ptr(nc2), None, s), "d3gs_blend_fwd (custom features)")
+            res[0, :, :, k:k + w] = img[:, :, :w]
+        return res
+
+    def _backward_custom_features(self, P, ctx, out, dfeat_img, rec):
+        """Adds the feature channels' share to rec[:, 0:6] and returns dcustom_features [N, F]."""
+        L, s = self._lib, self._stream()
+        Q = self._feature_params(P)
+        feat = ctx.custom_features.detach()
+        n, F = feat.shape
+        H, W = out.T.shape[1], out.T.shape[2]
+        dfeat = torch.empty((n, F), dtype=torch.float32, device=feat.device)
+        zero_dT = torch.zeros_like(out.T)
+        for k, w, tri in self._feature_triples(feat):
+            img = torch.zeros((H, W, 3), dtype=torch.float32, device=feat.device)
+            img[:, :, :w] = out.custom_features[0, :, :, k:k + w]
+            dimg = torch.zeros((H, W, 3), dtype=torch.float32, device=feat.device)
+            dimg[:, :, :w] = dfeat_img[0, :, :, k:k + w]
+            rec_k = torch.zeros_like(rec)
+            _capi.check(L.d3gs_blend_bwd(
+                C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(tri), None, _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
+                _capi.ptr(out.n_contrib), _capi.ptr(img), None, _capi.ptr(dimg), _capi.ptr(zero_dT), None,
+                _capi.ptr(rec_k), s), "d3gs_blend_bwd (custom features)")
+            rec[:, 0:6] += rec_k[:, 0:6]
+            dfeat[:, k:k + w] = rec_k[:, 6:6 + w]
+        return dfeat
+
     # ------------------------------------------------------- blend fwd / bwd
     def rasterize_forward_backward(self, model, ctx: GaussianSplatOpContext, out: GaussianSplatOutput,
                                    grad: GaussianSplatGradients | None = None, training: bool = False,
                                    render_depth: bool = False, custom_features=None, _params=None, _cameras=None):
         """render.py:1329-2316: blend forward when ``grad`` is None, else blend backward."""
-        if custom_features is not None:
-            raise NotImplementedError("custom_features are not supported")
         assert bool(render_depth) == bool(self._cfg.render_depth), "render_depth must match the op's config"
         L = self._lib
         P = _params
@@ -569,10 +638,8 @@ class GaussianSplatOp:
                  custom_features=None, prep_user_inputs=None):
         """render.py:2779-3374.  Returns ``(grad_model, duv | None, dcustom_features)``; ``grad_model``
         is a model-shaped dataclass holding the gradients of the raw tensors."""
-        if instance2world_T is not None or custom_features is not None or prep_user_inputs:
-            raise NotImplementedError("instance2world_T / custom_features / prep_user_inputs are not supported")
-        if grad.dcustom_features is not None:
-            raise NotImplementedError("custom feature gradients are not supported")
+        if instance2world_T is not None or prep_user_inputs:
+            raise NotImplementedError("instance2world_T / prep_user_inputs are not supported")
         if isinstance(ctx, GaussianSplatOpBatchContext):
             return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
         L = self._lib
@@ -582,6 +649,11 @@ class GaussianSplatOp:
         with self._stage("blend_bwd"):
             g = self.rasterize_forward_backward(model, ctx, out, grad, training=True,
                                                 render_depth=self._cfg.render_depth, _params=P)
+        dcustom = None
+        if ctx.custom_features is not None:
+            dfeat_img = grad.dcustom_features if grad.dcustom_features is not None else \
+                torch.zeros_like(out.custom_features)
+            dcustom = self._backward_custom_features(P, ctx, out, dfeat_img.contiguous(), g.records)
         with self._stage("preprocess_bwd"):
             dxyz = torch.empty_like(model.xyz)
             dquat = torch.empty_like(model.quaternion_xyzw)
@@ -600,22 +672,26 @@ class GaussianSplatOp:
                                          color_sh=dsh, color_sh_base=dsh_base)
         self.last_raster_grads = g
         if return_uv_grad:
-            return grad_model, g.duv.unsqueeze(0), None
-        return grad_model, None, None
+            return grad_model, g.duv.unsqueeze(0), dcustom
+        return grad_model, None, dcustom
 
 
 def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
     """Per-camera backward passes; the model gradients add up over the cameras, duv stays per camera."""
-    total, duvs = None, []
+    total, duvs, dcustom = None, [], None
     n = len(model)
     for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
         if ctx_b is None:       # nothing was rendered for this camera: zero gradient
             duvs.append(torch.zeros((1, n, 2), dtype=torch.float32, device=model.xyz.device))
             continue
-        g_b = GaussianSplatGradients(drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
-                                     ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous())
-        gm, duv, _ = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True)
+        g_b = GaussianSplatGradients(
+            drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
+            ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous(),
+            dcustom_features=None if grad.dcustom_features is None else grad.dcustom_features[b:b + 1].contiguous())
+        gm, duv, dcf = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True)
         duvs.append(duv)
+        if dcf is not None:
+            dcustom = dcf if dcustom is None else dcustom + dcf
         if total is None:
             total = gm
         else:
@@ -626,19 +702,19 @@ def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
     if total is None:
         zeros = {k: torch.zeros_like(v) for k, v in model.get_proxy_field_dict().items()}
         total = dataclasses.replace(model, **zeros)
-    return total, (torch.cat(duvs, 0) if return_uv_grad else None), None
+    return total, (torch.cat(duvs, 0) if return_uv_grad else None), dcustom
 
 
 class _RasterizeGaussians(torch.autograd.Function):
     """render.py:3376-3587, with saved tensors addressed by name."""
 
     @staticmethod
-    def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, mask, model_cls,
-                cameras, training, op: GaussianSplatOp, uv_grad_holder=None):
+    def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, custom_features,
+                mask, model_cls, cameras, training, op: GaussianSplatOp, uv_grad_holder=None):
         model = model_cls(xyz=xyz, color_sh=color_sh, color_sh_base=color_sh_base, scale=scale,
                           quaternion_xyzw=quaternion_xyzw, opacity=opacity, cur_sh_degree=cur_sh_degree,
                           act_applied=True)
-        out, fwd_ctx = op.forward(model, cameras, training, mask=mask)
+        out, fwd_ctx = op.forward(model, cameras, training, custom_features=custom_features, mask=mask)
         ctx.has_ctx = fwd_ctx is not None
         if fwd_ctx is not None:
             ctx.fwd_ctx = fwd_ctx
@@ -648,36 +724,39 @@ class _RasterizeGaussians(torch.autograd.Function):
         ctx.cameras = cameras
         ctx.return_uv_grad = uv_grad_holder is not None
         ctx.mark_non_differentiable(out.n_contrib, out.radii)
-        # same tuple as the reference (render.py:3493-3499); custom features are not supported
-        return out.color, out.depth, None, out.T, out.n_contrib, out.radii
+        # same tuple as the reference (render.py:3493-3499)
+        return out.color, out.depth, out.custom_features, out.T, out.n_contrib, out.radii
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, drgb, ddepth, dcustom_features, dT, dn_contrib, dradii):
         if not ctx.has_ctx:
-            return (None,) * 13
+            return (None,) * 14
         if drgb is None:
             drgb = torch.zeros_like(ctx.out.color)
         if dT is None:
             dT = torch.zeros_like(ctx.out.T)
         if ddepth is not None:
             ddepth = ddepth.contiguous()
-        grads = GaussianSplatGradients(drgb=drgb.contiguous(), dT=dT.contiguous(), ddepth=ddepth)
-        gm, duv, _ = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
-                                     return_uv_grad=ctx.return_uv_grad)
-        return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, None, None,
-                None, None, None, duv)
+        if dcustom_features is not None:
+            dcustom_features = dcustom_features.contiguous()
+        grads = GaussianSplatGradients(drgb=drgb.contiguous(), dT=dT.contiguous(), ddepth=ddepth,
+                                       dcustom_features=dcustom_features)
+        gm, duv, dcf = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
+                                       return_uv_grad=ctx.return_uv_grad)
+        return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, dcf, None,
+                None, None, None, None, duv)
 
 
 def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSplatOp, training=False,
                         uv_grad_holder: torch.Tensor | None = None, instance2world_T=None, custom_features=None,
                         mask=None) -> GaussianSplatOutput:
     """render.py:3783-3838."""
-    if instance2world_T is not None or custom_features is not None:
-        raise NotImplementedError("instance2world_T / custom_features are not supported")
+    if instance2world_T is not None:
+        raise NotImplementedError("instance2world_T is not supported")
     model = model.create_model_with_act()   # torch-side activations for the non-fused families
     res = _RasterizeGaussians.apply(model.xyz, model.color_sh, model.color_sh_base, model.scale,
-                                    model.quaternion_xyzw, model.opacity, model.cur_sh_degree, mask, type(model),
-                                    cameras, training, op, uv_grad_holder)
+                                    model.quaternion_xyzw, model.opacity, model.cur_sh_degree, custom_features, mask,
+                                    type(model), cameras, training, op, uv_grad_holder)
     return GaussianSplatOutput(color=res[0], depth=res[1], custom_features=res[2], T=res[3], n_contrib=res[4],
                                radii=res[5])

@@ -255,11 +255,62 @@ def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
     return out
 
 
-def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False, ddepth=None):
-    """Whole backward: K7 + K9 from the dict ``forward`` returned."""
+def _feature_params(P):
+    Q = OracleParams.from_buffer_copy(P)
+    Q.training, Q.render_depth, Q.render_rgba, Q.use_nchw = 1, 0, 0, 0
+    return Q
+
+
+def _feature_triples(feat):
+    feat = _f32(feat)
+    for k in range(0, feat.shape[1], 3):
+        w = min(3, feat.shape[1] - k)
+        tri = np.zeros((feat.shape[0], 3), np.float32)
+        tri[:, :w] = feat[:, k:k + w]
+        yield k, w, tri
+
+
+def blend_custom_features(P, fwd, feat):
+    """Custom feature image [H, W, F] (render.py:1571-1573, 1920-1923, 2268-2270): every channel is
+    accumulated as ``acc += weight * value`` with the colour channels' weights and written without
+    background or clamp, so three channels at a time go through the colour blend in training mode."""
+    Q = _feature_params(P)
+    out = np.zeros((P.height, P.width, feat.shape[1]), np.float32)
+    for k, w, tri in _feature_triples(feat):
+        img, _, _, _ = blend_fwd(Q, fwd["workload_ranges"], fwd["gaussian_idx_sorted"], fwd["uvs"],
+                                 fwd["conic_opacity"], tri)
+        out[:, :, k:k + w] = img[:, :, :w]
+    return out
+
+
+def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False, ddepth=None,
+             custom_features=None, custom_feature_image=None, dcustom_features=None):
+    """Whole backward: K7 + K9 from the dict ``forward`` returned.  With custom features
+    (render.py:1892-1895, 1952-1955, 1969-1972) the alpha gradient gains
+    ``dot(dfeat, T * feat - rest)`` and ``dcustom_features = sum weight * dfeat``: both are linear in
+    the channel values, so they are taken from colour-blend backward passes over three channels at a
+    time (zero dT) and added; ``g["dcustom_features"]`` is [N, F]."""
     g = blend_bwd(P, fwd["workload_ranges"], fwd["gaussian_idx_sorted"], fwd["uvs"], fwd["conic_opacity"],
                   fwd["rgb_gaussian"], fwd["T"], fwd["n_contrib"], fwd["color"], drgb, dT, fwd["depths"],
                   fwd["depth"], ddepth)
+    if custom_features is not None:
+        Q = _feature_params(P)
+        F = custom_features.shape[1]
+        g["dcustom_features"] = np.zeros((P.n, F), np.float64)
+        g["absmass_features"] = np.zeros((P.n, F), np.float64)
+        zero_dT = np.zeros((P.height, P.width), np.float32)
+        for k, w, tri in _feature_triples(custom_features):
+            img = np.zeros((P.height, P.width, 3), np.float32)
+            img[:, :, :w] = custom_feature_image[:, :, k:k + w]
+            dimg = np.zeros_like(img)
+            dimg[:, :, :w] = dcustom_features[:, :, k:k + w]
+            gk = blend_bwd(Q, fwd["workload_ranges"], fwd["gaussian_idx_sorted"], fwd["uvs"], fwd["conic_opacity"],
+                           tri, fwd["T"], fwd["n_contrib"], img, dimg, zero_dT)
+            for name in ("duv", "dconic", "dopacity"):
+                g[name] += gk[name]
+            g["absmass"][:, 0:6] += gk["absmass"][:, 0:6]
+            g["dcustom_features"][:, k:k + w] = gk["dcolor"][:, :w]
+            g["absmass_features"][:, k:k + w] = gk["absmass"][:, 6:6 + w]
     sh_in = sh
     pb = preprocess_bwd(P, xyz, quat, scale, opacity, sh_in, fwd["radii"], fwd["cov2d_vecs"], fwd["sh_to_rgb_ne_0"],
                         g["duv"].astype(np.float32), g["dconic"].astype(np.float32),

@@ -39,9 +39,10 @@ def _quat_to_R(q):
         torch.stack([2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)], -1)], -2)
 
 
-def _render_f64(scene, params, member, order, anti_aliasing=False):
+def _render_f64(scene, params, member, order, anti_aliasing=False, feat=None):
     """Dense float64 forward: `member[p, j]` says gaussian order[j] is in pixel p's tile list.
-    Returns colour, T, blended depth and blended alpha (the sum of the weights)."""
+    Returns colour, T, blended depth and blended alpha (the sum of the weights), and the blended
+    custom features when `feat` [N, F] is given."""
     xyz, quat, scale, opac, sh = params
     tw = torch.tensor(scene.to_world, dtype=torch.float64)
     W, c = tw[:3, :3].T, tw[:3, 3]
@@ -83,6 +84,7 @@ def _render_f64(scene, params, member, order, anti_aliasing=False):
     dep = torch.zeros(H * Wd, dtype=torch.float64)
     asum = torch.zeros(H * Wd, dtype=torch.float64)
     done = torch.zeros(H * Wd, dtype=torch.bool)
+    fimg = None if feat is None else torch.zeros(H * Wd, feat.shape[1], dtype=torch.float64)
     for j, g in enumerate(order):
         dx, dy = uv[g, 0] - px, uv[g, 1] - py
         power = -0.5 * (ca[g] * dx * dx + ccn[g] * dy * dy) - cb[g] * dx * dy
@@ -97,7 +99,12 @@ def _render_f64(scene, params, member, order, anti_aliasing=False):
         col = col + w[:, None] * rgb[g]
         dep = dep + w * z[g]
         asum = asum + w
+        if feat is not None:
+            fimg = fimg + w[:, None] * feat[g]
         Tcur = torch.where(use, nT, Tcur)
+    if feat is not None:
+        return col.reshape(H, Wd, 3), Tcur.reshape(H, Wd), dep.reshape(H, Wd), asum.reshape(H, Wd), \
+            fimg.reshape(H, Wd, -1)
     return col.reshape(H, Wd, 3), Tcur.reshape(H, Wd), dep.reshape(H, Wd), asum.reshape(H, Wd)
 
 
@@ -112,9 +119,10 @@ def _setup(seed_cfg=0, n=96, wh=(48, 32), filt=0, sh_cfg=None):
     return scene
 
 
-def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False):
-    """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) (+ sum(depth*ddepth)) w.r.t. the raw
-    model tensors.  A four-channel drgb also weights the blended alpha."""
+def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False, feat=None, feat_image=None, dfeat=None):
+    """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) (+ sum(depth*ddepth))
+    (+ sum(features*dfeat)) w.r.t. the raw model tensors (and the custom features, last in the list).
+    A four-channel drgb also weights the blended alpha."""
     # global depth order (stable) and per-pixel tile-list membership from the oracle's binning
     valid = np.flatnonzero(ref["radii"] > 0)
     order = valid[np.argsort(ref["depths"][valid].view(np.uint32), kind="stable")]
@@ -128,7 +136,13 @@ def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False):
 
     params = [torch.tensor(a, dtype=torch.float64, requires_grad=True)
               for a in (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)]
-    col, Tfin, dep, asum = _render_f64(scene, params, torch.from_numpy(member), order.tolist(), anti_aliasing)
+    fimg = None
+    if feat is not None:
+        params.append(torch.tensor(feat, dtype=torch.float64, requires_grad=True))
+        col, Tfin, dep, asum, fimg = _render_f64(scene, params[:5], torch.from_numpy(member), order.tolist(),
+                                                 anti_aliasing, params[5])
+    else:
+        col, Tfin, dep, asum = _render_f64(scene, params, torch.from_numpy(member), order.tolist(), anti_aliasing)
     # the float64 forward agrees with the oracle's float32 forward (no threshold flips on this scene)
     assert np.abs(col.detach().numpy() - ref["color"][..., :3]).max() <= 2e-5
     assert np.abs(Tfin.detach().numpy() - ref["T"]).max() <= 1e-5
@@ -140,6 +154,9 @@ def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False):
     if ddepth is not None:
         assert np.abs(dep.detach().numpy() - ref["depth"]).max() <= 1e-4
         loss = loss + (dep * torch.from_numpy(ddepth).double()).sum()
+    if fimg is not None:
+        assert np.abs(fimg.detach().numpy() - feat_image).max() <= 2e-5 * max(1.0, np.abs(feat).max())
+        loss = loss + (fimg * torch.from_numpy(dfeat).double()).sum()
     loss.backward()
     return [p.grad for p in params]
 
@@ -281,3 +298,36 @@ def test_channels_and_anti_aliasing_match_float64_autograd(oracle, aa, depth, rg
     grads = _f64_grads(scene, ref, drgb, dT, ddepth, aa)
     for i, name in enumerate(["dxyz", "dquat", "dscale", "dopacity", "dsh"]):
         _close(pb[name], grads[i], name)
+
+
+@pytest.mark.parametrize("F,depth", [(2, False), (3, False), (7, True)])
+def test_custom_features_match_float64_autograd(oracle, F, depth):
+    """Custom feature channels (render.py:1571-1573, 1892-1895, 1920-1923, 1952-1955, 1969-1972):
+    the blended feature image, its share of the geometry gradients and dcustom_features against
+    float64 autograd over the dense restatement.  F = 2 and 7 cover a partly filled last triple."""
+    scene = _setup()
+    P = oracle_params(oracle, scene, 0)
+    P.render_depth = int(depth)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    rng = np.random.default_rng(13)
+    feat = rng.standard_normal((scene.n, F)).astype(np.float32)
+    fimg = oracle.blend_custom_features(P, ref, feat)
+    assert fimg.shape == (scene.height, scene.width, F)
+    # a constant feature blends to the sum of the weights, 1 - T
+    ones = oracle.blend_custom_features(P, ref, np.ones((scene.n, 1), np.float32))
+    assert np.abs(ones[..., 0] + ref["T"] - 1.0).max() <= 1e-5
+    drgb = rng.standard_normal((scene.height, scene.width, 3)).astype(np.float32)
+    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    ddepth = rng.standard_normal((scene.height, scene.width)).astype(np.float32) if depth else None
+    dfeat = rng.standard_normal(fimg.shape).astype(np.float32)
+    g, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                            drgb, dT, ddepth=ddepth, custom_features=feat, custom_feature_image=fimg,
+                            dcustom_features=dfeat)
+    grads = _f64_grads(scene, ref, drgb, dT, ddepth, False, feat, fimg, dfeat)
+    for i, name in enumerate(["dxyz", "dquat", "dscale", "dopacity", "dsh"]):
+        _close(pb[name], grads[i], name)
+    _close(g["dcustom_features"], grads[5], "dcustom_features")
+    # the feature term matters: without it the geometry gradients are far from the autograd ones
+    _, pb0 = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                             drgb, dT, ddepth=ddepth)
+    assert np.abs(pb0["dxyz"] - grads[0].numpy()).max() > 1e-2 * np.abs(grads[0].numpy()).max()
