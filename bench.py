@@ -29,11 +29,17 @@ STAGE_BYTES = {
     # Together 108 + 221 B against the fused kernel's 297 B / gaussian.
     "preprocess": lambda N, M, P, T, passes: 108 * N,
     "sh_colors": lambda N, M, P, T, passes: 221 * N,
-    "depth_order": lambda N, M, P, T, passes: (4 + 12) * N + (8 + 24 * 4) * N,
+    # binning, priced at what this factorisation has to move (32-bit keys, 32-bit values), not at the
+    # reference's single sort of 64-bit keys, which would flatter these stages:
+    # depth order of the N gaussians: histogram reads the keys (4), first pass reads keys and writes
+    # keys + indices (12), three more passes read and write both (16 each)
+    "depth_order": lambda N, M, P, T, passes: (4 + 12 + 3 * 16) * N,
     "scan": lambda N, M, P, T, passes: (12 + 8) * N,
-    "make_keys": lambda N, M, P, T, passes: 36 * N + 12 * M,
-    "sort": lambda N, M, P, T, passes: (8 + 24 * passes) * M,
-    "tile_ranges": lambda N, M, P, T, passes: 8 * M + 8 * T,
+    # order, offset, kept-tile record, depth key per gaussian; tile key + gaussian index per pair
+    "make_keys": lambda N, M, P, T, passes: 28 * N + 8 * M,
+    # pair sort on the tile bits: histogram reads the keys, `passes` passes read and write key + value
+    "sort": lambda N, M, P, T, passes: (4 + 16 * passes) * M,
+    "tile_ranges": lambda N, M, P, T, passes: 4 * M + 12 * T,
     "blend_fwd": lambda N, M, P, T, passes: 40 * M + 20 * P,
     "blend_bwd": lambda N, M, P, T, passes: 76 * M + 36 * P,
     "preprocess_bwd": lambda N, M, P, T, passes: (236 + 50 + 236) * N,
@@ -116,8 +122,7 @@ def main():
 
     N, P_px, T_tiles = scene.n, scene.width * scene.height, ((scene.width + 15) // 16) * ((scene.height + 15) // 16)
     M = op.last_num_rendered
-    end_bit = 32 + int(T_tiles).bit_length()
-    passes = (end_bit + 7) // 8
+    passes = (int(T_tiles).bit_length() + 7) // 8      # radix passes of the pair sort (tile bits only)
     stages = {}
     for name, evs in op.stage_events.items():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
