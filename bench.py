@@ -64,6 +64,33 @@ def committed_traffic_bytes(stage, config_id):
     return None
 
 
+def hbm_copy_probe(torch, nbytes=1 << 30, reps=10):
+    """GB/s (bytes read + bytes written) of a 1 GiB device-to-device copy, HIP events, best of `reps`."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty_like(src)
+    src.zero_()
+    dst.copy_(src)
+    best = float("inf")
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        dst.copy_(src)
+        b.record()
+        b.synchronize()
+        best = min(best, a.elapsed_time(b))
+    return round(2 * nbytes / (best * 1e-3) / 1e9, 1)
+
+
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,7 +155,8 @@ def main():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
         avg = sum(ts) / len(ts)
         nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes)
-        stages[name] = {"ms": round(avg, 4), "ms_p50": round(ts[len(ts) // 2], 4), "alg_bytes": int(nbytes),
+        stages[name] = {"ms": round(avg, 4), "ms_p10": round(ts[len(ts) // 10], 4), "ms_p50": round(ts[len(ts) // 2], 4),
+                        "ms_p90": round(ts[(len(ts) * 9) // 10], 4), "alg_bytes": int(nbytes),
                         "gbs": round(nbytes / (avg * 1e-3) / 1e9, 1)}
     op.stage_events = None
     if "sh_colors" in stages:
@@ -136,9 +164,16 @@ def main():
     gpu_sum = sum(s["ms"] for s in stages.values() if not s.get("overlapped"))
     dom = max(stages, key=lambda k: stages[k]["ms"])
     achieved = stages[dom]["gbs"]
+    copy_gbs = hbm_copy_probe(torch)
     roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": committed_traffic_bytes(dom, args.config),
-                "pair_evals_per_s": round(256.0 * M / (stages[dom]["ms"] * 1e-3), 1)}
+                "pair_evals_per_s": round(256.0 * M / (stages[dom]["ms"] * 1e-3), 1),
+                # what a plain device-to-device copy reaches on this box (read + written bytes per second)
+                "measured_copy_gbs": copy_gbs, "frac_of_measured_copy": round(achieved / copy_gbs, 5)}
+    # tile list lengths of the last view (the blend kernels' work is their sum and their skew)
+    _, last_ctx = op.forward(model, cam, training=True)
+    lens = (last_ctx.workload_ranges[:, 1] - last_ctx.workload_ranges[:, 0]).to(torch.float64)
+    tile_lists = {"mean": round(float(lens.mean()), 1), "median": float(lens.median()), "max": int(lens.max())}
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -158,12 +193,24 @@ def main():
             fwd_ms.append((c1 - c0) * 1e3)
             bwd_ms.append((c2 - c1) * 1e3)
         med = lambda v: sorted(v)[len(v) // 2]
-        cpu_baseline = {"value": round(med(fwd_ms) + med(bwd_ms), 1), "unit": "ms/view", "cores": O.num_threads(),
+        spent = time.perf_counter() - t_start
+        # one view on a single thread as well (the scalar figure), if the threaded one says it fits in ~20 s
+        threads, single = O.num_threads(), None
+        if (med(fwd_ms) + med(bwd_ms)) * threads < 20e3:
+            O.set_num_threads(1)
+            c0 = time.perf_counter()
+            ref1 = O.forward(Pc, cs.xyz, cs.quaternion_xyzw, cs.scale, cs.opacity, cs.color_sh)
+            O.backward(Pc, ref1, cs.xyz, cs.quaternion_xyzw, cs.scale, cs.opacity, cs.color_sh, cs.drgb[0], cs.dT[0])
+            single = round((time.perf_counter() - c0) * 1e3, 1)
+            O.set_num_threads(threads)
+        cpu_baseline = {"value": round(med(fwd_ms) + med(bwd_ms), 1), "unit": "ms/view", "cores": threads,
                         "kind": "port", "fwd_ms": round(med(fwd_ms), 1), "bwd_ms": round(med(bwd_ms), 1),
+                        "single_thread_ms": single, "cpu": cpu_model_name(), "host_cpus": os.cpu_count(),
                         "sample": f"{len(fwd_ms)} views of config {args.config} with {cs.n} gaussians "
                                   f"({'full workload' if cs.n == scene.n else 'reduced gaussian count'}), "
                                   f"M={ref['num_rendered']}, median, OpenMP over {O.num_threads()} threads, "
-                                  f"{time.perf_counter() - t_start:.1f} s of CPU work"}
+                                  f"{spent:.1f} s of CPU work"
+                                  + ("" if single is None else "; single_thread_ms: one view on one thread")}
 
     line = {
         "metric": "fwd+bwd raster ms/view, 1M Gaussians @1080p, 1 MI355X" if args.config == 2
@@ -173,7 +220,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"config {args.config}: {scene.name}", "gaussians": N, "sh_degree": scene.sh_degree,
                    "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name, "pairs_M": int(M),
-                   "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles},
+                   "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists},
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
         "gpu_stage_sum_ms": round(gpu_sum, 4),
         "stages": stages,
