@@ -73,24 +73,45 @@ __device__ __forceinline__ float dpp_f(float v) {
 __device__ __forceinline__ int reduce_slot(int lane) {
     if (lane & 3) return -1;
     const int r = lane >> 4, h = (lane >> 3) & 1, k = (lane >> 2) & 1;
-    if (k) return (h == 0 && r == 0) ? 8 : (h == 0 && r == 2) ? 9 : -1;
-    const int rowmap = (r == 0) ? 0 : (r == 1) ? 2 : (r == 2) ? 1 : 3;
-    return rowmap + 4 * h;
+    if (r == 0) return h + 2 * k;
+    if (r == 2) return 4 + h + 2 * k;
+    if (r == 1 && k == 0) return 8 + h;
+    return -1;
 }
 
 __device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
-                                               float v7, float v8, float v9, bool hi8, bool hi4) {
-    // 64 -> 32: lower half keeps the first value of each pair, upper half the second
-    const float s01 = swap_add32(v0, v1), s23 = swap_add32(v2, v3), s45 = swap_add32(v4, v5),
-                s67 = swap_add32(v6, v7), s8 = swap_add32(v8, v9);
-    // 32 -> 16: rows (0,2) keep the first register of each pair, rows (1,3) the second
-    const float q0 = swap_add16(s01, s23), q1 = swap_add16(s45, s67);
-    float q2 = swap_add16(s8, 0.0f);
-    // 16 -> 8: lanes 0-7 of a row keep q0, lanes 8-15 keep q1 (row_ror:8 pairs lane i with i^8)
-    float x = (hi8 ? q1 : q0) + dpp_f<0x128>(hi8 ? q0 : q1);
-    q2 = q2 + dpp_f<0x128>(q2);
-    // 8 -> 4: lanes with bit 2 clear keep x, the others q2 (row_half_mirror pairs lane i with 7 - i)
-    float y = (hi4 ? q2 : x) + dpp_f<0x141>(hi4 ? x : q2);
+                                               float v7, float v8, float v9) {
+    // 16 -> 8 and 8 -> 4 inside each row of 16 lanes, while the most registers are live, with DPP adds whose
+    // bank mask writes only one half of the lanes: "b += b[partner]" on the lanes that keep b, then
+    // "b = a + a[partner]" on the lanes that keep a, merges a pair of registers in two instructions and no
+    // select.  row_ror:8 pairs lane i with i ^ 8 (banks 0,1 | 2,3), row_half_mirror pairs i with 7 - i inside
+    // each 8 lanes (banks 0,2 | 1,3).  The block opens and closes with two wait states: a DPP read needs
+    // them after a vector write of its source, and so does what follows; the compiler cannot see inside.
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %0, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %2, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %3, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %4, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        // now %0..%4 hold (v0|v1), (v2|v3), (v4|v5), (v6|v7), (v8|v9) in lanes (bit 3 clear | set)
+        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %4, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %1, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %3, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+        "s_nop 1"
+        : "+v"(v1), "+v"(v3), "+v"(v5), "+v"(v7), "+v"(v9)
+        : "v"(v0), "v"(v2), "v"(v4), "v"(v6), "v"(v8));
+    // v3: v0 v1 | v2 v3 by (bit 3, bit 2) of the lane; v7: v4 .. v7 likewise; v9: v8 | v9 by bit 3
+    // 64 -> 32: rows 0,1 keep the first register, rows 2,3 the second
+    const float e0 = swap_add32(v3, v7), e1 = swap_add32(v9, 0.0f);
+    // 32 -> 16: rows 0,2 keep e0, rows 1,3 keep e1
+    float y = swap_add16(e0, e1);
     // 4 -> 1 inside each quad
     y = y + dpp_f<0x4E>(y);
     y = y + dpp_f<0xB1>(y);
@@ -156,6 +177,20 @@ __device__ __forceinline__ unsigned long long uniform_u64(unsigned long long v) 
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return ((unsigned long long)hi << 32) | lo;
+}
+
+// Predicate codes of __builtin_amdgcn_fcmpf / __builtin_amdgcn_sicmp (LLVM's CmpInst::Predicate).
+constexpr int kFcmpOge = 3, kFcmpOle = 5, kIcmpSlt = 40;
+
+// a = mask ? a0 : 0 and b = mask ? b0 : 0 for a lane mask held in a scalar register pair.  The compiler has no
+// cheap way from a 64-bit integer back to a per-lane predicate, hence the instruction is written out; the
+// two wait states in front cover a vector instruction that has just written the mask registers.
+__device__ __forceinline__ void select2_or_zero(unsigned long long mask, float a0, float b0, float& a, float& b) {
+    asm("s_nop 1\n\t"
+        "v_cndmask_b32_e64 %0, 0, %2, %4\n\t"
+        "v_cndmask_b32_e64 %1, 0, %3, %4"
+        : "=&v"(a), "=&v"(b)
+        : "v"(a0), "v"(b0), "s"(mask));
 }
 
 // Index of channel ch of pixel pid in the colour image: [H,W,C] or, with use_nchw, [C,H,W].
@@ -340,7 +375,6 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const float dT_term = (-dT_val) * render_T;
     int slot = reduce_slot(lane);
     if (slot >= kValues) slot = -1;
-    const bool hi8 = (lane & 8) != 0, hi4 = (lane & 4) != 0;
     // wave-uniform by construction; readfirstlane tells the compiler, which keeps the gaussian
     // bit masks and loop bounds below in scalar registers
     const int wave_todo = __builtin_amdgcn_readfirstlane(wave_max_i32(contributor));
@@ -371,24 +405,19 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
           unsigned long long m = uniform_u64(s_mask[wave][chunk]);
           if (cnt - chunk * 64 < 64) m &= (1ull << (cnt - chunk * 64)) - 1ull;
           if (!m) continue;
-          // the next gaussian's record is fetched from LDS while the current one is evaluated
-          int j_next = chunk * 64 + __builtin_ctzll(m);
-          StagedGaussian sg_next = s_g[j_next];
-          float4 c_next = s_rgb[j_next];
           while (m) {
-            const int j = j_next;
-            const StagedGaussian sg = sg_next;
-            const float4 c = c_next;
+            const int j = chunk * 64 + __builtin_ctzll(m);
             m &= m - 1;
-            if (m) {
-                j_next = chunk * 64 + __builtin_ctzll(m);
-                sg_next = s_g[j_next];
-                c_next = s_rgb[j_next];
-            }
+            const StagedGaussian sg = s_g[j];
+            const float4 c = s_rgb[j];
             const float dx = sg.x - pxf, dy = sg.y - pyf;
             const float power = blend_power(sg, dx, dy);
-            const bool cand = (round * kBlock + j < contributor) && power >= sg.thr && power <= 0.0f;
-            if (!__any(cand)) continue;
+            // Per-lane conditions as 64-bit lane masks (one compare instruction each, combined with scalar
+            // instructions; ordered compares, a NaN fails them as it fails the C operators they stand for).
+            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBlock + j, contributor, kIcmpSlt) &
+                                              __builtin_amdgcn_fcmpf(power, sg.thr, kFcmpOge) &
+                                              __builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOle);
+            if (cand_m == 0) continue;
             // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
             // gaussian contributed to.  From here on every lane runs the same instructions: a lane the
             // gaussian did not contribute to carries G = alpha = 0, which leaves its running state
@@ -397,10 +426,10 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             // discarded by the select.)
             const float G0 = det_expf_inrange(power);   // candidates have power in [thr, 0]
             const float alpha0 = fminf(0.99f, sg.o * G0);
-            const bool valid = cand && alpha0 >= P.alpha_eps;
-            if (!__any(valid)) continue;
-            const float G = valid ? G0 : 0.0f;
-            const float alpha = valid ? alpha0 : 0.0f;
+            const unsigned long long valid_m = cand_m & __builtin_amdgcn_fcmpf(alpha0, P.alpha_eps, kFcmpOge);
+            if (valid_m == 0) continue;
+            float G, alpha;     // G = valid ? G0 : 0, alpha = valid ? alpha0 : 0
+            select2_or_zero(valid_m, G0, alpha0, G, alpha);
             // The per-pixel terms follow one fixed sequence of fused multiply-adds (the colour still
             // behind, T c - rr, cancels heavily, so a different rounding would already move a term by
             // ~1e-4): only the order of the sums over pixels differs from a sequential evaluation.
@@ -443,7 +472,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float g7 = w * dr1;
             const float g8 = w * dr2;
             // the wave totals land in different lanes: one LDS atomic instruction adds them all
-            const float total = wave_reduce10(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9, hi8, hi4);
+            const float total = wave_reduce10(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9);
             if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }
