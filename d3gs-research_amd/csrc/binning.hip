@@ -86,6 +86,150 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int32_t* __restrict_
 }
 
 // ---------------------------------------------------------------------------
+// Gather + inclusive scan in one launch: out[j] = sum_{i <= j} src[index[i]].
+// Chunks of 2048 are claimed from an atomic ticket, so a workgroup only waits on
+// chunks that started before it; each publishes its sum (aggregate), walks back
+// over its predecessors' status words until one that already knows its inclusive
+// prefix, and publishes its own.  Status word: flag in bits 62-63, value below.
+// Polling is bounded: past the limit the workgroup raises the error word and goes
+// on, and the grand total is reported as -1.
+// ---------------------------------------------------------------------------
+constexpr unsigned long long kScanAggregate = 1ull << 62, kScanPrefix = 2ull << 62, kScanValueMask = (1ull << 62) - 1ull;
+constexpr int kScanSpinLimit = 1 << 22;
+constexpr int kScanLookRounds = 4;
+
+// few items per thread: the gather is a dependent random read, and it is the number of wavefronts in flight
+// that hides its latency
+constexpr int kGatherScanItems = 2;
+constexpr int kGatherScanBlock = 1024;     // large workgroups: every chunk costs one (serialised) ticket atomic
+constexpr int kGatherScanWaves = kGatherScanBlock / 64;
+constexpr int kGatherScanChunk = kGatherScanBlock * kGatherScanItems;
+
+struct ScanWorkspace {
+    unsigned long long* status;  // [chunks]
+    uint32_t* ticket;            // [1]
+    uint32_t* error;             // [1]
+};
+
+__device__ __forceinline__ long long wave_sum_i64(long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(const int32_t* __restrict__ src, int src_n,
+                                                                       const int32_t* __restrict__ index, int n,
+                                                                       int32_t* __restrict__ out, ScanWorkspace ws,
+                                                                       int64_t* __restrict__ total_out) {
+    __shared__ int s_wave[kGatherScanWaves];
+    __shared__ unsigned s_chunk;
+    __shared__ long long s_prefix;
+    if (threadIdx.x == 0) s_chunk = atomicAdd(ws.ticket, 1u);
+    __syncthreads();
+    const int chunk = (int)s_chunk;
+    if (chunk >= (int)gridDim.x) return;   // the ticket counter was not zero: nothing sane to do
+    const int base = chunk * kGatherScanChunk + threadIdx.x * kGatherScanItems;
+    int v[kGatherScanItems];
+    int s = 0;
+#pragma unroll
+    for (int k = 0; k < kGatherScanItems; ++k) {
+        const int j = base + k;
+        int x = 0;
+        if (j < n) {
+            const int i = index ? index[j] : j;
+            if ((unsigned)i < (unsigned)src_n) x = src[i];   // a corrupt index must not become a wild read
+        }
+        v[k] = x;
+        s += x;
+    }
+    // exclusive scan of s over the workgroup
+    const int wlane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int incl = wave_incl_scan(s, wlane);
+    if (wlane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    int wave_base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kGatherScanWaves; ++w) {
+        const int c = s_wave[w];
+        if (w < wave) wave_base += c;
+        total += c;
+    }
+    int ex = wave_base + incl - s;
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        if (lane == 0)
+            __hip_atomic_store(ws.status + chunk, (chunk == 0 ? kScanPrefix : kScanAggregate) | (unsigned long long)total,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        long long prefix = 0;
+        if (chunk > 0) {
+            // lane l polls chunks pos - l - 64 r for r = 0 .. 3 with independent loads: 256 predecessors per
+            // round trip to memory, taken 64 at a time from the nearest on
+            int pos = chunk - 1;
+            int spins = 0;
+            bool walking = true;
+            while (walking) {
+                unsigned long long w[kScanLookRounds];
+#pragma unroll
+                for (int r = 0; r < kScanLookRounds; ++r) {
+                    const int t = pos - lane - 64 * r;
+                    w[r] = t >= 0 ? __hip_atomic_load(ws.status + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                  : kScanPrefix;   // before the first chunk: an empty prefix
+                }
+                int taken = 0;
+#pragma unroll
+                for (int r = 0; r < kScanLookRounds; ++r) {
+                    if (!walking || taken != 64 * r) continue;    // an earlier group stopped short
+                    const unsigned long long flag = w[r] & ~kScanValueMask;
+                    const unsigned long long not_ready = __ballot(flag == 0ull), is_prefix = __ballot(flag == kScanPrefix);
+                    const int first_nr = not_ready ? __builtin_ctzll(not_ready) : 64;
+                    const int first_p = is_prefix ? __builtin_ctzll(is_prefix) : 64;
+                    if (first_p < first_nr) {          // a chunk that knows its inclusive prefix: done
+                        prefix += wave_sum_i64(lane <= first_p ? (long long)(w[r] & kScanValueMask) : 0ll);
+                        walking = false;
+                    } else {                           // a run of aggregates (possibly empty): take them
+                        prefix += wave_sum_i64(lane < first_nr ? (long long)(w[r] & kScanValueMask) : 0ll);
+                        taken += first_nr;
+                    }
+                }
+                if (!walking) break;
+                pos -= taken;
+                if (taken > 0) {
+                    spins = 0;
+                } else if (++spins > kScanSpinLimit) {
+                    if (lane == 0) atomicOr(ws.error, 1u);
+                    __threadfence();
+                    walking = false;
+                } else {
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+        }
+        if (lane == 0) {
+            if (chunk > 0)
+                __hip_atomic_store(ws.status + chunk, kScanPrefix | ((unsigned long long)(prefix + total) & kScanValueMask),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_prefix = prefix;
+            if (chunk == (int)gridDim.x - 1 && total_out) {
+                const uint32_t err = __hip_atomic_load(ws.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *total_out = err ? -1ll : prefix + total;
+            }
+        }
+    }
+    __syncthreads();
+    ex += (int)s_prefix;
+#pragma unroll
+    for (int k = 0; k < kGatherScanItems; ++k) {
+        ex += v[k];
+        if (base + k < n) out[base + k] = ex;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void scan_clear_kernel(uint32_t* __restrict__ words, int count) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < count) words[i] = 0u;
+}
+
+// ---------------------------------------------------------------------------
 // Key expansion: one thread per gaussian, emits its (tile << 32 | depth bits)
 // keys at the offset the scan assigned (render.py:745-840).
 // ---------------------------------------------------------------------------
@@ -281,6 +425,48 @@ using namespace d3gs;
 extern "C" int d3gs_scan_workspace_bytes(int32_t n, size_t* bytes_out_host) {
     if (n < 0 || !bytes_out_host) { set_error("d3gs_scan_workspace_bytes: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
     *bytes_out_host = scan_ws_bytes(n);
+    return D3GS_OK;
+}
+
+static inline int gather_scan_chunks(long long n) { return (int)((n + kGatherScanChunk - 1) / kGatherScanChunk); }
+static size_t scan_gathered_ws_bytes(long long n) {
+    return align_up((size_t)std::max(1, gather_scan_chunks(n)) * sizeof(unsigned long long) + 2 * sizeof(uint32_t), 256);
+}
+
+extern "C" int d3gs_scan_gathered_workspace_bytes(int32_t n, size_t* bytes_out_host) {
+    if (n < 0 || !bytes_out_host) { set_error("d3gs_scan_gathered_workspace_bytes: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+    *bytes_out_host = scan_gathered_ws_bytes(n);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* out,
+                                  void* workspace, size_t workspace_bytes, int32_t workspace_is_zero, int64_t* total_dev,
+                                  d3gs_stream_t stream) {
+    if (n < 0 || src_n < 0 || !total_dev) { set_error("d3gs_scan_gathered: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
+    hipStream_t s = (hipStream_t)stream;
+    if (n == 0) {   // total = 0
+        hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, (int32_t*)nullptr, 0, total_dev);
+    } else {
+        if (!src || !out || !workspace) { set_error("d3gs_scan_gathered: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
+        if (workspace_bytes < scan_gathered_ws_bytes(n)) {
+            set_error("d3gs_scan_gathered: workspace %zu < required %zu", workspace_bytes, scan_gathered_ws_bytes(n));
+            return D3GS_ERR_INVALID_ARGUMENT;
+        }
+        const int nchunks = gather_scan_chunks(n);
+        ScanWorkspace ws;
+        ws.status = (unsigned long long*)workspace;
+        ws.ticket = (uint32_t*)(ws.status + nchunks);
+        ws.error = ws.ticket + 1;
+        if (!workspace_is_zero) {
+            const int words = 2 * nchunks + 2;
+            hipLaunchKernelGGL(scan_clear_kernel, dim3((words + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
+                               (uint32_t*)workspace, words);
+        }
+        hipLaunchKernelGGL(scan_gather_lookback_kernel, dim3(nchunks), dim3(kGatherScanBlock), 0, s, src, (int)src_n, index, (int)n,
+                           out, ws, total_dev);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_scan_gathered: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 

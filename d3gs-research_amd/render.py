@@ -373,9 +373,12 @@ class GaussianSplatOp:
         tile_bits = L.d3gs_higher_msb(num_tiles)
         spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
         align = lambda v: (v + 255) // 256 * 256
+        scan_ws_bytes = C.c_size_t(0)
+        _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(scan_ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
         sizes = [align(_sort_ws_bytes(n, 0, 32)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
-                 align(num_tiles * 8)]
+                 align(num_tiles * 8), align(scan_ws_bytes.value)]
         zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
+        zero_scan_ws = zero_pool[sum(sizes[:3]):]
         zero_ws_n = zero_pool[:sizes[0]]
         zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
         zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
@@ -389,15 +392,12 @@ class GaussianSplatOp:
                                                       values_are_indices=True, zero_ws=zero_ws_n)
 
         with self._stage("scan"):
+            # tile counts gathered into depth order and scanned in one launch
             counts_ordered = torch.empty(n, dtype=i32, device=dev)
-            _capi.check(L.d3gs_gather_i32(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
-                                          _capi.ptr(counts_ordered), s), "d3gs_gather_i32")
-            ws_bytes = C.c_size_t(0)
-            _capi.check(L.d3gs_scan_workspace_bytes(n, C.byref(ws_bytes)), "d3gs_scan_workspace_bytes")
-            scan_ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
             total = torch.empty(1, dtype=torch.int64, device=dev)
-            _capi.check(L.d3gs_scan_tiles(_capi.ptr(counts_ordered), n, _capi.ptr(scan_ws), ws_bytes.value,
-                                          _capi.ptr(total), s), "d3gs_scan_tiles")
+            _capi.check(L.d3gs_scan_gathered(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
+                                             _capi.ptr(counts_ordered), _capi.ptr(zero_scan_ws), zero_scan_ws.numel(), 1,
+                                             _capi.ptr(total), s), "d3gs_scan_gathered")
             # the count travels to pinned host memory behind the scan; the host looks at it only after
             # the rest of the forward pass has been enqueued
             if self._count_host is None:
@@ -483,6 +483,8 @@ class GaussianSplatOp:
             ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
         count_ready.synchronize()
         num_rendered = int(self._count_host[0])
+        if num_rendered < 0:
+            raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
         self.last_num_rendered = num_rendered
         self._pair_capacity = num_rendered + num_rendered // 4 + 4096
         if num_rendered == 0:

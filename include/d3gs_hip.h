@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 13
+#define D3GS_ABI_VERSION 14
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -121,6 +121,16 @@ int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const float* color_sh
 int d3gs_scan_workspace_bytes(int32_t n, size_t* bytes_out_host);
 int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t workspace_bytes, int64_t* total_dev,
                     d3gs_stream_t stream);
+
+/* K2 over a permutation, in one launch: out[j] = sum_{i <= j} src[index[i]] (index NULL: the identity), the same
+ * `cumsum_` (render.py:694-695) taken in the order K3 emits the pairs; the grand total goes to *total_dev
+ * (device int64; -1 if the kernel's bounded wait on an earlier chunk ran out).  An index outside [0, src_n)
+ * counts as 0.  The workspace (size from d3gs_scan_gathered_workspace_bytes) must be zero on entry:
+ * workspace_is_zero != 0 says the caller has cleared it, otherwise a fill kernel runs first. */
+int d3gs_scan_gathered_workspace_bytes(int32_t n, size_t* bytes_out_host);
+int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* out,
+                       void* workspace, size_t workspace_bytes, int32_t workspace_is_zero, int64_t* total_dev,
+                       d3gs_stream_t stream);
 
 /* K3 — replaces kernel_1d("prepare_sort_data_...") at render.py:739-840.
  * Without gaussian_order (NULL) this is the reference's call: offsets = the inclusive

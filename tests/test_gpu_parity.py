@@ -247,6 +247,38 @@ def test_scan_c_abi(n):
     assert int(total.item()) == int(x.sum())
 
 
+@pytest.mark.parametrize("n,permuted,dirty", [(0, False, False), (1, True, False), (63, False, True), (2048, True, True),
+                                              (2049, True, False), (1_000_003, True, True), (3_000_001, False, False)])
+def test_scan_gathered_c_abi(n, permuted, dirty):
+    """One-launch gather + scan against numpy's cumsum over the permuted counts; `dirty` hands over a
+    workspace that is not zero (the library clears it), and a corrupt index entry counts as zero."""
+    import torch
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    print(f"scan_gathered n={n} permuted={permuted} dirty={dirty}", flush=True)
+    rng = np.random.default_rng(n + 7)
+    x = rng.integers(0, 50, size=max(n, 1), dtype=np.int32)[:n]
+    perm = rng.permutation(n).astype(np.int32) if permuted else None
+    want_src = x[perm].astype(np.int64) if permuted else x.astype(np.int64)
+    if permuted and n > 10:
+        perm[5], perm[9] = -3, n + 100      # outside [0, n): counted as zero
+        want_src[5] = want_src[9] = 0
+    src = torch.from_numpy(x).cuda() if n else torch.empty(0, dtype=torch.int32, device="cuda")
+    idx = torch.from_numpy(perm).cuda() if permuted else None
+    out = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    nbytes = C.c_size_t(0)
+    _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(nbytes)), "ws")
+    ws = (torch.full if dirty else (lambda size, _v, **kw: torch.zeros(size, **kw)))((nbytes.value,), 0xAB, dtype=torch.uint8,
+                                                                                    device="cuda")
+    total = torch.full((1,), -7, dtype=torch.int64, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(2):      # the second call finds the first one's status words in the workspace
+        _capi.check(L.d3gs_scan_gathered(_capi.ptr(src), n, _capi.ptr(idx), n, _capi.ptr(out), _capi.ptr(ws), nbytes.value,
+                                         0, _capi.ptr(total), stream), "scan_gathered")
+        assert np.array_equal(out.cpu().numpy(), np.cumsum(want_src).astype(np.int32))
+        assert int(total.item()) == int(want_src.sum())
+
+
 @pytest.mark.parametrize("m,cap,begin,end,implicit", [(1000, 1000, 0, 13, False), (70001, 90000, 0, 32, True),
                                                       (0, 5000, 0, 13, False), (3_000_000, 3_100_000, 2, 15, True),
                                                       (9000, 5000, 0, 32, False)])
