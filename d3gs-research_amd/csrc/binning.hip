@@ -87,8 +87,7 @@ __global__ __launch_bounds__(kBlock) void scan_apply_kernel(int32_t* __restrict_
 
 // ---------------------------------------------------------------------------
 // Gather + inclusive scan in one launch: out[j] = sum_{i <= j} src[index[i]].
-// Chunks of 2048 are claimed from an atomic ticket, so a workgroup only waits on
-// chunks that started before it; each publishes its sum (aggregate), walks back
+// Each workgroup takes the chunk of 2048 with its own id, publishes its sum (aggregate), walks back
 // over its predecessors' status words until one that already knows its inclusive
 // prefix, and publishes its own.  Status word: flag in bits 62-63, value below.
 // Polling is bounded: past the limit the workgroup raises the error word and goes
@@ -101,13 +100,12 @@ constexpr int kScanLookRounds = 4;
 // few items per thread: the gather is a dependent random read, and it is the number of wavefronts in flight
 // that hides its latency
 constexpr int kGatherScanItems = 2;
-constexpr int kGatherScanBlock = 1024;     // large workgroups: every chunk costs one (serialised) ticket atomic
+constexpr int kGatherScanBlock = 1024;    // 2048-element chunks measured faster than 1024-element ones
 constexpr int kGatherScanWaves = kGatherScanBlock / 64;
 constexpr int kGatherScanChunk = kGatherScanBlock * kGatherScanItems;
 
 struct ScanWorkspace {
     unsigned long long* status;  // [chunks]
-    uint32_t* ticket;            // [1]
     uint32_t* error;             // [1]
 };
 
@@ -122,12 +120,12 @@ __global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(
                                                                        int32_t* __restrict__ out, ScanWorkspace ws,
                                                                        int64_t* __restrict__ total_out) {
     __shared__ int s_wave[kGatherScanWaves];
-    __shared__ unsigned s_chunk;
     __shared__ long long s_prefix;
-    if (threadIdx.x == 0) s_chunk = atomicAdd(ws.ticket, 1u);
-    __syncthreads();
-    const int chunk = (int)s_chunk;
-    if (chunk >= (int)gridDim.x) return;   // the ticket counter was not zero: nothing sane to do
+    // Chunk = workgroup id.  Workgroups of a 1-D grid are dispatched in id order (per XCD, which gets every
+    // 8th id), so every chunk this one waits on has been dispatched before it and finishes without help; an
+    // atomic ticket would put one chip-wide same-address atomic per workgroup (about 15 ns each, one after the
+    // other) in front of the launch.
+    const int chunk = blockIdx.x;
     const int base = chunk * kGatherScanChunk + threadIdx.x * kGatherScanItems;
     int v[kGatherScanItems];
     int s = 0;
@@ -455,8 +453,7 @@ extern "C" int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32
         const int nchunks = gather_scan_chunks(n);
         ScanWorkspace ws;
         ws.status = (unsigned long long*)workspace;
-        ws.ticket = (uint32_t*)(ws.status + nchunks);
-        ws.error = ws.ticket + 1;
+        ws.error = (uint32_t*)(ws.status + nchunks);
         if (!workspace_is_zero) {
             const int words = 2 * nchunks + 2;
             hipLaunchKernelGGL(scan_clear_kernel, dim3((words + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
