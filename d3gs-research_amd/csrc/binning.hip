@@ -358,47 +358,85 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
     if (i == m - 1) ranges[2 * t + 1] = (int32_t)m;
 }
 
-// Tile ids ordered by descending list length (counting sort over 256 length buckets, one
-// workgroup).  Order inside a bucket is arbitrary: the result only steers scheduling.
-__global__ __launch_bounds__(1024) void tile_order_kernel(const int32_t* __restrict__ work, int num_tiles,
-                                                          int32_t* __restrict__ order) {
-    __shared__ int s_max;
-    __shared__ int s_bin[256];
-    __shared__ int s_wave[4];
-    auto amount = [&](int t) { return work[2 * t + 1] - work[2 * t]; };
-    if (threadIdx.x == 0) s_max = 0;
-    if (threadIdx.x < 256) s_bin[threadIdx.x] = 0;
-    __syncthreads();
-    int mx = 0;
-    for (int t = threadIdx.x; t < num_tiles; t += 1024) mx = max(mx, amount(t));
-    atomicMax(&s_max, mx);
-    __syncthreads();
-    const long long denom = (long long)s_max + 1;
-    for (int t = threadIdx.x; t < num_tiles; t += 1024)
-        atomicAdd(&s_bin[255 - (int)((long long)max(amount(t), 0) * 256 / denom)], 1);
-    __syncthreads();
-    // exclusive scan of the 256 bucket counts by the first four wavefronts
-    int c = 0, incl = 0;
-    if (threadIdx.x < 256) {
-        c = s_bin[threadIdx.x];
-        incl = c;
-        const int lane = threadIdx.x & 63;
+// Tile ids ordered by descending list length (counting sort over 1024 length buckets, one workgroup; each
+// thread keeps its tiles' lengths in registers and takes its place inside a bucket from the counting atomic's
+// return value, so the lists are read once and every tile costs one LDS atomic).  Order inside a bucket is
+// arbitrary: the result only steers scheduling.
+constexpr int kOrderThreads = 1024, kOrderBuckets = 1024, kOrderPerThread = 8;
+
+__device__ __forceinline__ int order_wave_max(int v) {
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int v = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += v;
+    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+__global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t* __restrict__ work, int num_tiles,
+                                                                   int32_t* __restrict__ order) {
+    __shared__ int s_bin[kOrderBuckets];
+    __shared__ int s_wave[kOrderThreads / 64];
+    __shared__ int s_max[kOrderThreads / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int2* ranges = reinterpret_cast<const int2*>(work);
+    auto amount_of = [&](int t) { const int2 r = ranges[t]; return max(r.y - r.x, 0); };
+    auto bucket_of = [&](int a, float scale) { return kOrderBuckets - 1 - min(kOrderBuckets - 1, (int)((float)a * scale)); };
+    const bool in_registers = num_tiles <= kOrderThreads * kOrderPerThread;   // else the lists are read three times
+
+    int amount[kOrderPerThread];
+    int mx = 0;
+    if (in_registers) {
+#pragma unroll
+        for (int k = 0; k < kOrderPerThread; ++k) {
+            const int t = k * kOrderThreads + tid;
+            amount[k] = t < num_tiles ? amount_of(t) : 0;
+            mx = max(mx, amount[k]);
         }
-        if (lane == 63) s_wave[threadIdx.x >> 6] = incl;
+    } else {
+        for (int t = tid; t < num_tiles; t += kOrderThreads) mx = max(mx, amount_of(t));
+    }
+    s_bin[tid] = 0;
+    mx = order_wave_max(mx);
+    if (lane == 0) s_max[wave] = mx;
+    __syncthreads();
+    mx = 0;
+#pragma unroll
+    for (int w = 0; w < kOrderThreads / 64; ++w) mx = max(mx, s_max[w]);
+    const float scale = (float)kOrderBuckets / ((float)mx + 1.0f);
+
+    int bucket[kOrderPerThread], rank[kOrderPerThread];
+    if (in_registers) {
+#pragma unroll
+        for (int k = 0; k < kOrderPerThread; ++k) {
+            bucket[k] = bucket_of(amount[k], scale);
+            rank[k] = (k * kOrderThreads + tid < num_tiles) ? atomicAdd(&s_bin[bucket[k]], 1) : 0;
+        }
+    } else {
+        for (int t = tid; t < num_tiles; t += kOrderThreads) atomicAdd(&s_bin[bucket_of(amount_of(t), scale)], 1);
     }
     __syncthreads();
-    if (threadIdx.x < 256) {
-        int base = 0;
-        for (int w = 0; w < (int)(threadIdx.x >> 6); ++w) base += s_wave[w];
-        s_bin[threadIdx.x] = base + incl - c;
+    // exclusive scan of the bucket counts, one bucket per thread
+    const int c = s_bin[tid];
+    int incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int v = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += v;
     }
+    if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
-    for (int t = threadIdx.x; t < num_tiles; t += 1024)
-        order[atomicAdd(&s_bin[255 - (int)((long long)max(amount(t), 0) * 256 / denom)], 1)] = t;
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    s_bin[tid] = base + incl - c;
+    __syncthreads();
+    if (in_registers) {
+#pragma unroll
+        for (int k = 0; k < kOrderPerThread; ++k) {
+            const int t = k * kOrderThreads + tid;
+            if (t < num_tiles) order[s_bin[bucket[k]] + rank[k]] = t;
+        }
+    } else {
+        for (int t = tid; t < num_tiles; t += kOrderThreads)
+            order[atomicAdd(&s_bin[bucket_of(amount_of(t), scale)], 1)] = t;
+    }
 }
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -550,7 +588,7 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
                            (hipStream_t)stream, keys_sorted, (long long)m, (const long long*)m_device, workload_ranges,
                            (int)num_tiles);
     if (tile_order && num_tiles > 0)
-        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, workload_ranges,
+        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(kOrderThreads), 0, (hipStream_t)stream, workload_ranges,
                            (int)num_tiles, tile_order);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
