@@ -337,25 +337,45 @@ __device__ __forceinline__ uint32_t key_tile(Key k) {
     else return (uint32_t)k;
 }
 
+constexpr int kRangeItems = 4;   // consecutive keys per thread (one 16-byte load of 32-bit keys)
+
 template <typename Key>
 __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restrict__ keys, long long m,
                                                               const long long* __restrict__ m_device,
                                                               int32_t* __restrict__ ranges, int num_tiles) {
     if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the key buffer
-    const long long i = (long long)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= m) return;
-    const uint32_t t = key_tile<Key>(keys[i]);
-    if (t >= (uint32_t)num_tiles) return;  // corrupt key: never write outside the table
-    if (i == 0) {
-        ranges[2 * t] = 0;
-    } else {
-        const uint32_t tp = key_tile<Key>(keys[i - 1]);
-        if (t != tp) {
-            if (tp < (uint32_t)num_tiles) ranges[2 * tp + 1] = (int32_t)i;
-            ranges[2 * t] = (int32_t)i;
+    const long long i0 = ((long long)blockIdx.x * kBlock + threadIdx.x) * kRangeItems;
+    if (i0 >= m) return;
+    Key k[kRangeItems];
+    if (i0 + kRangeItems <= m) {
+        if constexpr (sizeof(Key) == 4) {
+            const uint4 v = *reinterpret_cast<const uint4*>(keys + i0);   // i0 is a multiple of 4
+            k[0] = v.x; k[1] = v.y; k[2] = v.z; k[3] = v.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < kRangeItems; ++j) k[j] = keys[i0 + j];
         }
+    } else {
+#pragma unroll
+        for (int j = 0; j < kRangeItems; ++j) k[j] = i0 + j < m ? keys[i0 + j] : (Key)0;
     }
-    if (i == m - 1) ranges[2 * t + 1] = (int32_t)m;
+    uint32_t tp = i0 > 0 ? key_tile<Key>(keys[i0 - 1]) : 0u;
+#pragma unroll
+    for (int j = 0; j < kRangeItems; ++j) {
+        const long long i = i0 + j;
+        if (i >= m) break;
+        const uint32_t t = key_tile<Key>(k[j]);
+        if (t < (uint32_t)num_tiles) {   // a corrupt key never writes outside the table
+            if (i == 0) {
+                ranges[2 * t] = 0;
+            } else if (t != tp) {
+                if (tp < (uint32_t)num_tiles) ranges[2 * tp + 1] = (int32_t)i;
+                ranges[2 * t] = (int32_t)i;
+            }
+            if (i == m - 1) ranges[2 * t + 1] = (int32_t)m;
+        }
+        tp = t;
+    }
 }
 
 // Tile ids ordered by descending list length (counting sort over 1024 length buckets, one workgroup; each
@@ -584,7 +604,8 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     if (m > 0)
-        hipLaunchKernelGGL(tile_ranges_kernel<Key>, dim3((unsigned)((m + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+        hipLaunchKernelGGL(tile_ranges_kernel<Key>,
+                           dim3((unsigned)((m + (long long)kBlock * kRangeItems - 1) / ((long long)kBlock * kRangeItems))), dim3(kBlock), 0,
                            (hipStream_t)stream, keys_sorted, (long long)m, (const long long*)m_device, workload_ranges,
                            (int)num_tiles);
     if (tile_order && num_tiles > 0)
