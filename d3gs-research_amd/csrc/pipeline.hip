@@ -1,0 +1,51 @@
+// Composite entry point: the whole binning of one view (depth order, offsets, key expansion, pair sort,
+// tile ranges and launch order) enqueued by one call.  Every step is one of the library's own entry points,
+// in the order a caller would issue them; doing it here takes the caller's per-launch cost (argument
+// marshalling in an interpreter, allocation between launches) off the stream's critical path, where the
+// kernels of this phase are short enough for that cost to leave the GPU idle between them.
+#include <hip/hip_runtime.h>
+
+#include "device_math.h"
+
+using namespace d3gs;
+
+extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                              const float* depths, const int32_t* tiles_touched, const uint64_t* tile_masks,
+                              uint32_t* depth_keys_a, uint32_t* depth_keys_b, int32_t* order_a, int32_t* order_b,
+                              void* depth_sort_ws, size_t depth_sort_ws_bytes, int32_t* offsets, void* scan_ws,
+                              size_t scan_ws_bytes, int64_t* total_dev, int64_t* total_host, int64_t capacity,
+                              uint32_t* tile_keys_a, uint32_t* tile_keys_b, int32_t* idx_a, int32_t* idx_b,
+                              void* pair_sort_ws, size_t pair_sort_ws_bytes, int32_t* workload_ranges,
+                              int32_t* tile_order, int32_t workspaces_are_zero, int32_t* order_in_b,
+                              int32_t* pairs_in_b, d3gs_stream_t stream) {
+    if (!p || !order_in_b || !pairs_in_b || !total_dev || capacity < 0) {
+        set_error("d3gs_bin_pairs: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const int32_t n = p->n;
+    const int32_t num_tiles = p->tiles_x * p->tiles_y;
+    int rc = d3gs_sort_pairs_u32(depth_keys_a, depth_keys_b, order_a, order_b, depth_sort_ws, depth_sort_ws_bytes, n,
+                                 nullptr, /*values_are_indices=*/1, workspaces_are_zero, 0, 32, order_in_b, stream);
+    if (rc) return rc;
+    const uint32_t* depth_keys_sorted = *order_in_b ? depth_keys_b : depth_keys_a;
+    const int32_t* order = *order_in_b ? order_b : order_a;
+    rc = d3gs_scan_gathered(tiles_touched, n, order, n, offsets, scan_ws, scan_ws_bytes, workspaces_are_zero, total_dev,
+                            stream);
+    if (rc) return rc;
+    if (total_host) {   // the pair count travels to the host behind the scan; nothing here waits for it
+        hipError_t e = hipMemcpyAsync(total_host, total_dev, sizeof(int64_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+        if (e != hipSuccess) {
+            set_error("d3gs_bin_pairs: copy of the pair count failed: %s", hipGetErrorString(e));
+            return D3GS_ERR_LAUNCH;
+        }
+    }
+    rc = d3gs_make_keys(p, radii, uvs, conic_opacity, depths, offsets, order, depth_keys_sorted, tile_masks, nullptr,
+                        tile_keys_a, idx_a, capacity, stream);
+    if (rc) return rc;
+    rc = d3gs_sort_pairs_u32(tile_keys_a, tile_keys_b, idx_a, idx_b, pair_sort_ws, pair_sort_ws_bytes, capacity,
+                             total_dev, /*values_are_indices=*/0, workspaces_are_zero, 0, d3gs_higher_msb((uint32_t)num_tiles),
+                             pairs_in_b, stream);
+    if (rc) return rc;
+    return d3gs_tile_ranges_u32(*pairs_in_b ? tile_keys_b : tile_keys_a, capacity, total_dev, workload_ranges, num_tiles,
+                                tile_order, stream);
+}

@@ -150,6 +150,8 @@ class GaussianSplatOp:
         # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
         self.overlap_sh_colors = True
         # size the pair buffers from the previous view's count instead of waiting for this view's
+        # the speculative binning of a view (depth order .. tile ranges) goes out as one library call
+        self.fused_binning = True
         self.speculative_pair_buffers = True
         self._pair_capacity = 0
         self._count_host: torch.Tensor | None = None
@@ -383,28 +385,61 @@ class GaussianSplatOp:
         zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
         zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
 
-        # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
-        # digits only depend on the gaussian, so the same stable order comes from sorting the N
-        # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
-        # tile digits only: 2 passes over M pairs instead of 6.
-        with self._stage("depth_order"):
-            depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, 32,
-                                                      values_are_indices=True, zero_ws=zero_ws_n)
-
-        with self._stage("scan"):
-            # tile counts gathered into depth order and scanned in one launch
-            counts_ordered = torch.empty(n, dtype=i32, device=dev)
+        # With buffers sized from the previous view and no stage timers, the whole binning is one call into the
+        # library (d3gs_bin_pairs): the launches of this phase are short, and issuing them one by one from
+        # Python leaves the GPU idle between them.
+        fused = bool(self.fused_binning and spec_capacity > 0 and self.stage_events is None)
+        fused_result = None
+        if self._count_host is None:
+            self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+        if fused:
+            cap = spec_capacity
+            up = lambda v: (v + 63) // 64 * 64          # 256-byte aligned slices of one int32 allocation
+            o_keys_b, o_ord_a, o_ord_b, o_offs = 0, up(n), 2 * up(n), 3 * up(n)
+            o_tk_a = 4 * up(n)
+            o_tk_b, o_ix_a, o_ix_b = o_tk_a + up(cap), o_tk_a + 2 * up(cap), o_tk_a + 3 * up(cap)
+            o_order = o_tk_a + 4 * up(cap)
+            pool = torch.empty(o_order + up(num_tiles), dtype=i32, device=dev)
+            base = pool.data_ptr()
+            at = lambda off: C.c_void_p(base + 4 * off)
             total = torch.empty(1, dtype=torch.int64, device=dev)
-            _capi.check(L.d3gs_scan_gathered(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
-                                             _capi.ptr(counts_ordered), _capi.ptr(zero_scan_ws), zero_scan_ws.numel(), 1,
-                                             _capi.ptr(total), s), "d3gs_scan_gathered")
-            # the count travels to pinned host memory behind the scan; the host looks at it only after
-            # the rest of the forward pass has been enqueued
-            if self._count_host is None:
-                self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
-            self._count_host.copy_(total, non_blocking=True)
+            order_in_b, pairs_in_b = C.c_int(0), C.c_int(0)
+            _capi.check(L.d3gs_bin_pairs(
+                C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(depths),
+                _capi.ptr(tiles_touched), _capi.ptr(tile_masks), _capi.ptr(depth_keys), at(o_keys_b), at(o_ord_a),
+                at(o_ord_b), _capi.ptr(zero_ws_n), zero_ws_n.numel(), at(o_offs), _capi.ptr(zero_scan_ws),
+                zero_scan_ws.numel(), _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), cap, at(o_tk_a),
+                at(o_tk_b), at(o_ix_a), at(o_ix_b), _capi.ptr(zero_ws_m), zero_ws_m.numel(), _capi.ptr(zero_ranges),
+                at(o_order), 1, C.byref(order_in_b), C.byref(pairs_in_b), s), "d3gs_bin_pairs")
             count_ready = torch.cuda.Event()
             count_ready.record()
+            # what a second, exactly sized binning of this view would start from
+            depth_keys_sorted = pool[o_keys_b:o_keys_b + n] if order_in_b.value else depth_keys
+            gaussian_order = pool[o_ord_b:o_ord_b + n] if order_in_b.value else pool[o_ord_a:o_ord_a + n]
+            counts_ordered = pool[o_offs:o_offs + n]
+            o_tk, o_ix = (o_tk_b, o_ix_b) if pairs_in_b.value else (o_tk_a, o_ix_a)
+            fused_result = (pool[o_tk:o_tk + cap], pool[o_ix:o_ix + cap], pool[o_order:o_order + num_tiles])
+        else:
+            # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
+            # digits only depend on the gaussian, so the same stable order comes from sorting the N
+            # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
+            # tile digits only: 2 passes over M pairs instead of 6.
+            with self._stage("depth_order"):
+                depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, 32,
+                                                          values_are_indices=True, zero_ws=zero_ws_n)
+
+            with self._stage("scan"):
+                # tile counts gathered into depth order and scanned in one launch
+                counts_ordered = torch.empty(n, dtype=i32, device=dev)
+                total = torch.empty(1, dtype=torch.int64, device=dev)
+                _capi.check(L.d3gs_scan_gathered(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
+                                                 _capi.ptr(counts_ordered), _capi.ptr(zero_scan_ws), zero_scan_ws.numel(), 1,
+                                                 _capi.ptr(total), s), "d3gs_scan_gathered")
+                # the count travels to pinned host memory behind the scan; the host looks at it only after
+                # the rest of the forward pass has been enqueued
+                self._count_host.copy_(total, non_blocking=True)
+                count_ready = torch.cuda.Event()
+                count_ready.record()
 
         final_T = torch.empty((1, height, width), dtype=f32, device=dev)
         n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
@@ -440,27 +475,32 @@ class GaussianSplatOp:
         def _bin_and_blend(capacity: int, count_on_device: bool):
             """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
             read the pair count from `total` on the device and nothing here waits for the host."""
-            m_dev = _capi.ptr(total) if count_on_device else None
-            # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
-            with self._stage("make_keys"):
-                tile_keys = torch.empty(capacity, dtype=i32, device=dev)
-                gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
-                _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                                             _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                             _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
-                                             _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
-                            "d3gs_make_keys")
-            with self._stage("sort"):
-                tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0, tile_bits, m_dev,
-                                                              zero_ws=zero_ws_m if count_on_device else None)
-            with self._stage("tile_ranges"):
-                # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
-                workload_ranges = zero_ranges if not pooled_ranges_used[0] else torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+            if fused_result is not None and count_on_device:
+                tile_keys_sorted, gaussian_idx_sorted, tile_order = fused_result
+                workload_ranges = zero_ranges
                 pooled_ranges_used[0] = True
-                tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
-                _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
-                                                   _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
-                            "d3gs_tile_ranges_u32")
+            else:
+                m_dev = _capi.ptr(total) if count_on_device else None
+                # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
+                with self._stage("make_keys"):
+                    tile_keys = torch.empty(capacity, dtype=i32, device=dev)
+                    gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
+                    _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                                                 _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
+                                                 _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
+                                                 _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
+                                "d3gs_make_keys")
+                with self._stage("sort"):
+                    tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0, tile_bits, m_dev,
+                                                                  zero_ws=zero_ws_m if count_on_device else None)
+                with self._stage("tile_ranges"):
+                    # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
+                    workload_ranges = zero_ranges if not pooled_ranges_used[0] else torch.zeros((num_tiles, 2), dtype=i32, device=dev)
+                    pooled_ranges_used[0] = True
+                    tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
+                    _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
+                                                       _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
+                                "d3gs_tile_ranges_u32")
             ctx = GaussianSplatOpContext(
                 conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 14
+#define D3GS_ABI_VERSION 15
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -194,6 +194,27 @@ int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* workload_r
 /* the same over 32-bit tile keys (see d3gs_make_keys); m_device as in d3gs_sort_pairs_u32 */
 int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
                          int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream);
+
+/* The binning of one view from K1's outputs to the tile ranges, enqueued by one call (no counterpart in the
+ * reference, whose host issues render.py:694-939 launch by launch): d3gs_sort_pairs_u32 of the N depth keys
+ * (depth_keys_a = K1's depth_sort_keys; values are the gaussian indices), d3gs_scan_gathered of tiles_touched in
+ * that order into offsets [N], d3gs_make_keys into tile_keys_a / idx_a [capacity], d3gs_sort_pairs_u32 on the
+ * tile bits with the pair count read from *total_dev, d3gs_tile_ranges_u32 (+ tile_order, may be NULL).
+ * Results: *order_in_b / *pairs_in_b say which of the a / b buffers hold the depth order and the sorted pairs;
+ * *total_dev the pair count M (the kernels touch min(M, capacity) pairs: a caller that sized capacity from a
+ * guess compares M with it afterwards and bins again when M is larger); total_host, when not NULL, is a pinned
+ * host word that receives M by an asynchronous copy.  Workspace sizes as for the single calls
+ * (d3gs_sort_workspace_bytes(n, 0, 32), d3gs_scan_gathered_workspace_bytes(n),
+ * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))); workspaces_are_zero != 0 says the caller has
+ * cleared all three.  workload_ranges must be zero on entry. */
+int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                   const float* depths, const int32_t* tiles_touched, const uint64_t* tile_masks,
+                   uint32_t* depth_keys_a, uint32_t* depth_keys_b, int32_t* order_a, int32_t* order_b,
+                   void* depth_sort_ws, size_t depth_sort_ws_bytes, int32_t* offsets, void* scan_ws,
+                   size_t scan_ws_bytes, int64_t* total_dev, int64_t* total_host, int64_t capacity,
+                   uint32_t* tile_keys_a, uint32_t* tile_keys_b, int32_t* idx_a, int32_t* idx_b, void* pair_sort_ws,
+                   size_t pair_sort_ws_bytes, int32_t* workload_ranges, int32_t* tile_order,
+                   int32_t workspaces_are_zero, int32_t* order_in_b, int32_t* pairs_in_b, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
  * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].

@@ -104,15 +104,19 @@ def test_forward_is_deterministic_and_backward_is_linear():
         assert med <= 1e-4 and p99 <= 1e-2, f"{name}: additivity per-gaussian median {med:.2e} p99 {p99:.2e}"
 
 
-def test_pair_buffers_sized_from_the_previous_view(oracle):
+@pytest.mark.parametrize("fused", [True, False])
+def test_pair_buffers_sized_from_the_previous_view(oracle, fused):
     """The operator sizes the pair buffers of a view from the previous view's count (no host wait
-    before binning).  A view that fits, one that outgrows the buffers (binned again), an empty one and
-    the unspeculative path must all equal the oracle."""
+    before binning) and, with `fused_binning`, enqueues the whole binning through d3gs_bin_pairs.  A view
+    that fits, one that outgrows the buffers (binned again), an empty one and the unspeculative path must
+    all equal the oracle, and the backward pass must run from the context either path leaves."""
     import torch
     from d3gs_research_amd.render import GaussianSplatOp
     from helpers import oracle_forward
     small, big = gen_scene(1, n=5000, wh=(250, 190), with_grad=False), gen_scene(1, n=40000, wh=(250, 190), with_grad=False)
     op = GaussianSplatOp(op_config(small, DFVT))
+    op.fused_binning = fused
+    print(f"speculative pair buffers, fused_binning={fused}", flush=True)
     refs = {id(sc): oracle_forward(oracle, sc, DFVT)[1] for sc in (small, big)}
     seq = [small, small, big, big, small]          # exact, fits, outgrown, fits, fits with large head room
     for k, sc in enumerate(seq):
@@ -124,6 +128,18 @@ def test_pair_buffers_sized_from_the_previous_view(oracle):
         assert np.array_equal(ctx.workload_ranges.cpu().numpy(), ref["workload_ranges"]), k
         assert np.array_equal(out.color.cpu().numpy()[0].view(np.uint32), ref["color"].view(np.uint32)), k
         assert np.array_equal(out.n_contrib.cpu().numpy()[0], ref["n_contrib"]), k
+        order = ctx.tile_order.long()
+        assert bool((torch.sort(order).values == torch.arange(order.numel(), device=order.device)).all()), k
+        keys = op._last_keys_sorted
+        assert np.array_equal(keys.cpu().numpy().view(np.uint64), ref["keys_sorted"]), k
+    from d3gs_research_amd.render import GaussianSplatGradients
+    model = torch_model(sc)
+    g = GaussianSplatGradients(drgb=torch.ones_like(out.color), dT=torch.zeros_like(out.T))
+    gm, _, _ = op.backward(model, sc.camera(), ctx, out, g)
+    plain = GaussianSplatOp(op_config(sc, DFVT))
+    out1, ctx1 = plain.forward(model, sc.camera(), training=True)
+    gm1, _, _ = plain.backward(model, sc.camera(), ctx1, out1, g)
+    assert float((gm.xyz - gm1.xyz).abs().max()) <= 1e-4 * float(gm1.xyz.abs().max())
     hidden = gen_scene(0, n=64, with_grad=False)
     hidden.xyz[:, 2] = -5.0
     out, ctx = op.forward(torch_model(hidden), hidden.camera(), training=True)
