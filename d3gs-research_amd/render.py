@@ -301,6 +301,28 @@ class GaussianSplatOp:
         s = self._stream()
         f32, i32 = torch.float32, torch.int32
 
+        def _sort_ws_bytes(count, begin_bit, end_bit):
+            nbytes = C.c_size_t(0)
+            _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
+                        "d3gs_sort_workspace_bytes")
+            return nbytes.value
+
+
+        # every zero-initialised work buffer of the forward pass comes out of one fill (the two sorts' and the
+        # scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later
+        tile_bits = L.d3gs_higher_msb(num_tiles)
+        spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
+        align = lambda v: (v + 255) // 256 * 256
+        scan_ws_bytes = C.c_size_t(0)
+        _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(scan_ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
+        sizes = [align(_sort_ws_bytes(n, 0, 32)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
+                 align(num_tiles * 8), align(scan_ws_bytes.value)]
+        zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
+        zero_scan_ws = zero_pool[sum(sizes[:3]):]
+        zero_ws_n = zero_pool[:sizes[0]]
+        zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
+        zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
+
         with self._stage("preprocess"):
             depths = torch.empty(n, dtype=f32, device=dev)
             radii = torch.empty(n, dtype=i32, device=dev)
@@ -348,12 +370,6 @@ class GaussianSplatOp:
             sh_done = torch.cuda.Event()
             sh_done.record(side)
 
-        def _sort_ws_bytes(count, begin_bit, end_bit):
-            nbytes = C.c_size_t(0)
-            _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
-                        "d3gs_sort_workspace_bytes")
-            return nbytes.value
-
         def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None):
             keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
             nbytes = _sort_ws_bytes(count, begin_bit, end_bit)
@@ -369,21 +385,6 @@ class GaussianSplatOp:
                                            int(zero_ws is not None), begin_bit, end_bit, C.byref(in_b), s)
             _capi.check(rc, "d3gs_sort_pairs")
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
-
-        # every zero-initialised work buffer of the forward pass comes out of one fill: the two sorts'
-        # workspaces and the tile ranges
-        tile_bits = L.d3gs_higher_msb(num_tiles)
-        spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
-        align = lambda v: (v + 255) // 256 * 256
-        scan_ws_bytes = C.c_size_t(0)
-        _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(scan_ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
-        sizes = [align(_sort_ws_bytes(n, 0, 32)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
-                 align(num_tiles * 8), align(scan_ws_bytes.value)]
-        zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
-        zero_scan_ws = zero_pool[sum(sizes[:3]):]
-        zero_ws_n = zero_pool[:sizes[0]]
-        zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
-        zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
 
         # With buffers sized from the previous view and no stage timers, the whole binning is one call into the
         # library (d3gs_bin_pairs): the launches of this phase are short, and issuing them one by one from
