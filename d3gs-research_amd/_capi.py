@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -51,7 +51,7 @@ _SIGNATURES = {
                                  _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, _VP, C.c_int32, C.POINTER(C.c_int),
                                  C.POINTER(C.c_int), _VP]),
     "d3gs_scan_gathered_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
-    "d3gs_scan_gathered": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP, C.c_size_t, C.c_int32, _VP, _VP]),
+    "d3gs_scan_gathered": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP, C.c_size_t, C.c_int32, _VP, _VP, _VP]),
     "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [C.c_int64, _VP]),
     "d3gs_depth_keys": (C.c_int, [_VP, C.c_int32, _VP, _VP, _VP]),
     "d3gs_gather_i32": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP]),

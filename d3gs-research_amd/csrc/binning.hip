@@ -118,7 +118,8 @@ __device__ __forceinline__ long long wave_sum_i64(long long v) {
 __global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(const int32_t* __restrict__ src, int src_n,
                                                                        const int32_t* __restrict__ index, int n,
                                                                        int32_t* __restrict__ out, ScanWorkspace ws,
-                                                                       int64_t* __restrict__ total_out) {
+                                                                       int64_t* __restrict__ total_out,
+                                                                       int64_t* __restrict__ total_host) {
     __shared__ int s_wave[kGatherScanWaves];
     __shared__ long long s_prefix;
     // Chunk = workgroup id.  Workgroups of a 1-D grid are dispatched in id order (per XCD, which gets every
@@ -207,9 +208,13 @@ __global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(
                 __hip_atomic_store(ws.status + chunk, kScanPrefix | ((unsigned long long)(prefix + total) & kScanValueMask),
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_prefix = prefix;
-            if (chunk == (int)gridDim.x - 1 && total_out) {
+            if (chunk == (int)gridDim.x - 1) {
                 const uint32_t err = __hip_atomic_load(ws.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                *total_out = err ? -1ll : prefix + total;
+                const long long grand = err ? -1ll : prefix + total;
+                if (total_out) *total_out = grand;
+                // pinned host memory is mapped into the device's address space: the count reaches the host with
+                // this store, and is visible there once the host has waited for the kernel
+                if (total_host) *total_host = grand;
             }
         }
     }
@@ -497,11 +502,12 @@ extern "C" int d3gs_scan_gathered_workspace_bytes(int32_t n, size_t* bytes_out_h
 
 extern "C" int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* out,
                                   void* workspace, size_t workspace_bytes, int32_t workspace_is_zero, int64_t* total_dev,
-                                  d3gs_stream_t stream) {
+                                  int64_t* total_host, d3gs_stream_t stream) {
     if (n < 0 || src_n < 0 || !total_dev) { set_error("d3gs_scan_gathered: bad argument"); return D3GS_ERR_INVALID_ARGUMENT; }
     hipStream_t s = (hipStream_t)stream;
     if (n == 0) {   // total = 0
         hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, (int32_t*)nullptr, 0, total_dev);
+        if (total_host) hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(kBlock), 0, s, (int32_t*)nullptr, 0, total_host);
     } else {
         if (!src || !out || !workspace) { set_error("d3gs_scan_gathered: NULL buffer"); return D3GS_ERR_INVALID_ARGUMENT; }
         if (workspace_bytes < scan_gathered_ws_bytes(n)) {
@@ -518,7 +524,7 @@ extern "C" int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32
                                (uint32_t*)workspace, words);
         }
         hipLaunchKernelGGL(scan_gather_lookback_kernel, dim3(nchunks), dim3(kGatherScanBlock), 0, s, src, (int)src_n, index, (int)n,
-                           out, ws, total_dev);
+                           out, ws, total_dev, total_host);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_scan_gathered: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

@@ -3,8 +3,6 @@
 // in the order a caller would issue them; doing it here takes the caller's per-launch cost (argument
 // marshalling in an interpreter, allocation between launches) off the stream's critical path, where the
 // kernels of this phase are short enough for that cost to leave the GPU idle between them.
-#include <hip/hip_runtime.h>
-
 #include "device_math.h"
 
 using namespace d3gs;
@@ -29,16 +27,10 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
     if (rc) return rc;
     const uint32_t* depth_keys_sorted = *order_in_b ? depth_keys_b : depth_keys_a;
     const int32_t* order = *order_in_b ? order_b : order_a;
+    // the pair count also goes to the host word, written by the scan itself; nothing here waits for it
     rc = d3gs_scan_gathered(tiles_touched, n, order, n, offsets, scan_ws, scan_ws_bytes, workspaces_are_zero, total_dev,
-                            stream);
+                            total_host, stream);
     if (rc) return rc;
-    if (total_host) {   // the pair count travels to the host behind the scan; nothing here waits for it
-        hipError_t e = hipMemcpyAsync(total_host, total_dev, sizeof(int64_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
-        if (e != hipSuccess) {
-            set_error("d3gs_bin_pairs: copy of the pair count failed: %s", hipGetErrorString(e));
-            return D3GS_ERR_LAUNCH;
-        }
-    }
     rc = d3gs_make_keys(p, radii, uvs, conic_opacity, depths, offsets, order, depth_keys_sorted, tile_masks, nullptr,
                         tile_keys_a, idx_a, capacity, stream);
     if (rc) return rc;

@@ -435,10 +435,10 @@ class GaussianSplatOp:
                 total = torch.empty(1, dtype=torch.int64, device=dev)
                 _capi.check(L.d3gs_scan_gathered(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
                                                  _capi.ptr(counts_ordered), _capi.ptr(zero_scan_ws), zero_scan_ws.numel(), 1,
-                                                 _capi.ptr(total), s), "d3gs_scan_gathered")
-                # the count travels to pinned host memory behind the scan; the host looks at it only after
-                # the rest of the forward pass has been enqueued
-                self._count_host.copy_(total, non_blocking=True)
+                                                 _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), s),
+                            "d3gs_scan_gathered")
+                # the scan also stores the count to pinned host memory; the host looks at it only after the
+                # rest of the forward pass has been enqueued
                 count_ready = torch.cuda.Event()
                 count_ready.record()
 

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 15
+#define D3GS_ABI_VERSION 16
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -124,13 +124,15 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
 
 /* K2 over a permutation, in one launch: out[j] = sum_{i <= j} src[index[i]] (index NULL: the identity), the same
  * `cumsum_` (render.py:694-695) taken in the order K3 emits the pairs; the grand total goes to *total_dev
- * (device int64; -1 if the kernel's bounded wait on an earlier chunk ran out).  An index outside [0, src_n)
+ * (device int64; -1 if the kernel's bounded wait on an earlier chunk ran out) and, when total_host is not NULL, to
+ * that word of pinned (device-mapped) host memory as well, stored by the kernel itself: the host may read it
+ * once it has waited for the stream to pass this call.  An index outside [0, src_n)
  * counts as 0.  The workspace (size from d3gs_scan_gathered_workspace_bytes) must be zero on entry:
  * workspace_is_zero != 0 says the caller has cleared it, otherwise a fill kernel runs first. */
 int d3gs_scan_gathered_workspace_bytes(int32_t n, size_t* bytes_out_host);
 int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* out,
                        void* workspace, size_t workspace_bytes, int32_t workspace_is_zero, int64_t* total_dev,
-                       d3gs_stream_t stream);
+                       int64_t* total_host, d3gs_stream_t stream);
 
 /* K3 — replaces kernel_1d("prepare_sort_data_...") at render.py:739-840.
  * Without gaussian_order (NULL) this is the reference's call: offsets = the inclusive
@@ -203,7 +205,7 @@ int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int6
  * Results: *order_in_b / *pairs_in_b say which of the a / b buffers hold the depth order and the sorted pairs;
  * *total_dev the pair count M (the kernels touch min(M, capacity) pairs: a caller that sized capacity from a
  * guess compares M with it afterwards and bins again when M is larger); total_host, when not NULL, is a pinned
- * host word that receives M by an asynchronous copy.  Workspace sizes as for the single calls
+ * host word that the scan kernel stores M to (see d3gs_scan_gathered).  Workspace sizes as for the single calls
  * (d3gs_sort_workspace_bytes(n, 0, 32), d3gs_scan_gathered_workspace_bytes(n),
  * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))); workspaces_are_zero != 0 says the caller has
  * cleared all three.  workload_ranges must be zero on entry. */

@@ -272,11 +272,13 @@ def test_scan_gathered_c_abi(n, permuted, dirty):
                                                                                     device="cuda")
     total = torch.full((1,), -7, dtype=torch.int64, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    host_total = torch.full((1,), -9, dtype=torch.int64).pin_memory()
     for _ in range(2):      # the second call finds the first one's status words in the workspace
         _capi.check(L.d3gs_scan_gathered(_capi.ptr(src), n, _capi.ptr(idx), n, _capi.ptr(out), _capi.ptr(ws), nbytes.value,
-                                         0, _capi.ptr(total), stream), "scan_gathered")
+                                         0, _capi.ptr(total), C.c_void_p(host_total.data_ptr()), stream), "scan_gathered")
         assert np.array_equal(out.cpu().numpy(), np.cumsum(want_src).astype(np.int32))
         assert int(total.item()) == int(want_src.sum())
+        assert int(host_total[0]) == int(want_src.sum())      # pinned host word, stored by the kernel
 
 
 @pytest.mark.parametrize("m,cap,begin,end,implicit", [(1000, 1000, 0, 13, False), (70001, 90000, 0, 32, True),
