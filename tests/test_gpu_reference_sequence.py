@@ -86,6 +86,41 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     assert torch.equal(out.color[0], color) and torch.equal(out.T[0], T) and torch.equal(out.n_contrib[0], nc)
     assert torch.equal(ctx.gaussian_idx_sorted, vs) and torch.equal(ctx.workload_ranges, ranges)
 
+    # the same binning through the one-call entry point (depth-first factorisation, 32-bit tile keys): the sorted
+    # gaussian indices, the ranges and the pair count must equal the plain sequence's
+    tile_masks = torch.empty((N, 2), dtype=torch.int64, device=dev)
+    dkeys_a, dkeys_b = torch.empty(N, dtype=i32, device=dev), torch.empty(N, dtype=i32, device=dev)
+    _capi.check(L.d3gs_preprocess_fwd(C.byref(P), p(model.xyz), p(model.quaternion_xyzw), p(model.scale), p(model.opacity),
+                                      p(model.color_sh), None, None, p(depths), p(radii), p(uvs), p(conic), p(touched),
+                                      p(rgb), p(cov2d), p(ne0), p(tile_masks), p(dkeys_a), s), "preprocess (masks, keys)")
+    cap = M + 1000
+    ord_a, ord_b, offs = (torch.empty(N, dtype=i32, device=dev) for _ in range(3))
+    tk_a, tk_b, ix_a, ix_b = (torch.empty(cap, dtype=i32, device=dev) for _ in range(4))
+    tile_bits = L.d3gs_higher_msb(tiles)
+    sizes = []
+    for call, args in ((L.d3gs_sort_workspace_bytes, (N, 0, 32)), (L.d3gs_scan_gathered_workspace_bytes, (N,)),
+                       (L.d3gs_sort_workspace_bytes, (cap, 0, tile_bits))):
+        _capi.check(call(*args, C.byref(nbytes)), "workspace size")
+        sizes.append(nbytes.value)
+    ws1, ws2, ws3 = (torch.full((b,), 0x5A, dtype=torch.uint8, device=dev) for b in sizes)   # not zero: the library clears
+    ranges2, order2 = torch.zeros((tiles, 2), dtype=i32, device=dev), torch.empty(tiles, dtype=i32, device=dev)
+    total2 = torch.empty(1, dtype=torch.int64, device=dev)
+    host_total = torch.full((1,), -1, dtype=torch.int64).pin_memory()
+    order_in_b, pairs_in_b = C.c_int(-1), C.c_int(-1)
+    _capi.check(L.d3gs_bin_pairs(C.byref(P), p(radii), p(uvs), p(conic), p(depths), p(touched), p(tile_masks), p(dkeys_a),
+                                 p(dkeys_b), p(ord_a), p(ord_b), p(ws1), sizes[0], p(offs), p(ws2), sizes[1], p(total2),
+                                 C.c_void_p(host_total.data_ptr()), cap, p(tk_a), p(tk_b), p(ix_a), p(ix_b), p(ws3), sizes[2],
+                                 p(ranges2), p(order2), 0, C.byref(order_in_b), C.byref(pairs_in_b), s), "bin_pairs")
+    torch.cuda.synchronize()
+    assert int(total2.item()) == M and int(host_total[0]) == M
+    assert order_in_b.value in (0, 1) and pairs_in_b.value in (0, 1)
+    vs2 = (ix_b if pairs_in_b.value else ix_a)[:M]
+    tks = (tk_b if pairs_in_b.value else tk_a)[:M]
+    assert np.array_equal(cpu(vs2), ref["gaussian_idx_sorted"])
+    assert np.array_equal(cpu(tks).astype(np.uint64), ref["keys_sorted"] >> np.uint64(32))
+    assert np.array_equal(cpu(ranges2), ref["workload_ranges"])
+    assert np.array_equal(np.sort(cpu(order2)), np.arange(tiles))
+
     # single-stream fused preprocess through the operator (overlap_sh_colors off)
     op2 = GaussianSplatOp(op_config(scene, filt))
     op2.overlap_sh_colors = False
