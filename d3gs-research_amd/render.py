@@ -52,6 +52,9 @@ class GaussianSplatOpContext:
     grad_records: torch.Tensor | None = None
     # custom feature channels of this view ([N, F]) kept for the backward pass
     custom_features: torch.Tensor | None = None
+    # disable_builtin_rgb: the image in the kernels' own layout ([1, H, W, 3 or 4], colour channels zero); the
+    # caller sees its alpha channel, or no channel at all, as out.color
+    kernel_color: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -167,7 +170,8 @@ class GaussianSplatOp:
             # back to front: not reproduced
             "render_inv_depth": c.render_inv_depth,
             "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
-            "disable_builtin_rgb": c.disable_builtin_rgb,
+            # builtin colours off: the kernels blend zeros in their place (render.py:262, 662, 1898-1931)
+            "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
             "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
             "use_int64_tile_touched": c.use_int64_tile_touched,
             "rasterize_backward_algo=PER_GAUSSIAN": c.rasterize_backward_algo != RasterizeBackwardAlgo.DEFAULT,
@@ -339,12 +343,17 @@ class GaussianSplatOp:
             if training and self.overlap_sh_colors:
                 grad_records = torch.empty((n, _capi.GRAD_RECORD_FLOATS), dtype=f32, device=dev)
             overlap = bool(self.overlap_sh_colors)
+            no_rgb = bool(self._cfg.disable_builtin_rgb)
+            if no_rgb:      # no SH evaluation: zero colours, nothing clamped
+                rgb_gaussian.zero_()
+                if ne0 is not None:
+                    ne0.zero_()
             _capi.check(L.d3gs_preprocess_fwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                _capi.ptr(tiles_touched), None if overlap else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
-                None if overlap else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), s),
+                _capi.ptr(tiles_touched), None if (overlap or no_rgb) else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
+                None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), s),
                 "d3gs_preprocess_fwd")
         sh_done = None
         if overlap:
@@ -353,13 +362,14 @@ class GaussianSplatOp:
             main = torch.cuda.current_stream()
             side = self._side_stream
             side.wait_stream(main)          # radii (and the buffers' allocation) are ready
-            ta = torch.cuda.Event(enable_timing=True) if self.stage_events is not None else None
+            ta = torch.cuda.Event(enable_timing=True) if (self.stage_events is not None and not no_rgb) else None
             if ta is not None:
                 ta.record(side)
-            _capi.check(L.d3gs_sh_colors(
-                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
-                _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), C.c_void_p(side.cuda_stream)),
-                "d3gs_sh_colors")
+            if not no_rgb:
+                _capi.check(L.d3gs_sh_colors(
+                    C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
+                    _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), C.c_void_p(side.cuda_stream)),
+                    "d3gs_sh_colors")
             tb = torch.cuda.Event(enable_timing=True) if ta is not None else None
             if tb is not None:
                 tb.record(side)
@@ -444,12 +454,14 @@ class GaussianSplatOp:
 
         final_T = torch.empty((1, height, width), dtype=f32, device=dev)
         n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
-        channels = self._cfg.num_channels
+        channels = 4 if self._cfg.render_rgba else 3       # what the kernels write
         color_shape = (1, channels, height, width) if self._cfg.use_nchw else (1, height, width, channels)
         out_color = torch.empty(color_shape, dtype=f32, device=dev)
         out_depth = torch.empty((1, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
-        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color, depth=out_depth,
-                                  n_contrib=n_contrib, radii=radii)
+        # disable_builtin_rgb: the caller's colour image is the alpha channel alone, or has no channel
+        # (config_def.py:152-157)
+        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color[..., 3:] if no_rgb else out_color,
+                                  depth=out_depth, n_contrib=n_contrib, radii=radii)
 
         def _empty_result():
             if custom_features is not None:
@@ -506,7 +518,7 @@ class GaussianSplatOp:
                 conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
-                tile_order=tile_order, grad_records=grad_records)
+                tile_order=tile_order, grad_records=grad_records, kernel_color=out_color if no_rgb else None)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
@@ -645,16 +657,21 @@ class GaussianSplatOp:
             P = self.make_params(model, _cameras, training)
         s = self._stream()
         n, dev = P.n, ctx.uvs.device
+        color = ctx.kernel_color if ctx.kernel_color is not None else out.color
         if grad is None:
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
-                _capi.ptr(ctx.tile_order), _capi.ptr(out.color), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
+                _capi.ptr(ctx.tile_order), _capi.ptr(color), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
                 _capi.ptr(out.depth), s), "d3gs_blend_fwd")
             return None
         drgb = grad.drgb
-        assert drgb.is_contiguous(), "drgb must be contiguous"
         assert drgb.shape == out.color.shape, "drgb must have the shape of the colour image"
+        if ctx.kernel_color is not None:      # gradient of the alpha channel only; the colour channels carry none
+            full = torch.zeros_like(color)
+            full[..., 3:] = drgb
+            drgb = full
+        assert drgb.is_contiguous(), "drgb must be contiguous"
         assert grad.dT.is_contiguous(), "dT must be contiguous"
         ddepth = None
         if render_depth:
@@ -668,7 +685,7 @@ class GaussianSplatOp:
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
             _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
-            _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(out.color),
+            _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
             _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec), s),
             "d3gs_blend_bwd")
         res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
