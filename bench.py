@@ -96,7 +96,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE config id (2 = headline 1M @1080p)")
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration id (2 = headline 1M @1080p)")
     ap.add_argument("--filter", type=str, default="OBB_DFVT", help="early_filter_algo: NONE, AABB, ELLIPSE, OBB, OBB_DFVT")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")

@@ -28,7 +28,7 @@ CASES = [
     (0, None, None, ELLIPSE),
     (2, 100000, (640, 360), ELLIPSE),
     (4, 30000, (960, 540), ELLIPSE),
-    # BASELINE.json's full sizes (the CPU oracle renders these in a few seconds on the box's host cores)
+    # the benchmark's full sizes (the CPU oracle renders these in a few seconds on the box's host cores)
     (2, None, None, DFVT),
     (3, None, None, AABB),
     (4, None, None, DFVT),
