@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration id (2 = headline 1M @1080p)")
     ap.add_argument("--filter", type=str, default="OBB_DFVT", help="early_filter_algo: NONE, AABB, ELLIPSE, OBB, OBB_DFVT")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--late-gradient-clear", action="store_true",
+                    help="let the preprocess backward write the zero gradients itself instead of clearing the arrays "
+                         "beside the forward pass (for comparison)")
     ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="only run a plain 256 MiB -> 256 MiB elementwise copy 5 times (reference reading for "
@@ -128,6 +131,7 @@ def main():
     scene = gen_scene(args.config)
     cam = scene.camera()
     op = GaussianSplatOp(scene_config(scene, filt))
+    op.clear_gradients_early = not args.late_gradient_clear
     model = scene_model(scene, "cuda:0")
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
 

@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 20
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -62,9 +62,9 @@ _SIGNATURES = {
                                       C.POINTER(C.c_int), _VP]),
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
-    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP]),
+    "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),
     "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
-    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int32] + [_VP] * 6 + [_VP]),
+    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int32, C.c_int32] + [_VP] * 6 + [_VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -210,7 +210,15 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                                                             const int32_t* __restrict__ tile_order,
                                                             float* __restrict__ color, float* __restrict__ final_T,
                                                             int32_t* __restrict__ n_contrib,
-                                                            float* __restrict__ final_depth) {
+                                                            float* __restrict__ final_depth,
+                                                            uint4* __restrict__ clear_vec, size_t clear_count) {
+    // Optional service to the backward pass: this kernel hardly uses the memory pipes, so it clears the
+    // caller's accumulator arrays (16-byte units, spread over all workgroups) on the side.
+    if (clear_vec) {
+        const size_t step = (size_t)gridDim.x * kBlock;
+        for (size_t q = (size_t)blockIdx.x * kBlock + threadIdx.x; q < clear_count; q += step)
+            clear_vec[q] = make_uint4(0u, 0u, 0u, 0u);
+    }
     __shared__ StagedGaussian s_g[kBlock];
     __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
@@ -516,9 +524,14 @@ static int finish_launch(const char* who) {
 extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                               const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
                               const float* depths, const int32_t* tile_order, float* color, float* final_T,
-                              int32_t* n_contrib, float* final_depth, d3gs_stream_t stream) {
+                              int32_t* n_contrib, float* final_depth, void* clear_ptr, size_t clear_bytes,
+                              d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_fwd");
     if (rc) return rc;
+    if (clear_ptr && ((((uintptr_t)clear_ptr) | clear_bytes) & 15u)) {
+        set_error("d3gs_blend_fwd: clear_ptr / clear_bytes must be multiples of 16");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib ||
         (p->render_depth && (!depths || !final_depth))) {
         set_error("d3gs_blend_fwd: NULL buffer");
@@ -527,7 +540,7 @@ extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_rang
 #define D3GS_LAUNCH_FWD(D, A)                                                                                       \
     hipLaunchKernelGGL((blend_fwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
                        workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
-                       color, final_T, n_contrib, final_depth)
+                       color, final_T, n_contrib, final_depth, (uint4*)clear_ptr, clear_bytes / 16)
     if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true); else D3GS_LAUNCH_FWD(true, false); }
     else                 { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true); else D3GS_LAUNCH_FWD(false, false); }
 #undef D3GS_LAUNCH_FWD

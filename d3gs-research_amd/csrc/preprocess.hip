@@ -43,12 +43,21 @@ constexpr int kShColorBlocks = 512;   // two workgroups per CU for the SH colour
 // Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
 // consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
 // different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
+// row_active (LDS, one byte per row, may be NULL): groups of four elements that lie entirely in rows marked 0
+// are neither read nor written.
+__device__ __forceinline__ bool rows_group_skipped(const unsigned char* row_active, int e4, int total, float inv) {
+    if (!row_active) return false;
+    const int g0 = (int)(((float)e4 + 0.5f) * inv), g1 = (int)(((float)min(e4 + 3, total - 1) + 0.5f) * inv);
+    return !row_active[g0] && !row_active[g1];
+}
+
 __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
-                                                   int stride) {
+                                                   int stride, const unsigned char* row_active = nullptr) {
     const int total = nrows * rowlen;
     const float inv = 1.0f / (float)rowlen;
     const bool vec = ((uintptr_t)src & 15u) == 0;
     for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
+        if (rows_group_skipped(row_active, e4, total, inv)) continue;
         float v[4];
         if (vec && e4 + 3 < total) {
             const float4 t = *reinterpret_cast<const float4*>(src + e4);
@@ -69,11 +78,12 @@ __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src
 }
 
 __device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, const float* lds, int nrows, int rowlen,
-                                                   int stride) {
+                                                   int stride, const unsigned char* row_active = nullptr) {
     const int total = nrows * rowlen;
     const float inv = 1.0f / (float)rowlen;
     const bool vec = ((uintptr_t)dst & 15u) == 0;
     for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
+        if (rows_group_skipped(row_active, e4, total, inv)) continue;
         float v[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -283,26 +293,15 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
 __device__ __forceinline__ void preprocess_bwd_one(
     const d3gs_params& P, const int i, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const int32_t* __restrict__ radii,
-    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0, const float* __restrict__ grad_records,
+    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
+    // the blend backward's record of this gaussian: duv(2) dconic(3) dopacity dcolor(3) dz
+    const float4 ra, const float4 rb, const float4 rc,
     const int sh_mask_compat,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* shrow, float* __restrict__ dsh_base) {
     const int K = P.sh_stride;
     float* dshp = shrow;
 
-    if (radii[i] == 0) {
-        dxyz[3 * i] = dxyz[3 * i + 1] = dxyz[3 * i + 2] = 0.0f;
-        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        dscale[3 * i] = dscale[3 * i + 1] = dscale[3 * i + 2] = 0.0f;
-        dopacity_out[i] = 0.0f;
-        for (int k = 0; k < K * 3; ++k) dshp[k] = 0.0f;
-        if (dsh_base) dsh_base[3 * i] = dsh_base[3 * i + 1] = dsh_base[3 * i + 2] = 0.0f;
-        return;
-    }
-
-    // the blend backward's record of this gaussian: duv(2) dconic(3) dopacity dcolor(3) dz
-    const float4* rec4 = reinterpret_cast<const float4*>(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * i);
-    const float4 ra = rec4[0], rb = rec4[1], rc = rec4[2];
     const float* W = P.w2c;
     float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
     float pc[3] = {dot3(W + 0, d), dot3(W + 3, d), dot3(W + 6, d)};
@@ -526,25 +525,127 @@ __device__ __forceinline__ void preprocess_bwd_one(
     dxyz[3 * i + 2] = gx[2] + (ddir[2] - dirv[2] * dd) / dn;
 }
 
-__global__ __launch_bounds__(kPrepBlock) void preprocess_bwd_kernel(
+// A gaussian whose record is all zero -- culled in the forward pass, or in tile lists but never reached before
+// its pixels saturated, which is most of a dense scene -- has an all-zero gradient: nothing of it is read beyond
+// the record, and with outputs_are_zero (the caller cleared the gradient arrays beforehand) nothing is written.
+// The others are compacted inside the workgroup (kPer gaussians per thread, so that what is left still fills
+// whole wavefronts) and worked off kBwdBlock at a time: thread t takes the t-th of them, their SH rows are
+// staged in LDS and leave as gradient rows.
+constexpr int kBwdBlock = 256;
+
+// element e of a block of `cnt` staged rows <-> element of the global [N][rowlen] array, for the gaussians
+// first + list[0 .. cnt)
+template <bool kToLds>
+__device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float* lds, const unsigned short* list, int cnt,
+                                              int first, int rowlen, int stride) {
+    if ((rowlen & 3) == 0 && ((uintptr_t)global & 15u) == 0) {
+        const int per_row = rowlen >> 2;
+        for (int q = threadIdx.x; q < cnt * per_row; q += kBwdBlock) {
+            const int r = q / per_row, c = (q - r * per_row) * 4;
+            float4* gp = reinterpret_cast<float4*>(global + (size_t)(first + list[r]) * rowlen + c);
+            float* lp = lds + r * stride + c;
+            if (kToLds) {
+                const float4 t = *gp;
+                lp[0] = t.x; lp[1] = t.y; lp[2] = t.z; lp[3] = t.w;
+            } else {
+                *gp = make_float4(lp[0], lp[1], lp[2], lp[3]);
+            }
+        }
+    } else {
+        for (int e = threadIdx.x; e < cnt * rowlen; e += kBwdBlock) {
+            const int r = e / rowlen, c = e - r * rowlen;
+            float* gp = global + (size_t)(first + list[r]) * rowlen + c;
+            if (kToLds) lds[r * stride + c] = *gp;
+            else *gp = lds[r * stride + c];
+        }
+    }
+}
+
+__device__ __forceinline__ bool record_is_zero(const float4 ra, const float4 rb, const float4 rc) {
+    return ra.x == 0.0f && ra.y == 0.0f && ra.z == 0.0f && ra.w == 0.0f && rb.x == 0.0f && rb.y == 0.0f &&
+           rb.z == 0.0f && rb.w == 0.0f && rc.x == 0.0f && rc.y == 0.0f;
+}
+
+template <int kPer>
+__global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ grad_records, const int sh_mask_compat,
+    const float* __restrict__ grad_records, const int sh_mask_compat, const int outputs_are_zero,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
-    extern __shared__ float s_rows[];
+    constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
+    extern __shared__ float s_rows[];                    // kBwdBlock rows of `stride` floats
+    __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
+    __shared__ unsigned char s_active[kSpan];
+    __shared__ int s_count[kPer * kWaves];
     const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
-    const int first = blockIdx.x * kPrepBlock;
-    const int nrows = min(kPrepBlock, P.n - first);
-    rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
+    const int first = blockIdx.x * kSpan;
+    const int nrows = min(kSpan, P.n - first);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float4* rec4 = reinterpret_cast<const float4*>(grad_records);
+    bool active[kPer];
+    unsigned long long mates[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int local = k * kBwdBlock + tid;
+        const size_t i = (size_t)first + local;
+        active[k] = false;
+        if (local < nrows && radii[i] != 0) active[k] = !record_is_zero(rec4[4 * i], rec4[4 * i + 1], rec4[4 * i + 2]);
+        mates[k] = __ballot(active[k]);
+        if (lane == 0) s_count[k * kWaves + wave] = __popcll(mates[k]);
+        s_active[local] = active[k] ? 1 : 0;
+    }
     __syncthreads();
-    if ((int)threadIdx.x < nrows)
-        preprocess_bwd_one(P, first + threadIdx.x, xyz, quat, scale, opacity, radii, cov2d, ne0, grad_records,
-                           sh_mask_compat, dxyz, dquat, dscale, dopacity_out, s_rows + threadIdx.x * stride,
-                           dsh_base);
+    int nactive = 0;
+    int before[kPer];      // entries of the list ahead of this wavefront's group k
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) before[k] = 0;
+#pragma unroll
+    for (int q = 0; q < kPer * kWaves; ++q) {
+        const int c = s_count[q];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k)
+            if (q < k * kWaves + wave) before[k] += c;
+        nactive += c;
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k)
+        if (active[k])
+            s_list[before[k] + __popcll(mates[k] & ((1ull << lane) - 1ull))] = (unsigned short)(k * kBwdBlock + tid);
+    if (!outputs_are_zero) {   // the zero gradients of the gaussians without work
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+            const int local = k * kBwdBlock + tid;
+            const size_t i = (size_t)first + local;
+            if (local < nrows && !active[k]) {
+                dxyz[3 * i] = dxyz[3 * i + 1] = dxyz[3 * i + 2] = 0.0f;
+                *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                dscale[3 * i] = dscale[3 * i + 1] = dscale[3 * i + 2] = 0.0f;
+                dopacity_out[i] = 0.0f;
+                if (dsh_base) dsh_base[3 * i] = dsh_base[3 * i + 1] = dsh_base[3 * i + 2] = 0.0f;
+            }
+        }
+        float* block_dsh = dsh + (size_t)first * rowlen;
+        const float inv = 1.0f / (float)rowlen;
+        for (int e = tid; e < nrows * rowlen; e += kBwdBlock)
+            if (!s_active[(int)(((float)e + 0.5f) * inv)]) block_dsh[e] = 0.0f;
+    }
     __syncthreads();
-    rows_lds_to_global(dsh + (size_t)first * rowlen, s_rows, nrows, rowlen, stride);
+    for (int base = 0; base < nactive; base += kBwdBlock) {
+        const int cnt = min(kBwdBlock, nactive - base);
+        bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride);
+        __syncthreads();
+        if (tid < cnt) {
+            const int g = first + s_list[base + tid];
+            preprocess_bwd_one(P, g, xyz, quat, scale, opacity, radii, cov2d, ne0, rec4[4 * (size_t)g],
+                               rec4[4 * (size_t)g + 1], rec4[4 * (size_t)g + 2], sh_mask_compat, dxyz, dquat, dscale,
+                               dopacity_out, s_rows + tid * stride, dsh_base);
+        }
+        __syncthreads();
+        bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride);
+        __syncthreads();
+    }
 }
 
 int check_params(const d3gs_params* p, const char* who) {
@@ -633,9 +734,9 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
 extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
                                    const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
-                                   const float* grad_records, int32_t sh_mask_compat, float* dxyz,
-                                   float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
-                                   float* dcolor_sh_base, d3gs_stream_t stream) {
+                                   const float* grad_records, int32_t sh_mask_compat, int32_t outputs_are_zero,
+                                   float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
+                                   float* dcolor_sh, float* dcolor_sh_base, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_bwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -645,12 +746,19 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
-    const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
-    hipLaunchKernelGGL(preprocess_bwd_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
-                       scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,
-                       (int)sh_mask_compat, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
-                       dcolor_sh_base);
+    const size_t lds_bytes = (size_t)kBwdBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    // four gaussians per thread once there are enough workgroups to fill the chip that way
+    if (p->n >= 512 * kBwdBlock * 4) {
+        hipLaunchKernelGGL(preprocess_bwd_kernel<4>, dim3((p->n + kBwdBlock * 4 - 1) / (kBwdBlock * 4)), dim3(kBwdBlock),
+                           lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale, opacity, color_sh, radii,
+                           cov2d_vecs, sh_to_rgb_ne_0, grad_records, (int)sh_mask_compat, (int)outputs_are_zero, dxyz,
+                           dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
+    } else {
+        hipLaunchKernelGGL(preprocess_bwd_kernel<1>, dim3((p->n + kBwdBlock - 1) / kBwdBlock), dim3(kBwdBlock), lds_bytes,
+                           (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs,
+                           sh_to_rgb_ne_0, grad_records, (int)sh_mask_compat, (int)outputs_are_zero, dxyz,
+                           dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

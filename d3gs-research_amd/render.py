@@ -50,6 +50,10 @@ class GaussianSplatOpContext:
     # not in the reference: the backward's [N, 16] gradient records, zero-filled during the forward pass
     # on the second stream (consumed by the first backward over this context)
     grad_records: torch.Tensor | None = None
+    # float32 pool for the model gradients of this view, cleared beside the forward pass (see _grad_views)
+    grad_pool: torch.Tensor | None = None
+    # the allocation behind grad_records and grad_pool, until the forward blend has been asked to clear it
+    grad_clear: torch.Tensor | None = None
     # custom feature channels of this view ([N, F]) kept for the backward pass
     custom_features: torch.Tensor | None = None
     # disable_builtin_rgb: the image in the kernels' own layout ([1, H, W, 3 or 4], colour channels zero); the
@@ -155,6 +159,8 @@ class GaussianSplatOp:
         # size the pair buffers from the previous view's count instead of waiting for this view's
         # the speculative binning of a view (depth order .. tile ranges) goes out as one library call
         self.fused_binning = True
+        # training: the model-gradient arrays are allocated with the forward pass and cleared beside it
+        self.clear_gradients_early = True
         self.speculative_pair_buffers = True
         self._pair_capacity = 0
         self._count_host: torch.Tensor | None = None
@@ -339,11 +345,21 @@ class GaussianSplatOp:
             # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
             tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
             depth_keys = torch.empty(n, dtype=i32, device=dev)      # float bits of the depths: the depth sort's keys
-            grad_records = None
-            if training and self.overlap_sh_colors:
-                grad_records = torch.empty((n, _capi.GRAD_RECORD_FLOATS), dtype=f32, device=dev)
+            # The backward's accumulators (one record per gaussian) and, with clear_gradients_early, the model
+            # gradient arrays: one allocation that the forward blend kernel clears while it runs (it leaves the
+            # memory pipes idle).  Most gaussians of a view end with an all-zero gradient (culled, or never reached
+            # before their pixels saturated), which the preprocess backward then need not write.
+            grad_records = grad_pool = grad_clear = None
+            if training:
+                rec_floats = n * _capi.GRAD_RECORD_FLOATS
+                pool_floats = self._grad_pool_floats(model) if self.clear_gradients_early else 0
+                grad_clear = torch.empty(rec_floats + pool_floats, dtype=f32, device=dev)
+                grad_records = grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
+                grad_pool = grad_clear[rec_floats:] if pool_floats else None
             overlap = bool(self.overlap_sh_colors)
             no_rgb = bool(self._cfg.disable_builtin_rgb)
+            if overlap and (self._side_stream is None or self._side_stream.device != dev):
+                self._side_stream = torch.cuda.Stream(device=dev)   # default priority
             if no_rgb:      # no SH evaluation: zero colours, nothing clamped
                 rgb_gaussian.zero_()
                 if ne0 is not None:
@@ -357,8 +373,6 @@ class GaussianSplatOp:
                 "d3gs_preprocess_fwd")
         sh_done = None
         if overlap:
-            if self._side_stream is None or self._side_stream.device != dev:
-                self._side_stream = torch.cuda.Stream(device=dev)   # default priority
             main = torch.cuda.current_stream()
             side = self._side_stream
             side.wait_stream(main)          # radii (and the buffers' allocation) are ready
@@ -374,9 +388,6 @@ class GaussianSplatOp:
             if tb is not None:
                 tb.record(side)
                 self.stage_events.setdefault("sh_colors", []).append((ta, tb))
-            if grad_records is not None:
-                with torch.cuda.stream(side):
-                    grad_records.zero_()      # the backward's accumulators, cleared while the sort runs
             sh_done = torch.cuda.Event()
             sh_done.record(side)
 
@@ -518,7 +529,8 @@ class GaussianSplatOp:
                 conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
-                tile_order=tile_order, grad_records=grad_records, kernel_color=out_color if no_rgb else None)
+                tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
+                kernel_color=out_color if no_rgb else None)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
@@ -585,6 +597,28 @@ class GaussianSplatOp:
     def _backward_bundle(self, model, ctx, out, grad, return_uv_grad):
         return _backward_bundle_impl(self, model, ctx, out, grad, return_uv_grad)
 
+    # ------------------------------------------------------- gradient pool
+    @staticmethod
+    def _grad_fields(model):
+        fields = [("xyz", model.xyz), ("quaternion_xyzw", model.quaternion_xyzw), ("scale", model.scale),
+                  ("opacity", model.opacity), ("color_sh", model.color_sh)]
+        if model.color_sh_base is not None:
+            fields.append(("color_sh_base", model.color_sh_base))
+        return fields
+
+    @classmethod
+    def _grad_pool_floats(cls, model) -> int:
+        return sum((t.numel() + 63) // 64 * 64 for _, t in cls._grad_fields(model))
+
+    @classmethod
+    def _grad_views(cls, model, pool):
+        """The model-shaped gradient tensors as 256-byte aligned slices of one allocation."""
+        views, off = {}, 0
+        for name, t in cls._grad_fields(model):
+            views[name] = pool[off:off + t.numel()].view(t.shape)
+            off += (t.numel() + 63) // 64 * 64
+        return views
+
     # ------------------------------------------------------- custom features
     # The blend is linear in the per-gaussian channel values and every channel shares the weights
     # alpha * T, so F custom feature channels (render.py:1536-1539, 1892-1923, 1952-1971) are blended by
@@ -616,7 +650,7 @@ class GaussianSplatOp:
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(tri), None, _capi.ptr(ctx.tile_order), _capi.ptr(img),
-                _capi.ptr(T2), _capi.ptr(nc2), None, s), "d3gs_blend_fwd (custom features)")
+                _capi.ptr(T2), _capi.ptr(nc2), None, None, 0, s), "d3gs_blend_fwd (custom features)")
             res[0, :, :, k:k + w] = img[:, :, :w]
         return res
 
@@ -659,11 +693,12 @@ class GaussianSplatOp:
         n, dev = P.n, ctx.uvs.device
         color = ctx.kernel_color if ctx.kernel_color is not None else out.color
         if grad is None:
+            clear, ctx.grad_clear = ctx.grad_clear, None
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
                 _capi.ptr(ctx.tile_order), _capi.ptr(color), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
-                _capi.ptr(out.depth), s), "d3gs_blend_fwd")
+                _capi.ptr(out.depth), _capi.ptr(clear), 0 if clear is None else clear.numel() * 4, s), "d3gs_blend_fwd")
             return None
         drgb = grad.drgb
         assert drgb.shape == out.color.shape, "drgb must have the shape of the colour image"
@@ -715,18 +750,19 @@ class GaussianSplatOp:
                 torch.zeros_like(out.custom_features)
             dcustom = self._backward_custom_features(P, ctx, out, dfeat_img.contiguous(), g.records)
         with self._stage("preprocess_bwd"):
-            dxyz = torch.empty_like(model.xyz)
-            dquat = torch.empty_like(model.quaternion_xyzw)
-            dscale = torch.empty_like(model.scale)
-            dsh = torch.empty_like(model.color_sh)
-            dsh_base = torch.empty_like(model.color_sh_base) if model.color_sh_base is not None else None
-            dopacity = torch.empty_like(model.opacity)
+            pool, ctx.grad_pool = ctx.grad_pool, None
+            prezeroed = pool is not None and pool.numel() == self._grad_pool_floats(model)
+            if not prezeroed:
+                pool = torch.empty(self._grad_pool_floats(model), dtype=torch.float32, device=dev)
+            gv = self._grad_views(model, pool)
+            dxyz, dquat, dscale, dopacity, dsh = (gv[k] for k in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh"))
+            dsh_base = gv.get("color_sh_base")
             _capi.check(L.d3gs_preprocess_bwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
                 _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), int(self._cfg.compat_ref_sh_mask_bitorder),
-                _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh),
-                _capi.ptr(dsh_base), s),
+                int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity),
+                _capi.ptr(dsh), _capi.ptr(dsh_base), s),
                 "d3gs_preprocess_bwd")
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,
                                          color_sh=dsh, color_sh_base=dsh_base)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 16
+#define D3GS_ABI_VERSION 20
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -222,11 +222,16 @@ int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs,
  * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].
  * depths [N] (K1's output) and final_depth [H,W] are read / written only when p->render_depth and may be
  * NULL otherwise.  In inference the depth is divided by the accumulated opacity, which makes it NaN (0/0)
- * for a pixel nothing reached, as in the reference (render.py:2244-2250). */
+ * for a pixel nothing reached, as in the reference (render.py:2244-2250).
+ * clear_ptr (may be NULL; no counterpart in the reference): clear_bytes of device memory, both multiples of
+ * 16, that the kernel sets to zero while it runs -- meant for the arrays the backward pass accumulates into
+ * (grad_records, and the gradient arrays handed to d3gs_preprocess_bwd with outputs_are_zero): the blend is
+ * bound by arithmetic and leaves the memory pipes idle, so the clear costs nothing here. */
 int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                    const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
                    const int32_t* tile_order /* from d3gs_tile_ranges, or NULL for raster order */, float* color,
-                   float* final_T, int32_t* n_contrib, float* final_depth, d3gs_stream_t stream);
+                   float* final_T, int32_t* n_contrib, float* final_depth, void* clear_ptr, size_t clear_bytes,
+                   d3gs_stream_t stream);
 
 /* Per-gaussian gradient record written by K7 and read by K9: one 64-byte line per gaussian so that
  * the sixteen lanes flushing one gaussian issue a single line-wide atomic request.  The reference keeps
@@ -254,14 +259,18 @@ int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const i
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from K7's records (duv, dconic, dopacity, dcolor
  * [, dz]) to the raw model tensors, including the fused activation gradients.
- * Gradients of gaussians with radii == 0 are written as zeros.  The *_base
+ * Gradients of gaussians with radii == 0, and of gaussians whose record is all
+ * zero (in no tile list, or never reached before their pixels saturated), are
+ * zeros; nothing but the record is read for them.  outputs_are_zero != 0 (no
+ * counterpart in the reference) says the caller has cleared the six gradient
+ * arrays beforehand: those zeros are then not written again.  The *_base
  * pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
  * reference's reversed bit order (render.py:3344-3350). */
 int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
                         const uint8_t* sh_to_rgb_ne_0, const float* grad_records, int32_t sh_mask_compat,
-                        float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
-                        float* dcolor_sh_base, d3gs_stream_t stream);
+                        int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw, float* dscale,
+                        float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base, d3gs_stream_t stream);
 
 #ifdef __cplusplus
 }

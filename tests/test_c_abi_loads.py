@@ -32,7 +32,7 @@ def test_params_struct_matches_header_layout():
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 16
+    assert L.d3gs_abi_version() == 20
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
 
@@ -42,7 +42,7 @@ def test_error_codes_without_compute():
     L = _capi.lib()
     P = _capi.Params()
     P.n, P.width, P.height, P.tiles_x, P.tiles_y, P.sh_stride = 4, 32, 32, 3, 2, 1   # wrong tile counts
-    nul = [None] * 12
+    nul = [None] * 11 + [None, 0, None]     # eleven buffers, the optional clear region, the stream
     rc = L.d3gs_blend_fwd(C.byref(P), *nul)
     assert rc == -1 and b"tiles_x" in L.d3gs_last_error_string()
     P.tiles_x = 2
@@ -50,6 +50,8 @@ def test_error_codes_without_compute():
     assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"early_filter_algo" in L.d3gs_last_error_string()
     P.filter_algo = 1
     assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"NULL" in L.d3gs_last_error_string()
+    odd = [None] * 11 + [C.c_void_p(24), 32, None]     # clear region not on a 16-byte boundary
+    assert L.d3gs_blend_fwd(C.byref(P), *odd) == -1 and b"multiples of 16" in L.d3gs_last_error_string()
     P.sh_degree, P.sh_stride = 3, 4
     assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"sh_stride" in L.d3gs_last_error_string()
     n = C.c_size_t(0)

@@ -152,12 +152,25 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
     _capi.check(L.d3gs_preprocess_bwd(
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
         _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, stream), "d3gs_preprocess_bwd")
     torch.cuda.synchronize()
     for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", dop_io), ("dsh", o_sh)):
         ok, worst, nbad = grad_close(cpu(got), pb_ref[name], rel=1e-6, abs_frac=1e-7)
         assert ok, f"isolated {name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+    # outputs cleared by the caller: gaussians with an all-zero record are left alone, the rest must match
+    z_xyz, z_q, z_s, z_op, z_sh = (torch.zeros_like(t) for t in (o_xyz, o_q, o_s, dop_io, o_sh))
+    _capi.check(L.d3gs_preprocess_bwd(
+        C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+        _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 1, _capi.ptr(z_xyz), _capi.ptr(z_q),
+        _capi.ptr(z_s), _capi.ptr(z_op), _capi.ptr(z_sh), None, stream), "d3gs_preprocess_bwd (cleared outputs)")
+    torch.cuda.synchronize()
+    for a, b in ((o_xyz, z_xyz), (o_q, z_q), (o_s, z_s), (dop_io, z_op), (o_sh, z_sh)):
+        assert torch.equal(a, b), "cleared-output mode changed a gradient"
+    silent = (rec_np == 0).all(axis=1)
+    assert silent.any() and not silent.all()
+    assert float(o_sh[torch.from_numpy(silent).cuda()].abs().max()) == 0.0
 
 
 def test_autograd_entry_point(oracle):

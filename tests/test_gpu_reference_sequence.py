@@ -74,12 +74,14 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     H, W = scene.height, scene.width
     color = torch.empty((H, W, 3), dtype=f32, device=dev)
     T, nc = torch.empty((H, W), dtype=f32, device=dev), torch.empty((H, W), dtype=i32, device=dev)
+    scratch = torch.full((4096 + 3,), 7.0, dtype=f32, device=dev)[:4096]     # a region for the kernel to clear
     _capi.check(L.d3gs_blend_fwd(C.byref(P), p(ranges), p(vs), p(uvs), p(conic), p(rgb), None, None, p(color), p(T), p(nc),
-                                 None, s), "blend_fwd")
+                                 None, p(scratch), 4096 * 4, s), "blend_fwd")
     torch.cuda.synchronize()
     assert np.array_equal(cpu(nc), ref["n_contrib"])
     assert np.array_equal(cpu(color).view(np.uint32), ref["color"].view(np.uint32))
     assert np.array_equal(cpu(T).view(np.uint32), ref["T"].view(np.uint32))
+    assert float(scratch.abs().max()) == 0.0
 
     # and the operator's fast path gives the same image
     out, ctx = op.forward(model, scene.camera(), training=True)
