@@ -42,7 +42,10 @@ STAGE_BYTES = {
     "tile_ranges": lambda N, M, P, T, passes: 4 * M + 12 * T,
     "blend_fwd": lambda N, M, P, T, passes: 40 * M + 20 * P,
     "blend_bwd": lambda N, M, P, T, passes: 76 * M + 36 * P,
-    "preprocess_bwd": lambda N, M, P, T, passes: (236 + 50 + 236) * N,
+    # every gaussian's record and radius are read (68 B); only gaussians with a non-zero record (A of them) are
+    # worked on: 250 B of parameters and SH read, 236 B of gradients written.  With A = N this is the 522 B x N of
+    # a kernel that treats every gaussian alike.
+    "preprocess_bwd": lambda N, M, P, T, passes, A=None: 68 * N + (250 + 236) * (N if A is None else A),
 }
 
 
@@ -160,11 +163,14 @@ def main():
     N, P_px, T_tiles = scene.n, scene.width * scene.height, ((scene.width + 15) // 16) * ((scene.height + 15) // 16)
     M = op.last_num_rendered
     passes = (int(T_tiles).bit_length() + 7) // 8      # radix passes of the pair sort (tile bits only)
+    # gaussians whose gradient record is not all zero after the last view's blend backward
+    active = int((op.last_raster_grads.records != 0).any(dim=1).sum())
     stages = {}
     for name, evs in op.stage_events.items():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
         avg = sum(ts) / len(ts)
-        nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes)
+        nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes) if name != "preprocess_bwd" else \
+            STAGE_BYTES[name](N, M, P_px, T_tiles, passes, active)
         stages[name] = {"ms": round(avg, 4), "ms_p10": round(ts[len(ts) // 10], 4), "ms_p50": round(ts[len(ts) // 2], 4),
                         "ms_p90": round(ts[(len(ts) * 9) // 10], 4), "alg_bytes": int(nbytes),
                         "gbs": round(nbytes / (avg * 1e-3) / 1e9, 1)}
@@ -230,7 +236,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"config {args.config}: {scene.name}", "gaussians": N, "sh_degree": scene.sh_degree,
                    "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name, "pairs_M": int(M),
-                   "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists},
+                   "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists,
+                   "gaussians_with_gradient": active},
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
         "gpu_stage_sum_ms": round(gpu_sum, 4),
         "stages": stages,

@@ -532,6 +532,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
 // whole wavefronts) and worked off kBwdBlock at a time: thread t takes the t-th of them, their SH rows are
 // staged in LDS and leave as gradient rows.
 constexpr int kBwdBlock = 256;
+constexpr int kBwdRows = 176;   // gaussians worked off per pass: with their LDS rows (34 KB) four workgroups share a CU
 
 // element e of a block of `cnt` staged rows <-> element of the global [N][rowlen] array, for the gaussians
 // first + list[0 .. cnt)
@@ -575,7 +576,7 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
-    extern __shared__ float s_rows[];                    // kBwdBlock rows of `stride` floats
+    extern __shared__ float s_rows[];                    // kBwdRows rows of `stride` floats
     __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
     __shared__ unsigned char s_active[kSpan];
     __shared__ int s_count[kPer * kWaves];
@@ -586,12 +587,28 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const float4* rec4 = reinterpret_cast<const float4*>(grad_records);
     bool active[kPer];
     unsigned long long mates[kPer];
+    // all radii first, then all records: two round trips to memory instead of two per gaussian
+    int rad[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
         const int local = k * kBwdBlock + tid;
-        const size_t i = (size_t)first + local;
-        active[k] = false;
-        if (local < nrows && radii[i] != 0) active[k] = !record_is_zero(rec4[4 * i], rec4[4 * i + 1], rec4[4 * i + 2]);
+        rad[k] = local < nrows ? radii[(size_t)first + local] : 0;
+    }
+    float4 ra[kPer], rb[kPer], rc[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const size_t i = (size_t)first + k * kBwdBlock + tid;
+        ra[k] = rb[k] = rc[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (rad[k] != 0) {
+            ra[k] = rec4[4 * i];
+            rb[k] = rec4[4 * i + 1];
+            rc[k] = rec4[4 * i + 2];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        const int local = k * kBwdBlock + tid;
+        active[k] = rad[k] != 0 && !record_is_zero(ra[k], rb[k], rc[k]);
         mates[k] = __ballot(active[k]);
         if (lane == 0) s_count[k * kWaves + wave] = __popcll(mates[k]);
         s_active[local] = active[k] ? 1 : 0;
@@ -632,8 +649,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
             if (!s_active[(int)(((float)e + 0.5f) * inv)]) block_dsh[e] = 0.0f;
     }
     __syncthreads();
-    for (int base = 0; base < nactive; base += kBwdBlock) {
-        const int cnt = min(kBwdBlock, nactive - base);
+    for (int base = 0; base < nactive; base += kBwdRows) {
+        const int cnt = min(kBwdRows, nactive - base);
         bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride);
         __syncthreads();
         if (tid < cnt) {
@@ -746,7 +763,7 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    const size_t lds_bytes = (size_t)kBwdBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
+    const size_t lds_bytes = (size_t)kBwdRows * ((p->sh_stride * 3) | 1) * sizeof(float);
     // four gaussians per thread once there are enough workgroups to fill the chip that way
     if (p->n >= 512 * kBwdBlock * 4) {
         hipLaunchKernelGGL(preprocess_bwd_kernel<4>, dim3((p->n + kBwdBlock * 4 - 1) / (kBwdBlock * 4)), dim3(kBwdBlock),
