@@ -180,7 +180,9 @@ class GaussianSplatOp:
             "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
             "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
             "use_int64_tile_touched": c.use_int64_tile_touched,
-            "rasterize_backward_algo=PER_GAUSSIAN": c.rasterize_backward_algo != RasterizeBackwardAlgo.DEFAULT,
+            # rasterize_backward_algo = PER_GAUSSIAN is accepted: the reference's second backward
+            # (render.py:2319-2776) computes the same gradient with fewer atomics per gaussian, which the one
+            # backward kernel here already has (one record-wide atomic per tile and gaussian)
         }
         bad = [k for k, v in unsupported.items() if v]
         if bad:

@@ -4,6 +4,8 @@ import ctypes as C
 import os
 import re
 
+import pytest
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -69,3 +71,19 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_capi, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _capi.lib()
+
+
+def test_operator_config_gate():
+    """Options the operator carries out construct; the ones it does not raise at construction, by name."""
+    import numpy as np
+    from d3gs_research_amd.config_def import GaussianSplatConfig, RasterizeBackwardAlgo
+    from d3gs_research_amd.render import GaussianSplatOp
+    GaussianSplatOp(GaussianSplatConfig())
+    GaussianSplatOp(GaussianSplatConfig(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN))
+    GaussianSplatOp(GaussianSplatConfig(disable_builtin_rgb=True, render_rgba=True, render_depth=True,
+                                        enable_anti_aliasing=True))
+    for kw, word in ((dict(sparse_mode=True), "sparse_mode"), (dict(render_inv_depth=True), "render_inv_depth"),
+                     (dict(enable_32bit_sort=True), "enable_32bit_sort"), (dict(tile_size=(8, 8)), "tile_size"),
+                     (dict(disable_builtin_rgb=True, use_nchw=True), "use_nchw")):
+        with pytest.raises(NotImplementedError, match=word):
+            GaussianSplatOp(GaussianSplatConfig(**kw))
