@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -38,13 +38,18 @@ class Params(C.Structure):
     ]
 
 
+class Instances(C.Structure):
+    """Mirror of ``d3gs_instances``: per-gaussian instance ids and one camera (12 floats) per instance."""
+    _fields_ = [("instance_ids", C.c_void_p), ("instance_cameras", C.c_void_p), ("num_instances", C.c_int32)]
+
+
 _VP = C.c_void_p
 _SIGNATURES = {
     "d3gs_abi_version": (C.c_int, []),
     "d3gs_last_error_string": (C.c_char_p, []),
     "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
-    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [_VP]),
-    "d3gs_sh_colors": (C.c_int, [C.POINTER(Params)] + [_VP] * 6 + [_VP]),
+    "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [C.POINTER(Instances), _VP]),
+    "d3gs_sh_colors": (C.c_int, [C.POINTER(Params)] + [_VP] * 6 + [C.POINTER(Instances), _VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_tiles": (C.c_int, [_VP, C.c_int32, _VP, C.c_size_t, _VP, _VP]),
     "d3gs_bin_pairs": (C.c_int, [C.POINTER(Params)] + [_VP] * 10 + [_VP, C.c_size_t, _VP, _VP, C.c_size_t, _VP, _VP, C.c_int64,
@@ -64,7 +69,8 @@ _SIGNATURES = {
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),
     "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
-    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int32, C.c_int32] + [_VP] * 6 + [_VP]),
+    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int32, C.c_int32] + [_VP] * 6 +
+                            [C.POINTER(Instances), _VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -101,10 +101,30 @@ __device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, cons
     }
 }
 
+// Per-gaussian camera for instance rendering (render.py:346-356): a gaussian with instance id k >= 0 lives in
+// the frame of instance k and is seen by the camera expressed in that frame, cameras[k] = 9 floats of the
+// world-to-camera rotation (row major) followed by the camera centre; the others keep the view's camera.
+struct InstanceView {
+    const int32_t* ids;     // [N], may be NULL
+    const float* cameras;   // [count][12]
+    int count;
+};
+
+__device__ __forceinline__ void apply_instance(d3gs_params& P, const InstanceView& inst, int i) {
+    const int id = inst.ids[i];
+    if (id >= 0 && id < inst.count) {
+        const float* m = inst.cameras + 12 * (size_t)id;
+#pragma unroll
+        for (int k = 0; k < 9; ++k) P.w2c[k] = m[k];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) P.cam_center[k] = m[9 + k];
+    }
+}
+
 // kWithSh = false leaves the SH colour to sh_colors_kernel: no LDS, twice the resident wavefronts.
-template <bool kWithSh>
+template <bool kWithSh, bool kInstances>
 __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
-    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const d3gs_params P0, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const float* __restrict__ sh_base, const uint8_t* __restrict__ invalid_mask, float* __restrict__ depths,
     int32_t* __restrict__ radii, float* __restrict__ uvs, float* __restrict__ conic_opacity,
@@ -113,16 +133,18 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     uint32_t* __restrict__ depth_sort_keys) {
     // SH rows of this workgroup's gaussians: coalesced global read into LDS, then per-thread rows
     extern __shared__ float s_rows[];
-    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    const int rowlen = P0.sh_stride * 3, stride = rowlen | 1;
     if constexpr (kWithSh) {
         const int first = blockIdx.x * kPrepBlock;
-        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P.n - first), rowlen, stride);
+        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
         __syncthreads();
     }
     // no early return: every lane of the wavefront takes part in the cooperative tile count
     const int i_raw = blockIdx.x * kPrepBlock + threadIdx.x;
-    const bool in_range = i_raw < P.n;
-    const int i = in_range ? i_raw : P.n - 1;
+    const bool in_range = i_raw < P0.n;
+    const int i = in_range ? i_raw : P0.n - 1;
+    d3gs_params P = P0;     // with instances: this lane's camera
+    if constexpr (kInstances) apply_instance(P, inst, i);
 
     bool valid = true;
     float z = 0.0f, u = 0.0f, v = 0.0f, con0 = 0.0f, con1 = 0.0f, con2 = 0.0f, op = 0.0f;
@@ -248,20 +270,23 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
 
 // SH colour of the gaussians the preprocess kernel accepted (radii > 0), the part of K1 that
 // streams the 192-byte SH rows: same operations as the fused kernel, zeros for rejected gaussians.
+template <bool kInstances>
 __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
-    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ sh,
+    const d3gs_params P0, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ sh,
     const float* __restrict__ sh_base, const int32_t* __restrict__ radii, float* __restrict__ rgb_out,
     uint8_t* __restrict__ ne0_out) {
     extern __shared__ float s_rows[];
-    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    const int rowlen = P0.sh_stride * 3, stride = rowlen | 1;
     // grid-stride over 128-gaussian chunks: a small grid leaves most of every CU to the kernels this
     // one runs beside
-    for (int first = blockIdx.x * kPrepBlock; first < P.n; first += gridDim.x * kPrepBlock) {
+    for (int first = blockIdx.x * kPrepBlock; first < P0.n; first += gridDim.x * kPrepBlock) {
         __syncthreads();   // the previous chunk's rows have been read
-        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P.n - first), rowlen, stride);
+        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
         __syncthreads();
         const int i = first + threadIdx.x;
-        if (i >= P.n) continue;
+        if (i >= P0.n) continue;
+        d3gs_params P = P0;
+        if constexpr (kInstances) apply_instance(P, inst, i);
         float rgb[3] = {0.0f, 0.0f, 0.0f};
         uint32_t ne0 = 0;
         if (radii[i] > 0) {
@@ -567,9 +592,9 @@ __device__ __forceinline__ bool record_is_zero(const float4 ra, const float4 rb,
            rb.z == 0.0f && rb.w == 0.0f && rc.x == 0.0f && rc.y == 0.0f;
 }
 
-template <int kPer>
+template <int kPer, bool kInstances>
 __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
-    const d3gs_params P, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const d3gs_params P, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
     const float* __restrict__ grad_records, const int sh_mask_compat, const int outputs_are_zero,
@@ -655,7 +680,9 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         __syncthreads();
         if (tid < cnt) {
             const int g = first + s_list[base + tid];
-            preprocess_bwd_one(P, g, xyz, quat, scale, opacity, radii, cov2d, ne0, rec4[4 * (size_t)g],
+            d3gs_params Pg = P;
+            if constexpr (kInstances) apply_instance(Pg, inst, g);
+            preprocess_bwd_one(Pg, g, xyz, quat, scale, opacity, radii, cov2d, ne0, rec4[4 * (size_t)g],
                                rec4[4 * (size_t)g + 1], rec4[4 * (size_t)g + 2], sh_mask_compat, dxyz, dquat, dscale,
                                dopacity_out, s_rows + tid * stride, dsh_base);
         }
@@ -696,12 +723,29 @@ int check_params(const d3gs_params* p, const char* who) {
 
 using namespace d3gs;
 
+// host view of the optional instance table -> what the kernels take; returns false on a malformed table
+static bool instance_view(const d3gs_instances* in, InstanceView* out, const char* who) {
+    out->ids = nullptr;
+    out->cameras = nullptr;
+    out->count = 0;
+    if (!in || !in->instance_ids) return true;
+    if (in->num_instances < 0 || (in->num_instances > 0 && !in->instance_cameras)) {
+        set_error("%s: instance table with %d entries and no cameras", who, in->num_instances);
+        return false;
+    }
+    out->ids = in->instance_ids;
+    out->cameras = in->instance_cameras;
+    out->count = in->num_instances;
+    return true;
+}
+
 extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
                                    const float* color_sh_base, const uint8_t* invalid_mask, float* depths,
                                    int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
                                    float* rgb_gaussian, float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0,
-                                   uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream) {
+                                   uint64_t* tile_masks, uint32_t* depth_sort_keys, const d3gs_instances* instances,
+                                   d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_fwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -711,26 +755,26 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
+    InstanceView inst;
+    if (!instance_view(instances, &inst, "d3gs_preprocess_fwd")) return D3GS_ERR_INVALID_ARGUMENT;
     dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
-    if (with_sh) {
-        const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
-        hipLaunchKernelGGL(preprocess_fwd_kernel<true>, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz,
-                           quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs,
-                           conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,
-                           (unsigned long long*)tile_masks, depth_sort_keys);
-    } else {
-        hipLaunchKernelGGL(preprocess_fwd_kernel<false>, grid, block, 0, (hipStream_t)stream, *p, xyz, quaternion_xyzw,
-                           scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, conic_opacity,
-                           tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0, (unsigned long long*)tile_masks,
-                           depth_sort_keys);
-    }
+    const size_t lds_bytes = with_sh ? (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float) : 0;
+#define D3GS_LAUNCH_K1(SH, INST)                                                                                      \
+    hipLaunchKernelGGL((preprocess_fwd_kernel<SH, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,   \
+                       quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs,     \
+                       conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,                         \
+                       (unsigned long long*)tile_masks, depth_sort_keys)
+    if (with_sh) { if (inst.ids) D3GS_LAUNCH_K1(true, true); else D3GS_LAUNCH_K1(true, false); }
+    else         { if (inst.ids) D3GS_LAUNCH_K1(false, true); else D3GS_LAUNCH_K1(false, false); }
+#undef D3GS_LAUNCH_K1
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 
 extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const float* color_sh, const float* color_sh_base,
-                              const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+                              const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0,
+                              const d3gs_instances* instances, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_sh_colors");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -738,11 +782,17 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
         set_error("d3gs_sh_colors: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
+    InstanceView inst;
+    if (!instance_view(instances, &inst, "d3gs_sh_colors")) return D3GS_ERR_INVALID_ARGUMENT;
     const int chunks = (p->n + kPrepBlock - 1) / kPrepBlock;
     dim3 grid(chunks < kShColorBlocks ? chunks : kShColorBlocks), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
-    hipLaunchKernelGGL(sh_colors_kernel, grid, block, lds_bytes, (hipStream_t)stream, *p, xyz, color_sh, color_sh_base,
-                       radii, rgb_gaussian, sh_to_rgb_ne_0);
+    if (inst.ids)
+        hipLaunchKernelGGL(sh_colors_kernel<true>, grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz, color_sh,
+                           color_sh_base, radii, rgb_gaussian, sh_to_rgb_ne_0);
+    else
+        hipLaunchKernelGGL(sh_colors_kernel<false>, grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz, color_sh,
+                           color_sh_base, radii, rgb_gaussian, sh_to_rgb_ne_0);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_sh_colors: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
@@ -753,7 +803,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
                                    const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
                                    const float* grad_records, int32_t sh_mask_compat, int32_t outputs_are_zero,
                                    float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
-                                   float* dcolor_sh, float* dcolor_sh_base, d3gs_stream_t stream) {
+                                   float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
+                                   d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_bwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -763,19 +814,21 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
+    InstanceView inst;
+    if (!instance_view(instances, &inst, "d3gs_preprocess_bwd")) return D3GS_ERR_INVALID_ARGUMENT;
     const size_t lds_bytes = (size_t)kBwdRows * ((p->sh_stride * 3) | 1) * sizeof(float);
     // four gaussians per thread once there are enough workgroups to fill the chip that way
-    if (p->n >= 512 * kBwdBlock * 4) {
-        hipLaunchKernelGGL(preprocess_bwd_kernel<4>, dim3((p->n + kBwdBlock * 4 - 1) / (kBwdBlock * 4)), dim3(kBwdBlock),
-                           lds_bytes, (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale, opacity, color_sh, radii,
-                           cov2d_vecs, sh_to_rgb_ne_0, grad_records, (int)sh_mask_compat, (int)outputs_are_zero, dxyz,
-                           dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
-    } else {
-        hipLaunchKernelGGL(preprocess_bwd_kernel<1>, dim3((p->n + kBwdBlock - 1) / kBwdBlock), dim3(kBwdBlock), lds_bytes,
-                           (hipStream_t)stream, *p, xyz, quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs,
-                           sh_to_rgb_ne_0, grad_records, (int)sh_mask_compat, (int)outputs_are_zero, dxyz,
-                           dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base);
-    }
+    const bool wide = p->n >= 512 * kBwdBlock * 4;
+    const int per = wide ? 4 : 1;
+    dim3 grid((p->n + kBwdBlock * per - 1) / (kBwdBlock * per)), block(kBwdBlock);
+#define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
+    hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,  \
+                       quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
+                       (int)sh_mask_compat, (int)outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out,       \
+                       dcolor_sh, dcolor_sh_base)
+    if (wide) { if (inst.ids) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }
+    else      { if (inst.ids) D3GS_LAUNCH_K9(1, true); else D3GS_LAUNCH_K9(1, false); }
+#undef D3GS_LAUNCH_K9
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;

@@ -59,6 +59,9 @@ class GaussianSplatOpContext:
     # disable_builtin_rgb: the image in the kernels' own layout ([1, H, W, 3 or 4], colour channels zero); the
     # caller sees its alpha channel, or no channel at all, as out.color
     kernel_color: torch.Tensor | None = None
+    # instance rendering: the view's camera in every instance frame ([I, 12] float32) and the int32 ids
+    instance_cameras: torch.Tensor | None = None
+    instance_ids: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -235,6 +238,42 @@ class GaussianSplatOp:
             raise TypeError(f"unsupported camera type {type(cameras)}")
         return focal, pp, c2w_T, cameras.image_shape_wh
 
+    def instance_table(self, model, cameras, instance2world_T):
+        """Instance rendering (render.py:207-220, 346-356): gaussians with ``model.instance_id[i] = k >= 0`` live
+        in the frame of object instance k, whose pose this frame is ``instance2world_T[frame][k]`` ([4, 3]: three
+        rows holding the columns of the rotation, then the translation; rigid).  The reference composes
+        cam2instance = world2instance o cam2world per gaussian inside its kernels; here it is done once per
+        instance, in float64 on the device, and the kernels read a [I, 12] float32 table: the world-to-camera
+        rotation in the instance frame (row major) and the camera centre in the instance frame.
+        Returns ``(instance_ids int32 [N], instance_cameras float32 [I, 12])``."""
+        assert model.instance_id is not None, "instance_id must be provided in model when render with instance"
+        T = instance2world_T
+        if T.ndim == 4:      # [num_frame, num_instance, 4, 3]
+            if isinstance(cameras, BasicPinholeCamera):
+                assert cameras.frame_local_id is not None, "frame_local_id must be set when render with instance"
+                T = T[int(cameras.frame_local_id)]
+            else:
+                assert cameras.frame_ids is not None, "frame_ids must be provided when render with instance"
+                T = T[cameras.frame_ids[0].to(device=T.device, dtype=torch.long)]
+        assert T.ndim == 3 and tuple(T.shape[1:]) == (4, 3), \
+            "instance2world_T must be [num_frame, num_instance, 4, 3] (or [num_instance, 4, 3] for one frame)"
+        dev = model.xyz.device
+        T = T.detach().to(device=dev, dtype=torch.float64)
+        cw = torch.from_numpy(self._camera_arrays(cameras)[2].astype(np.float64)).to(dev)
+        rot_T = T[:, :3, :]                                   # R_i^T: world -> instance
+        w2c = cw[:3] @ rot_T.transpose(1, 2)                  # R_c^T R_i
+        centre = rot_T @ (cw[3] - T[:, 3, :]).unsqueeze(-1)   # R_i^T (c - t_i)
+        table = torch.cat([w2c.reshape(-1, 9), centre.reshape(-1, 3)], 1).to(torch.float32).contiguous()
+        ids = model.instance_id.detach().to(device=dev, dtype=torch.int32).contiguous()
+        assert ids.numel() == len(model), "instance_id must hold one id per gaussian"
+        return ids, table
+
+    @staticmethod
+    def _instances_arg(ids, table):
+        if table is None:
+            return None
+        return C.byref(_capi.Instances(ids.data_ptr(), table.data_ptr(), int(table.shape[0])))
+
     def make_params(self, model: GaussianModelOriginBase, cameras, training: bool) -> _capi.Params:
         """Scalars the reference bakes into kernel source (render.py:198-230, 333-358)."""
         c = self._cfg
@@ -292,8 +331,8 @@ class GaussianSplatOp:
         if isinstance(cameras, CameraBundle) and len(cameras) != 1:
             return self._forward_bundle(model, cameras, training, instance2world_T, custom_features, mask,
                                         prep_user_inputs)
-        if instance2world_T is not None or prep_user_inputs:
-            raise NotImplementedError("instance2world_T / prep_user_inputs are not supported")
+        if prep_user_inputs:
+            raise NotImplementedError("prep_user_inputs is not supported")
         self._check_model(model)
         if custom_features is not None:
             assert not self.is_nchw, "custom feat don't support nchw, set use_nchw=False in config."   # render.py:246
@@ -307,6 +346,10 @@ class GaussianSplatOp:
                 mask = mask.view(torch.uint8)
         L = self._lib
         P = self.make_params(model, cameras, training)
+        inst_ids = inst_cams = None
+        if instance2world_T is not None:
+            inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
+        inst = self._instances_arg(inst_ids, inst_cams)
         n, dev = P.n, model.xyz.device
         width, height = P.width, P.height
         num_tiles = P.tiles_x * P.tiles_y
@@ -371,7 +414,7 @@ class GaussianSplatOp:
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                 _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                 _capi.ptr(tiles_touched), None if (overlap or no_rgb) else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
-                None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), s),
+                None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), inst, s),
                 "d3gs_preprocess_fwd")
         sh_done = None
         if overlap:
@@ -384,7 +427,7 @@ class GaussianSplatOp:
             if not no_rgb:
                 _capi.check(L.d3gs_sh_colors(
                     C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
-                    _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), C.c_void_p(side.cuda_stream)),
+                    _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), inst, C.c_void_p(side.cuda_stream)),
                     "d3gs_sh_colors")
             tb = torch.cuda.Event(enable_timing=True) if ta is not None else None
             if tb is not None:
@@ -532,7 +575,7 @@ class GaussianSplatOp:
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
                 tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
-                kernel_color=out_color if no_rgb else None)
+                kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
@@ -735,8 +778,8 @@ class GaussianSplatOp:
                  custom_features=None, prep_user_inputs=None):
         """render.py:2779-3374.  Returns ``(grad_model, duv | None, dcustom_features)``; ``grad_model``
         is a model-shaped dataclass holding the gradients of the raw tensors."""
-        if instance2world_T is not None or prep_user_inputs:
-            raise NotImplementedError("instance2world_T / prep_user_inputs are not supported")
+        if prep_user_inputs:
+            raise NotImplementedError("prep_user_inputs is not supported")
         if isinstance(ctx, GaussianSplatOpBatchContext):
             return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
         L = self._lib
@@ -759,12 +802,17 @@ class GaussianSplatOp:
             gv = self._grad_views(model, pool)
             dxyz, dquat, dscale, dopacity, dsh = (gv[k] for k in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh"))
             dsh_base = gv.get("color_sh_base")
+            # the cameras of the forward pass; a context from a pass without instances takes the argument
+            inst_ids, inst_cams = ctx.instance_ids, ctx.instance_cameras
+            if inst_cams is None and instance2world_T is not None:
+                inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
+            inst = self._instances_arg(inst_ids, inst_cams)
             _capi.check(L.d3gs_preprocess_bwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
                 _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), int(self._cfg.compat_ref_sh_mask_bitorder),
                 int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity),
-                _capi.ptr(dsh), _capi.ptr(dsh_base), s),
+                _capi.ptr(dsh), _capi.ptr(dsh_base), inst, s),
                 "d3gs_preprocess_bwd")
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,
                                          color_sh=dsh, color_sh_base=dsh_base)
@@ -808,11 +856,13 @@ class _RasterizeGaussians(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, xyz, color_sh, color_sh_base, scale, quaternion_xyzw, opacity, cur_sh_degree, custom_features,
-                mask, model_cls, cameras, training, op: GaussianSplatOp, uv_grad_holder=None):
+                mask, model_cls, cameras, training, op: GaussianSplatOp, uv_grad_holder=None, instance_id=None,
+                instance2world_T=None):
         model = model_cls(xyz=xyz, color_sh=color_sh, color_sh_base=color_sh_base, scale=scale,
                           quaternion_xyzw=quaternion_xyzw, opacity=opacity, cur_sh_degree=cur_sh_degree,
-                          act_applied=True)
-        out, fwd_ctx = op.forward(model, cameras, training, custom_features=custom_features, mask=mask)
+                          instance_id=instance_id, act_applied=True)
+        out, fwd_ctx = op.forward(model, cameras, training, instance2world_T, custom_features=custom_features,
+                                  mask=mask)
         ctx.has_ctx = fwd_ctx is not None
         if fwd_ctx is not None:
             ctx.fwd_ctx = fwd_ctx
@@ -829,7 +879,7 @@ class _RasterizeGaussians(torch.autograd.Function):
     @torch.autograd.function.once_differentiable
     def backward(ctx, drgb, ddepth, dcustom_features, dT, dn_contrib, dradii):
         if not ctx.has_ctx:
-            return (None,) * 14
+            return (None,) * 16
         if drgb is None:
             drgb = torch.zeros_like(ctx.out.color)
         if dT is None:
@@ -842,19 +892,19 @@ class _RasterizeGaussians(torch.autograd.Function):
                                        dcustom_features=dcustom_features)
         gm, duv, dcf = ctx.op.backward(ctx.model, ctx.cameras, ctx.fwd_ctx, ctx.out, grads,
                                        return_uv_grad=ctx.return_uv_grad)
+        # no gradient reaches the instance poses (render.py:3584-3587 returns None for them as well)
         return (gm.xyz, gm.color_sh, gm.color_sh_base, gm.scale, gm.quaternion_xyzw, gm.opacity, None, dcf, None,
-                None, None, None, None, duv)
+                None, None, None, None, duv, None, None)
 
 
 def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSplatOp, training=False,
                         uv_grad_holder: torch.Tensor | None = None, instance2world_T=None, custom_features=None,
                         mask=None) -> GaussianSplatOutput:
     """render.py:3783-3838."""
-    if instance2world_T is not None:
-        raise NotImplementedError("instance2world_T is not supported")
     model = model.create_model_with_act()   # torch-side activations for the non-fused families
     res = _RasterizeGaussians.apply(model.xyz, model.color_sh, model.color_sh_base, model.scale,
                                     model.quaternion_xyzw, model.opacity, model.cur_sh_degree, custom_features, mask,
-                                    type(model), cameras, training, op, uv_grad_holder)
+                                    type(model), cameras, training, op, uv_grad_holder, model.instance_id,
+                                    instance2world_T)
     return GaussianSplatOutput(color=res[0], depth=res[1], custom_features=res[2], T=res[3], n_contrib=res[4],
                                radii=res[5])

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 20
+#define D3GS_ABI_VERSION 21
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -89,6 +89,19 @@ const char* d3gs_last_error_string(void);
 /* DeviceSort.get_higher_msb — devsort.py:131-149: bit length of n. */
 int d3gs_higher_msb(uint32_t n);
 
+/* Instance rendering (render.py:207-220, 346-356): a gaussian with instance_ids[i] = k >= 0 belongs to object
+ * instance k, its parameters are given in that object's frame, and it is seen by the camera expressed in that
+ * frame: instance_cameras[k] holds the 9 floats of the world-to-camera rotation in the instance frame (row
+ * major, the layout of d3gs_params.w2c) followed by the camera centre in the instance frame, i.e.
+ * cam2instance = world2instance o cam2world, which the reference derives from instance2world_T[frame][k] inside
+ * its kernels and the caller derives here.  Gaussians with a negative (or out of range) id use the view's own
+ * camera.  Passed by pointer to K1, the SH colours and K9; NULL, or instance_ids == NULL, means no instances. */
+typedef struct d3gs_instances {
+    const int32_t* instance_ids;     /* [N] device */
+    const float* instance_cameras;   /* [num_instances][12] device */
+    int32_t num_instances;
+} d3gs_instances;
+
 /* K1 — replaces kernel_raw("gs3d_preprocess_...") at render.py:629-681 (body
  * 421-476, 569-619).  One pass over the gaussians: fused activations, projection,
  * EWA covariance, conic, radius, tile rect, validity, tile count under the chosen
@@ -107,13 +120,14 @@ int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* qua
                         const uint8_t* invalid_mask, float* depths,
                         int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_gaussian,
                         float* cov2d_vecs, uint8_t* sh_to_rgb_ne_0, uint64_t* tile_masks, uint32_t* depth_sort_keys,
-                        d3gs_stream_t stream);
+                        const d3gs_instances* instances, d3gs_stream_t stream);
 
 /* The SH-colour part of K1 on its own (render.py:569-613): rgb_gaussian [N,3] and, when not NULL, the
  * clamp mask sh_to_rgb_ne_0 [N] of the gaussians with radii > 0, zeros for the rest.  Same values as the
  * fused call. */
 int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const float* color_sh, const float* color_sh_base,
-                   const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
+                   const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, const d3gs_instances* instances,
+                   d3gs_stream_t stream);
 
 /* K2 — replaces `tiles_touched.cumsum_(0)` + `.item()` at render.py:694-695.
  * In-place inclusive scan; the grand total is written to *total_dev (device
@@ -270,7 +284,8 @@ int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* qua
                         const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
                         const uint8_t* sh_to_rgb_ne_0, const float* grad_records, int32_t sh_mask_compat,
                         int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw, float* dscale,
-                        float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base, d3gs_stream_t stream);
+                        float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
+                        d3gs_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -33,6 +33,11 @@
 //   orc_blend_fwd                : float64 dense per-pixel restatement in numpy
 //   orc_blend_bwd / orc_preprocess_bwd : float64 torch autograd of the forward
 //                                  (straight-through alpha clamp) + finite differences
+//   instance cameras             : identity poses / negative ids are no-ops, one instance equals
+//                                  the plain render by the composed camera, an SH-0 render equals
+//                                  the render of the gaussians moved to the world frame; the
+//                                  reference composes the pose in float32 with third-party cumm
+//                                  array ops whose rounding is absent here -> "parity unpinned"
 //   exp used in the blend        : the reference uses CUDA __expf (approximate,
 //                                  rounding unspecified); this oracle and the HIP
 //                                  kernels use orc_expf's exact operation sequence so
@@ -392,14 +397,33 @@ static inline int tile_walk(const orc_params* P, const TileWalkIn& g, F&& f) {
 // Outputs of invalid gaussians are zero-filled (the reference leaves them
 // uninitialised).
 // ---------------------------------------------------------------------------
-ORC_API int orc_preprocess_fwd(const orc_params* P, const float* xyz, const float* quat, const float* scale,
+// Instance rendering (render.py:346-356): gaussian i with instance_ids[i] = k in [0, num_instances) is seen by
+// the camera expressed in the frame of instance k, instance_cameras[k] = world-to-camera rotation (9, row major) +
+// camera centre (3) in that frame; the others by the view's camera.
+static inline orc_params with_instance(const orc_params* P, const int32_t* instance_ids, const float* instance_cameras,
+                                       int32_t num_instances, int i) {
+    orc_params L = *P;
+    if (instance_ids) {
+        const int id = instance_ids[i];
+        if (id >= 0 && id < num_instances) {
+            for (int k = 0; k < 9; ++k) L.w2c[k] = instance_cameras[12 * (size_t)id + k];
+            for (int k = 0; k < 3; ++k) L.cam_center[k] = instance_cameras[12 * (size_t)id + 9 + k];
+        }
+    }
+    return L;
+}
+
+ORC_API int orc_preprocess_fwd(const orc_params* P0, const float* xyz, const float* quat, const float* scale,
                        const float* opacity, const float* sh, const float* sh_base, const uint8_t* invalid_mask,
                        float* depths, int32_t* radii,
                        float* uvs, float* conic_opacity, int32_t* tiles_touched, float* rgb_out, float* cov2d_out,
-                       uint8_t* ne0_out) {
-    const int n = P->n;
+                       uint8_t* ne0_out, const int32_t* instance_ids, const float* instance_cameras,
+                       int32_t num_instances) {
+    const int n = P0->n;
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int i = 0; i < n; ++i) {
+        const orc_params Pl = with_instance(P0, instance_ids, instance_cameras, num_instances, i);
+        const orc_params* P = &Pl;
         depths[i] = 0.0f;
         radii[i] = 0;
         uvs[2 * i] = uvs[2 * i + 1] = 0.0f;
@@ -805,15 +829,18 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
 // (render.py:608 vs 3344-3350); 0 uses the consistent mapping.
 // Gradients of gaussians with radii == 0 are zero.
 // ---------------------------------------------------------------------------
-ORC_API void orc_preprocess_bwd(const orc_params* P, const float* xyz, const float* quat, const float* scale,
+ORC_API void orc_preprocess_bwd(const orc_params* P0, const float* xyz, const float* quat, const float* scale,
                         const float* opacity, const float* sh, const int32_t* radii, const float* cov2d,
                         const uint8_t* ne0, const float* duv, const float* dconic, const float* dopacity_in,
                         const float* dcolor, const float* dz, int32_t sh_mask_compat, float* dxyz, float* dquat,
-                        float* dscale, float* dopacity_out, float* dsh, float* dsh_base) {
-    const int n = P->n;
-    const int K = P->sh_stride;
+                        float* dscale, float* dopacity_out, float* dsh, float* dsh_base, const int32_t* instance_ids,
+                        const float* instance_cameras, int32_t num_instances) {
+    const int n = P0->n;
+    const int K = P0->sh_stride;
 #pragma omp parallel for schedule(dynamic, 1024)
     for (int i = 0; i < n; ++i) {
+        const orc_params Pl = with_instance(P0, instance_ids, instance_cameras, num_instances, i);
+        const orc_params* P = &Pl;
         for (int k = 0; k < 3; ++k) dxyz[3 * i + k] = 0.0f;
         for (int k = 0; k < 4; ++k) dquat[4 * i + k] = 0.0f;
         for (int k = 0; k < 3; ++k) dscale[3 * i + k] = 0.0f;

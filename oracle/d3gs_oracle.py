@@ -139,7 +139,32 @@ def _f32(a):
     return None if a is None else np.ascontiguousarray(a, np.float32)
 
 
-def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
+def _instances(instances):
+    """(instance_ids [N] int32, instance_cameras [I, 12] float32) or None -> the three C arguments."""
+    if instances is None:
+        return None, None, C.c_int32(0), ()
+    ids = np.ascontiguousarray(instances[0], np.int32)
+    cams = np.ascontiguousarray(instances[1], np.float32).reshape(-1, 12)
+    return _p(ids), _p(cams), C.c_int32(cams.shape[0]), (ids, cams)
+
+
+def instance_cameras(cam2world_T, instance2world_T):
+    """Cameras in the instances' frames, [I, 12] float32 (9 of the world-to-camera rotation, row major, then
+    the camera centre), from the view's cam2world_T [4, 3] (rows 0-2: columns of the camera-to-world rotation,
+    row 3: centre) and instance2world_T [I, 4, 3] in the same layout: cam2instance = world2instance o cam2world
+    (render.py:350-354), evaluated in float64."""
+    cw = np.asarray(cam2world_T, np.float64)
+    iw = np.asarray(instance2world_T, np.float64).reshape(-1, 4, 3)
+    Rc_T, c = cw[:3], cw[3]                 # R_c^T (world -> camera), camera centre
+    out = np.empty((iw.shape[0], 12), np.float64)
+    for k, T in enumerate(iw):
+        Ri, ti = T[:3].T, T[3]              # instance -> world rotation and translation
+        out[k, :9] = (Rc_T @ Ri).reshape(-1)
+        out[k, 9:] = Ri.T @ (c - ti)
+    return out.astype(np.float32)
+
+
+def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None, instances=None):
     n = P.n
     out = dict(
         depths=np.empty(n, np.float32), radii=np.empty(n, np.int32), uvs=np.empty((n, 2), np.float32),
@@ -151,7 +176,7 @@ def preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=
     rc = lib().orc_preprocess_fwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(sh_base), _p(mask),
                                   _p(out["depths"]), _p(out["radii"]), _p(out["uvs"]), _p(out["conic_opacity"]),
                                   _p(out["tiles_touched"]), _p(out["rgb_gaussian"]), _p(out["cov2d_vecs"]),
-                                  _p(out["sh_to_rgb_ne_0"]))
+                                  _p(out["sh_to_rgb_ne_0"]), *_instances(instances)[:3])
     if rc != 0:
         raise ValueError("oracle: unsupported early_filter_algo")
     return out
@@ -224,7 +249,7 @@ def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib
 
 
 def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dconic, dopacity, dcolor, dz=None,
-                   sh_mask_compat=False):
+                   sh_mask_compat=False, instances=None):
     n, K = P.n, P.sh_stride
     xyz, quat, scale, opacity, sh, cov2d, duv, dconic, dopacity, dcolor, dz = map(
         _f32, (xyz, quat, scale, opacity, sh, cov2d, duv, dconic, dopacity, dcolor, dz))
@@ -235,13 +260,13 @@ def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dco
     lib().orc_preprocess_bwd(C.byref(P), _p(xyz), _p(quat), _p(scale), _p(opacity), _p(sh), _p(radii), _p(cov2d),
                              _p(ne0), _p(duv), _p(dconic), _p(dopacity), _p(dcolor), _p(dz),
                              C.c_int32(int(sh_mask_compat)), _p(out["dxyz"]), _p(out["dquat"]), _p(out["dscale"]),
-                             _p(out["dopacity"]), _p(out["dsh"]), _p(out["dsh_base"]))
+                             _p(out["dopacity"]), _p(out["dsh"]), _p(out["dsh_base"]), *_instances(instances)[:3])
     return out
 
 
-def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None):
+def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None, instances=None):
     """Whole forward: K1 .. K6.  Returns every intermediate the op context holds."""
-    pre = preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base, invalid_mask)
+    pre = preprocess_fwd(P, xyz, quat, scale, opacity, sh, sh_base, invalid_mask, instances)
     offsets, m = scan(pre["tiles_touched"])
     num_tiles = P.tiles_x * P.tiles_y
     keys, vals = make_keys(P, pre["radii"], pre["uvs"], pre["conic_opacity"], pre["depths"], offsets, m)
@@ -284,7 +309,7 @@ def blend_custom_features(P, fwd, feat):
 
 
 def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_mask_compat=False, ddepth=None,
-             custom_features=None, custom_feature_image=None, dcustom_features=None):
+             custom_features=None, custom_feature_image=None, dcustom_features=None, instances=None):
     """Whole backward: K7 + K9 from the dict ``forward`` returned.  With custom features
     (render.py:1892-1895, 1952-1955, 1969-1972) the alpha gradient gains
     ``dot(dfeat, T * feat - rest)`` and ``dcustom_features = sum weight * dfeat``: both are linear in
@@ -315,5 +340,6 @@ def backward(P, fwd, xyz, quat, scale, opacity, sh, drgb, dT, sh_base=None, sh_m
     pb = preprocess_bwd(P, xyz, quat, scale, opacity, sh_in, fwd["radii"], fwd["cov2d_vecs"], fwd["sh_to_rgb_ne_0"],
                         g["duv"].astype(np.float32), g["dconic"].astype(np.float32),
                         g["dopacity"].astype(np.float32), g["dcolor"].astype(np.float32),
-                        dz=None if g["dz"] is None else g["dz"].astype(np.float32), sh_mask_compat=sh_mask_compat)
+                        dz=None if g["dz"] is None else g["dz"].astype(np.float32), sh_mask_compat=sh_mask_compat,
+                        instances=instances)
     return g, pb

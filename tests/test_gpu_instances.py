@@ -1,0 +1,165 @@
+"""GPU parity for instance rendering (render.py:207-220, 346-356, 3031-3040, 3261-3270): gaussians that carry an
+instance id are seen by the camera expressed in their object's frame.  Forward stages bit-exact against the
+oracle given the same camera table, gradients to the bars of the plain path, the table itself against the
+oracle's float64 composition, and the autograd entry point with a [num_frame, num_instance, 4, 3] pose tensor."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import gen_scene, grad_close, op_config, oracle_params, torch_model
+from test_oracle_instances import _poses
+
+pytestmark = pytest.mark.gpu
+
+AABB, DFVT = 1, 4
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+def _setup(scene, K, seed, frames=2, frame=1):
+    import torch
+    rng = np.random.default_rng(seed)
+    T = np.stack([_poses(rng, K)[3] for _ in range(frames)])       # [F, K, 4, 3]
+    ids = rng.integers(-1, K, scene.n).astype(np.int32)
+    model = torch_model(scene)
+    model.instance_id = torch.from_numpy(ids).cuda()
+    cam = scene.camera()
+    cam.frame_local_id = frame
+    return T, ids, model, cam
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt,K", [(0, None, None, AABB, 3), (1, 30000, (320, 240), DFVT, 5),
+                                                (2, 200000, (960, 540), DFVT, 17)])
+def test_instances_forward_and_backward(oracle, cfg_id, n, wh, filt, K):
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    print(f"instances cfg={cfg_id} n={scene.n} K={K}", flush=True)
+    T, ids, model, cam = _setup(scene, K, 40 + cfg_id)
+    op = GaussianSplatOp(op_config(scene, filt))
+    T_dev = torch.from_numpy(T).cuda()
+
+    # the table: device float64 composition against the oracle's numpy one (both rounded to float32 once)
+    ids_dev, table = op.instance_table(model, cam, T_dev)
+    table_np = table.cpu().numpy()
+    want = oracle.instance_cameras(scene.cam2world_T, T[1])
+    assert ids_dev.dtype == torch.int32 and np.array_equal(ids_dev.cpu().numpy(), ids)
+    assert table_np.shape == (K, 12) and np.abs(table_np - want).max() <= 2e-7 * max(1.0, np.abs(want).max())
+
+    inst = (ids, table_np)
+    P = oracle_params(oracle, scene, filt)
+    args = (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    ref = oracle.forward(P, *args, instances=inst)
+    out, ctx = op.forward(model, cam, training=True, instance2world_T=T_dev)
+    torch.cuda.synchronize()
+    cpu = lambda t: t.detach().cpu().numpy()
+    assert op.last_num_rendered == ref["num_rendered"] > 0
+    assert np.array_equal(cpu(ctx.radii), ref["radii"])
+    for name, got in (("uvs", ctx.uvs), ("conic_opacity", ctx.conic_opacity), ("depths", ctx.depths),
+                      ("rgb_gaussian", ctx.rgb_gaussian), ("cov2d_vecs", ctx.cov2d_vecs)):
+        vis = ref["radii"] > 0
+        assert np.array_equal(_bits(cpu(got))[vis], _bits(ref[name])[vis]), name
+    assert np.array_equal(cpu(ctx.sh_to_rgb_ne_0), ref["sh_to_rgb_ne_0"])
+    M = ref["num_rendered"]
+    assert np.array_equal(cpu(ctx.gaussian_idx_sorted)[:M], ref["gaussian_idx_sorted"][:M])
+    assert np.array_equal(cpu(ctx.workload_ranges), ref["workload_ranges"])
+    assert np.abs(cpu(out.color)[0] - ref["color"]).max() <= 1e-5
+    assert np.abs(cpu(out.T)[0] - ref["T"]).max() <= 1e-5
+    # differs from the render without instances
+    plain = oracle.forward(P, *args)
+    assert not np.array_equal(plain["radii"], ref["radii"])
+
+    g_ref, pb_ref = oracle.backward(P, ref, *args, scene.drgb[0], scene.dT[0], instances=inst)
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    gm, _, _ = op.backward(model, cam, ctx, out, grads)
+    torch.cuda.synchronize()
+    for name, got in (("dxyz", gm.xyz), ("dquat", gm.quaternion_xyzw), ("dscale", gm.scale),
+                      ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
+        a = cpu(got).astype(np.float64).reshape(scene.n, -1)
+        b = pb_ref[name].astype(np.float64).reshape(scene.n, -1)
+        rn = np.linalg.norm(b, axis=1)
+        e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
+        med, p99 = np.quantile(e, [0.5, 0.99])
+        assert med <= 1e-4 and p99 <= 5e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
+        assert not (np.abs(a[rn == 0]) > 0).any(), f"{name}: gradient on a gaussian the oracle leaves at zero"
+
+    # preprocess backward alone, fed the oracle's blend gradients: same inputs, same operation order
+    from d3gs_research_amd import _capi
+    L = _capi.lib()
+    Pg = op.make_params(model, cam, True)
+    rec_np = np.zeros((scene.n, _capi.GRAD_RECORD_FLOATS), np.float32)
+    rec_np[:, 0:2], rec_np[:, 2:5], rec_np[:, 5], rec_np[:, 6:9] = g_ref["duv"], g_ref["dconic"], g_ref["dopacity"], g_ref["dcolor"]
+    rec = torch.from_numpy(rec_np).cuda()
+    o_xyz, o_q, o_s = torch.empty_like(model.xyz), torch.empty_like(model.quaternion_xyzw), torch.empty_like(model.scale)
+    o_op, o_sh = torch.empty_like(model.opacity), torch.empty_like(model.color_sh)
+    arg = C.byref(_capi.Instances(ids_dev.data_ptr(), table.data_ptr(), K))
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _capi.check(L.d3gs_preprocess_bwd(
+        C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+        _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q), _capi.ptr(o_s),
+        _capi.ptr(o_op), _capi.ptr(o_sh), None, arg, stream), "d3gs_preprocess_bwd (instances)")
+    torch.cuda.synchronize()
+    for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", o_op), ("dsh", o_sh)):
+        ok, worst, nbad = grad_close(cpu(got), pb_ref[name], rel=1e-4, abs_frac=1e-6)
+        assert ok, f"K9 {name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
+
+
+def test_instances_inference_and_a_single_frame_table(oracle):
+    """Inference pass (no context), a [num_instance, 4, 3] pose tensor, the combined SH kernel path."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    T, ids, model, cam = _setup(scene, 4, 51, frames=1, frame=0)
+    cam.frame_local_id = None          # not needed for a single-frame tensor
+    op = GaussianSplatOp(op_config(scene, DFVT))
+    op.overlap_sh_colors = False
+    T_dev = torch.from_numpy(T[0]).cuda()
+    _, table = op.instance_table(model, cam, T_dev)
+    P = oracle_params(oracle, scene, DFVT, training=False)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                         instances=(ids, table.cpu().numpy()))
+    out, ctx = op.forward(model, cam, training=False, instance2world_T=T_dev)
+    assert ctx is None
+    assert np.array_equal(out.radii.cpu().numpy().reshape(-1), ref["radii"])
+    assert np.abs(out.color.cpu().numpy()[0] - ref["color"]).max() <= 1e-5
+    assert np.array_equal(out.n_contrib.cpu().numpy()[0], ref["n_contrib"])
+
+
+def test_instances_through_autograd_entry_point_and_bundle(oracle):
+    """rasterize_gaussians with instance poses; a two-camera bundle picks each camera's frame by frame_ids."""
+    import torch
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatOp, rasterize_gaussians
+    scene = gen_scene(0)
+    T, ids, model, cam = _setup(scene, 3, 52, frames=3, frame=2)
+    op = GaussianSplatOp(op_config(scene, AABB))
+    T_dev = torch.from_numpy(T).cuda()
+    model.act_applied = False
+    model.set_requires_grad(True)
+    out = rasterize_gaussians(model, cam, op, training=True, instance2world_T=T_dev)
+    (out.color * torch.from_numpy(scene.drgb).cuda()).sum().backward()
+
+    P = oracle_params(oracle, scene, AABB)
+    args = (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    inst = (ids, oracle.instance_cameras(scene.cam2world_T, T[2]))
+    ref = oracle.forward(P, *args, instances=inst)
+    assert np.abs(out.color.detach().cpu().numpy()[0] - ref["color"]).max() <= 1e-5
+    _, pb = oracle.backward(P, ref, *args, scene.drgb[0], np.zeros_like(scene.dT[0]), instances=inst)
+    for name, tns in (("dxyz", model.xyz), ("dscale", model.scale), ("dquat", model.quaternion_xyzw),
+                      ("dopacity", model.opacity)):
+        ok, worst, nbad = grad_close(tns.grad.cpu().numpy(), pb[name], rel=1e-3, abs_frac=1e-4)
+        assert ok, f"{name}: {nbad} bad (worst {worst:.2f}x)"
+
+    # bundle: camera 0 renders frame 2, camera 1 renders frame 0
+    bundle = CameraBundle.from_pinhole_cams([cam, cam])
+    bundle.frame_ids = torch.tensor([2, 0], dtype=torch.int64, device="cuda")
+    model.set_requires_grad(False)
+    model.act_applied = True
+    out_b, _ = op.forward(model, bundle, training=False, instance2world_T=T_dev)
+    ref0 = oracle.forward(P, *args, instances=(ids, oracle.instance_cameras(scene.cam2world_T, T[0])))
+    got = out_b.color.cpu().numpy()
+    assert np.abs(got[0] - ref["color"]).max() <= 1e-5 and np.abs(got[1] - ref0["color"]).max() <= 1e-5
+    assert np.abs(ref["color"] - ref0["color"]).max() > 1e-2

@@ -153,7 +153,7 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
         _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
-        _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, stream), "d3gs_preprocess_bwd")
+        _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, None, stream), "d3gs_preprocess_bwd")
     torch.cuda.synchronize()
     for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", dop_io), ("dsh", o_sh)):
         ok, worst, nbad = grad_close(cpu(got), pb_ref[name], rel=1e-6, abs_frac=1e-7)
@@ -164,7 +164,7 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
         _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 1, _capi.ptr(z_xyz), _capi.ptr(z_q),
-        _capi.ptr(z_s), _capi.ptr(z_op), _capi.ptr(z_sh), None, stream), "d3gs_preprocess_bwd (cleared outputs)")
+        _capi.ptr(z_s), _capi.ptr(z_op), _capi.ptr(z_sh), None, None, stream), "d3gs_preprocess_bwd (cleared outputs)")
     torch.cuda.synchronize()
     for a, b in ((o_xyz, z_xyz), (o_q, z_q), (o_s, z_s), (dop_io, z_op), (o_sh, z_sh)):
         assert torch.equal(a, b), "cleared-output mode changed a gradient"

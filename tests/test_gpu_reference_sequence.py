@@ -35,7 +35,7 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     cov2d, ne0 = torch.empty((N, 3), dtype=f32, device=dev), torch.empty(N, dtype=torch.uint8, device=dev)
     _capi.check(L.d3gs_preprocess_fwd(C.byref(P), p(model.xyz), p(model.quaternion_xyzw), p(model.scale), p(model.opacity),
                                       p(model.color_sh), None, None, p(depths), p(radii), p(uvs), p(conic), p(touched),
-                                      p(rgb), p(cov2d), p(ne0), None, None, s), "preprocess")
+                                      p(rgb), p(cov2d), p(ne0), None, None, None, s), "preprocess")
     cpu = lambda t: t.cpu().numpy()
     assert np.array_equal(cpu(touched), ref["tiles_touched"])
     assert np.array_equal(cpu(rgb).view(np.uint32), ref["rgb_gaussian"].view(np.uint32))
@@ -94,7 +94,7 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     dkeys_a, dkeys_b = torch.empty(N, dtype=i32, device=dev), torch.empty(N, dtype=i32, device=dev)
     _capi.check(L.d3gs_preprocess_fwd(C.byref(P), p(model.xyz), p(model.quaternion_xyzw), p(model.scale), p(model.opacity),
                                       p(model.color_sh), None, None, p(depths), p(radii), p(uvs), p(conic), p(touched),
-                                      p(rgb), p(cov2d), p(ne0), p(tile_masks), p(dkeys_a), s), "preprocess (masks, keys)")
+                                      p(rgb), p(cov2d), p(ne0), p(tile_masks), p(dkeys_a), None, s), "preprocess (masks, keys)")
     cap = M + 1000
     ord_a, ord_b, offs = (torch.empty(N, dtype=i32, device=dev) for _ in range(3))
     tk_a, tk_b, ix_a, ix_b = (torch.empty(cap, dtype=i32, device=dev) for _ in range(4))
