@@ -1,8 +1,8 @@
 // Per-gaussian kernels: preprocess forward (projection, EWA covariance, conic,
-// radius, tile count, SH colour) and preprocess backward (chain rule back to the
-// raw model tensors).  One thread per gaussian, 128-thread workgroups whose SH rows
-// (and SH gradient rows) pass through LDS so that global traffic is coalesced; both
-// are single streaming passes bound by HBM bandwidth.
+// radius, tile count), the SH colours, and preprocess backward (chain rule back to the
+// raw model tensors).  One thread per gaussian; the SH rows (and, in the backward, the SH
+// gradient rows of the gaussians that carry gradient) pass through LDS so that global
+// traffic is coalesced.  All are single streaming passes over the model arrays.
 //
 // Reference: d3sim/algos/d3gs/render.py:421-476, 569-619 (forward) and
 // 3217-3356 (backward); math in d3sim/csrc/gs3d.py and d3sim/csrc/camera.py.
@@ -40,24 +40,15 @@ __device__ __forceinline__ float sh_channel(int degree, float x, float y, float 
 constexpr int kPrepBlock = 128;   // gaussians (= threads) per workgroup of the per-gaussian kernels
 constexpr int kShColorBlocks = 512;   // two workgroups per CU for the SH colour kernel
 
-// Rows of `rowlen` floats per gaussian move between global memory and LDS with consecutive threads on
+// Rows of `rowlen` floats per gaussian move from global memory into LDS with consecutive threads on
 // consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
 // different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
-// row_active (LDS, one byte per row, may be NULL): groups of four elements that lie entirely in rows marked 0
-// are neither read nor written.
-__device__ __forceinline__ bool rows_group_skipped(const unsigned char* row_active, int e4, int total, float inv) {
-    if (!row_active) return false;
-    const int g0 = (int)(((float)e4 + 0.5f) * inv), g1 = (int)(((float)min(e4 + 3, total - 1) + 0.5f) * inv);
-    return !row_active[g0] && !row_active[g1];
-}
-
 __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
-                                                   int stride, const unsigned char* row_active = nullptr) {
+                                                   int stride) {
     const int total = nrows * rowlen;
     const float inv = 1.0f / (float)rowlen;
     const bool vec = ((uintptr_t)src & 15u) == 0;
     for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
-        if (rows_group_skipped(row_active, e4, total, inv)) continue;
         float v[4];
         if (vec && e4 + 3 < total) {
             const float4 t = *reinterpret_cast<const float4*>(src + e4);
@@ -73,30 +64,6 @@ __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src
                 const int g = (int)(((float)e + 0.5f) * inv);
                 lds[g * stride + (e - g * rowlen)] = v[c];
             }
-        }
-    }
-}
-
-__device__ __forceinline__ void rows_lds_to_global(float* __restrict__ dst, const float* lds, int nrows, int rowlen,
-                                                   int stride, const unsigned char* row_active = nullptr) {
-    const int total = nrows * rowlen;
-    const float inv = 1.0f / (float)rowlen;
-    const bool vec = ((uintptr_t)dst & 15u) == 0;
-    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
-        if (rows_group_skipped(row_active, e4, total, inv)) continue;
-        float v[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int e = min(e4 + c, total - 1);
-            const int g = (int)(((float)e + 0.5f) * inv);
-            v[c] = lds[g * stride + (e - g * rowlen)];
-        }
-        if (vec && e4 + 3 < total) {
-            *reinterpret_cast<float4*>(dst + e4) = make_float4(v[0], v[1], v[2], v[3]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                if (e4 + c < total) dst[e4 + c] = v[c];
         }
     }
 }
@@ -317,15 +284,14 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
 // registers before that channel's gradients overwrite them).
 __device__ __forceinline__ void preprocess_bwd_one(
     const d3gs_params& P, const int i, const float* __restrict__ xyz, const float* __restrict__ quat,
-    const float* __restrict__ scale, const float* __restrict__ opacity, const int32_t* __restrict__ radii,
-    const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
+    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ cov2d,
+    const uint8_t* __restrict__ ne0,
     // the blend backward's record of this gaussian: duv(2) dconic(3) dopacity dcolor(3) dz
     const float4 ra, const float4 rb, const float4 rc,
     const int sh_mask_compat,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* shrow, float* __restrict__ dsh_base) {
     const int K = P.sh_stride;
-    float* dshp = shrow;
 
     const float* W = P.w2c;
     float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
@@ -475,10 +441,9 @@ __device__ __forceinline__ void preprocess_bwd_one(
         cg[1] = rb.w * ((m & 2) ? 0.0f : 1.0f);
         cg[2] = rc.x * ((m & 1) ? 0.0f : 1.0f);
     }
-    const float* shp = shrow;
-    const float* rest = P.has_sh_base ? shp : shp + 3;
-    float* drest = P.has_sh_base ? dshp : dshp + 3;
-    float* dbase = P.has_sh_base ? dsh_base + 3 * i : dshp;
+    const float* rest = P.has_sh_base ? shrow : shrow + 3;
+    float* drest = P.has_sh_base ? shrow : shrow + 3;
+    float* dbase = P.has_sh_base ? dsh_base + 3 * i : shrow;
     const int deg = P.sh_degree;
     // coefficients above the evaluated degree receive zero gradient
     const int used = (deg + 1) * (deg + 1) - 1;
@@ -682,7 +647,7 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
             const int g = first + s_list[base + tid];
             d3gs_params Pg = P;
             if constexpr (kInstances) apply_instance(Pg, inst, g);
-            preprocess_bwd_one(Pg, g, xyz, quat, scale, opacity, radii, cov2d, ne0, rec4[4 * (size_t)g],
+            preprocess_bwd_one(Pg, g, xyz, quat, scale, opacity, cov2d, ne0, rec4[4 * (size_t)g],
                                rec4[4 * (size_t)g + 1], rec4[4 * (size_t)g + 2], sh_mask_compat, dxyz, dquat, dscale,
                                dopacity_out, s_rows + tid * stride, dsh_base);
         }

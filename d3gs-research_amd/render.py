@@ -47,10 +47,10 @@ class GaussianSplatOpContext:
     per_gaussian_snap: None = None
     # not in the reference: tile ids by descending list length, the blend kernels' launch order
     tile_order: torch.Tensor | None = None
-    # not in the reference: the backward's [N, 16] gradient records, zero-filled during the forward pass
-    # on the second stream (consumed by the first backward over this context)
+    # not in the reference: the backward's [N, 16] gradient records, cleared by the forward blend kernel
+    # (consumed by the first backward over this context)
     grad_records: torch.Tensor | None = None
-    # float32 pool for the model gradients of this view, cleared beside the forward pass (see _grad_views)
+    # float32 pool for the model gradients of this view, cleared with the records (see _grad_views)
     grad_pool: torch.Tensor | None = None
     # the allocation behind grad_records and grad_pool, until the forward blend has been asked to clear it
     grad_clear: torch.Tensor | None = None
@@ -160,11 +160,11 @@ class GaussianSplatOp:
         # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
         self.overlap_sh_colors = True
         # size the pair buffers from the previous view's count instead of waiting for this view's
-        # the speculative binning of a view (depth order .. tile ranges) goes out as one library call
-        self.fused_binning = True
-        # training: the model-gradient arrays are allocated with the forward pass and cleared beside it
-        self.clear_gradients_early = True
         self.speculative_pair_buffers = True
+        # the binning of such a view (depth order .. tile ranges) goes out as one library call
+        self.fused_binning = True
+        # training: the model-gradient arrays are allocated with the forward pass and cleared by its blend kernel
+        self.clear_gradients_early = True
         self._pair_capacity = 0
         self._count_host: torch.Tensor | None = None
         self._side_stream: torch.cuda.Stream | None = None
@@ -181,9 +181,13 @@ class GaussianSplatOp:
             "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
             # builtin colours off: the kernels blend zeros in their place (render.py:262, 662, 1898-1931)
             "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
-            "move_opacity_in_grad_to_prep": c.move_opacity_in_grad_to_prep,
-            "use_int64_tile_touched": c.use_int64_tile_touched,
-            # rasterize_backward_algo = PER_GAUSSIAN is accepted: the reference's second backward
+            # Accepted without a code path of their own, because they change how the reference computes and not
+            # what: move_opacity_in_grad_to_prep (render.py:1973-1990, 2995-3003) takes the factors opacity, -1/2
+            # and -1 out of the per-pixel gradient terms and applies them once per gaussian -- the same gradient up
+            # to rounding; the blend backward here applies the conic factors once per tile and gaussian in any
+            # case, and taking the opacity out as well measured no gain; use_int64_tile_touched (render.py:657-660)
+            # widens the tile counters for views beyond 2^31 pairs, while this build stops at 2^30 pairs per
+            # camera with an error; rasterize_backward_algo = PER_GAUSSIAN is accepted: the reference's second backward
             # (render.py:2319-2776) computes the same gradient with fewer atomics per gaussian, which the one
             # backward kernel here already has (one record-wide atomic per tile and gaussian)
         }

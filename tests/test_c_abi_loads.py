@@ -82,6 +82,7 @@ def test_operator_config_gate():
     GaussianSplatOp(GaussianSplatConfig(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN))
     GaussianSplatOp(GaussianSplatConfig(disable_builtin_rgb=True, render_rgba=True, render_depth=True,
                                         enable_anti_aliasing=True))
+    GaussianSplatOp(GaussianSplatConfig(move_opacity_in_grad_to_prep=True, use_int64_tile_touched=True))
     for kw, word in ((dict(sparse_mode=True), "sparse_mode"), (dict(render_inv_depth=True), "render_inv_depth"),
                      (dict(enable_32bit_sort=True), "enable_32bit_sort"), (dict(tile_size=(8, 8)), "tile_size"),
                      (dict(disable_builtin_rgb=True, use_nchw=True), "use_nchw")):
