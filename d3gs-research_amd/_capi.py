@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -34,7 +34,7 @@ class Params(C.Structure):
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
-        ("enable_anti_aliasing", C.c_int32),
+        ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
     ]
 
 

@@ -15,6 +15,7 @@
 
 namespace d3gs {
 
+constexpr int kDepthStepBits = 18;  // depth bits of the 32-bit sort key (render.py:737, 768)
 constexpr int kTile = 16;          // tile edge in pixels (config tile_size, config_def.py:79)
 constexpr int kBlock = 256;        // threads per tile / per 1-D block (csrc/inliner.py:38)
 
@@ -510,5 +511,12 @@ __device__ constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f,
 void set_error(const char* fmt, ...);
 // Validates sizes / enum values of a params block (defined in preprocess.hip).
 int check_params(const d3gs_params* p, const char* who);
+
+// Depth part of a gaussian's sort key (render.py:767-775): the float bits (positive floats order like their
+// bit patterns), or with enable_32bit_sort the depth in steps of depth_32bit_prec, truncated to 18 bits.
+__device__ __forceinline__ uint32_t depth_sort_key(const d3gs_params& P, float z) {
+    if (P.enable_32bit_sort) return (uint32_t)(z / P.depth_32bit_prec) & ((1u << kDepthStepBits) - 1u);
+    return __float_as_uint(z);
+}
 
 }  // namespace d3gs

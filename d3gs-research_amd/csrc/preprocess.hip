@@ -213,7 +213,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     if (!in_range) return;
 
     depths[i] = z;
-    if (depth_sort_keys) depth_sort_keys[i] = __float_as_uint(z);   // positive floats order like their bits
+    if (depth_sort_keys) depth_sort_keys[i] = depth_sort_key(P, z);
     radii[i] = (int)radius;
     *reinterpret_cast<float2*>(uvs + 2 * i) = make_float2(u, v);
     *reinterpret_cast<float4*>(conic_opacity + 4 * i) = make_float4(con0, con1, con2, op);
@@ -679,6 +679,11 @@ int check_params(const d3gs_params* p, const char* who) {
     }
     if (p->filter_algo < 0 || p->filter_algo > 4) {
         set_error("%s: unknown early_filter_algo %d", who, p->filter_algo);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p->enable_32bit_sort && (!(p->depth_32bit_prec > 0.0f) || p->tiles_x * p->tiles_y >= (1 << 14))) {
+        // render.py:227-228: 14 bits of tile index above the 18 depth bits
+        set_error("%s: enable_32bit_sort needs depth_32bit_prec > 0 and fewer than 2^14 tiles", who);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     return D3GS_OK;

@@ -174,7 +174,6 @@ class GaussianSplatOp:
         c = self._cfg
         unsupported = {
             "tile_size != (16, 16)": tuple(c.tile_size) != (16, 16),
-            "enable_32bit_sort": c.enable_32bit_sort,
             # the reference stores 1/z in the buffer it also sorts by (render.py:582, 773), which blends
             # back to front: not reproduced
             "render_inv_depth": c.render_inv_depth,
@@ -200,6 +199,9 @@ class GaussianSplatOp:
         """The reference's sorted 64-bit keys, (tile << 32) | depth bits, rebuilt from the last forward's
         sorted tile keys and gaussian indices (parity tests compare them with the oracle's)."""
         tile_keys, idx, depths = self._last_sorted
+        if self._cfg.enable_32bit_sort:     # render.py:767-770, 820: (tile << 18) | depth steps
+            steps = (depths / torch.tensor(self._cfg.depth_32bit_prec, dtype=torch.float32, device=depths.device))
+            return (tile_keys.long() << 18) | (steps.long()[idx.long()] & 0x3FFFF)
         bits = depths.view(torch.int32)[idx.long()].long() & 0xFFFFFFFF
         return (tile_keys.long() << 32) | bits
 
@@ -309,6 +311,9 @@ class GaussianSplatOp:
         P.fused_activation = int(isinstance(model, GaussianModelOriginFused))
         P.render_depth, P.render_rgba = int(c.render_depth), int(c.render_rgba)
         P.use_nchw, P.enable_anti_aliasing = int(c.use_nchw), int(c.enable_anti_aliasing)
+        P.enable_32bit_sort, P.depth_32bit_prec = int(c.enable_32bit_sort), float(c.depth_32bit_prec)
+        if c.enable_32bit_sort:
+            assert P.tiles_x * P.tiles_y < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
         return P
 
     @staticmethod
@@ -370,11 +375,12 @@ class GaussianSplatOp:
         # every zero-initialised work buffer of the forward pass comes out of one fill (the two sorts' and the
         # scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later
         tile_bits = L.d3gs_higher_msb(num_tiles)
+        depth_bits = 18 if P.enable_32bit_sort else 32      # the depth sort's key width (render.py:737)
         spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
         align = lambda v: (v + 255) // 256 * 256
         scan_ws_bytes = C.c_size_t(0)
         _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(scan_ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
-        sizes = [align(_sort_ws_bytes(n, 0, 32)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
+        sizes = [align(_sort_ws_bytes(n, 0, depth_bits)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
                  align(num_tiles * 8), align(scan_ws_bytes.value)]
         zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
         zero_scan_ws = zero_pool[sum(sizes[:3]):]
@@ -496,8 +502,8 @@ class GaussianSplatOp:
             # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
             # tile digits only: 2 passes over M pairs instead of 6.
             with self._stage("depth_order"):
-                depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, 32,
-                                                          values_are_indices=True, zero_ws=zero_ws_n)
+                depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0,
+                                                          depth_bits, values_are_indices=True, zero_ws=zero_ws_n)
 
             with self._stage("scan"):
                 # tile counts gathered into depth order and scanned in one launch

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 21
+#define D3GS_ABI_VERSION 22
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -81,6 +81,10 @@ typedef struct d3gs_params {
     int32_t render_rgba;          /* colour has a fourth channel, the sum of the blend weights (render.py:1899-1906) */
     int32_t use_nchw;             /* colour / drgb stored [C,H,W] instead of [H,W,C] (render.py:702, 2272-2294) */
     int32_t enable_anti_aliasing; /* conic without eps and opacity *= sqrt(det / det_lowpass) (render.py:391-407) */
+    int32_t enable_32bit_sort;    /* the depth part of the sort key is uint32(depth / depth_32bit_prec) & 0x3FFFF instead
+                                     of the float bits (render.py:767-770, 853-854): gaussians of a tile that fall into
+                                     the same depth step are blended in index order.  At most 2^14 tiles. */
+    float depth_32bit_prec;       /* config_def.py:91, default 0.001 */
 } d3gs_params;
 
 int d3gs_abi_version(void);
@@ -113,8 +117,9 @@ typedef struct d3gs_instances {
  * d3gs_make_keys expands instead of repeating the per-tile tests.
  * rgb_gaussian may be NULL: the SH colour (and sh_to_rgb_ne_0) is then left to d3gs_sh_colors, which a
  * caller can run on a second stream beside the sort, the only consumer being the blend.
- * depth_sort_keys (uint32[N], may be NULL): the float bits of depths, the keys of the depth sort
- * (saves the d3gs_depth_keys pass). */
+ * depth_sort_keys (uint32[N], may be NULL): the keys of the depth sort, the float bits of depths or, with
+ * enable_32bit_sort, the 18-bit depth steps (saves the d3gs_depth_keys pass; the depth sort then runs on bits
+ * [0, 32) or [0, 18)). */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const float* color_sh_base,
                         const uint8_t* invalid_mask, float* depths,

@@ -29,7 +29,8 @@
 //                                  stated invariant, render.py:1051-1072); the
 //                                  third-party cumm OBBCornersGridOverlap::inc_step
 //                                  rounding is absent here -> "parity unpinned"
-//   orc_scan/make_keys/sort/ranges : numpy cumsum + stable argsort, partition invariants
+//   orc_scan/make_keys/sort/ranges : numpy cumsum + stable argsort, partition invariants; the 32-bit
+//                                  key mode against numpy float32 division + stable lexsort
 //   orc_blend_fwd                : float64 dense per-pixel restatement in numpy
 //   orc_blend_bwd / orc_preprocess_bwd : float64 torch autograd of the forward
 //                                  (straight-through alpha clamp) + finite differences
@@ -90,6 +91,8 @@ struct orc_params {
     int32_t render_rgba;           // fourth colour channel = sum of blend weights (render.py:1899-1906)
     int32_t use_nchw;              // colour image stored [C,H,W] instead of [H,W,C] (render.py:702)
     int32_t enable_anti_aliasing;  // opacity scaled by sqrt(det / det_lowpass) (render.py:391-407)
+    int32_t enable_32bit_sort;     // key = (tile << 18) | (uint32(depth / prec) & 0x3FFFF) (render.py:767-770, 820)
+    float depth_32bit_prec;        // config_def.py:91
 };
 
 // ---------------------------------------------------------------------------
@@ -553,11 +556,14 @@ ORC_API void orc_make_keys(const orc_params* P, const int32_t* radii, const floa
         int64_t off = i == 0 ? 0 : offsets[i - 1];
         uint32_t dbits;
         memcpy(&dbits, depths + i, 4);
+        // render.py:767-775: the float bits, or the depth in steps of depth_32bit_prec cut to 18 bits
+        if (P->enable_32bit_sort) dbits = (uint32_t)(depths[i] / P->depth_32bit_prec) & 0x3FFFFu;
+        const int shift = P->enable_32bit_sort ? 18 : 32;   // render.py:737
         TileWalkIn g{uvs[2 * i], uvs[2 * i + 1], (float)radii[i],
                      {conic_opacity[4 * i], conic_opacity[4 * i + 1], conic_opacity[4 * i + 2]}, conic_opacity[4 * i + 3]};
         tile_walk(P, g, [&](int x, int y) {
             uint64_t key = (uint64_t)(y * P->tiles_x + x);
-            keys[off] = (key << 32) | dbits;
+            keys[off] = (key << shift) | dbits;
             vals[off] = i;
             ++off;
         });
@@ -595,14 +601,14 @@ ORC_API void orc_sort_pairs(const uint64_t* keys_in, const int32_t* vals_in, uin
 }
 
 // K5: per-tile [start,end) in the sorted list (render.py:897-939). ranges must be zero-filled.
-ORC_API void orc_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* ranges, int32_t num_tiles) {
+ORC_API void orc_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t* ranges, int32_t num_tiles, int32_t shift) {
     (void)num_tiles;
     for (int64_t i = 0; i < m; ++i) {
-        uint32_t t = (uint32_t)(keys_sorted[i] >> 32);
+        uint32_t t = (uint32_t)(keys_sorted[i] >> shift);
         if (i == 0) {
             ranges[2 * t] = 0;
         } else {
-            uint32_t tp = (uint32_t)(keys_sorted[i - 1] >> 32);
+            uint32_t tp = (uint32_t)(keys_sorted[i - 1] >> shift);
             if (t != tp) {
                 ranges[2 * tp + 1] = (int32_t)i;
                 ranges[2 * t] = (int32_t)i;

@@ -33,7 +33,7 @@ class OracleParams(C.Structure):
         ("lowpass", C.c_float), ("alpha_eps", C.c_float), ("transmittance_eps", C.c_float),
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
-        ("enable_anti_aliasing", C.c_int32),
+        ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
     ]
 
 
@@ -75,7 +75,8 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
                 has_sh_base=False, filter_algo=FILTER_NONE, training=True, near=0.2, far=10000.0, eps=1e-6,
                 radii_eigen_eps=0.1, clamp_factor=1.3, std_sigma=3.0, lowpass=0.3, alpha_eps=1.0 / 255.0,
                 transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0), fused_activation=True,
-                render_depth=False, render_rgba=False, use_nchw=False, enable_anti_aliasing=False) -> OracleParams:
+                render_depth=False, render_rgba=False, use_nchw=False, enable_anti_aliasing=False,
+                enable_32bit_sort=False, depth_32bit_prec=0.001) -> OracleParams:
     """cam2world_T is the 4x3 matrix ``to_world[:3].T`` (render.py:205-206)."""
     P = OracleParams()
     P.n, P.width, P.height = int(n), int(width), int(height)
@@ -99,6 +100,9 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
     P.fused_activation = int(bool(fused_activation))
     P.render_depth, P.render_rgba = int(bool(render_depth)), int(bool(render_rgba))
     P.use_nchw, P.enable_anti_aliasing = int(bool(use_nchw)), int(bool(enable_anti_aliasing))
+    P.enable_32bit_sort, P.depth_32bit_prec = int(bool(enable_32bit_sort)), float(depth_32bit_prec)
+    if P.enable_32bit_sort:
+        assert P.tiles_x * P.tiles_y < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
     return P
 
 
@@ -204,9 +208,11 @@ def sort_pairs(keys, vals, begin_bit, end_bit):
     return ko, vo
 
 
-def tile_ranges(keys_sorted, num_tiles):
+def tile_ranges(keys_sorted, num_tiles, shift=32):
+    """shift: where the tile index starts in the key, 32 or (32-bit sort) 18 (render.py:900)."""
     r = np.zeros((num_tiles, 2), np.int32)
-    lib().orc_tile_ranges(_p(keys_sorted), C.c_int64(keys_sorted.shape[0]), _p(r), C.c_int32(num_tiles))
+    lib().orc_tile_ranges(_p(keys_sorted), C.c_int64(keys_sorted.shape[0]), _p(r), C.c_int32(num_tiles),
+                          C.c_int32(shift))
     return r
 
 
@@ -270,9 +276,10 @@ def forward(P, xyz, quat, scale, opacity, sh, sh_base=None, invalid_mask=None, i
     offsets, m = scan(pre["tiles_touched"])
     num_tiles = P.tiles_x * P.tiles_y
     keys, vals = make_keys(P, pre["radii"], pre["uvs"], pre["conic_opacity"], pre["depths"], offsets, m)
-    end_bit = 32 + higher_msb(num_tiles)
+    # render.py:850-854, 900: 64-bit keys are sorted up to the tile bits in use, 32-bit keys whole
+    end_bit = 32 if P.enable_32bit_sort else 32 + higher_msb(num_tiles)
     ks, vs = sort_pairs(keys, vals, 0, end_bit)
-    ranges = tile_ranges(ks, num_tiles)
+    ranges = tile_ranges(ks, num_tiles, 18 if P.enable_32bit_sort else 32)
     color, T, nc, depth = blend_fwd(P, ranges, vs, pre["uvs"], pre["conic_opacity"], pre["rgb_gaussian"], pre["depths"])
     out = dict(pre)
     out.update(offsets=offsets, num_rendered=m, keys=keys, vals=vals, keys_sorted=ks, gaussian_idx_sorted=vs,

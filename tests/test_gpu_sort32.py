@@ -1,0 +1,78 @@
+"""GPU parity for enable_32bit_sort (render.py:227-228, 737, 767-770, 820, 853-854, 900): the sort key carries 18
+bits of depth steps under the tile index, gaussians of a tile within one step blend in index order.  Sorted keys,
+tile lists and ranges bit-exact against the oracle, images and gradients to the bars of the default path, on both
+binning paths (one library call from the second view on, launch by launch on the first)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import gen_scene, grad_close, op_config, oracle_forward, torch_model
+
+pytestmark = pytest.mark.gpu
+
+AABB, DFVT = 1, 4
+
+
+@pytest.mark.parametrize("cfg_id,n,wh,filt,prec", [(0, None, None, AABB, 0.001), (1, 20000, (250, 190), DFVT, 0.05),
+                                                   (2, 200000, (960, 540), DFVT, 0.001), (2, None, None, DFVT, 0.001)])
+def test_32bit_sort_forward_and_backward(oracle, cfg_id, n, wh, filt, prec):
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    print(f"32-bit sort cfg={cfg_id} n={scene.n} prec={prec}", flush=True)
+    P, ref = oracle_forward(oracle, scene, filt, enable_32bit_sort=True, depth_32bit_prec=prec)
+    op = GaussianSplatOp(op_config(scene, filt, enable_32bit_sort=True, depth_32bit_prec=prec))
+    model = torch_model(scene)
+    cpu = lambda t: t.detach().cpu().numpy()
+    for view in range(2):       # the second view sizes its buffers from the first and bins in one call
+        out, ctx = op.forward(model, scene.camera(), training=True)
+        torch.cuda.synchronize()
+        assert op.last_num_rendered == ref["num_rendered"] > 0
+        assert np.array_equal(cpu(op._last_keys_sorted).view(np.uint64), ref["keys_sorted"]), view
+        assert np.array_equal(cpu(ctx.gaussian_idx_sorted), ref["gaussian_idx_sorted"]), view
+        assert np.array_equal(cpu(ctx.workload_ranges), ref["workload_ranges"]), view
+        assert np.array_equal(cpu(out.n_contrib)[0], ref["n_contrib"])
+        assert np.array_equal(cpu(out.color)[0].view(np.uint32), ref["color"].view(np.uint32))
+        assert np.array_equal(cpu(out.T)[0].view(np.uint32), ref["T"].view(np.uint32))
+    g_ref, pb_ref = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                    scene.color_sh, scene.drgb[0], scene.dT[0])
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    gm, _, _ = op.backward(model, scene.camera(), ctx, out, grads)
+    torch.cuda.synchronize()
+    g = op.last_raster_grads
+    mass = g_ref["absmass"]
+    for name, got, cols in (("duv", g.duv, slice(0, 2)), ("dconic", g.dconic, slice(2, 5)),
+                            ("dopacity", g.dopacity, slice(5, 6)), ("dcolor", g.dcolor, slice(6, 9))):
+        a, b = cpu(got).astype(np.float64).reshape(scene.n, -1), g_ref[name].reshape(scene.n, -1)
+        assert (np.abs(a - b) <= 1e-4 * mass[:, cols] + 1e-30).all(), name
+    for name, got in (("dxyz", gm.xyz), ("dscale", gm.scale), ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
+        a = cpu(got).astype(np.float64).reshape(scene.n, -1)
+        b = pb_ref[name].astype(np.float64).reshape(scene.n, -1)
+        rn = np.linalg.norm(b, axis=1)
+        e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
+        med, p99 = np.quantile(e, [0.5, 0.99])
+        assert med <= 1e-4 and p99 <= 5e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
+
+
+def test_32bit_sort_differs_from_the_default_order_and_rejects_large_tile_grids(oracle):
+    import torch
+    from d3gs_research_amd import _capi
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    model = torch_model(scene)
+    a = GaussianSplatOp(op_config(scene, AABB, enable_32bit_sort=True, depth_32bit_prec=0.05))
+    b = GaussianSplatOp(op_config(scene, AABB))
+    _, ca = a.forward(model, scene.camera(), training=True)
+    _, cb = b.forward(model, scene.camera(), training=True)
+    assert torch.equal(ca.workload_ranges, cb.workload_ranges)
+    assert not torch.equal(ca.gaussian_idx_sorted, cb.gaussian_idx_sorted)
+    # 3840x2160 has 32400 tiles: more than 14 bits (render.py:227-228)
+    big = gen_scene(4, n=1000)
+    with pytest.raises(AssertionError, match="14 bits"):
+        GaussianSplatOp(op_config(big, AABB, enable_32bit_sort=True)).forward(torch_model(big), big.camera())
+    P = GaussianSplatOp(op_config(big, AABB)).make_params(torch_model(big), big.camera(), False)
+    P.enable_32bit_sort, P.depth_32bit_prec = 1, 0.001
+    L = _capi.lib()
+    assert L.d3gs_blend_fwd(C.byref(P), *([None] * 11 + [None, 0, None])) == -1
+    assert b"2^14 tiles" in L.d3gs_last_error_string()

@@ -166,3 +166,48 @@ def test_ellipse_filter_is_the_exact_ellipse_box_test(oracle, make):
             decided += 1
             dropped += t not in s_ell[g]
     assert decided > 1000 and dropped > 50
+
+
+@pytest.mark.parametrize("prec", [0.001, 0.05])
+def test_32bit_sort_keys_order_and_ties(oracle, prec):
+    """enable_32bit_sort (render.py:227-228, 737, 767-770, 820, 853-854, 900): key = (tile << 18) |
+    (uint32(depth / prec) & 0x3FFFF), sorted whole as 32 bits by a stable sort, so gaussians of a tile that share
+    a depth step keep index order.  Pinned with numpy: float32 division, truncation, stable lexsort."""
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    P64, ref64 = oracle_forward(oracle, scene, AABB)
+    P, ref = oracle_forward(oracle, scene, AABB, enable_32bit_sort=True, depth_32bit_prec=prec)
+    m = ref["num_rendered"]
+    assert m == ref64["num_rendered"] > 0 and np.array_equal(ref["vals"], ref64["vals"])
+    # the unsorted keys: same tiles as the 64-bit keys, depth steps from the depths
+    tiles = (ref64["keys"] >> np.uint64(32)).astype(np.uint64)
+    steps = (ref["depths"] / np.float32(prec)).astype(np.uint32) & np.uint32(0x3FFFF)
+    assert np.array_equal(ref["keys"], (tiles << np.uint64(18)) | steps[ref["vals"]].astype(np.uint64))
+    assert int(ref["keys"].max()) < 2 ** 32
+    # stable sort on the whole key == lexsort by (tile, step), ties in emission order (ascending gaussian index)
+    order = np.lexsort((np.arange(m), steps[ref["vals"]], tiles))
+    assert np.array_equal(ref["keys_sorted"], ref["keys"][order])
+    assert np.array_equal(ref["gaussian_idx_sorted"], ref["vals"][order])
+    assert np.array_equal(ref["workload_ranges"], ref64["workload_ranges"])
+    # inside a tile: steps ascend, and equal steps list ascending gaussian indices
+    lo, hi = max(ref["workload_ranges"], key=lambda r: r[1] - r[0])
+    seg_steps, seg_idx = steps[ref["gaussian_idx_sorted"][lo:hi]], ref["gaussian_idx_sorted"][lo:hi]
+    assert hi - lo > 20 and (np.diff(seg_steps.astype(np.int64)) >= 0).all()
+    same = np.diff(seg_steps.astype(np.int64)) == 0
+    assert (np.diff(seg_idx)[same] > 0).all()
+    if prec > 0.01:
+        # coarse steps: ties exist and reorder the lists against the exact depth order, so the image moves
+        assert same.any() and not np.array_equal(ref["gaussian_idx_sorted"], ref64["gaussian_idx_sorted"])
+        assert np.abs(ref["color"] - ref64["color"]).max() > 1e-4
+    else:
+        # 1 mm steps on this scene: a few ties at most, the image stays within blending-order noise
+        assert np.abs(ref["color"] - ref64["color"]).max() < 0.2
+
+
+def test_32bit_sort_depth_steps_wrap_at_18_bits(oracle):
+    """Depth steps beyond 2^18 wrap (the mask in render.py:769): with 1e-5 steps a depth of 3 sorts as 300000 - 262144."""
+    scene = gen_scene(0, n=800)
+    P, ref = oracle_forward(oracle, scene, NONE, enable_32bit_sort=True, depth_32bit_prec=1e-5)
+    steps = (ref["depths"] / np.float32(1e-5)).astype(np.uint32)
+    assert (steps[ref["radii"] > 0] >= 2 ** 18).any()
+    got = (ref["keys"] & np.uint64(0x3FFFF)).astype(np.uint32)
+    assert np.array_equal(got, (steps & np.uint32(0x3FFFF))[ref["vals"]])
