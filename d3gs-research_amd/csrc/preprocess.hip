@@ -721,7 +721,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     if (p->n == 0) return D3GS_OK;
     const bool with_sh = rgb_gaussian != nullptr;
     if (!xyz || !quaternion_xyzw || !scale || !opacity || !depths || !radii || !uvs || !conic_opacity ||
-        !tiles_touched || (with_sh && (!color_sh || (p->has_sh_base && !color_sh_base)))) {
+        !tiles_touched || (with_sh && ((!color_sh && p->sh_stride > 0) || (p->has_sh_base && !color_sh_base)))) {
         set_error("d3gs_preprocess_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
@@ -748,7 +748,7 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
     int rc = check_params(p, "d3gs_sh_colors");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
-    if (!xyz || !color_sh || !radii || !rgb_gaussian || (p->has_sh_base && !color_sh_base)) {
+    if (!xyz || (!color_sh && p->sh_stride > 0) || !radii || !rgb_gaussian || (p->has_sh_base && !color_sh_base)) {
         set_error("d3gs_sh_colors: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
@@ -778,9 +778,10 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
     int rc = check_params(p, "d3gs_preprocess_bwd");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
-    if (!xyz || !quaternion_xyzw || !scale || !opacity || !color_sh || !radii || !cov2d_vecs || !sh_to_rgb_ne_0 ||
+    // a model whose only colour coefficient is the split-off DC term has empty color_sh arrays (sh_stride 0)
+    if (!xyz || !quaternion_xyzw || !scale || !opacity || !radii || !cov2d_vecs || !sh_to_rgb_ne_0 ||
         !grad_records || !dxyz || !dquaternion_xyzw || !dscale || !dopacity_out ||
-        !dcolor_sh || (p->has_sh_base && !dcolor_sh_base)) {
+        ((!color_sh || !dcolor_sh) && p->sh_stride > 0) || (p->has_sh_base && !dcolor_sh_base)) {
         set_error("d3gs_preprocess_bwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }

@@ -120,3 +120,38 @@ def test_non_fused_model_family(oracle, cfg_id, n, wh, filt):
         e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = np.quantile(e, [0.5, 0.99])
         assert med <= 1e-4 and p99 <= 5e-3, f"{name}: fused vs torch-activated median {med:.2e} p99 {p99:.2e}"
+
+
+def test_dc_only_model_with_split_base(oracle):
+    """A degree-0 model that keeps its one colour coefficient in color_sh_base has an empty color_sh [N, 0, 3]
+    (origin/model.py:34-48): it renders and differentiates like the unsplit model, bit for bit."""
+    import torch
+    from d3gs_research_amd.model import GaussianModelOriginFused
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(0)
+    op = GaussianSplatOp(op_config(scene, AABB))
+    whole = torch_model(scene)
+    split = GaussianModelOriginFused(xyz=whole.xyz, quaternion_xyzw=whole.quaternion_xyzw, scale=whole.scale,
+                                     opacity=whole.opacity, color_sh=whole.color_sh[:, 1:].contiguous(),
+                                     color_sh_base=whole.color_sh[:, 0].contiguous(), cur_sh_degree=0, act_applied=True)
+    assert tuple(split.color_sh.shape) == (scene.n, 0, 3) and split.color_sh_degree == 0
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    res = []
+    for model in (whole, split):
+        for overlap in (True, False):       # SH colours on their own stream, or inside the preprocess kernel
+            op.overlap_sh_colors = overlap
+            out, ctx = op.forward(model, scene.camera(), training=True)
+            gm, _, _ = op.backward(model, scene.camera(), ctx, out, grads)
+            torch.cuda.synchronize()
+            res.append((out, gm))
+    (o0, g0), (o2, g2) = res[0], res[2]
+    # images bit for bit; gradients up to the order of the backward's atomic float sums
+    close = lambda a, b: torch.allclose(a, b, rtol=1e-4, atol=1e-5 * float(b.abs().max()))
+    for o, g in (res[1], res[2], res[3]):
+        assert torch.equal(o.color, o0.color) and torch.equal(o.T, o0.T)
+        assert close(g.xyz, g0.xyz) and close(g.opacity, g0.opacity) and close(g.scale, g0.scale)
+    assert close(g2.color_sh_base, g0.color_sh[:, 0]) and g2.color_sh.numel() == 0
+    P = oracle_params(oracle, scene, AABB, sh_stride=0, has_sh_base=True)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                         np.zeros((scene.n, 0, 3), np.float32), sh_base=np.ascontiguousarray(scene.color_sh[:, 0]))
+    assert np.array_equal(o2.color.cpu().numpy()[0].view(np.uint32), ref["color"].view(np.uint32))
