@@ -271,9 +271,10 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : depth_sort_key(P, depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
     unsigned long long kept = 0ull, meta = 0ull;
-    if (tile_masks && active) {
-        meta = tile_masks[2 * (size_t)i + 1];
-        if (meta & kTileMaskHas) kept = tile_masks[2 * (size_t)i];
+    if (tile_masks && active) {     // both words in one 16-byte load: one round trip, not two dependent ones
+        const ulonglong2 rec = *reinterpret_cast<const ulonglong2*>(tile_masks + 2 * (size_t)i);
+        kept = rec.x;
+        meta = rec.y;
     }
     const bool has_mask = (meta & kTileMaskHas) != 0;
     const bool walk_again = active && !has_mask;
@@ -561,6 +562,10 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
     if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
         !gaussian_idx) {
         set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if ((uintptr_t)tile_masks & 15u) {     // the two words of a gaussian are read as one 16-byte load
+        set_error("d3gs_make_keys: tile_masks must be 16-byte aligned");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     const dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);

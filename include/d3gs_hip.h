@@ -112,7 +112,7 @@ typedef struct d3gs_instances {
  * early filter, SH colour.  Outputs of rejected gaussians are written as zeros.
  * cov2d_vecs and sh_to_rgb_ne_0 may be NULL (inference). sh_base may be NULL.
  * invalid_mask (uint8[N], may be NULL): non-zero rejects the gaussian (render.py:306-308).
- * tile_masks (uint64[N][2], may be NULL; no counterpart in the reference): a record of the tiles the
+ * tile_masks (uint64[N][2], 16-byte aligned, may be NULL; no counterpart in the reference): a record of the tiles the
  * early filter kept for each gaussian (word 0: bit mask over its candidate rect, word 1: the rect), which
  * d3gs_make_keys expands instead of repeating the per-tile tests.
  * rgb_gaussian may be NULL: the SH colour (and sh_to_rgb_ne_0) is then left to d3gs_sh_colors, which a
