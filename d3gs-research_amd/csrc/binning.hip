@@ -253,6 +253,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                                                             long long m) {
     __shared__ Key s_key[kBlock / 64][kKeyStage];
     __shared__ int32_t s_val[kBlock / 64][kKeyStage];
+    __shared__ int s_start[kBlock / 64][64], s_slot[kBlock / 64][64];
     // no early return: every lane takes part in the cooperative emission of large gaussians
     const int j_raw = blockIdx.x * kBlock + threadIdx.x;
     const bool in_range = j_raw < P.n;
@@ -278,32 +279,47 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     }
     const bool has_mask = (meta & kTileMaskHas) != 0;
     const bool walk_again = active && !has_mask;
-    // The slots of a wavefront's gaussians are consecutive.  When they all come from masks and fit the
-    // staging buffer they are assembled in LDS and leave as whole coalesced segments; otherwise each
-    // lane writes its own run.
-    const long long wave_base = __shfl(off, 0, 64);
-    const long long wave_end = __shfl(end, 63, 64);
-    const bool staged = !__any(walk_again) && !__any(in_range && !sane) && wave_end - wave_base <= kKeyStage &&
-                        wave_end <= m && wave_end >= wave_base;
-    if (staged) {
-        if (has_mask)
-            mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
-                s_key[wave][slot - wave_base] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
-                s_val[wave][slot - wave_base] = i;
-            });
-        __builtin_amdgcn_wave_barrier();
-        const int total = (int)(wave_end - wave_base);
-        for (int sidx = lane; sidx < total; sidx += 64) {
-            keys[wave_base + sidx] = s_key[wave][sidx];
-            vals[wave_base + sidx] = s_val[wave][sidx];
-        }
-        return;   // wave-uniform
+    // The pairs of the wavefront's gaussians that come from masks are assembled in LDS, packed, and leave as
+    // coalesced segments: consecutive lanes write consecutive slots, stepping over the runs of the (few, large)
+    // gaussians that are walked again below.  The owner of packed element e is the last lane whose packed start
+    // is <= e (lanes without pairs share their successor's start), found by a binary search over the starts.
+    const int my_cnt = (active && has_mask) ? (int)(end - off) : 0;
+    int incl = my_cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int t = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += t;
     }
-    if (has_mask)
+    const int start = incl - my_cnt, packed_total = __shfl(incl, 63, 64);
+    const long long wave_base = __shfl(off, 0, 64);
+    const bool staged = packed_total <= kKeyStage && !__any(in_range && !sane);
+    if (staged) {
+        s_start[wave][lane] = start;
+        s_slot[wave][lane] = (int)(off - wave_base);    // a wavefront's slots span far less than 2^31
+        if (has_mask)
+            mask_tile_emit(kept, meta, P.tiles_x, dbits, (long long)start, (long long)(start + my_cnt),
+                           [&](long long e, uint64_t key) {
+                               s_key[wave][e] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
+                               s_val[wave][e] = i;
+                           });
+        __builtin_amdgcn_wave_barrier();
+        for (int e = lane; e < packed_total; e += 64) {
+            int lo = 0, hi = 63;
+#pragma unroll
+            for (int step = 0; step < 6; ++step) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (s_start[wave][mid] <= e) lo = mid; else hi = mid - 1;
+            }
+            const long long slot = wave_base + s_slot[wave][lo] + (e - s_start[wave][lo]);
+            keys[slot] = s_key[wave][e];
+            vals[slot] = s_val[wave][e];
+        }
+    } else if (has_mask) {
         mask_tile_emit(kept, meta, P.tiles_x, dbits, off, end, [&](long long slot, uint64_t key) {
             keys[slot] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
             vals[slot] = i;
         });
+    }
     if (!__any(walk_again)) return;   // wave-uniform
     TileWalk walk = {};
     if (walk_again) {
