@@ -115,7 +115,6 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    import numpy as np
     import torch
     if args.pmc_calibrate:
         x = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")

@@ -23,7 +23,7 @@ import torch
 
 from . import _capi
 from .camera import BasicPinholeCamera
-from .config_def import EarlyFilterAlgo, GaussianSplatConfig, RasterizeBackwardAlgo
+from .config_def import GaussianSplatConfig
 from .model import GaussianModelOriginBase, GaussianModelOriginFused
 
 

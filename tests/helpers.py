@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from d3gs_research_amd.config_def import EarlyFilterAlgo, GaussianSplatConfig
+from d3gs_research_amd.config_def import GaussianSplatConfig
 from d3gs_research_amd.synthetic import Scene, gen_scene, scene_config, scene_model  # noqa: F401
 
 

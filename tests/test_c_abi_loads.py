@@ -75,7 +75,6 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
 
 def test_operator_config_gate():
     """Options the operator carries out construct; the ones it does not raise at construction, by name."""
-    import numpy as np
     from d3gs_research_amd.config_def import GaussianSplatConfig, RasterizeBackwardAlgo
     from d3gs_research_amd.render import GaussianSplatOp
     GaussianSplatOp(GaussianSplatConfig())

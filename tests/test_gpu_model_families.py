@@ -4,7 +4,7 @@
 import numpy as np
 import pytest
 
-from helpers import gen_scene, grad_close, op_config, oracle_forward, oracle_params, torch_model
+from helpers import gen_scene, grad_close, op_config, oracle_params, torch_model
 
 pytestmark = pytest.mark.gpu
 

@@ -7,7 +7,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from helpers import gen_scene, grad_close, op_config, oracle_forward, torch_model
+from helpers import gen_scene, op_config, oracle_forward, torch_model
 
 pytestmark = pytest.mark.gpu
 

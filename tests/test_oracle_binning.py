@@ -4,7 +4,6 @@ argsort for the integer stages, and structural invariants of the result."""
 import numpy as np
 import pytest
 
-from f64_reference import preprocess_f64
 from helpers import gen_scene, oracle_forward
 
 NONE, AABB, ELLIPSE, OBB, DFVT = 0, 1, 2, 3, 4
@@ -77,7 +76,6 @@ def test_scan_keys_sort_ranges(oracle, cfg_id, n, wh, filt):
     assert np.array_equal(ref["offsets"], np.cumsum(tt, dtype=np.int64).astype(np.int32)) and m == int(tt.sum())
     # keys: emitted at [offset[i-1], offset[i]) with value i, low word = float bits of the depth,
     # high word = tile id in row-major order (render.py:773, 809, 830-833)
-    starts = np.concatenate([[0], ref["offsets"][:-1]])
     owner = np.repeat(np.arange(scene.n, dtype=np.int32), tt)
     assert np.array_equal(ref["vals"], owner)
     low = (ref["keys"] & np.uint64(0xFFFFFFFF)).astype(np.uint32)

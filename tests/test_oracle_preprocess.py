@@ -6,7 +6,7 @@ import pytest
 from scipy.spatial.transform import Rotation
 
 from f64_reference import preprocess_f64
-from helpers import gen_scene, oracle_forward, oracle_params
+from helpers import gen_scene, oracle_params
 
 
 def _posed_scene(cfg_id, n, wh=None):

@@ -11,8 +11,7 @@ from scipy.spatial.transform import Rotation
 from d3gs_research_amd import config_def
 from d3gs_research_amd.model import GaussianModelOrigin, GaussianModelOriginFused
 from d3gs_research_amd.render import GaussianSplatOutput
-from d3gs_research_amd.strategy import (GaussianStrategyOrigin, GaussianTrainState, quat_xyzw_to_rotmat,
-                                        reset_param_in_optim)
+from d3gs_research_amd.strategy import GaussianStrategyOrigin, GaussianTrainState, quat_xyzw_to_rotmat
 from d3gs_research_amd.tools import create_origin_3dgs_optimizer
 from d3gs_research_amd.train import ssim
 
