@@ -18,8 +18,8 @@
 // in LDS, then written out by consecutive threads, so equal-digit runs leave as
 // contiguous segments.
 //
-// Look-back protocol: tiles are claimed from an atomic ticket, so a workgroup
-// only ever waits on tiles that started before it.  A status word carries a
+// Look-back protocol: a workgroup's tile is its id, and workgroups are dispatched in
+// id order, so a workgroup only ever waits on tiles that started before it.  A status word carries a
 // 30-bit count and two flag bits (aggregate of this tile / inclusive prefix up
 // to this tile); words are read and written with relaxed device-scope atomics.
 // Polling is bounded: past the limit the workgroup raises an error flag and
@@ -41,7 +41,6 @@ constexpr int kLookWindow = 16;  // predecessor tiles polled per look-back step
 
 struct SortWorkspace {
     uint32_t* hist;     // [passes][256] digit totals of the whole input
-    uint32_t* tickets;  // [passes] next tile to hand out
     uint32_t* error;    // [1] set when a look-back gave up
     uint32_t* status;   // [passes][ntiles][256]
 };
@@ -117,7 +116,6 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
                                                               const long long* __restrict__ m_device, int shift,
                                                               uint32_t mask, int ntiles,
                                                               const uint32_t* __restrict__ hist /* this pass, [256] */,
-                                                              uint32_t* __restrict__ ticket,
                                                               uint32_t* __restrict__ status,
                                                               uint32_t* __restrict__ error) {
     __shared__ int wave_cnt[kOsWaves][kOsRadix];  // running, then exclusive-over-waves, per-wave digit counts
@@ -278,8 +276,6 @@ static size_t os_layout(int64_t m, int passes, SortWorkspace* ws, void* base) {
     char* b = (char*)base;
     if (ws) ws->hist = (uint32_t*)(b + off);
     off += os_align((size_t)passes * kOsRadix * 4);
-    if (ws) ws->tickets = (uint32_t*)(b + off);
-    off += os_align((size_t)passes * 4);
     if (ws) ws->error = (uint32_t*)(b + off);
     off += 256;
     if (ws) ws->status = (uint32_t*)(b + off);
@@ -343,7 +339,7 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         const int nb = std::min(8, end_bit - bit);
         const uint32_t mask = (1u << nb) - 1u;
         hipLaunchKernelGGL(os_pass_kernel<Key>, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
-                           (const long long*)m_device, bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix, ws.tickets + p,
+                           (const long long*)m_device, bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix,
                            ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
         std::swap(kin, kout);
         vin = vout;
