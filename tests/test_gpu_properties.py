@@ -180,3 +180,29 @@ def test_every_optional_acceleration_off_gives_the_same_result():
             # a gaussian without gradient has exactly none on both paths
             assert torch.equal(a.reshape(scene.n, -1).abs().sum(1) == 0, b.reshape(scene.n, -1).abs().sum(1) == 0), name
         assert float((u1 - u2).abs().max()) <= 1e-4 * float(u2.abs().max())
+
+
+def test_runs_on_the_callers_stream():
+    """Everything is enqueued on torch's current stream (the SH colours on the operator's second stream, joined
+    back before the blend): a forward and backward issued inside a non-default stream, with the default stream
+    kept busy, give the results of the default-stream run."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients
+    scene = gen_scene(1, n=60000, wh=(400, 300))
+    op, model, out, ctx = _forward(scene, DFVT)
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    gm, _, _ = op.backward(model, scene.camera(), ctx, out, grads)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()          # default priority
+    busy = torch.empty(1 << 26, device="cuda")
+    for view in range(3):
+        for _ in range(8):
+            busy.normal_()              # work on the default stream that the side stream must not wait for or race
+        with torch.cuda.stream(side):
+            out2, ctx2 = op.forward(model, scene.camera(), training=True)
+            gm2, _, _ = op.backward(model, scene.camera(), ctx2, out2, grads)
+        side.synchronize()
+        assert torch.equal(out2.color.view(torch.int32), out.color.view(torch.int32)), view
+        assert torch.equal(ctx2.gaussian_idx_sorted, ctx.gaussian_idx_sorted)
+        assert torch.allclose(gm2.xyz, gm.xyz, rtol=1e-3, atol=1e-5 * float(gm.xyz.abs().max()))
+    torch.cuda.synchronize()
