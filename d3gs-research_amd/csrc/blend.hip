@@ -232,22 +232,24 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
     const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
     const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
     const bool inside = px < P.width && py < P.height;
-    const float pxf = (float)px, pyf = (float)py;
+    const float pyf = (float)py;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
 
     const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
     const int len = r1 - r0;
     const int rounds = (len + kBlock - 1) / kBlock;
 
-    // "this pixel is finished" lives in a vector register as an integer: a loop-carried bool would be kept
-    // as a lane mask in scalar registers and merged with scalar instructions on every iteration
-    int done = inside ? 0 : 1;
+    // "This pixel is finished" is kept in the pixel's x coordinate: a finished pixel's becomes NaN, which makes
+    // its power NaN and fails the one ordered compare `power >= thr` that every visited gaussian pays for
+    // anyway, so no separate test of a flag is needed.  (A loop-carried bool would live as a lane mask in
+    // scalar registers and be merged with scalar instructions on every iteration.)
+    float pxf = inside ? (float)px : __builtin_nanf("");
     float T = 1.0f;
     float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f, depth_accum = 0.0f;
     int contributor = 0;
 
     for (int round = 0; round < rounds; ++round) {
-        if (__syncthreads_count(done != 0) == kBlock) break;
+        if (__syncthreads_count(pxf != pxf) == kBlock) break;
         const int src = r0 + round * kBlock + tid;
         uint32_t bits = 0;
         if (src < r1) {
@@ -259,7 +261,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         }
         publish_masks(bits, wave, lane, s_mask);
         __syncthreads();
-        if (__all(done != 0)) continue;
+        if (__all(pxf != pxf)) continue;
         for (int chunk = 0; chunk < 4; ++chunk) {
             unsigned long long m = uniform_u64(s_mask[wave][chunk]);
             while (m) {
@@ -268,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 const StagedGaussian sg = s_g[j];
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
                 const float power = blend_power(sg, dx, dy);
-                const bool live = done == 0 && power >= sg.thr;
+                const bool live = power >= sg.thr;      // false for a finished pixel (NaN)
                 if (!__any(live)) continue;
                 // From here on every lane runs the same instructions and the outcome is applied with
                 // selects (w = 0 leaves the accumulators untouched): far fewer scalar mask operations
@@ -292,8 +294,8 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 acc2 = __builtin_fmaf(w, c.z, acc2);
                 if constexpr (kRgba) acc3 = acc3 + w;
                 if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
-                done = stop ? 1 : done;
-                if (__any(stop) && __all(done != 0)) goto wave_finished;
+                pxf = stop ? __builtin_nanf("") : pxf;
+                if (__any(stop) && __all(pxf != pxf)) goto wave_finished;
             }
         }
     wave_finished:;
