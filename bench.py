@@ -97,7 +97,7 @@ def cpu_model_name():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration id (2 = headline 1M @1080p)")
     ap.add_argument("--filter", type=str, default="OBB_DFVT", help="early_filter_algo: NONE, AABB, ELLIPSE, OBB, OBB_DFVT")
@@ -161,7 +161,7 @@ def main():
         step()
     torch.cuda.synchronize()
     op.stage_events = {}
-    for _ in range(args.steps):
+    for _ in range(min(args.steps, 20)):
         step()
     torch.cuda.synchronize()
 
