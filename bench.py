@@ -32,8 +32,8 @@ STAGE_BYTES = {
     # binning, priced at what this factorisation has to move (32-bit keys, 32-bit values), not at the
     # reference's single sort of 64-bit keys, which would flatter these stages:
     # depth order of the N gaussians: histogram reads the keys (4), first pass reads keys and writes
-    # keys + indices (12), three more passes read and write both (16 each)
-    "depth_order": lambda N, M, P, T, passes: (4 + 12 + 3 * 16) * N,
+    # keys + indices (12), the other passes read and write both (16 each); D passes (3 for 27-bit depth keys)
+    "depth_order": lambda N, M, P, T, passes, D=4: (4 + 12 + (D - 1) * 16) * N,
     "scan": lambda N, M, P, T, passes: (12 + 8) * N,
     # order, offset, kept-tile record, depth key per gaussian; tile key + gaussian index per pair
     "make_keys": lambda N, M, P, T, passes: 28 * N + 8 * M,
@@ -167,7 +167,11 @@ def main():
 
     N, P_px, T_tiles = scene.n, scene.width * scene.height, ((scene.width + 15) // 16) * ((scene.height + 15) // 16)
     M = op.last_num_rendered
-    passes = (int(T_tiles).bit_length() + 7) // 8      # radix passes of the pair sort (tile bits only)
+    radix_passes = lambda bits: min((bits + 7) // 8, (bits + 8) // 9)     # 8-bit digits, 9-bit where that saves a pass
+    passes = radix_passes(int(T_tiles).bit_length())      # the pair sort (tile bits only)
+    from d3gs_research_amd import _capi
+    import ctypes
+    depth_passes = radix_passes(_capi.lib().d3gs_depth_key_bits(ctypes.byref(op.make_params(model, cam, True))))
     # gaussians whose gradient record is not all zero after the last view's blend backward
     active = int((op.last_raster_grads.records != 0).any(dim=1).sum())
     stages = {}
@@ -177,8 +181,8 @@ def main():
         # the median: such samples are left out of the average and counted
         kept = [t for t in ts if t <= 5.0 * ts[len(ts) // 2]]
         avg = sum(kept) / len(kept)
-        nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes) if name != "preprocess_bwd" else \
-            STAGE_BYTES[name](N, M, P_px, T_tiles, passes, active)
+        extra = {"preprocess_bwd": (active,), "depth_order": (depth_passes,)}.get(name, ())
+        nbytes = STAGE_BYTES[name](N, M, P_px, T_tiles, passes, *extra)
         stages[name] = {"ms": round(avg, 4), "ms_p10": round(ts[len(ts) // 10], 4), "ms_p50": round(ts[len(ts) // 2], 4),
                         "ms_p90": round(ts[(len(ts) * 9) // 10], 4), "stalled_samples_left_out": len(ts) - len(kept),
                         "alg_bytes": int(nbytes),

@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -48,6 +48,7 @@ _SIGNATURES = {
     "d3gs_abi_version": (C.c_int, []),
     "d3gs_last_error_string": (C.c_char_p, []),
     "d3gs_higher_msb": (C.c_int, [C.c_uint32]),
+    "d3gs_depth_key_bits": (C.c_int, [C.POINTER(Params)]),
     "d3gs_preprocess_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [C.POINTER(Instances), _VP]),
     "d3gs_sh_colors": (C.c_int, [C.POINTER(Params)] + [_VP] * 6 + [C.POINTER(Instances), _VP]),
     "d3gs_scan_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),

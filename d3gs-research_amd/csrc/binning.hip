@@ -269,7 +269,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     // a gaussian with no tiles has an empty slot range; a caller that passed a smaller buffer than
     // the scan total must never be written past
     const bool active = in_range && sane && end > off && end <= m;
-    const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : depth_sort_key(P, depths[i]);
+    const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : reference_depth_bits(P, depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
     unsigned long long kept = 0ull, meta = 0ull;
     if (tile_masks && active) {     // both words in one 16-byte load: one round trip, not two dependent ones

@@ -31,3 +31,15 @@ extern "C" int d3gs_higher_msb(uint32_t n) {
     }
     return b;
 }
+
+// Significant bits of the keys d3gs_preprocess_fwd writes to depth_sort_keys (see depth_sort_key()).
+extern "C" int d3gs_depth_key_bits(const d3gs_params* p) {
+    if (!p) return 32;
+    if (p->enable_32bit_sort) return d3gs::kDepthStepBits;
+    union { float f; uint32_t u; } far_bits;
+    far_bits.f = p->z_far;
+    const uint32_t base = d3gs::depth_key_base(*p);
+    if (!(p->z_far > 0.0f) || far_bits.u < base) return 1;    // nothing is accepted: every key is 0
+    const int bits = d3gs_higher_msb(far_bits.u - base);
+    return bits > 0 ? bits : 1;
+}

@@ -512,11 +512,25 @@ void set_error(const char* fmt, ...);
 // Validates sizes / enum values of a params block (defined in preprocess.hip).
 int check_params(const d3gs_params* p, const char* who);
 
-// Depth part of a gaussian's sort key (render.py:767-775): the float bits (positive floats order like their
+// Depth part of the reference's sort key (render.py:767-775): the float bits (positive floats order like their
 // bit patterns), or with enable_32bit_sort the depth in steps of depth_32bit_prec, truncated to 18 bits.
-__device__ __forceinline__ uint32_t depth_sort_key(const d3gs_params& P, float z) {
+__device__ __forceinline__ uint32_t reference_depth_bits(const d3gs_params& P, float z) {
     if (P.enable_32bit_sort) return (uint32_t)(z / P.depth_32bit_prec) & ((1u << kDepthStepBits) - 1u);
     return __float_as_uint(z);
+}
+
+// Key of the depth sort that orders the gaussians ahead of the pair sort: the same order as the reference's
+// depth bits in fewer significant bits.  Accepted depths lie in [z_near, z_far], so their float bits minus those
+// of z_near fit d3gs_depth_key_bits() bits (27 for the default planes, three 9-bit digits instead of four
+// 8-bit ones); rejected gaussians (depth written as 0) get key 0.
+__host__ __device__ __forceinline__ uint32_t depth_key_base(const d3gs_params& P) {
+    union { float f; uint32_t u; } near_bits;
+    near_bits.f = P.z_near;
+    return P.z_near > 0.0f ? near_bits.u : 0u;
+}
+__device__ __forceinline__ uint32_t depth_sort_key(const d3gs_params& P, float z) {
+    if (P.enable_32bit_sort) return reference_depth_bits(P, z);
+    return z >= P.z_near && z > 0.0f ? __float_as_uint(z) - depth_key_base(P) : 0u;
 }
 
 }  // namespace d3gs

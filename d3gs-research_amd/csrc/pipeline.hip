@@ -24,7 +24,7 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
     const int32_t num_tiles = p->tiles_x * p->tiles_y;
     int rc = d3gs_sort_pairs_u32(depth_keys_a, depth_keys_b, order_a, order_b, depth_sort_ws, depth_sort_ws_bytes, n,
                                  nullptr, /*values_are_indices=*/1, workspaces_are_zero, 0,
-                                 p->enable_32bit_sort ? kDepthStepBits : 32, order_in_b, stream);
+                                 d3gs_depth_key_bits(p), order_in_b, stream);
     if (rc) return rc;
     const uint32_t* depth_keys_sorted = *order_in_b ? depth_keys_b : depth_keys_a;
     const int32_t* order = *order_in_b ? order_b : order_a;

@@ -3,7 +3,7 @@
 // (d3sim/csrc/devsort.py:38-129, call site d3sim/algos/d3gs/render.py:846-887).
 //
 // Single-sweep design: one kernel histograms every digit of every pass in one
-// read of the keys; then each 8-bit pass is ONE kernel that reads a pair once
+// read of the keys; then each pass (one 8- or 9-bit digit) is ONE kernel that reads a pair once
 // and writes it once (24 B per pair per pass).  A workgroup owns 4096
 // consecutive keys, ranks them in LDS, and learns where its digits start in the
 // output from the workgroups before it through a decoupled look-back over
@@ -32,7 +32,12 @@ constexpr int kOsThreads = 512;
 constexpr int kOsWaves = kOsThreads / 64;
 constexpr int kOsItems = 8;
 constexpr int kOsTile = kOsThreads * kOsItems;  // 4096 pairs per workgroup
-constexpr int kOsRadix = 256;
+// Digits are 8 bits wide, or 9 where that saves a pass (18 or 27 key bits: the depth keys of the gaussians).
+constexpr int kOsMaxRadix = 512;
+static inline int os_digit_bits(int begin_bit, int end_bit) {
+    const int bits = end_bit - begin_bit;
+    return (bits + 8) / 9 < (bits + 7) / 8 ? 9 : 8;
+}
 constexpr uint32_t kFlagAggregate = 1u << 30;
 constexpr uint32_t kFlagPrefix = 2u << 30;
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
@@ -40,9 +45,9 @@ constexpr int kSpinLimit = 1 << 22;
 constexpr int kLookWindow = 16;  // predecessor tiles polled per look-back step
 
 struct SortWorkspace {
-    uint32_t* hist;     // [passes][256] digit totals of the whole input
+    uint32_t* hist;     // [passes][radix] digit totals of the whole input
     uint32_t* error;    // [1] set when a look-back gave up
-    uint32_t* status;   // [passes][ntiles][256]
+    uint32_t* status;   // [passes][ntiles][radix]
 };
 
 __device__ __forceinline__ int os_wave_incl_scan(int v, int lane) {
@@ -79,53 +84,55 @@ __global__ __launch_bounds__(kBlock) void os_clear_kernel(uint32_t* __restrict__
 // same-address conflicts of skewed digits (the exponent byte of a depth takes a handful of values).
 constexpr int kHistThreads = 1024;
 constexpr int kHistCopies = 8;
-template <typename Key>
+template <typename Key, int kBits>
 __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __restrict__ keys, long long m,
                                                                 const long long* __restrict__ m_device,
-                                                                int begin_bit, int end_bit, int passes,
+                                                                int begin_bit, int end_bit, int passes, int copies,
                                                                 uint32_t* __restrict__ hist) {
+    constexpr int kRadix = 1 << kBits;
     if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the buffers
-    extern __shared__ uint32_t h[];  // [kHistCopies][passes][256]
-    const int table = passes * kOsRadix;
-    for (int k = threadIdx.x; k < kHistCopies * table; k += kHistThreads) h[k] = 0u;
+    extern __shared__ uint32_t h[];  // [copies][passes][kRadix]; copies is a power of two
+    const int table = passes * kRadix;
+    for (int k = threadIdx.x; k < copies * table; k += kHistThreads) h[k] = 0u;
     __syncthreads();
-    uint32_t* mine = h + (threadIdx.x & (kHistCopies - 1)) * table;
+    uint32_t* mine = h + (threadIdx.x & (copies - 1)) * table;
     const long long stride = (long long)gridDim.x * kHistThreads;
     for (long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x; i < m; i += stride) {
         const Key key = keys[i];
         for (int p = 0; p < passes; ++p) {
-            const int bit = begin_bit + 8 * p;
-            const int nb = min(8, end_bit - bit);
-            atomicAdd(&mine[p * kOsRadix + ((uint32_t)(key >> bit) & ((1u << nb) - 1u))], 1u);
+            const int bit = begin_bit + kBits * p;
+            const int nb = min(kBits, end_bit - bit);
+            atomicAdd(&mine[p * kRadix + ((uint32_t)(key >> bit) & ((1u << nb) - 1u))], 1u);
         }
     }
     __syncthreads();
     for (int k = threadIdx.x; k < table; k += kHistThreads) {
         uint32_t c = 0;
-#pragma unroll
-        for (int q = 0; q < kHistCopies; ++q) c += h[q * table + k];
+        for (int q = 0; q < copies; ++q) c += h[q * table + k];
         if (c) atomicAdd(&hist[k], c);
     }
 }
 
-template <typename Key>
+template <typename Key, int kBits>
 __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restrict__ keys_in,
                                                               const int32_t* __restrict__ vals_in,
                                                               Key* __restrict__ keys_out,
                                                               int32_t* __restrict__ vals_out, long long m,
                                                               const long long* __restrict__ m_device, int shift,
                                                               uint32_t mask, int ntiles,
-                                                              const uint32_t* __restrict__ hist /* this pass, [256] */,
+                                                              const uint32_t* __restrict__ hist /* this pass, [radix] */,
                                                               uint32_t* __restrict__ status,
                                                               uint32_t* __restrict__ error) {
-    __shared__ int wave_cnt[kOsWaves][kOsRadix];  // running, then exclusive-over-waves, per-wave digit counts
-    __shared__ int digit_out[kOsRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
+    constexpr int kRadix = 1 << kBits;
+    static_assert(kRadix <= kOsThreads && kRadix <= kOsMaxRadix, "one thread owns one digit");
+    __shared__ int wave_cnt[kOsWaves][kRadix];  // running, then exclusive-over-waves, per-wave digit counts
+    __shared__ int digit_out[kRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
     __shared__ Key s_keys[kOsTile];
     __shared__ uint16_t s_src[kOsTile];  // tile-local input index of the pair at each sorted position
     __shared__ int s_scan[kOsWaves];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int k = tid; k < kOsWaves * kOsRadix; k += kOsThreads) (&wave_cnt[0][0])[k] = 0;
+    for (int k = tid; k < kOsWaves * kRadix; k += kOsThreads) (&wave_cnt[0][0])[k] = 0;
     __syncthreads();
     // Tile = workgroup id.  Workgroups of a 1-D grid are dispatched in id order (per XCD, which gets
     // every 8th id), so every tile this one waits on has been dispatched before it; an atomic ticket
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
         const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
         uint64_t peers = __ballot(in);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < kBits; ++b) {
             const uint64_t bal = __ballot((d >> b) & 1u);
             peers &= ((d >> b) & 1u) ? bal : ~bal;
         }
@@ -167,11 +174,11 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
     }
     __syncthreads();
 
-    // threads 0..255 each own one digit
-    const bool owner = tid < kOsRadix;
+    // the first kRadix threads each own one digit
+    const bool owner = tid < kRadix;
     int c[kOsWaves];
     uint32_t total = 0;
-    uint32_t* my_status = status + (size_t)tile * kOsRadix + (owner ? tid : 0);
+    uint32_t* my_status = status + (size_t)tile * kRadix + (owner ? tid : 0);
     if (owner) {
 #pragma unroll
         for (int w = 0; w < kOsWaves; ++w) {
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
 #pragma unroll
                 for (int i = 0; i < kLookWindow; ++i) {
                     const int tt = t - i;
-                    s[i] = tt >= 0 ? __hip_atomic_load(status + (size_t)tt * kOsRadix + tid, __ATOMIC_RELAXED,
+                    s[i] = tt >= 0 ? __hip_atomic_load(status + (size_t)tt * kRadix + tid, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT)
                                    : kFlagPrefix;  // before the first tile: an empty inclusive prefix
                 }
@@ -268,18 +275,21 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
 
 static inline size_t os_align(size_t v) { return (v + 255) / 256 * 256; }
 static inline int os_tiles(int64_t m) { return (int)((m + kOsTile - 1) / kOsTile); }
-static inline int os_passes(int begin_bit, int end_bit) { return (end_bit - begin_bit + 7) / 8; }
+static inline int os_passes(int begin_bit, int end_bit) {
+    const int digit = os_digit_bits(begin_bit, end_bit);
+    return (end_bit - begin_bit + digit - 1) / digit;
+}
 
-static size_t os_layout(int64_t m, int passes, SortWorkspace* ws, void* base) {
+static size_t os_layout(int64_t m, int passes, int radix, SortWorkspace* ws, void* base) {
     const int ntiles = os_tiles(m) > 0 ? os_tiles(m) : 1;
     size_t off = 0;
     char* b = (char*)base;
     if (ws) ws->hist = (uint32_t*)(b + off);
-    off += os_align((size_t)passes * kOsRadix * 4);
+    off += os_align((size_t)passes * radix * 4);
     if (ws) ws->error = (uint32_t*)(b + off);
     off += 256;
     if (ws) ws->status = (uint32_t*)(b + off);
-    off += os_align((size_t)passes * ntiles * kOsRadix * 4);
+    off += os_align((size_t)passes * ntiles * radix * 4);
     return off;
 }
 
@@ -293,7 +303,7 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     const int passes = os_passes(begin_bit, end_bit) > 0 ? os_passes(begin_bit, end_bit) : 1;
-    *bytes_out_host = os_layout(m, passes, nullptr, nullptr);
+    *bytes_out_host = os_layout(m, passes, 1 << os_digit_bits(begin_bit, end_bit), nullptr, nullptr);
     return D3GS_OK;
 }
 
@@ -314,8 +324,9 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     const int passes = os_passes(begin_bit, end_bit);
+    const int digit = os_digit_bits(begin_bit, end_bit), radix = 1 << digit;
     SortWorkspace ws;
-    const size_t need = os_layout(m, passes, &ws, workspace);
+    const size_t need = os_layout(m, passes, radix, &ws, workspace);
     if (workspace_bytes < need) {
         set_error("%s: workspace %zu < required %zu", who, workspace_bytes, need);
         return D3GS_ERR_WORKSPACE_TOO_SMALL;
@@ -326,21 +337,35 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
     if (!workspace_is_zero)
         hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
     const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
-    hipLaunchKernelGGL(os_hist_kernel<Key>, dim3(hist_blocks), dim3(kHistThreads),
-                       (size_t)kHistCopies * passes * kOsRadix * sizeof(uint32_t), s, keys_a, (long long)m,
-                       (const long long*)m_device, begin_bit, end_bit, passes, ws.hist);
+    // as many LDS copies of the histogram table as fit in 64 KB (a power of two, at most kHistCopies)
+    int copies = kHistCopies;
+    while (copies > 1 && (size_t)copies * passes * radix * sizeof(uint32_t) > 64 * 1024) copies >>= 1;
+    const size_t hist_lds = (size_t)copies * passes * radix * sizeof(uint32_t);
+    if (digit == 9)
+        hipLaunchKernelGGL((os_hist_kernel<Key, 9>), dim3(hist_blocks), dim3(kHistThreads), hist_lds, s, keys_a,
+                           (long long)m, (const long long*)m_device, begin_bit, end_bit, passes, copies, ws.hist);
+    else
+        hipLaunchKernelGGL((os_hist_kernel<Key, 8>), dim3(hist_blocks), dim3(kHistThreads), hist_lds, s, keys_a,
+                           (long long)m, (const long long*)m_device, begin_bit, end_bit, passes, copies, ws.hist);
     Key* kin = keys_a;
     Key* kout = keys_b;
     const int32_t* vin = values_are_indices ? nullptr : vals_a;   // first pass only
     int32_t* vout = vals_b;
     int in_b = 0;
     for (int p = 0; p < passes; ++p) {
-        const int bit = begin_bit + 8 * p;
-        const int nb = std::min(8, end_bit - bit);
+        const int bit = begin_bit + digit * p;
+        const int nb = std::min(digit, end_bit - bit);
         const uint32_t mask = (1u << nb) - 1u;
-        hipLaunchKernelGGL(os_pass_kernel<Key>, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
-                           (const long long*)m_device, bit, mask, ntiles, ws.hist + (size_t)p * kOsRadix,
-                           ws.status + (size_t)p * ntiles * kOsRadix, ws.error);
+        const uint32_t* pass_hist = ws.hist + (size_t)p * radix;
+        uint32_t* pass_status = ws.status + (size_t)p * ntiles * radix;
+        if (digit == 9)
+            hipLaunchKernelGGL((os_pass_kernel<Key, 9>), dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout,
+                               (long long)m, (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status,
+                               ws.error);
+        else
+            hipLaunchKernelGGL((os_pass_kernel<Key, 8>), dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout,
+                               (long long)m, (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status,
+                               ws.error);
         std::swap(kin, kout);
         vin = vout;
         vout = in_b ? vals_b : vals_a;

@@ -375,7 +375,7 @@ class GaussianSplatOp:
         # every zero-initialised work buffer of the forward pass comes out of one fill (the two sorts' and the
         # scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later
         tile_bits = L.d3gs_higher_msb(num_tiles)
-        depth_bits = 18 if P.enable_32bit_sort else 32      # the depth sort's key width (render.py:737)
+        depth_bits = L.d3gs_depth_key_bits(C.byref(P))      # the depth sort's key width: 27 bits for the default planes
         spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
         align = lambda v: (v + 255) // 256 * 256
         scan_ws_bytes = C.c_size_t(0)

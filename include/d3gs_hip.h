@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 22
+#define D3GS_ABI_VERSION 23
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -93,6 +93,12 @@ const char* d3gs_last_error_string(void);
 /* DeviceSort.get_higher_msb — devsort.py:131-149: bit length of n. */
 int d3gs_higher_msb(uint32_t n);
 
+/* Number of significant bits of the depth-sort keys that d3gs_preprocess_fwd writes to depth_sort_keys (no
+ * counterpart in the reference): accepted depths lie in [z_near, z_far], so the key is the depth's float bits
+ * minus those of z_near -- the same order in fewer bits (27 for the default planes 0.2 and 1e4) -- or, with
+ * enable_32bit_sort, the 18-bit depth step.  The depth sort runs on bits [0, d3gs_depth_key_bits(p)). */
+int d3gs_depth_key_bits(const d3gs_params* p);
+
 /* Instance rendering (render.py:207-220, 346-356): a gaussian with instance_ids[i] = k >= 0 belongs to object
  * instance k, its parameters are given in that object's frame, and it is seen by the camera expressed in that
  * frame: instance_cameras[k] holds the 9 floats of the world-to-camera rotation in the instance frame (row
@@ -117,9 +123,9 @@ typedef struct d3gs_instances {
  * d3gs_make_keys expands instead of repeating the per-tile tests.
  * rgb_gaussian may be NULL: the SH colour (and sh_to_rgb_ne_0) is then left to d3gs_sh_colors, which a
  * caller can run on a second stream beside the sort, the only consumer being the blend.
- * depth_sort_keys (uint32[N], may be NULL): the keys of the depth sort, the float bits of depths or, with
- * enable_32bit_sort, the 18-bit depth steps (saves the d3gs_depth_keys pass; the depth sort then runs on bits
- * [0, 32) or [0, 18)). */
+ * depth_sort_keys (uint32[N], may be NULL): the keys of the depth sort, the float bits of depths relative to
+ * those of z_near or, with enable_32bit_sort, the 18-bit depth steps (saves the d3gs_depth_keys pass; the depth
+ * sort then runs on bits [0, d3gs_depth_key_bits(p))). */
 int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const float* color_sh_base,
                         const uint8_t* invalid_mask, float* depths,
@@ -225,7 +231,7 @@ int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int6
  * *total_dev the pair count M (the kernels touch min(M, capacity) pairs: a caller that sized capacity from a
  * guess compares M with it afterwards and bins again when M is larger); total_host, when not NULL, is a pinned
  * host word that the scan kernel stores M to (see d3gs_scan_gathered).  Workspace sizes as for the single calls
- * (d3gs_sort_workspace_bytes(n, 0, 32), d3gs_scan_gathered_workspace_bytes(n),
+ * (d3gs_sort_workspace_bytes(n, 0, d3gs_depth_key_bits(p)), d3gs_scan_gathered_workspace_bytes(n),
  * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))); workspaces_are_zero != 0 says the caller has
  * cleared all three.  workload_ranges must be zero on entry. */
 int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,

@@ -34,9 +34,19 @@ def test_params_struct_matches_header_layout():
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 22
+    assert L.d3gs_abi_version() == 23
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
+    # depth-sort key width: float bits of z_far minus those of z_near, or the 18 depth-step bits
+    P = _capi.Params()
+    widths = []
+    for near, far, sort32 in ((0.2, 1e4, 0), (0.01, 100.0, 0), (1.0, 2.0, 0), (0.2, 1e4, 1), (5.0, 1.0, 0), (0.0, 1e4, 0)):
+        P.z_near, P.z_far, P.enable_32bit_sort = near, far, sort32
+        widths.append(L.d3gs_depth_key_bits(C.byref(P)))
+    import struct
+    bits = lambda v: struct.unpack("<I", struct.pack("<f", v))[0]
+    assert widths == [(bits(1e4) - bits(0.2)).bit_length(), (bits(100.0) - bits(0.01)).bit_length(), 24, 18, 1,
+                      bits(1e4).bit_length()] and widths[0] == 27
 
 
 def test_error_codes_without_compute():

@@ -100,7 +100,8 @@ def test_reference_call_sequence(oracle, cfg_id, n, wh, filt):
     tk_a, tk_b, ix_a, ix_b = (torch.empty(cap, dtype=i32, device=dev) for _ in range(4))
     tile_bits = L.d3gs_higher_msb(tiles)
     sizes = []
-    for call, args in ((L.d3gs_sort_workspace_bytes, (N, 0, 32)), (L.d3gs_scan_gathered_workspace_bytes, (N,)),
+    for call, args in ((L.d3gs_sort_workspace_bytes, (N, 0, L.d3gs_depth_key_bits(C.byref(P)))),
+                       (L.d3gs_scan_gathered_workspace_bytes, (N,)),
                        (L.d3gs_sort_workspace_bytes, (cap, 0, tile_bits))):
         _capi.check(call(*args, C.byref(nbytes)), "workspace size")
         sizes.append(nbytes.value)
