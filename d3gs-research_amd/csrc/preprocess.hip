@@ -522,7 +522,18 @@ __device__ __forceinline__ void preprocess_bwd_one(
 // whole wavefronts) and worked off kBwdBlock at a time: thread t takes the t-th of them, their SH rows are
 // staged in LDS and leave as gradient rows.
 constexpr int kBwdBlock = 256;
-constexpr int kBwdRows = 176;   // gaussians worked off per pass: with their LDS rows (34 KB) four workgroups share a CU
+// Gaussians worked off per pass: as many LDS rows as leave room for four workgroups on a CU (160 KB of LDS, and the
+// kernel's registers allow four as well), at most one per thread: 192 rows of 48 coefficients, 209 of 45 (split
+// DC term).  A workgroup of a dense view holds about 170 gaussians with gradient; those beyond the rows of a
+// pass cost a second, nearly empty one (176 -> 192 rows: -2 us; keeping the DC term out of LDS to reach 209: no
+// further gain).
+constexpr int kBwdLdsBudget = 160 * 1024 / 4;
+constexpr int kBwdStaticLds = 3328;     // s_list, s_active, s_count, with some slack
+static inline int bwd_rows_per_pass(int sh_stride) {
+    const int row_bytes = ((sh_stride * 3) | 1) * (int)sizeof(float);
+    const int rows = (kBwdLdsBudget - kBwdStaticLds) / row_bytes;
+    return rows < kBwdBlock ? rows : kBwdBlock;
+}
 
 // element e of a block of `cnt` staged rows <-> element of the global [N][rowlen] array, for the gaussians
 // first + list[0 .. cnt)
@@ -562,11 +573,11 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const d3gs_params P, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ grad_records, const int sh_mask_compat, const int outputs_are_zero,
+    const float* __restrict__ grad_records, const int sh_mask_compat, const int outputs_are_zero, const int rows_per_pass,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
-    extern __shared__ float s_rows[];                    // kBwdRows rows of `stride` floats
+    extern __shared__ float s_rows[];                    // rows_per_pass rows of `stride` floats
     __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
     __shared__ unsigned char s_active[kSpan];
     __shared__ int s_count[kPer * kWaves];
@@ -639,8 +650,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
             if (!s_active[(int)(((float)e + 0.5f) * inv)]) block_dsh[e] = 0.0f;
     }
     __syncthreads();
-    for (int base = 0; base < nactive; base += kBwdRows) {
-        const int cnt = min(kBwdRows, nactive - base);
+    for (int base = 0; base < nactive; base += rows_per_pass) {
+        const int cnt = min(rows_per_pass, nactive - base);
         bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride);
         __syncthreads();
         if (tid < cnt) {
@@ -787,7 +798,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
     }
     InstanceView inst;
     if (!instance_view(instances, &inst, "d3gs_preprocess_bwd")) return D3GS_ERR_INVALID_ARGUMENT;
-    const size_t lds_bytes = (size_t)kBwdRows * ((p->sh_stride * 3) | 1) * sizeof(float);
+    const int rows_per_pass = bwd_rows_per_pass(p->sh_stride);
+    const size_t lds_bytes = (size_t)rows_per_pass * ((p->sh_stride * 3) | 1) * sizeof(float);
     // four gaussians per thread once there are enough workgroups to fill the chip that way
     const bool wide = p->n >= 512 * kBwdBlock * 4;
     const int per = wide ? 4 : 1;
@@ -795,7 +807,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
 #define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
     hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,  \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
-                       (int)sh_mask_compat, (int)outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out,       \
+                       (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, dxyz, dquaternion_xyzw, dscale,      \
+                       dopacity_out,                                                                                   \
                        dcolor_sh, dcolor_sh_base)
     if (wide) { if (inst.ids) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }
     else      { if (inst.ids) D3GS_LAUNCH_K9(1, true); else D3GS_LAUNCH_K9(1, false); }
