@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 
 
@@ -69,8 +69,8 @@ _SIGNATURES = {
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),
-    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
-    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [C.c_int32, C.c_int32] + [_VP] * 6 +
+    "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
+    "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 10 + [C.c_int32, C.c_int32] + [_VP] * 6 +
                             [C.POINTER(Instances), _VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const float* __restrict__ depths, const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
     const int32_t* __restrict__ n_contrib, const float* __restrict__ color, const float* __restrict__ final_depth,
     const float* __restrict__ drgb, const float* __restrict__ dT, const float* __restrict__ ddepth,
-    float* __restrict__ grad_records) {
+    float* __restrict__ grad_records, uint8_t* __restrict__ touched) {
     constexpr int kValues = kDepth ? 10 : 9;
     constexpr int kChannels = kRgba ? 4 : 3;
     __shared__ StagedGaussian s_g[kBlock];
@@ -502,10 +502,13 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         // side sees one line-wide atomic request per (tile, gaussian) instead of one per value.
         const int slot_k = tid & 15;
         for (int gl = tid >> 4; gl < flush_cnt; gl += kBlock / 16) {
-            if (slot_k < kValues) {
-                const float v = s_grad[slot_k][gl];
-                if (v != 0.0f)
-                    unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * s_id[gl] + slot_k, v);
+            const float v = slot_k < kValues ? s_grad[slot_k][gl] : 0.0f;
+            if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * s_id[gl] + slot_k, v);
+            // one byte per gaussian that received anything: the preprocess backward finds its work in this
+            // dense array instead of reading every record
+            if (touched) {
+                const unsigned long long nz = __ballot(v != 0.0f);
+                if (slot_k == 0 && ((nz >> (tid & 48)) & 0xFFFFull)) touched[s_id[gl]] = 1;
             }
         }
     }
@@ -554,7 +557,7 @@ extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_rang
                               const float* depths, const int32_t* tile_order, const float* final_T,
                               const int32_t* n_contrib, const float* color, const float* final_depth,
                               const float* drgb, const float* dT, const float* ddepth, float* grad_records,
-                              d3gs_stream_t stream) {
+                              uint8_t* touched, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_bwd");
     if (rc) return rc;
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb ||
@@ -565,7 +568,7 @@ extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_rang
 #define D3GS_LAUNCH_BWD(D, A)                                                                                       \
     hipLaunchKernelGGL((blend_bwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
                        workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
-                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, grad_records)
+                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, grad_records, touched)
     if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_BWD(true, true); else D3GS_LAUNCH_BWD(true, false); }
     else                 { if (p->render_rgba) D3GS_LAUNCH_BWD(false, true); else D3GS_LAUNCH_BWD(false, false); }
 #undef D3GS_LAUNCH_BWD

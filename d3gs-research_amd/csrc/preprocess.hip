@@ -573,7 +573,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const d3gs_params P, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ grad_records, const int sh_mask_compat, const int outputs_are_zero, const int rows_per_pass,
+    const float* __restrict__ grad_records, const uint8_t* __restrict__ touched, const int sh_mask_compat,
+    const int outputs_are_zero, const int rows_per_pass,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
@@ -588,12 +589,14 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const float4* rec4 = reinterpret_cast<const float4*>(grad_records);
     bool active[kPer];
     unsigned long long mates[kPer];
-    // all radii first, then all records: two round trips to memory instead of two per gaussian
+    // all radii first, then all records: two round trips to memory instead of two per gaussian.  With the blend
+    // backward's `touched` bytes a gaussian it did not mark counts as culled, and its record is never read.
     int rad[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
         const int local = k * kBwdBlock + tid;
         rad[k] = local < nrows ? radii[(size_t)first + local] : 0;
+        if (touched && local < nrows && !touched[(size_t)first + local]) rad[k] = 0;
     }
     float4 ra[kPer], rb[kPer], rc[kPer];
 #pragma unroll
@@ -782,7 +785,8 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
 extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
                                    const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
-                                   const float* grad_records, int32_t sh_mask_compat, int32_t outputs_are_zero,
+                                   const float* grad_records, const uint8_t* touched, int32_t sh_mask_compat,
+                                   int32_t outputs_are_zero,
                                    float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
                                    float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                                    d3gs_stream_t stream) {
@@ -807,6 +811,7 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
 #define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
     hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,  \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
+                       touched,                                                                                        \
                        (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, dxyz, dquaternion_xyzw, dscale,      \
                        dopacity_out,                                                                                   \
                        dcolor_sh, dcolor_sh_base)

@@ -54,6 +54,8 @@ class GaussianSplatOpContext:
     grad_pool: torch.Tensor | None = None
     # the allocation behind grad_records and grad_pool, until the forward blend has been asked to clear it
     grad_clear: torch.Tensor | None = None
+    # one byte per gaussian, set by the blend backward where a record received anything (cleared with the records)
+    grad_touched: torch.Tensor | None = None
     # custom feature channels of this view ([N, F]) kept for the backward pass
     custom_features: torch.Tensor | None = None
     # disable_builtin_rgb: the image in the kernels' own layout ([1, H, W, 3 or 4], colour channels zero); the
@@ -108,6 +110,8 @@ class RasterizeGradientOutput:
     dz: torch.Tensor | None = None
     # not in the reference: the [N, 16] buffer the tensors above are strided views of
     records: torch.Tensor | None = None
+    # not in the reference: one byte per gaussian, non-zero where the record received anything (or None)
+    touched: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -404,13 +408,15 @@ class GaussianSplatOp:
             # gradient arrays: one allocation that the forward blend kernel clears while it runs (it leaves the
             # memory pipes idle).  Most gaussians of a view end with an all-zero gradient (culled, or never reached
             # before their pixels saturated), which the preprocess backward then need not write.
-            grad_records = grad_pool = grad_clear = None
+            grad_records = grad_pool = grad_clear = grad_touched = None
             if training:
                 rec_floats = n * _capi.GRAD_RECORD_FLOATS
                 pool_floats = self._grad_pool_floats(model) if self.clear_gradients_early else 0
-                grad_clear = torch.empty(rec_floats + pool_floats, dtype=f32, device=dev)
+                mark_floats = (n + 15) // 16 * 4          # n bytes, in whole 16-byte units
+                grad_clear = torch.empty(rec_floats + pool_floats + mark_floats, dtype=f32, device=dev)
                 grad_records = grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
-                grad_pool = grad_clear[rec_floats:] if pool_floats else None
+                grad_pool = grad_clear[rec_floats:rec_floats + pool_floats] if pool_floats else None
+                grad_touched = grad_clear[rec_floats + pool_floats:].view(torch.uint8)[:n]
             overlap = bool(self.overlap_sh_colors)
             no_rgb = bool(self._cfg.disable_builtin_rgb)
             if overlap and (self._side_stream is None or self._side_stream.device != dev):
@@ -585,6 +591,7 @@ class GaussianSplatOp:
                 gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
                 tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
+                grad_touched=grad_touched,
                 kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
@@ -709,8 +716,9 @@ class GaussianSplatOp:
             res[0, :, :, k:k + w] = img[:, :, :w]
         return res
 
-    def _backward_custom_features(self, P, ctx, out, dfeat_img, rec):
-        """Adds the feature channels' share to rec[:, 0:6] and returns dcustom_features [N, F]."""
+    def _backward_custom_features(self, P, ctx, out, dfeat_img, rec, touched=None):
+        """Adds the feature channels' share to rec[:, 0:6] and returns dcustom_features [N, F]; gaussians that
+        receive anything are marked in ``touched`` as in the colour pass."""
         L, s = self._lib, self._stream()
         Q = self._feature_params(P)
         feat = ctx.custom_features.detach()
@@ -728,7 +736,7 @@ class GaussianSplatOp:
                 C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(tri), None, _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
                 _capi.ptr(out.n_contrib), _capi.ptr(img), None, _capi.ptr(dimg), _capi.ptr(zero_dT), None,
-                _capi.ptr(rec_k), s), "d3gs_blend_bwd (custom features)")
+                _capi.ptr(rec_k), _capi.ptr(touched), s), "d3gs_blend_bwd (custom features)")
             rec[:, 0:6] += rec_k[:, 0:6]
             dfeat[:, k:k + w] = rec_k[:, 6:6 + w]
         return dfeat
@@ -770,16 +778,18 @@ class GaussianSplatOp:
         # one 64-byte record per gaussian (see D3GS_GRAD_RECORD_FLOATS); the reference's four tensors
         # and dz are strided views of it
         rec, ctx.grad_records = ctx.grad_records, None
-        if rec is None:
+        touched, ctx.grad_touched = ctx.grad_touched, None
+        if rec is None:     # a second backward over this context: fresh records, work found from the records
             rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
+            touched = None
         _capi.check(L.d3gs_blend_bwd(
             C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
             _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
             _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
-            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec), s),
-            "d3gs_blend_bwd")
+            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec),
+            _capi.ptr(touched), s), "d3gs_blend_bwd")
         res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
-                                      dz=rec[:, 9] if render_depth else None, records=rec)
+                                      dz=rec[:, 9] if render_depth else None, records=rec, touched=touched)
         return res
 
     # --------------------------------------------------------------- backward
@@ -803,7 +813,7 @@ class GaussianSplatOp:
         if ctx.custom_features is not None:
             dfeat_img = grad.dcustom_features if grad.dcustom_features is not None else \
                 torch.zeros_like(out.custom_features)
-            dcustom = self._backward_custom_features(P, ctx, out, dfeat_img.contiguous(), g.records)
+            dcustom = self._backward_custom_features(P, ctx, out, dfeat_img.contiguous(), g.records, g.touched)
         with self._stage("preprocess_bwd"):
             pool, ctx.grad_pool = ctx.grad_pool, None
             prezeroed = pool is not None and pool.numel() == self._grad_pool_floats(model)
@@ -820,8 +830,8 @@ class GaussianSplatOp:
             _capi.check(L.d3gs_preprocess_bwd(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                 _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), int(self._cfg.compat_ref_sh_mask_bitorder),
-                int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity),
+                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), _capi.ptr(g.touched),
+                int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity),
                 _capi.ptr(dsh), _capi.ptr(dsh_base), inst, s),
                 "d3gs_preprocess_bwd")
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 23
+#define D3GS_ABI_VERSION 24
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -274,12 +274,15 @@ int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const i
  * reference's backward_reduction_balanced_factor <= 0 branch, render.py:2024-2050,
  * 2182-2210).  grad_records [N][D3GS_GRAD_RECORD_FLOATS] is accumulated with
  * atomics: zero-fill it first.  drgb has the layout of color; final_depth /
- * ddepth [H,W] may be NULL without p->render_depth. */
+ * ddepth [H,W] may be NULL without p->render_depth.
+ * touched (uint8[N], may be NULL; no counterpart in the reference): set to 1 for every gaussian whose record
+ * received a non-zero value; zero-fill it with the records.  d3gs_preprocess_bwd takes it to find the gaussians
+ * with work without reading all records. */
 int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                    const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
                    const int32_t* tile_order, const float* final_T, const int32_t* n_contrib, const float* color,
                    const float* final_depth, const float* drgb, const float* dT, const float* ddepth,
-                   float* grad_records, d3gs_stream_t stream);
+                   float* grad_records, uint8_t* touched, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from K7's records (duv, dconic, dopacity, dcolor
@@ -288,13 +291,15 @@ int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const i
  * zero (in no tile list, or never reached before their pixels saturated), are
  * zeros; nothing but the record is read for them.  outputs_are_zero != 0 (no
  * counterpart in the reference) says the caller has cleared the six gradient
- * arrays beforehand: those zeros are then not written again.  The *_base
- * pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
+ * arrays beforehand: those zeros are then not written again.  touched (uint8[N],
+ * may be NULL; no counterpart in the reference) is d3gs_blend_bwd's array of the
+ * same name: gaussians it marks 0 are taken to have an all-zero record, which is
+ * then not read.  The *_base pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
  * reference's reversed bit order (render.py:3344-3350). */
 int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
-                        const uint8_t* sh_to_rgb_ne_0, const float* grad_records, int32_t sh_mask_compat,
-                        int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw, float* dscale,
+                        const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
+                        int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw, float* dscale,
                         float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                         d3gs_stream_t stream);
 

@@ -100,7 +100,7 @@ def test_instances_forward_and_backward(oracle, cfg_id, n, wh, filt, K):
     _capi.check(L.d3gs_preprocess_bwd(
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q), _capi.ptr(o_s),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), None, 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q), _capi.ptr(o_s),
         _capi.ptr(o_op), _capi.ptr(o_sh), None, arg, stream), "d3gs_preprocess_bwd (instances)")
     torch.cuda.synchronize()
     for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", o_op), ("dsh", o_sh)):

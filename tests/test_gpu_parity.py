@@ -152,7 +152,7 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
     _capi.check(L.d3gs_preprocess_bwd(
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), None, 0, 0, _capi.ptr(o_xyz), _capi.ptr(o_q),
         _capi.ptr(o_s), _capi.ptr(dop_io), _capi.ptr(o_sh), None, None, stream), "d3gs_preprocess_bwd")
     torch.cuda.synchronize()
     for name, got in (("dxyz", o_xyz), ("dquat", o_q), ("dscale", o_s), ("dopacity", dop_io), ("dsh", o_sh)):
@@ -160,10 +160,12 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt):
         assert ok, f"isolated {name}: {nbad} elements outside tolerance (worst {worst:.2f}x)"
     # outputs cleared by the caller: gaussians with an all-zero record are left alone, the rest must match
     z_xyz, z_q, z_s, z_op, z_sh = (torch.zeros_like(t) for t in (o_xyz, o_q, o_s, dop_io, o_sh))
+    # ... and with the bytes that say which records hold anything, as the blend backward writes them
+    marks = (rec != 0).any(dim=1).to(torch.uint8).contiguous()
     _capi.check(L.d3gs_preprocess_bwd(
         C.byref(Pg), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
         _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), 0, 1, _capi.ptr(z_xyz), _capi.ptr(z_q),
+        _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(rec), _capi.ptr(marks), 0, 1, _capi.ptr(z_xyz), _capi.ptr(z_q),
         _capi.ptr(z_s), _capi.ptr(z_op), _capi.ptr(z_sh), None, None, stream), "d3gs_preprocess_bwd (cleared outputs)")
     torch.cuda.synchronize()
     for a, b in ((o_xyz, z_xyz), (o_q, z_q), (o_s, z_s), (dop_io, z_op), (o_sh, z_sh)):
