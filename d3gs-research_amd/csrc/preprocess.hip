@@ -279,22 +279,45 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
 // ---------------------------------------------------------------------------
 // Preprocess backward.
 // ---------------------------------------------------------------------------
+// What the backward of one gaussian reads besides its SH row: loaded ahead of the rows' way through LDS, so that
+// these scattered reads and the row copy are in flight together.
+struct BwdInputs {
+    float xyz[3], s[3], cov[3], opacity;
+    float4 q, ra, rb, rc;      // quaternion; the blend backward's record: duv(2) dconic(3) dopacity dcolor(3) dz
+    uint32_t ne0;
+};
+__device__ __forceinline__ BwdInputs load_bwd_inputs(const int i, const float* __restrict__ xyz,
+                                                     const float* __restrict__ quat, const float* __restrict__ scale,
+                                                     const float* __restrict__ opacity, const float* __restrict__ cov2d,
+                                                     const uint8_t* __restrict__ ne0, const float4* __restrict__ rec4) {
+    BwdInputs in;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        in.xyz[k] = xyz[3 * i + k];
+        in.s[k] = scale[3 * i + k];
+        in.cov[k] = cov2d[3 * i + k];
+    }
+    in.opacity = opacity[i];
+    in.q = *reinterpret_cast<const float4*>(quat + 4 * i);
+    in.ra = rec4[4 * (size_t)i];
+    in.rb = rec4[4 * (size_t)i + 1];
+    in.rc = rec4[4 * (size_t)i + 2];
+    in.ne0 = ne0[i];
+    return in;
+}
+
 // One gaussian of the preprocess backward.  `shrow` is this gaussian's SH row staged in LDS: it holds
 // the coefficients on entry and receives their gradients (each channel's coefficients are read into
 // registers before that channel's gradients overwrite them).
 __device__ __forceinline__ void preprocess_bwd_one(
-    const d3gs_params& P, const int i, const float* __restrict__ xyz, const float* __restrict__ quat,
-    const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ cov2d,
-    const uint8_t* __restrict__ ne0,
-    // the blend backward's record of this gaussian: duv(2) dconic(3) dopacity dcolor(3) dz
-    const float4 ra, const float4 rb, const float4 rc,
-    const int sh_mask_compat,
+    const d3gs_params& P, const int i, const BwdInputs& in, const int sh_mask_compat,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* shrow, float* __restrict__ dsh_base) {
+    const float4 ra = in.ra, rb = in.rb, rc = in.rc;
     const int K = P.sh_stride;
 
     const float* W = P.w2c;
-    float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+    float d[3] = {in.xyz[0] - P.cam_center[0], in.xyz[1] - P.cam_center[1], in.xyz[2] - P.cam_center[2]};
     float pc[3] = {dot3(W + 0, d), dot3(W + 3, d), dot3(W + 6, d)};
     float z = pc[2];
     // pinhole backward (camera.py:357-369)
@@ -304,7 +327,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
     float dpc[3] = {gu * zi, gv * zi, (dzin + ((-gu) * pc[0]) * zi2) + ((-gv) * pc[1]) * zi2};
 
     // conic -> cov2d backward (gs3d.py:571-586)
-    float a = cov2d[3 * i], b = cov2d[3 * i + 1], c = cov2d[3 * i + 2];
+    float a = in.cov[0], b = in.cov[1], c = in.cov[2];
     float g0 = ra.z, g1 = ra.w, g2 = rb.x;
     float det = a * c - b * b;
     float k2 = 1.0f / (det * det + 1e-8f);
@@ -319,7 +342,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
         const float a0 = a - lf, c0 = c - lf;
         const float ratio = (a0 * c0 - b * b) / det;
         const float comp = sqrtf(fmaxf(0.000025f, ratio));
-        const float op_act = P.fused_activation ? det_sigmoid(opacity[i]) : opacity[i];
+        const float op_act = P.fused_activation ? det_sigmoid(in.opacity) : in.opacity;
         const float dcomp = dop_in * op_act;
         const float dratio = ratio <= 0.000025f ? 0.0f : (dcomp * 0.5f) / comp;
         const float gm = dratio * k2;
@@ -329,10 +352,10 @@ __device__ __forceinline__ void preprocess_bwd_one(
         dop_in = dop_in * comp;
     }
 
-    const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
+    const float4 qr = in.q;
     float qn = 1.0f;
     float q[4] = {qr.x, qr.y, qr.z, qr.w};
-    float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+    float s[3] = {in.s[0], in.s[1], in.s[2]};
     if (P.fused_activation) {
         qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
         q[0] = qr.x / qn; q[1] = qr.y / qn; q[2] = qr.z / qn; q[3] = qr.w / qn;
@@ -416,7 +439,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
         float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
         *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
                                                                 (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
-        float o = det_sigmoid(opacity[i]);
+        float o = det_sigmoid(in.opacity);
         dopacity_out[i] = dop_in * (o * (1.0f - o));
     } else {
         // inputs were activated by the caller: gradients w.r.t. the activated values
@@ -430,7 +453,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
     // SH backward (gs3d.py:262-364)
     float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
     float x = d[0] / dn, y = d[1] / dn, zd = d[2] / dn;
-    uint32_t m = ne0[i];
+    uint32_t m = in.ne0;
     float cg[3];
     if (sh_mask_compat) {
         cg[0] = rb.z * ((m & 1) ? 0.0f : 1.0f);
@@ -655,15 +678,16 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     __syncthreads();
     for (int base = 0; base < nactive; base += rows_per_pass) {
         const int cnt = min(rows_per_pass, nactive - base);
+        const int g = first + s_list[base + min(tid, cnt - 1)];
+        BwdInputs in = {};
+        if (tid < cnt) in = load_bwd_inputs(g, xyz, quat, scale, opacity, cov2d, ne0, rec4);
         bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride);
         __syncthreads();
         if (tid < cnt) {
-            const int g = first + s_list[base + tid];
             d3gs_params Pg = P;
             if constexpr (kInstances) apply_instance(Pg, inst, g);
-            preprocess_bwd_one(Pg, g, xyz, quat, scale, opacity, cov2d, ne0, rec4[4 * (size_t)g],
-                               rec4[4 * (size_t)g + 1], rec4[4 * (size_t)g + 2], sh_mask_compat, dxyz, dquat, dscale,
-                               dopacity_out, s_rows + tid * stride, dsh_base);
+            preprocess_bwd_one(Pg, g, in, sh_mask_compat, dxyz, dquat, dscale, dopacity_out, s_rows + tid * stride,
+                               dsh_base);
         }
         __syncthreads();
         bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride);
