@@ -42,10 +42,10 @@ STAGE_BYTES = {
     "tile_ranges": lambda N, M, P, T, passes: 4 * M + 12 * T,
     "blend_fwd": lambda N, M, P, T, passes: 40 * M + 20 * P,
     "blend_bwd": lambda N, M, P, T, passes: 76 * M + 36 * P,
-    # every gaussian's record and radius are read (68 B); only gaussians with a non-zero record (A of them) are
-    # worked on: 250 B of parameters and SH read, 236 B of gradients written.  With A = N this is the 522 B x N of
-    # a kernel that treats every gaussian alike.
-    "preprocess_bwd": lambda N, M, P, T, passes, A=None: 68 * N + (250 + 236) * (N if A is None else A),
+    # every gaussian's radius and mark are read (5 B); only gaussians whose record received anything (A of them)
+    # are worked on: 64 B of record, 250 B of parameters and SH read, 236 B of gradients written.  With A = N this
+    # is, up to the marks, the 522 B x N of a kernel that treats every gaussian alike.
+    "preprocess_bwd": lambda N, M, P, T, passes, A=None: 5 * N + (64 + 250 + 236) * (N if A is None else A),
 }
 
 
