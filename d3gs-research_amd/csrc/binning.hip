@@ -254,6 +254,7 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     __shared__ Key s_key[kBlock / 64][kKeyStage];
     __shared__ int32_t s_val[kBlock / 64][kKeyStage];
     __shared__ int s_start[kBlock / 64][64], s_slot[kBlock / 64][64];
+    __shared__ unsigned char s_owner[kBlock / 64][kKeyStage];
     // no early return: every lane takes part in the cooperative emission of large gaussians
     const int j_raw = blockIdx.x * kBlock + threadIdx.x;
     const bool in_range = j_raw < P.n;
@@ -281,8 +282,8 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     const bool walk_again = active && !has_mask;
     // The pairs of the wavefront's gaussians that come from masks are assembled in LDS, packed, and leave as
     // coalesced segments: consecutive lanes write consecutive slots, stepping over the runs of the (few, large)
-    // gaussians that are walked again below.  The owner of packed element e is the last lane whose packed start
-    // is <= e (lanes without pairs share their successor's start), found by a binary search over the starts.
+    // gaussians that are walked again below.  Each packed element carries the lane it came from, which gives its
+    // slot: the lane's first slot plus the element's place in the lane's run.
     const int my_cnt = (active && has_mask) ? (int)(end - off) : 0;
     int incl = my_cnt;
 #pragma unroll
@@ -301,15 +302,11 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
                            [&](long long e, uint64_t key) {
                                s_key[wave][e] = sizeof(Key) == 8 ? (Key)key : (Key)(key >> 32);
                                s_val[wave][e] = i;
+                               s_owner[wave][e] = (unsigned char)lane;
                            });
         __builtin_amdgcn_wave_barrier();
         for (int e = lane; e < packed_total; e += 64) {
-            int lo = 0, hi = 63;
-#pragma unroll
-            for (int step = 0; step < 6; ++step) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (s_start[wave][mid] <= e) lo = mid; else hi = mid - 1;
-            }
+            const int lo = s_owner[wave][e];
             const long long slot = wave_base + s_slot[wave][lo] + (e - s_start[wave][lo]);
             keys[slot] = s_key[wave][e];
             vals[slot] = s_val[wave][e];
