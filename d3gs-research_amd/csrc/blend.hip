@@ -295,10 +295,15 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 if constexpr (kRgba) acc3 = acc3 + w;
                 if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
                 pxf = stop ? __builtin_nanf("") : pxf;
-                if (__any(stop) && __all(pxf != pxf)) goto wave_finished;
+                // every pixel of the patch finished: both loops end at their next test (one way out of the
+                // loops keeps the scalar control flow short; the scalar unit is shared by the CU's four SIMDs
+                // and this kernel issues two scalar instructions for every three vector ones)
+                if (__any(stop) && __all(pxf != pxf)) {
+                    m = 0ull;
+                    chunk = 4;
+                }
             }
         }
-    wave_finished:;
     }
 
     if (inside) {
