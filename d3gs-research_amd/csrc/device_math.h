@@ -379,6 +379,7 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
     }
     int count = 0;
     const bool big = area > kSmallWalk;
+    const float my_inv_bw = 1.0f / (float)w.bw;
     if (!big) {
         int lx = 0, ly = 0;
         for (int t = 0; t < area; ++t) {
@@ -397,7 +398,9 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
         const int a = ws.bw * ws.bh;
         int c = 0;
         unsigned long long first = 0ull;
-        const float inv_bw = 1.0f / (float)ws.bw;   // row of candidate t: exact for the rect sizes a screen can hold
+        // row of candidate t: exact for the rect sizes a screen can hold.  Every lane divides once for its own
+        // gaussian (below the loop); dividing here would be one division per large gaussian, one after the other.
+        const float inv_bw = bcast_f(my_inv_bw, src);
         for (int base = 0; base < a; base += 64) {
             const int t = base + lane;
             bool k = false;
@@ -465,6 +468,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
     }
     const int lane = threadIdx.x & 63;
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
+    const float my_inv_bw = 1.0f / (float)w.bw;
     unsigned long long todo = __ballot(big);
     while (todo) {
         const int src = __builtin_ctzll(todo);
@@ -475,7 +479,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
         long long o = ((long long)bcast_i((int)(off >> 32), src) << 32) | (uint32_t)bcast_i((int)off, src);
         const long long e = ((long long)bcast_i((int)(end >> 32), src) << 32) | (uint32_t)bcast_i((int)end, src);
         const int a = ws.bw * ws.bh;
-        const float inv_bw = 1.0f / (float)ws.bw;
+        const float inv_bw = bcast_f(my_inv_bw, src);   // one division per lane, not one per large gaussian
         for (int base = 0; base < a; base += 64) {
             const int t = base + lane;
             bool k = false;
