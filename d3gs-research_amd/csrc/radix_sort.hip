@@ -32,11 +32,16 @@ constexpr int kOsThreads = 512;
 constexpr int kOsWaves = kOsThreads / 64;
 constexpr int kOsItems = 8;
 constexpr int kOsTile = kOsThreads * kOsItems;  // 4096 pairs per workgroup
-// Digits are 8 bits wide, or 9 where that saves a pass (18 or 27 key bits: the depth keys of the gaussians).
+// Digits are 7, 8 or 9 bits wide: the narrowest width that reaches the fewest passes.  9 saves a pass on 18 or 27
+// key bits (the depth keys of the gaussians); 7 costs none on 9 to 14 bits (the tile ids of an image of up to
+// 16384 tiles) and makes the ranking one ballot shorter and a digit's run in the output twice as long.
 constexpr int kOsMaxRadix = 512;
 static inline int os_digit_bits(int begin_bit, int end_bit) {
     const int bits = end_bit - begin_bit;
-    return (bits + 8) / 9 < (bits + 7) / 8 ? 9 : 8;
+    const int fewest = (bits + 8) / 9;
+    for (int d = 7; d < 9; ++d)
+        if ((bits + d - 1) / d == fewest) return d;
+    return 9;
 }
 constexpr uint32_t kFlagAggregate = 1u << 30;
 constexpr uint32_t kFlagPrefix = 2u << 30;
@@ -341,12 +346,10 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
     int copies = kHistCopies;
     while (copies > 1 && (size_t)copies * passes * radix * sizeof(uint32_t) > 64 * 1024) copies >>= 1;
     const size_t hist_lds = (size_t)copies * passes * radix * sizeof(uint32_t);
-    if (digit == 9)
-        hipLaunchKernelGGL((os_hist_kernel<Key, 9>), dim3(hist_blocks), dim3(kHistThreads), hist_lds, s, keys_a,
-                           (long long)m, (const long long*)m_device, begin_bit, end_bit, passes, copies, ws.hist);
-    else
-        hipLaunchKernelGGL((os_hist_kernel<Key, 8>), dim3(hist_blocks), dim3(kHistThreads), hist_lds, s, keys_a,
-                           (long long)m, (const long long*)m_device, begin_bit, end_bit, passes, copies, ws.hist);
+    auto hist_kernel = digit == 9 ? os_hist_kernel<Key, 9> : digit == 8 ? os_hist_kernel<Key, 8> : os_hist_kernel<Key, 7>;
+    auto pass_kernel = digit == 9 ? os_pass_kernel<Key, 9> : digit == 8 ? os_pass_kernel<Key, 8> : os_pass_kernel<Key, 7>;
+    hipLaunchKernelGGL(hist_kernel, dim3(hist_blocks), dim3(kHistThreads), hist_lds, s, keys_a, (long long)m,
+                       (const long long*)m_device, begin_bit, end_bit, passes, copies, ws.hist);
     Key* kin = keys_a;
     Key* kout = keys_b;
     const int32_t* vin = values_are_indices ? nullptr : vals_a;   // first pass only
@@ -358,14 +361,8 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         const uint32_t mask = (1u << nb) - 1u;
         const uint32_t* pass_hist = ws.hist + (size_t)p * radix;
         uint32_t* pass_status = ws.status + (size_t)p * ntiles * radix;
-        if (digit == 9)
-            hipLaunchKernelGGL((os_pass_kernel<Key, 9>), dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout,
-                               (long long)m, (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status,
-                               ws.error);
-        else
-            hipLaunchKernelGGL((os_pass_kernel<Key, 8>), dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout,
-                               (long long)m, (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status,
-                               ws.error);
+        hipLaunchKernelGGL(pass_kernel, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
+                           (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status, ws.error);
         std::swap(kin, kout);
         vin = vout;
         vout = in_b ? vals_b : vals_a;

@@ -299,7 +299,7 @@ def test_scan_gathered_c_abi(n, permuted, dirty):
 @pytest.mark.parametrize("m,cap,begin,end,implicit", [(1000, 1000, 0, 13, False), (70001, 90000, 0, 32, True),
                                                       (0, 5000, 0, 13, False), (3_000_000, 3_100_000, 2, 15, True),
                                                       (9000, 5000, 0, 32, False),
-                                                      # 27 and 18 key bits take 9-bit digits (3 and 2 passes)
+                                                      # 27 and 18 key bits take 9-bit digits (3 and 2 passes), 13 bits 7-bit digits
                                                       (70001, 90000, 0, 27, True), (1_000_000, 1_000_000, 0, 27, True),
                                                       (5000, 5000, 0, 18, False), (300_000, 300_000, 3, 30, True)])
 def test_sort_pairs_u32_c_abi(m, cap, begin, end, implicit):
