@@ -89,6 +89,7 @@ __global__ __launch_bounds__(kBlock) void os_clear_kernel(uint32_t* __restrict__
 // same-address conflicts of skewed digits (the exponent byte of a depth takes a handful of values).
 constexpr int kHistThreads = 1024;
 constexpr int kHistCopies = 8;
+constexpr int kHistMaxBlocks = 256, kHistKeysPerThread = 4;   // 128 workgroups were no faster, 64 slower
 template <typename Key, int kBits>
 __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __restrict__ keys, long long m,
                                                                 const long long* __restrict__ m_device,
@@ -102,14 +103,23 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __rest
     __syncthreads();
     uint32_t* mine = h + (threadIdx.x & (copies - 1)) * table;
     const long long stride = (long long)gridDim.x * kHistThreads;
-    for (long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x; i < m; i += stride) {
-        const Key key = keys[i];
+    auto count = [&](Key key) {
         for (int p = 0; p < passes; ++p) {
             const int bit = begin_bit + kBits * p;
             const int nb = min(kBits, end_bit - bit);
             atomicAdd(&mine[p * kRadix + ((uint32_t)(key >> bit) & ((1u << nb) - 1u))], 1u);
         }
+    };
+    // four independent loads in flight per thread: with one, a workgroup per CU waits a memory round trip per key
+    long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x;
+    for (; i + 3 * stride < m; i += 4 * stride) {
+        const Key k0 = keys[i], k1 = keys[i + stride], k2 = keys[i + 2 * stride], k3 = keys[i + 3 * stride];
+        count(k0);
+        count(k1);
+        count(k2);
+        count(k3);
     }
+    for (; i < m; i += stride) count(keys[i]);
     __syncthreads();
     for (int k = threadIdx.x; k < table; k += kHistThreads) {
         uint32_t c = 0;
@@ -341,7 +351,7 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
     // a fill kernel, not a memset node, so the call can be captured in a graph
     if (!workspace_is_zero)
         hipLaunchKernelGGL(os_clear_kernel, dim3(512), dim3(kBlock), 0, s, (uint32_t*)workspace, need / 4);
-    const int hist_blocks = (int)std::min<int64_t>(256, (m + kHistThreads * 4 - 1) / (kHistThreads * 4));
+    const int hist_blocks = (int)std::min<int64_t>(kHistMaxBlocks, (m + kHistThreads * kHistKeysPerThread - 1) / (kHistThreads * kHistKeysPerThread));
     // as many LDS copies of the histogram table as fit in 64 KB (a power of two, at most kHistCopies)
     int copies = kHistCopies;
     while (copies > 1 && (size_t)copies * passes * radix * sizeof(uint32_t) > 64 * 1024) copies >>= 1;
