@@ -15,8 +15,10 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
+ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
+COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP = -1, -2
 
 
 class Params(C.Structure):
@@ -66,6 +68,8 @@ _SIGNATURES = {
                                   C.POINTER(C.c_int), _VP]),
     "d3gs_sort_pairs_u32": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_size_t, C.c_int64, _VP, C.c_int, C.c_int, C.c_int, C.c_int,
                                       C.POINTER(C.c_int), _VP]),
+    "d3gs_sort_error_offset": (C.c_int, [C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
+    "d3gs_sort_status": (C.c_int, [_VP, C.c_size_t, C.c_int64, C.c_int, C.c_int, _VP, _VP, _VP]),
     "d3gs_tile_ranges": (C.c_int, [_VP, C.c_int64, _VP, C.c_int32, _VP, _VP]),
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),

@@ -210,7 +210,7 @@ __global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(
             s_prefix = prefix;
             if (chunk == (int)gridDim.x - 1) {
                 const uint32_t err = __hip_atomic_load(ws.error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const long long grand = err ? -1ll : prefix + total;
+                const long long grand = err ? (long long)D3GS_COUNT_SCAN_GAVE_UP : prefix + total;
                 if (total_out) *total_out = grand;
                 // pinned host memory is mapped into the device's address space: the count reaches the host with
                 // this store, and is visible there once the host has waited for the kernel
@@ -409,8 +409,31 @@ __device__ __forceinline__ int order_wave_max(int v) {
     return v;
 }
 
+// What a caller reads back in place of the pair count when one of the sorts that built the lists gave up
+// a look-back: the error words of the two sort workspaces are folded into the count words (device and
+// pinned host) by the last kernel of the binning, so a mis-sorted list never passes for a result.
+struct BinStatus {
+    const uint32_t* sort_error[2];   // error words of the depth sort and the pair sort (either may be NULL)
+    int64_t* total_dev;              // count words to poison (either may be NULL)
+    int64_t* total_host;
+};
+
+__device__ __forceinline__ void fold_sort_errors(const BinStatus& st) {
+    uint32_t err = 0;
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+        if (st.sort_error[k]) err |= __hip_atomic_load(st.sort_error[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (err) {
+        if (st.total_dev) *st.total_dev = D3GS_COUNT_SORT_GAVE_UP;
+        if (st.total_host) *st.total_host = D3GS_COUNT_SORT_GAVE_UP;
+    }
+}
+
+__global__ void bin_status_kernel(BinStatus st) { fold_sort_errors(st); }
+
 __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t* __restrict__ work, int num_tiles,
-                                                                   int32_t* __restrict__ order) {
+                                                                   int32_t* __restrict__ order, BinStatus st) {
+    if (threadIdx.x == 0) fold_sort_errors(st);
     __shared__ int s_bin[kOrderBuckets];
     __shared__ int s_wave[kOrderThreads / 64];
     __shared__ int s_max[kOrderThreads / 64];
@@ -621,7 +644,9 @@ extern "C" int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t*
 
 template <typename Key>
 static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, const int64_t* m_device,
-                            int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream) {
+                            int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream,
+                            BinStatus status = BinStatus{{nullptr, nullptr}, nullptr, nullptr}) {
+    const bool report = (status.sort_error[0] || status.sort_error[1]) && (status.total_dev || status.total_host);
     if (m < 0 || num_tiles < 0) { set_error("%s: bad argument", who); return D3GS_ERR_INVALID_ARGUMENT; }
     if ((m > 0 && !keys_sorted) || (num_tiles > 0 && !workload_ranges)) {
         set_error("%s: NULL buffer", who);
@@ -634,7 +659,9 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
                            (int)num_tiles);
     if (tile_order && num_tiles > 0)
         hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(kOrderThreads), 0, (hipStream_t)stream, workload_ranges,
-                           (int)num_tiles, tile_order);
+                           (int)num_tiles, tile_order, status);
+    else if (report)
+        hipLaunchKernelGGL(bin_status_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, status);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
@@ -645,6 +672,17 @@ extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t*
     return tile_ranges_impl<uint64_t>("d3gs_tile_ranges", keys_sorted, m, nullptr, workload_ranges, num_tiles, tile_order,
                                       stream);
 }
+
+namespace d3gs {
+int tile_ranges_u32_with_status(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
+                                int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
+                                const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
+                                int64_t* total_host, d3gs_stream_t stream) {
+    return tile_ranges_impl<uint32_t>("d3gs_bin_pairs (tile ranges)", tile_keys_sorted, m, m_device, workload_ranges,
+                                      num_tiles, tile_order, stream,
+                                      BinStatus{{sort_error_a, sort_error_b}, total_dev, total_host});
+}
+}  // namespace d3gs
 
 extern "C" int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
                                     int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,

@@ -405,10 +405,16 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read or write
+            if ((unsigned)g < (unsigned)P.n) {
                 s_id[tid] = g;
                 bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
                 s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
+            } else {
+                // a corrupt index list must not become a wild read or write: the slot is staged as a gaussian
+                // nobody visits (bits = 0) with finite parameters, and id -1 keeps the flush away from it
+                s_id[tid] = -1;
+                s_g[tid] = StagedGaussian{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                s_rgb[tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             }
         }
         publish_masks(bits, wave, lane, s_mask);
@@ -507,13 +513,14 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         // side sees one line-wide atomic request per (tile, gaussian) instead of one per value.
         const int slot_k = tid & 15;
         for (int gl = tid >> 4; gl < flush_cnt; gl += kBlock / 16) {
-            const float v = slot_k < kValues ? s_grad[slot_k][gl] : 0.0f;
-            if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * s_id[gl] + slot_k, v);
+            const int gid = s_id[gl];
+            const float v = (slot_k < kValues && gid >= 0) ? s_grad[slot_k][gl] : 0.0f;
+            if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * gid + slot_k, v);
             // one byte per gaussian that received anything: the preprocess backward finds its work in this
             // dense array instead of reading every record
             if (touched) {
                 const unsigned long long nz = __ballot(v != 0.0f);
-                if (slot_k == 0 && ((nz >> (tid & 48)) & 0xFFFFull)) touched[s_id[gl]] = 1;
+                if (slot_k == 0 && ((nz >> (tid & 48)) & 0xFFFFull)) touched[gid] = 1;
             }
         }
     }

@@ -39,6 +39,12 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
                              total_dev, /*values_are_indices=*/0, workspaces_are_zero, 0, d3gs_higher_msb((uint32_t)num_tiles),
                              pairs_in_b, stream);
     if (rc) return rc;
-    return d3gs_tile_ranges_u32(*pairs_in_b ? tile_keys_b : tile_keys_a, capacity, total_dev, workload_ranges, num_tiles,
-                                tile_order, stream);
+    // the last kernel replaces the pair count by D3GS_COUNT_SORT_GAVE_UP when either sort raised its error word
+    size_t err_depth = 0, err_pairs = 0;
+    d3gs_sort_error_offset(n, 0, d3gs_depth_key_bits(p), &err_depth);
+    d3gs_sort_error_offset(capacity, 0, d3gs_higher_msb((uint32_t)num_tiles), &err_pairs);
+    const uint32_t* e_depth = n > 0 && depth_sort_ws ? (const uint32_t*)((const char*)depth_sort_ws + err_depth) : nullptr;
+    const uint32_t* e_pairs = capacity > 0 && pair_sort_ws ? (const uint32_t*)((const char*)pair_sort_ws + err_pairs) : nullptr;
+    return tile_ranges_u32_with_status(*pairs_in_b ? tile_keys_b : tile_keys_a, capacity, total_dev, workload_ranges,
+                                       num_tiles, tile_order, e_depth, e_pairs, total_dev, total_host, stream);
 }

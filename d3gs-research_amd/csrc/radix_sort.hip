@@ -288,6 +288,15 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
     }
 }
 
+// Reports a finished sort's error word: 0, or D3GS_ERR_SORT_LOOKBACK when a workgroup's bounded wait ran out
+// (the output is then not sorted).  One thread; the host word is pinned, device-mapped memory.
+__global__ void os_status_kernel(const uint32_t* __restrict__ error, int32_t* __restrict__ status_dev,
+                                 int32_t* __restrict__ status_host) {
+    const int32_t st = __hip_atomic_load(error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ? D3GS_ERR_SORT_LOOKBACK : 0;
+    if (status_dev) *status_dev = st;
+    if (status_host) *status_host = st;
+}
+
 static inline size_t os_align(size_t v) { return (v + 255) / 256 * 256; }
 static inline int os_tiles(int64_t m) { return (int)((m + kOsTile - 1) / kOsTile); }
 static inline int os_passes(int begin_bit, int end_bit) {
@@ -319,6 +328,33 @@ extern "C" int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, 
     }
     const int passes = os_passes(begin_bit, end_bit) > 0 ? os_passes(begin_bit, end_bit) : 1;
     *bytes_out_host = os_layout(m, passes, 1 << os_digit_bits(begin_bit, end_bit), nullptr, nullptr);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sort_error_offset(int64_t m, int begin_bit, int end_bit, size_t* offset_out_host) {
+    if (m < 0 || begin_bit < 0 || end_bit > 64 || begin_bit > end_bit || !offset_out_host) {
+        set_error("d3gs_sort_error_offset: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const int passes = os_passes(begin_bit, end_bit) > 0 ? os_passes(begin_bit, end_bit) : 1;
+    // the error word follows the digit histograms (os_layout)
+    *offset_out_host = os_align((size_t)passes * (1 << os_digit_bits(begin_bit, end_bit)) * 4);
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sort_status(const void* workspace, size_t workspace_bytes, int64_t m, int begin_bit, int end_bit,
+                                int32_t* status_dev, int32_t* status_host, d3gs_stream_t stream) {
+    size_t off = 0;
+    int rc = d3gs_sort_error_offset(m, begin_bit, end_bit, &off);
+    if (rc) return rc;
+    if (!workspace || workspace_bytes < off + sizeof(uint32_t) || (!status_dev && !status_host)) {
+        set_error("d3gs_sort_status: NULL or short workspace, or no status word to write");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(os_status_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream,
+                       (const uint32_t*)((const char*)workspace + off), status_dev, status_host);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_sort_status: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 

@@ -160,6 +160,7 @@ class GaussianSplatOp:
         # optional per-stage timing: set to a dict to collect torch.cuda.Event pairs
         self.stage_events: dict[str, list] | None = None
         self.last_num_rendered = 0
+        self.last_forward_fused = False
         # The SH colours are only read by the blend, so they are computed on a second stream beside the
         # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
         self.overlap_sh_colors = True
@@ -170,7 +171,12 @@ class GaussianSplatOp:
         # training: the model-gradient arrays are allocated with the forward pass and cleared by its blend kernel
         self.clear_gradients_early = True
         self._pair_capacity = 0
+        # Pinned host words the kernels report into (the pair count; the two sorts' status on the launch-by-launch
+        # path).  One set per op: an op serves one forward at a time -- two forwards of the same op that overlap
+        # (two host threads, or two streams) would race on these words and on _pair_capacity.  Use one op per
+        # stream.
         self._count_host: torch.Tensor | None = None
+        self._sort_status_host: torch.Tensor | None = None
         self._side_stream: torch.cuda.Stream | None = None
 
     # ------------------------------------------------------------------ utils
@@ -452,12 +458,15 @@ class GaussianSplatOp:
             sh_done = torch.cuda.Event()
             sh_done.record(side)
 
-        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None):
+        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None,
+                  status_slot=None):
             keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
             nbytes = _sort_ws_bytes(count, begin_bit, end_bit)
             ws = zero_ws if zero_ws is not None else torch.empty(nbytes, dtype=torch.uint8, device=dev)
             assert ws.numel() >= nbytes
             in_b = C.c_int(0)
+            if status_slot is not None:
+                self._sort_status_host[status_slot] = 0
             if keys_a.dtype == torch.int64:
                 rc = L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
                                        _capi.ptr(ws), nbytes, count, begin_bit, end_bit, C.byref(in_b), s)
@@ -466,15 +475,35 @@ class GaussianSplatOp:
                                            _capi.ptr(ws), nbytes, count, count_dev, int(values_are_indices),
                                            int(zero_ws is not None), begin_bit, end_bit, C.byref(in_b), s)
             _capi.check(rc, "d3gs_sort_pairs")
+            if status_slot is not None and count > 0 and end_bit > begin_bit:
+                status_pending.append((ws, nbytes, count, begin_bit, end_bit, status_slot))
             return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
+
+        status_pending = []
+
+        def _report_sort_status():
+            """The error word of every sort issued since the last call (a look-back that gave up) goes to its
+            pinned host word, by a one-thread kernel behind the sort (outside the stage timers)."""
+            while status_pending:
+                ws, nbytes, count, begin_bit, end_bit, slot = status_pending.pop()
+                _capi.check(L.d3gs_sort_status(_capi.ptr(ws), nbytes, count, begin_bit, end_bit, None,
+                                               C.c_void_p(self._sort_status_host.data_ptr() + 4 * slot), s),
+                            "d3gs_sort_status")
+
+        def _check_sort_status(slot, what):
+            if int(self._sort_status_host[slot]) != 0:
+                raise RuntimeError(f"d3gs_sort_pairs_u32 ({what}): a workgroup's bounded wait on an earlier tile ran "
+                                   "out; the list is not sorted")
 
         # With buffers sized from the previous view and no stage timers, the whole binning is one call into the
         # library (d3gs_bin_pairs): the launches of this phase are short, and issuing them one by one from
         # Python leaves the GPU idle between them.
         fused = bool(self.fused_binning and spec_capacity > 0 and self.stage_events is None)
+        self.last_forward_fused = fused      # which of the two binning paths this view took (tests look at it)
         fused_result = None
         if self._count_host is None:
             self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+            self._sort_status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
         if fused:
             cap = spec_capacity
             up = lambda v: (v + 63) // 64 * 64          # 256-byte aligned slices of one int32 allocation
@@ -509,7 +538,9 @@ class GaussianSplatOp:
             # tile digits only: 2 passes over M pairs instead of 6.
             with self._stage("depth_order"):
                 depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0,
-                                                          depth_bits, values_are_indices=True, zero_ws=zero_ws_n)
+                                                          depth_bits, values_are_indices=True, zero_ws=zero_ws_n,
+                                                          status_slot=0)
+            _report_sort_status()
 
             with self._stage("scan"):
                 # tile counts gathered into depth order and scanned in one launch
@@ -556,6 +587,7 @@ class GaussianSplatOp:
             return out, None
 
         pooled_ranges_used = [False]
+        pair_sort_done = [None]      # launch-by-launch path: recorded behind the pair sort's status word
 
         def _bin_and_blend(capacity: int, count_on_device: bool):
             """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
@@ -577,7 +609,11 @@ class GaussianSplatOp:
                                 "d3gs_make_keys")
                 with self._stage("sort"):
                     tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0, tile_bits, m_dev,
-                                                                  zero_ws=zero_ws_m if count_on_device else None)
+                                                                  zero_ws=zero_ws_m if count_on_device else None,
+                                                                  status_slot=1)
+                _report_sort_status()
+                pair_sort_done[0] = torch.cuda.Event()
+                pair_sort_done[0].record()
                 with self._stage("tile_ranges"):
                     # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
                     workload_ranges = zero_ranges if not pooled_ranges_used[0] else torch.zeros((num_tiles, 2), dtype=i32, device=dev)
@@ -610,14 +646,23 @@ class GaussianSplatOp:
             ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
         count_ready.synchronize()
         num_rendered = int(self._count_host[0])
+        if num_rendered == _capi.COUNT_SORT_GAVE_UP:
+            raise RuntimeError("d3gs_bin_pairs: a sort workgroup's bounded wait on an earlier tile ran out; "
+                               "the tile lists are not sorted")
         if num_rendered < 0:
             raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
+        if not fused:
+            _check_sort_status(0, "depth order")
         self.last_num_rendered = num_rendered
         self._pair_capacity = num_rendered + num_rendered // 4 + 4096
         if num_rendered == 0:
             return _empty_result()
         if ctx is None or num_rendered > capacity:
             ctx, tile_keys_sorted = _bin_and_blend(num_rendered, False)
+        if pair_sort_done[0] is not None:
+            # everything is enqueued; the host only waits for the pair sort's status word, the blend runs on
+            pair_sort_done[0].synchronize()
+            _check_sort_status(1, "tile lists")
         ctx.gaussian_idx_sorted = ctx.gaussian_idx_sorted[:num_rendered]
         if custom_features is not None:
             out.custom_features = self._blend_custom_features(P, ctx, out, custom_features)

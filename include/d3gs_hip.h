@@ -31,13 +31,19 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 24
+#define D3GS_ABI_VERSION 25
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
 #define D3GS_ERR_UNSUPPORTED (-2)
 #define D3GS_ERR_WORKSPACE_TOO_SMALL (-3)
 #define D3GS_ERR_LAUNCH (-4)
+#define D3GS_ERR_SORT_LOOKBACK (-5) /* status word of d3gs_sort_status: a workgroup's bounded wait ran out */
+
+/* Values a pair-count word (total_dev / total_host of d3gs_scan_gathered and d3gs_bin_pairs) takes in place of
+ * the count when a kernel's bounded wait on an earlier workgroup ran out; the lists are then not valid. */
+#define D3GS_COUNT_SCAN_GAVE_UP (-1)
+#define D3GS_COUNT_SORT_GAVE_UP (-2)
 
 /* EarlyFilterAlgo, d3sim/algos/d3gs/config_def.py:59-70 */
 #define D3GS_FILTER_NONE 0
@@ -149,7 +155,7 @@ int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t w
 
 /* K2 over a permutation, in one launch: out[j] = sum_{i <= j} src[index[i]] (index NULL: the identity), the same
  * `cumsum_` (render.py:694-695) taken in the order K3 emits the pairs; the grand total goes to *total_dev
- * (device int64; -1 if the kernel's bounded wait on an earlier chunk ran out) and, when total_host is not NULL, to
+ * (device int64; D3GS_COUNT_SCAN_GAVE_UP if the kernel's bounded wait on an earlier chunk ran out) and, when total_host is not NULL, to
  * that word of pinned (device-mapped) host memory as well, stored by the kernel itself: the host may read it
  * once it has waited for the stream to pass this call.  An index outside [0, src_n)
  * counts as 0.  The workspace (size from d3gs_scan_gathered_workspace_bytes) must be zero on entry:
@@ -211,6 +217,18 @@ int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int
                         int workspace_is_zero, int begin_bit, int end_bit, int* result_in_b_host,
                         d3gs_stream_t stream);
 
+/* Error report of a sort (the reference's sort throws through TV_THROW_RT_ERR, devsort.py:34-37).  The pass
+ * kernels learn where their digits start from the workgroups before them by polling status words; the polling is
+ * bounded, and a workgroup whose wait runs out raises an error word in the workspace and carries on, so the
+ * grid always drains but the output is not sorted.  d3gs_sort_status enqueues, behind the sort on `stream`, a
+ * one-thread kernel that writes 0 or D3GS_ERR_SORT_LOOKBACK to *status_dev (device) and *status_host (pinned,
+ * device-mapped host memory; the host reads it once it has waited for the stream to pass this call); either
+ * may be NULL.  workspace, m and the bit range are those of the sort call.  d3gs_sort_error_offset gives the
+ * byte offset of that uint32 error word inside the workspace for callers that copy it out themselves. */
+int d3gs_sort_error_offset(int64_t m, int begin_bit, int end_bit, size_t* offset_out_host);
+int d3gs_sort_status(const void* workspace, size_t workspace_bytes, int64_t m, int begin_bit, int end_bit,
+                     int32_t* status_dev, int32_t* status_host, d3gs_stream_t stream);
+
 /* K5 — replaces kernel_1d("prepare_workload_range_...") at render.py:896-939.
  * ranges[num_tiles][2] must be zero-filled by the caller.  tile_order (int32[num_tiles],
  * may be NULL) receives the tile ids sorted by descending list length: a launch order
@@ -230,7 +248,10 @@ int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int6
  * Results: *order_in_b / *pairs_in_b say which of the a / b buffers hold the depth order and the sorted pairs;
  * *total_dev the pair count M (the kernels touch min(M, capacity) pairs: a caller that sized capacity from a
  * guess compares M with it afterwards and bins again when M is larger); total_host, when not NULL, is a pinned
- * host word that the scan kernel stores M to (see d3gs_scan_gathered).  Workspace sizes as for the single calls
+ * host word that the scan kernel stores M to (see d3gs_scan_gathered).  When either sort raised its error word
+ * (see d3gs_sort_status) the last kernel of the call replaces the count in *total_dev and *total_host by
+ * D3GS_COUNT_SORT_GAVE_UP, so a caller that checks the count for a negative value never takes a mis-sorted list
+ * for a result.  Workspace sizes as for the single calls
  * (d3gs_sort_workspace_bytes(n, 0, d3gs_depth_key_bits(p)), d3gs_scan_gathered_workspace_bytes(n),
  * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))); workspaces_are_zero != 0 says the caller has
  * cleared all three.  workload_ranges must be zero on entry. */

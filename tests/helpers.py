@@ -34,3 +34,35 @@ def grad_close(a, b, rel=1e-4, abs_frac=1e-5):
     bad = err > tol
     worst = float((err / np.maximum(tol, 1e-300)).max()) if b.size else 0.0
     return (not bad.any()), worst, int(bad.sum())
+
+
+def per_gaussian_rel_err(a, b):
+    """Relative L2 error of each gaussian's gradient vector (rows of a against rows of b), over the gaussians
+    whose reference gradient is not zero; the denominator has a floor of 1e-6 of the largest norm."""
+    n = b.shape[0]
+    a = np.asarray(a, np.float64).reshape(n, -1)
+    b = np.asarray(b, np.float64).reshape(n, -1)
+    rn = np.linalg.norm(b, axis=1)
+    return (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
+
+
+def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11):
+    """What rounding noise in the blend backward's sums does to the preprocess backward, measured on the
+    oracle.  A float32 sum of the per-pixel terms, in whatever order, carries an error of the order of
+    2^-24 * sum|terms| ("absmass", which the oracle returns next to its float64 sums).  The oracle's own
+    preprocess backward is run again on the screen-space gradients perturbed by N(0, 1) * ulps * 2^-24 * absmass;
+    returned: {gradient name: (median, 99th percentile)} of the per-gaussian relative error it induces.  The
+    spread beyond the input noise is the conditioning of the chain rule itself (near-degenerate projected
+    covariances: gradients that are small differences of large terms)."""
+    rng = np.random.default_rng(seed)
+    eps = ulps * 2.0 ** -24
+    m = g_ref["absmass"]
+    noisy = {"duv": g_ref["duv"] + rng.standard_normal(g_ref["duv"].shape) * eps * m[:, 0:2],
+             "dconic": g_ref["dconic"] + rng.standard_normal(g_ref["dconic"].shape) * eps * m[:, 2:5],
+             "dopacity": g_ref["dopacity"] + rng.standard_normal(g_ref["dopacity"].shape) * eps * m[:, 5],
+             "dcolor": g_ref["dcolor"] + rng.standard_normal(g_ref["dcolor"].shape) * eps * m[:, 6:9]}
+    pert = O.preprocess_bwd(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                            ref["radii"], ref["cov2d_vecs"], ref["sh_to_rgb_ne_0"],
+                            *(noisy[k].astype(np.float32) for k in ("duv", "dconic", "dopacity", "dcolor")))
+    return {k: tuple(np.quantile(per_gaussian_rel_err(pert[k], pb_ref[k]), [0.5, 0.99]))
+            for k in ("dxyz", "dquat", "dscale", "dopacity", "dsh")}

@@ -104,7 +104,7 @@ def test_non_fused_model_family(oracle, cfg_id, n, wh, filt):
         rn = np.linalg.norm(b, axis=1)
         e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = np.quantile(e, [0.5, 0.99])
-        assert med <= 1e-4 and p99 <= 5e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
+        assert med <= 1e-5 and p99 <= 1e-3, f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}"
 
     # raw-tensor gradients through torch's activations == the fused kernels' raw-tensor gradients
     def raw_grads(model):
@@ -119,6 +119,8 @@ def test_non_fused_model_family(oracle, cfg_id, n, wh, filt):
         rn = np.linalg.norm(b, axis=1)
         e = (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = np.quantile(e, [0.5, 0.99])
+        # two different forward passes (torch's exp / normalize / sigmoid against the kernels' own): the rendered
+        # inputs themselves differ by a few ulp, hence the wider bar than against the oracle on identical inputs
         assert med <= 1e-4 and p99 <= 5e-3, f"{name}: fused vs torch-activated median {med:.2e} p99 {p99:.2e}"
 
 

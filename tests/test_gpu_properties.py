@@ -101,7 +101,7 @@ def test_forward_is_deterministic_and_backward_is_linear():
         rn = c.norm(dim=1)
         e = ((a + b - c).norm(dim=1) / (rn + 1e-6 * rn.max()))[rn > 0]
         med, p99 = float(e.quantile(0.5)), float(torch.quantile(e[:: max(1, e.numel() // 1_000_000)], 0.99))
-        assert med <= 1e-4 and p99 <= 1e-2, f"{name}: additivity per-gaussian median {med:.2e} p99 {p99:.2e}"
+        assert med <= 1e-5 and p99 <= 2e-3, f"{name}: additivity per-gaussian median {med:.2e} p99 {p99:.2e}"
 
 
 @pytest.mark.parametrize("fused", [True, False])
