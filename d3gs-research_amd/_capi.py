@@ -19,6 +19,7 @@ ABI_VERSION = 25
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
 COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP = -1, -2
+SCAN_NOALLOC_MAX_N = 1 << 24   # D3GS_SCAN_NOALLOC_MAX_N
 
 
 class Params(C.Structure):
@@ -60,6 +61,7 @@ _SIGNATURES = {
                                  C.POINTER(C.c_int), _VP]),
     "d3gs_scan_gathered_workspace_bytes": (C.c_int, [C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_scan_gathered": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP, C.c_size_t, C.c_int32, _VP, _VP, _VP]),
+    "d3gs_scan_gathered_noalloc": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP, _VP, _VP]),
     "d3gs_make_keys": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [C.c_int64, _VP]),
     "d3gs_depth_keys": (C.c_int, [_VP, C.c_int32, _VP, _VP, _VP]),
     "d3gs_gather_i32": (C.c_int, [_VP, C.c_int32, _VP, C.c_int32, _VP, _VP]),

@@ -5,6 +5,8 @@
 //
 // Reference: d3sim/algos/d3gs/render.py:694-695 (cumsum), 739-840 (keys),
 // 845-887 + d3sim/csrc/devsort.py:38-149 (CUB radix sort), 896-939 (ranges).
+#include <mutex>
+
 #include "device_math.h"
 
 namespace d3gs {
@@ -566,6 +568,64 @@ extern "C" int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_scan_gathered: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
+}
+
+// ---------------------------------------------------------------------------
+// d3gs_scan_gathered for callers that cannot allocate (code under graph capture, serving loops, harnesses that
+// forbid hipMalloc): the look-back's status words and error word live in a file-scope device array instead of a
+// caller workspace.  Every GPU the library runs on holds its own copy of the array, at its own address, until
+// the process ends; the address is resolved once per device, with that device current.
+// ---------------------------------------------------------------------------
+constexpr int kScratchMaxN = D3GS_SCAN_NOALLOC_MAX_N;
+constexpr size_t kScratchBytes =
+    ((size_t)((kScratchMaxN + d3gs::kGatherScanChunk - 1) / d3gs::kGatherScanChunk) * sizeof(unsigned long long) +
+     2 * sizeof(uint32_t) + 255) / 256 * 256;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kScratchMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kScratchMaxDevices] = {};
+
+// Device address of `scratch` on the current device (NULL and an error text on failure).  In host code the
+// array's name is only a handle for the runtime: everything that touches the memory goes through this pointer.
+static void* scratch_on_current_device(const char* who) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kScratchMaxDevices) {
+        set_error("%s: cannot tell the current device (%s)", who, e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+
+extern "C" int d3gs_scan_gathered_noalloc(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n,
+                                          int32_t* out, int64_t* total_dev, int64_t* total_host,
+                                          d3gs_stream_t stream) {
+    if (n < 0 || src_n < 0 || !total_dev) {
+        set_error("d3gs_scan_gathered_noalloc: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (n > kScratchMaxN) {
+        set_error("d3gs_scan_gathered_noalloc: n = %d exceeds the built-in scratch (at most %d elements); use "
+                  "d3gs_scan_gathered with a caller workspace", n, kScratchMaxN);
+        return D3GS_ERR_WORKSPACE_TOO_SMALL;
+    }
+    void* ws = scratch_on_current_device("d3gs_scan_gathered_noalloc");
+    if (!ws) return D3GS_ERR_LAUNCH;
+    // the array keeps the previous call's status words: workspace_is_zero = 0 clears the part this call uses,
+    // with a fill kernel (not a memset node) so that the call can be captured in a graph
+    return d3gs_scan_gathered(src, src_n, index, n, out, ws, kScratchBytes, /*workspace_is_zero=*/0, total_dev,
+                              total_host, stream);
 }
 
 extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspace, size_t workspace_bytes,

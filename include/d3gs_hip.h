@@ -165,6 +165,19 @@ int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, 
                        void* workspace, size_t workspace_bytes, int32_t workspace_is_zero, int64_t* total_dev,
                        int64_t* total_host, d3gs_stream_t stream);
 
+/* d3gs_scan_gathered without a workspace argument, for callers that cannot allocate one.  It has no counterpart
+ * in the reference (whose `cumsum_` allocates its temporary storage inside torch); it is meant for code under HIP
+ * graph capture, tight serving loops and harnesses that forbid hipMalloc.  The look-back's status words live in
+ * a file-scope device array of the library (64 KiB + 256 B per GPU, held until the process ends), so n is limited
+ * to D3GS_SCAN_NOALLOC_MAX_N elements (a larger n returns D3GS_ERR_WORKSPACE_TOO_SMALL).  The call allocates and
+ * frees nothing; it clears the part of the array it uses with a fill kernel on `stream` and then runs the same
+ * kernel as d3gs_scan_gathered: same outputs bit for bit.  The array is resolved for the device that is
+ * current at the first call on that device (make that first call outside a graph capture).  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams) race; calls on one stream are safe. */
+#define D3GS_SCAN_NOALLOC_MAX_N (1 << 24)
+int d3gs_scan_gathered_noalloc(const int32_t* src, int32_t src_n, const int32_t* index, int32_t n, int32_t* out,
+                               int64_t* total_dev, int64_t* total_host, d3gs_stream_t stream);
+
 /* K3 — replaces kernel_1d("prepare_sort_data_...") at render.py:739-840.
  * Without gaussian_order (NULL) this is the reference's call: offsets = the inclusive
  * scan of tiles_touched from d3gs_scan_tiles, m = its total, pairs are emitted in
