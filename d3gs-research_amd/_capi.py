@@ -15,8 +15,9 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
+BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
 ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
 COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP = -1, -2
 SCAN_NOALLOC_MAX_N = 1 << 24   # D3GS_SCAN_NOALLOC_MAX_N
@@ -38,6 +39,7 @@ class Params(C.Structure):
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
         ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
+        ("batch_size", C.c_int32), ("reserved0", C.c_int32), ("batch_cameras", C.c_void_p),
     ]
 
 
@@ -78,6 +80,8 @@ _SIGNATURES = {
     "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
     "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 10 + [C.c_int32, C.c_int32] + [_VP] * 6 +
                             [C.POINTER(Instances), _VP]),
+    "d3gs_preprocess_bwd_camera": (C.c_int, [C.POINTER(Params), C.c_int32, C.c_int32] + [_VP] * 10 +
+                                   [C.c_int32, C.c_int32] + [_VP] * 6 + [C.POINTER(Instances), _VP]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

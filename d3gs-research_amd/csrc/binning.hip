@@ -259,13 +259,14 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     __shared__ unsigned char s_owner[kBlock / 64][kKeyStage];
     // no early return: every lane takes part in the cooperative emission of large gaussians
     const int j_raw = blockIdx.x * kBlock + threadIdx.x;
-    const bool in_range = j_raw < P.n;
-    const int j = in_range ? j_raw : P.n - 1;
+    const int items = item_count(P);     // gaussians x cameras of a bundle
+    const bool in_range = j_raw < items;
+    const int j = in_range ? j_raw : items - 1;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // slot j of the emission order holds gaussian order[j] (identity without an order table);
     // `offsets` is the inclusive scan of the tile counts taken in that same order
     int i = order ? order[j] : j;
-    const bool sane = (unsigned)i < (unsigned)P.n;
+    const bool sane = (unsigned)i < (unsigned)items;
     i = sane ? i : 0;
     const long long end = offsets[j];
     long long off = !in_range ? end : (j == 0 ? 0 : offsets[j - 1]);   // lanes past the end: an empty range at the total
@@ -326,6 +327,12 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
         const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
         TileWalkIn g{uv.x, uv.y, (float)radii[i], co.x, co.y, co.z, co.w};
         walk = tile_walk_setup(P, g);
+        // camera b of a bundle owns the tile rows from b * tiles_y on (render.py:787, 809); the shift moves the
+        // 3-sigma rect and the candidate rect together, so the per-tile decisions are the single camera's
+        const int shift = P.batch_size > 1 ? (i / P.n) * P.tiles_y : 0;
+        walk.bminy += shift;
+        walk.rminy += shift;
+        walk.rmaxy += shift;
     }
     wave_tile_emit<Key>(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
 }
@@ -655,6 +662,10 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
     if (p->n == 0 || m == 0) return D3GS_OK;
+    if (p->batch_size > 1 && p->enable_32bit_sort) {
+        set_error("d3gs_make_keys: a camera bundle with enable_32bit_sort is not supported");
+        return D3GS_ERR_UNSUPPORTED;
+    }
     if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
         !gaussian_idx) {
         set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");
@@ -664,7 +675,7 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
         set_error("d3gs_make_keys: tile_masks must be 16-byte aligned");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    const dim3 grid((p->n + kBlock - 1) / kBlock), block(kBlock);
+    const dim3 grid((item_count(*p) + kBlock - 1) / kBlock), block(kBlock);
     if (keys)
         hipLaunchKernelGGL(make_keys_kernel<uint64_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
                            depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,

@@ -193,9 +193,24 @@ __device__ __forceinline__ void select2_or_zero(unsigned long long mask, float a
         : "v"(a0), "v"(b0), "s"(mask));
 }
 
-// Index of channel ch of pixel pid in the colour image: [H,W,C] or, with use_nchw, [C,H,W].
-__device__ __forceinline__ size_t color_index(const d3gs_params& P, size_t pid, int ch, int channels) {
-    return P.use_nchw ? (size_t)ch * P.width * P.height + pid : pid * channels + ch;
+// Index of channel ch of pixel pid (= y * W + x) of image `batch` in the colour images: [B,H,W,C] or, with
+// use_nchw, [B,C,H,W].
+__device__ __forceinline__ size_t color_index(const d3gs_params& P, int batch, size_t pid, int ch, int channels) {
+    const size_t plane = (size_t)P.width * P.height;
+    return P.use_nchw ? ((size_t)batch * channels + ch) * plane + pid : ((size_t)batch * plane + pid) * channels + ch;
+}
+
+// Which camera of a bundle and which of its tiles a tile id b * tiles + y * tiles_x + x names (render.py:1515-1522,
+// 1561); a single camera has batch 0.
+struct TilePlace { int batch, tx, ty; };
+__device__ __forceinline__ TilePlace place_tile(const d3gs_params& P, int tile) {
+    const int per_view = P.tiles_x * P.tiles_y;
+    TilePlace t;
+    t.batch = P.batch_size > 1 ? tile / per_view : 0;
+    const int local = tile - t.batch * per_view;
+    t.ty = local / P.tiles_x;
+    t.tx = local - t.ty * P.tiles_x;
+    return t;
 }
 
 // kDepth: blend the camera-space depth as one more channel (render.py:1532-1539, 1915-1919).
@@ -224,10 +239,12 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
     constexpr int kChannels = kRgba ? 4 : 3;
 
-    const int ntiles = P.tiles_x * P.tiles_y;
+    const int ntiles = P.tiles_x * P.tiles_y * batch_count(P);
+    const int items = item_count(P);
     const int tile = tile_for_block(blockIdx.x, tile_order);
     if (tile < 0 || tile >= ntiles) return;
-    const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
+    const TilePlace place = place_tile(P, tile);
+    const int tx = place.tx, ty = place.ty;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
     const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
@@ -254,7 +271,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            if ((unsigned)g < (unsigned)P.n) {  // a corrupt index list must not become a wild read
+            if ((unsigned)g < (unsigned)items) {  // a corrupt index list must not become a wild read
                 bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
                 s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
             }
@@ -308,17 +325,18 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
 
     if (inside) {
         const size_t pid = (size_t)py * P.width + px;
-        final_T[pid] = T;
-        n_contrib[pid] = contributor;
+        const size_t gpid = (size_t)place.batch * P.width * P.height + pid;     // pixel of the [B,H,W] images
+        final_T[gpid] = T;
+        n_contrib[gpid] = contributor;
         if constexpr (kDepth)  // inference normalises by the opacity (render.py:2244-2254)
-            final_depth[pid] = P.training ? depth_accum : depth_accum / ((1e-10f + 1.0f) - T);
+            final_depth[gpid] = P.training ? depth_accum : depth_accum / ((1e-10f + 1.0f) - T);
         const float acc[4] = {acc0, acc1, acc2, acc3};
 #pragma unroll
         for (int ch = 0; ch < kChannels; ++ch) {
             float v = acc[ch];
             // the alpha channel has no background (render.py:2227-2229)
             if (!P.training) v = fminf(fmaxf(v + T * (ch < 3 ? P.bg[ch] : 0.0f), 0.0f), 1.0f);
-            color[color_index(P, pid, ch, kChannels)] = v;
+            color[color_index(P, place.batch, pid, ch, kChannels)] = v;
         }
     }
 }
@@ -348,10 +366,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     __shared__ int s_wmax[4];
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 
-    const int ntiles = P.tiles_x * P.tiles_y;
+    const int ntiles = P.tiles_x * P.tiles_y * batch_count(P);
+    const int items = item_count(P);
     const int tile = tile_for_block(blockIdx.x, tile_order);
     if (tile < 0 || tile >= ntiles) return;
-    const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
+    const TilePlace place = place_tile(P, tile);
+    const int tx = place.tx, ty = place.ty;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int px = tx * kTile + (wave & 1) * 8 + (lane & 7);
     const int py = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
@@ -359,6 +379,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     const float pxf = (float)px, pyf = (float)py;
     const float tile_x0 = (float)(tx * kTile), tile_y0 = (float)(ty * kTile);
     const size_t pid = (size_t)py * P.width + px;
+    const size_t gpid = (size_t)place.batch * P.width * P.height + pid;     // pixel of the [B,H,W] images
 
     const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
     const int len = r1 - r0;
@@ -369,22 +390,22 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     float rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f, rr3 = 0.0f, dr0 = 0.0f, dr1 = 0.0f, dr2 = 0.0f, dr3 = 0.0f;
     float rdep = 0.0f, ddep = 0.0f;
     if (inside) {
-        contributor = min(n_contrib[pid] + 1, len);
-        render_T = final_T[pid];
-        dT_val = dT[pid];
-        rr0 = color[color_index(P, pid, 0, kChannels)];
-        rr1 = color[color_index(P, pid, 1, kChannels)];
-        rr2 = color[color_index(P, pid, 2, kChannels)];
-        dr0 = drgb[color_index(P, pid, 0, kChannels)];
-        dr1 = drgb[color_index(P, pid, 1, kChannels)];
-        dr2 = drgb[color_index(P, pid, 2, kChannels)];
+        contributor = min(n_contrib[gpid] + 1, len);
+        render_T = final_T[gpid];
+        dT_val = dT[gpid];
+        rr0 = color[color_index(P, place.batch, pid, 0, kChannels)];
+        rr1 = color[color_index(P, place.batch, pid, 1, kChannels)];
+        rr2 = color[color_index(P, place.batch, pid, 2, kChannels)];
+        dr0 = drgb[color_index(P, place.batch, pid, 0, kChannels)];
+        dr1 = drgb[color_index(P, place.batch, pid, 1, kChannels)];
+        dr2 = drgb[color_index(P, place.batch, pid, 2, kChannels)];
         if constexpr (kRgba) {
-            rr3 = color[color_index(P, pid, 3, kChannels)];
-            dr3 = drgb[color_index(P, pid, 3, kChannels)];
+            rr3 = color[color_index(P, place.batch, pid, 3, kChannels)];
+            dr3 = drgb[color_index(P, place.batch, pid, 3, kChannels)];
         }
         if constexpr (kDepth) {
-            rdep = final_depth[pid];
-            ddep = ddepth[pid];
+            rdep = final_depth[gpid];
+            ddep = ddepth[gpid];
         }
     }
     const float dT_term = (-dT_val) * render_T;
@@ -405,7 +426,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         uint32_t bits = 0;
         if (src < r1) {
             const int g = idx_sorted[src];
-            if ((unsigned)g < (unsigned)P.n) {
+            if ((unsigned)g < (unsigned)items) {
                 s_id[tid] = g;
                 bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
                 s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
@@ -530,7 +551,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
 
 using namespace d3gs;
 
-static int blend_grid(const d3gs_params* p) { return p->tiles_x * p->tiles_y; }
+static int blend_grid(const d3gs_params* p) { return p->tiles_x * p->tiles_y * batch_count(*p); }
 
 static int finish_launch(const char* who) {
     hipError_t e = hipGetLastError();

@@ -511,6 +511,25 @@ __device__ constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f,
                                        0.3731763325901154f, -0.4570457994644658f, 1.445305721320277f,
                                        -0.5900435899266435f};
 
+// Camera bundles: a call with batch_size = B > 1 works on B * n render items, item i = b * n + g.
+__host__ __device__ __forceinline__ int batch_count(const d3gs_params& P) { return P.batch_size > 1 ? P.batch_size : 1; }
+__host__ __device__ __forceinline__ int item_count(const d3gs_params& P) { return P.n * batch_count(P); }
+// Camera b of the bundle into the per-camera fields (what make_params fills for a single camera); tan_fov is
+// 0.5 * resolution / focal in float32, as the host computes it (render.py:358).
+__device__ __forceinline__ void apply_batch_camera(d3gs_params& P, int b) {
+    const float* m = P.batch_cameras + D3GS_BATCH_CAMERA_FLOATS * (size_t)b;
+#pragma unroll
+    for (int k = 0; k < 9; ++k) P.w2c[k] = m[k];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) P.cam_center[k] = m[9 + k];
+    P.fx = m[12];
+    P.fy = m[13];
+    P.cx = m[14];
+    P.cy = m[15];
+    P.tan_fovx = (0.5f * (float)P.width) / P.fx;
+    P.tan_fovy = (0.5f * (float)P.height) / P.fy;
+}
+
 // Thread-local error string helpers live in capi.hip.
 void set_error(const char* fmt, ...);
 // Validates sizes / enum values of a params block (defined in preprocess.hip).

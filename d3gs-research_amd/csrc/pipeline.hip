@@ -20,8 +20,8 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
         set_error("d3gs_bin_pairs: bad argument");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    const int32_t n = p->n;
-    const int32_t num_tiles = p->tiles_x * p->tiles_y;
+    const int32_t n = item_count(*p);                               // render items: gaussians x cameras of a bundle
+    const int32_t num_tiles = p->tiles_x * p->tiles_y * batch_count(*p);
     int rc = d3gs_sort_pairs_u32(depth_keys_a, depth_keys_b, order_a, order_b, depth_sort_ws, depth_sort_ws_bytes, n,
                                  nullptr, /*values_are_indices=*/1, workspaces_are_zero, 0,
                                  d3gs_depth_key_bits(p), order_in_b, stream);

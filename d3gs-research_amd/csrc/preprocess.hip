@@ -78,6 +78,7 @@ struct InstanceView {
 };
 
 __device__ __forceinline__ void apply_instance(d3gs_params& P, const InstanceView& inst, int i) {
+    if (!inst.ids) return;
     const int id = inst.ids[i];
     if (id >= 0 && id < inst.count) {
         const float* m = inst.cameras + 12 * (size_t)id;
@@ -108,10 +109,19 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     }
     // no early return: every lane of the wavefront takes part in the cooperative tile count
     const int i_raw = blockIdx.x * kPrepBlock + threadIdx.x;
-    const bool in_range = i_raw < P0.n;
-    const int i = in_range ? i_raw : P0.n - 1;
-    d3gs_params P = P0;     // with instances: this lane's camera
-    if constexpr (kInstances) apply_instance(P, inst, i);
+    const int items = item_count(P0);
+    const bool in_range = i_raw < items;
+    const int i = in_range ? i_raw : items - 1;     // render item: outputs and the reject mask are indexed by it
+    d3gs_params P = P0;     // with instances or a camera bundle: this lane's camera
+    int g = i, batch = 0;   // gaussian (row of the model arrays) and camera of the item
+    if constexpr (kInstances) {
+        if (P0.batch_size > 1) {
+            batch = i / P0.n;
+            g = i - batch * P0.n;
+            apply_batch_camera(P, batch);
+        }
+        if (inst.ids) apply_instance(P, inst, g);
+    }
 
     bool valid = true;
     float z = 0.0f, u = 0.0f, v = 0.0f, con0 = 0.0f, con1 = 0.0f, con2 = 0.0f, op = 0.0f;
@@ -121,7 +131,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     float rgb[3] = {0.0f, 0.0f, 0.0f};
     uint32_t ne0 = 0;
 
-    float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+    float d[3] = {xyz[3 * g] - P.cam_center[0], xyz[3 * g + 1] - P.cam_center[1], xyz[3 * g + 2] - P.cam_center[2]};
     float pc[3] = {dot3(P.w2c + 0, d), dot3(P.w2c + 3, d), dot3(P.w2c + 6, d)};
     z = pc[2];
     valid = in_range && (z >= P.z_near && z <= P.z_far) && !(invalid_mask && invalid_mask[i]);
@@ -129,9 +139,9 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         u = ((pc[0] / z) * P.fx + P.cx) - 0.5f;
         v = ((pc[1] / z) * P.fy + P.cy) - 0.5f;
 
-        const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * i);
+        const float4 qr = *reinterpret_cast<const float4*>(quat + 4 * g);
         float q[4] = {qr.x, qr.y, qr.z, qr.w};
-        float s[3] = {scale[3 * i], scale[3 * i + 1], scale[3 * i + 2]};
+        float s[3] = {scale[3 * g], scale[3 * g + 1], scale[3 * g + 2]};
         if (P.fused_activation) {
             float qn = sqrtf(((qr.x * qr.x + qr.y * qr.y) + qr.z * qr.z) + qr.w * qr.w);
             q[0] = qr.x / qn; q[1] = qr.y / qn; q[2] = qr.z / qn; q[3] = qr.w / qn;
@@ -156,7 +166,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         c = dot3(t1, v1) + P.lowpass;
 
         float det;
-        op = P.fused_activation ? det_sigmoid(opacity[i]) : opacity[i];
+        op = P.fused_activation ? det_sigmoid(opacity[g]) : opacity[g];
         if (P.enable_anti_aliasing) {
             // gs3d.py:592-617: exact inverse of the low-passed covariance; the determinant handed on to
             // the radius and the det > 0 test is the one without the low-pass term (render.py:466-476);
@@ -195,13 +205,16 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         if (valid) walk = tile_walk_setup(P, g);
         bool has_mask;
         count = wave_tile_count(P.filter_algo, valid, walk, kept_mask, has_mask);
+        // the tile rows of camera b start at b * tiles_y: the record's origin carries the camera, so that key
+        // expansion emits b * tiles + y * tiles_x + x (render.py:787, 809) without knowing about bundles
+        walk.bminy += batch * P.tiles_y;
         kept_meta = tile_mask_meta(walk, has_mask);
     }
     if (valid && kWithSh) {
         float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
         float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
         const float* shp = s_rows + threadIdx.x * stride;
-        const float* base = P.has_sh_base ? sh_base + 3 * i : shp;
+        const float* base = P.has_sh_base ? sh_base + 3 * g : shp;     // (the fused colours run without a bundle: g = i)
         const float* rest = P.has_sh_base ? shp : shp + 3;
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch) rgb[ch] = sh_channel(P.sh_degree, dx, dy, dz, base[ch], rest, ch);
@@ -246,22 +259,30 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
     const int rowlen = P0.sh_stride * 3, stride = rowlen | 1;
     // grid-stride over 128-gaussian chunks: a small grid leaves most of every CU to the kernels this
     // one runs beside
-    for (int first = blockIdx.x * kPrepBlock; first < P0.n; first += gridDim.x * kPrepBlock) {
+    // (with a camera bundle: the chunks of camera 0, then those of camera 1, ...; a chunk never spans two cameras)
+    const int chunks_per_view = (P0.n + kPrepBlock - 1) / kPrepBlock;
+    for (int chunk = blockIdx.x; chunk < chunks_per_view * batch_count(P0); chunk += gridDim.x) {
+        const int batch = chunk / chunks_per_view;
+        const int first = (chunk - batch * chunks_per_view) * kPrepBlock;      // first gaussian of the chunk
         __syncthreads();   // the previous chunk's rows have been read
         rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
         __syncthreads();
-        const int i = first + threadIdx.x;
-        if (i >= P0.n) continue;
+        const int g = first + threadIdx.x;
+        if (g >= P0.n) continue;
+        const int i = batch * P0.n + g;     // render item
         d3gs_params P = P0;
-        if constexpr (kInstances) apply_instance(P, inst, i);
+        if constexpr (kInstances) {
+            if (P0.batch_size > 1) apply_batch_camera(P, batch);
+            if (inst.ids) apply_instance(P, inst, g);
+        }
         float rgb[3] = {0.0f, 0.0f, 0.0f};
         uint32_t ne0 = 0;
         if (radii[i] > 0) {
-            float d[3] = {xyz[3 * i] - P.cam_center[0], xyz[3 * i + 1] - P.cam_center[1], xyz[3 * i + 2] - P.cam_center[2]};
+            float d[3] = {xyz[3 * g] - P.cam_center[0], xyz[3 * g + 1] - P.cam_center[1], xyz[3 * g + 2] - P.cam_center[2]};
             float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
             float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
             const float* shp = s_rows + threadIdx.x * stride;
-            const float* base = P.has_sh_base ? sh_base + 3 * i : shp;
+            const float* base = P.has_sh_base ? sh_base + 3 * g : shp;
             const float* rest = P.has_sh_base ? shp : shp + 3;
 #pragma unroll
             for (int ch = 0; ch < 3; ++ch) rgb[ch] = sh_channel(P.sh_degree, dx, dy, dz, base[ch], rest, ch);
@@ -310,9 +331,11 @@ __device__ __forceinline__ BwdInputs load_bwd_inputs(const int i, const float* _
 // the coefficients on entry and receives their gradients (each channel's coefficients are read into
 // registers before that channel's gradients overwrite them).
 __device__ __forceinline__ void preprocess_bwd_one(
-    const d3gs_params& P, const int i, const BwdInputs& in, const int sh_mask_compat,
+    const d3gs_params& P, const int i, const BwdInputs& in, const int sh_mask_compat, const bool accumulate,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* shrow, float* __restrict__ dsh_base) {
+    // accumulate: the gradient arrays already hold the sum over the cameras before this one (camera bundles)
+    auto put = [accumulate](float* dst, float v) { *dst = accumulate ? *dst + v : v; };
     const float4 ra = in.ra, rb = in.rb, rc = in.rc;
     const int K = P.sh_stride;
 
@@ -432,23 +455,29 @@ __device__ __forceinline__ void preprocess_bwd_one(
     dq[2] = 2.0f * (((qx * (dR[2] + dR[6]) + qy * (dR[5] + dR[7])) - (2.0f * qz) * (dR[0] + dR[4])) + qw * (dR[3] - dR[1]));
     dq[3] = 2.0f * ((qz * (dR[3] - dR[1]) + qy * (dR[2] - dR[6])) + qx * (dR[7] - dR[5]));
     // activation backward: exp, normalize, sigmoid (origin/model.py:332-383)
+    float4 gq;
     if (P.fused_activation) {
-        dscale[3 * i + 0] = ds[0] * s[0];
-        dscale[3 * i + 1] = ds[1] * s[1];
-        dscale[3 * i + 2] = ds[2] * s[2];
+        put(dscale + 3 * i + 0, ds[0] * s[0]);
+        put(dscale + 3 * i + 1, ds[1] * s[1]);
+        put(dscale + 3 * i + 2, ds[2] * s[2]);
         float qd = ((q[0] * dq[0] + q[1] * dq[1]) + q[2] * dq[2]) + q[3] * dq[3];
-        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn,
-                                                                (dq[2] - q[2] * qd) / qn, (dq[3] - q[3] * qd) / qn);
+        gq = make_float4((dq[0] - q[0] * qd) / qn, (dq[1] - q[1] * qd) / qn, (dq[2] - q[2] * qd) / qn,
+                         (dq[3] - q[3] * qd) / qn);
         float o = det_sigmoid(in.opacity);
-        dopacity_out[i] = dop_in * (o * (1.0f - o));
+        put(dopacity_out + i, dop_in * (o * (1.0f - o)));
     } else {
         // inputs were activated by the caller: gradients w.r.t. the activated values
-        dscale[3 * i + 0] = ds[0];
-        dscale[3 * i + 1] = ds[1];
-        dscale[3 * i + 2] = ds[2];
-        *reinterpret_cast<float4*>(dquat + 4 * i) = make_float4(dq[0], dq[1], dq[2], dq[3]);
-        dopacity_out[i] = dop_in;
+        put(dscale + 3 * i + 0, ds[0]);
+        put(dscale + 3 * i + 1, ds[1]);
+        put(dscale + 3 * i + 2, ds[2]);
+        gq = make_float4(dq[0], dq[1], dq[2], dq[3]);
+        put(dopacity_out + i, dop_in);
     }
+    if (accumulate) {
+        const float4 old = *reinterpret_cast<const float4*>(dquat + 4 * i);
+        gq = make_float4(old.x + gq.x, old.y + gq.y, old.z + gq.z, old.w + gq.w);
+    }
+    *reinterpret_cast<float4*>(dquat + 4 * i) = gq;
 
     // SH backward (gs3d.py:262-364)
     float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
@@ -482,7 +511,8 @@ __device__ __forceinline__ void preprocess_bwd_one(
         float sv[15];
 #pragma unroll
         for (int k = 0; k < 15; ++k) sv[k] = k < used ? rest[k * 3 + ch] : 0.0f;
-        dbase[ch] = kShC0 * gch;
+        if (P.has_sh_base) put(dbase + ch, kShC0 * gch);   // global array; without a split base the row in LDS
+        else dbase[ch] = kShC0 * gch;
         float dx_ = 0.0f, dy_ = 0.0f, dz_ = 0.0f;
         if (deg > 0) {
             drest[0 * 3 + ch] = (-kShC1 * y) * gch;
@@ -533,9 +563,9 @@ __device__ __forceinline__ void preprocess_bwd_one(
     }
     float dirv[3] = {x, y, zd};
     float dd = (dirv[0] * ddir[0] + dirv[1] * ddir[1]) + dirv[2] * ddir[2];
-    dxyz[3 * i + 0] = gx[0] + (ddir[0] - dirv[0] * dd) / dn;
-    dxyz[3 * i + 1] = gx[1] + (ddir[1] - dirv[1] * dd) / dn;
-    dxyz[3 * i + 2] = gx[2] + (ddir[2] - dirv[2] * dd) / dn;
+    put(dxyz + 3 * i + 0, gx[0] + (ddir[0] - dirv[0] * dd) / dn);
+    put(dxyz + 3 * i + 1, gx[1] + (ddir[1] - dirv[1] * dd) / dn);
+    put(dxyz + 3 * i + 2, gx[2] + (ddir[2] - dirv[2] * dd) / dn);
 }
 
 // A gaussian whose record is all zero -- culled in the forward pass, or in tile lists but never reached before
@@ -562,7 +592,7 @@ static inline int bwd_rows_per_pass(int sh_stride) {
 // first + list[0 .. cnt)
 template <bool kToLds>
 __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float* lds, const unsigned short* list, int cnt,
-                                              int first, int rowlen, int stride) {
+                                              int first, int rowlen, int stride, bool accumulate = false) {
     if ((rowlen & 3) == 0 && ((uintptr_t)global & 15u) == 0) {
         const int per_row = rowlen >> 2;
         for (int q = threadIdx.x; q < cnt * per_row; q += kBwdBlock) {
@@ -572,6 +602,9 @@ __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float*
             if (kToLds) {
                 const float4 t = *gp;
                 lp[0] = t.x; lp[1] = t.y; lp[2] = t.z; lp[3] = t.w;
+            } else if (accumulate) {
+                const float4 t = *gp;
+                *gp = make_float4(t.x + lp[0], t.y + lp[1], t.z + lp[2], t.w + lp[3]);
             } else {
                 *gp = make_float4(lp[0], lp[1], lp[2], lp[3]);
             }
@@ -581,7 +614,7 @@ __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float*
             const int r = e / rowlen, c = e - r * rowlen;
             float* gp = global + (size_t)(first + list[r]) * rowlen + c;
             if (kToLds) lds[r * stride + c] = *gp;
-            else *gp = lds[r * stride + c];
+            else *gp = accumulate ? *gp + lds[r * stride + c] : lds[r * stride + c];
         }
     }
 }
@@ -593,7 +626,7 @@ __device__ __forceinline__ bool record_is_zero(const float4 ra, const float4 rb,
 
 template <int kPer, bool kInstances>
 __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
-    const d3gs_params P, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const d3gs_params P_in, const int batch_index, const int accumulate, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
     const float* __restrict__ grad_records, const uint8_t* __restrict__ touched, const int sh_mask_compat,
@@ -601,6 +634,10 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
+    // one camera per launch: with a bundle, camera batch_index from the table (every per-item array comes in
+    // offset to that camera's rows by the host side of the call)
+    d3gs_params P = P_in;
+    if (P_in.batch_size > 1) apply_batch_camera(P, batch_index);
     extern __shared__ float s_rows[];                    // rows_per_pass rows of `stride` floats
     __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
     __shared__ unsigned char s_active[kSpan];
@@ -657,7 +694,7 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     for (int k = 0; k < kPer; ++k)
         if (active[k])
             s_list[before[k] + __popcll(mates[k] & ((1ull << lane) - 1ull))] = (unsigned short)(k * kBwdBlock + tid);
-    if (!outputs_are_zero) {   // the zero gradients of the gaussians without work
+    if (!outputs_are_zero && !accumulate) {   // the zero gradients of the gaussians without work
 #pragma unroll
         for (int k = 0; k < kPer; ++k) {
             const int local = k * kBwdBlock + tid;
@@ -686,11 +723,11 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         if (tid < cnt) {
             d3gs_params Pg = P;
             if constexpr (kInstances) apply_instance(Pg, inst, g);
-            preprocess_bwd_one(Pg, g, in, sh_mask_compat, dxyz, dquat, dscale, dopacity_out, s_rows + tid * stride,
-                               dsh_base);
+            preprocess_bwd_one(Pg, g, in, sh_mask_compat, accumulate != 0, dxyz, dquat, dscale, dopacity_out,
+                               s_rows + tid * stride, dsh_base);
         }
         __syncthreads();
-        bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride);
+        bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride, accumulate != 0);
         __syncthreads();
     }
 }
@@ -719,7 +756,18 @@ int check_params(const d3gs_params* p, const char* who) {
         set_error("%s: unknown early_filter_algo %d", who, p->filter_algo);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    if (p->enable_32bit_sort && (!(p->depth_32bit_prec > 0.0f) || p->tiles_x * p->tiles_y >= (1 << 14))) {
+    if (p->batch_size < 0 || (p->batch_size > 1 && !p->batch_cameras)) {
+        set_error("%s: batch_size %d needs batch_cameras", who, p->batch_size);
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if ((long long)p->n * batch_count(*p) >= (1ll << 31) ||
+        (long long)p->tiles_y * batch_count(*p) >= (1ll << 16) ||
+        (long long)p->tiles_x * p->tiles_y * batch_count(*p) >= (1ll << 31)) {
+        set_error("%s: bundle of %d cameras is too large (render items and tiles must fit 31 bits, tile rows 16)", who,
+                  p->batch_size);
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    if (p->enable_32bit_sort && (!(p->depth_32bit_prec > 0.0f) || p->tiles_x * p->tiles_y * batch_count(*p) >= (1 << 14))) {
         // render.py:227-228: 14 bits of tile index above the 18 depth bits
         set_error("%s: enable_32bit_sort needs depth_32bit_prec > 0 and fewer than 2^14 tiles", who);
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -765,7 +813,13 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     }
     InstanceView inst;
     if (!instance_view(instances, &inst, "d3gs_preprocess_fwd")) return D3GS_ERR_INVALID_ARGUMENT;
-    dim3 grid((p->n + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
+    const bool bundle = p->batch_size > 1;
+    if (bundle && (with_sh || inst.ids)) {
+        set_error("d3gs_preprocess_fwd: a camera bundle takes its colours from d3gs_sh_colors (rgb_gaussian = NULL) "
+                  "and no instance table");
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    dim3 grid((item_count(*p) + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
     const size_t lds_bytes = with_sh ? (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float) : 0;
 #define D3GS_LAUNCH_K1(SH, INST)                                                                                      \
     hipLaunchKernelGGL((preprocess_fwd_kernel<SH, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,   \
@@ -773,7 +827,7 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
                        conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,                         \
                        (unsigned long long*)tile_masks, depth_sort_keys)
     if (with_sh) { if (inst.ids) D3GS_LAUNCH_K1(true, true); else D3GS_LAUNCH_K1(true, false); }
-    else         { if (inst.ids) D3GS_LAUNCH_K1(false, true); else D3GS_LAUNCH_K1(false, false); }
+    else         { if (inst.ids || bundle) D3GS_LAUNCH_K1(false, true); else D3GS_LAUNCH_K1(false, false); }
 #undef D3GS_LAUNCH_K1
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
@@ -792,10 +846,14 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
     }
     InstanceView inst;
     if (!instance_view(instances, &inst, "d3gs_sh_colors")) return D3GS_ERR_INVALID_ARGUMENT;
-    const int chunks = (p->n + kPrepBlock - 1) / kPrepBlock;
+    if (p->batch_size > 1 && inst.ids) {
+        set_error("d3gs_sh_colors: a camera bundle takes no instance table");
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    const int chunks = ((p->n + kPrepBlock - 1) / kPrepBlock) * batch_count(*p);
     dim3 grid(chunks < kShColorBlocks ? chunks : kShColorBlocks), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
-    if (inst.ids)
+    if (inst.ids || p->batch_size > 1)
         hipLaunchKernelGGL(sh_colors_kernel<true>, grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz, color_sh,
                            color_sh_base, radii, rgb_gaussian, sh_to_rgb_ne_0);
     else
@@ -814,8 +872,29 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
                                    float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
                                    float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                                    d3gs_stream_t stream) {
+    if (p && p->batch_size > 1) {
+        set_error("d3gs_preprocess_bwd: a camera bundle goes through d3gs_preprocess_bwd_camera, one call per camera");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    return d3gs_preprocess_bwd_camera(p, 0, 0, xyz, quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs,
+                                      sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat, outputs_are_zero, dxyz,
+                                      dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base, instances, stream);
+}
+
+extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,
+                                          const float* quaternion_xyzw, const float* scale, const float* opacity,
+                                          const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                                          const uint8_t* sh_to_rgb_ne_0, const float* grad_records,
+                                          const uint8_t* touched, int32_t sh_mask_compat, int32_t outputs_are_zero,
+                                          float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
+                                          float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
+                                          d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_bwd");
     if (rc) return rc;
+    if (batch_index < 0 || batch_index >= batch_count(*p)) {
+        set_error("d3gs_preprocess_bwd_camera: batch_index %d outside the bundle of %d", batch_index, batch_count(*p));
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
     if (p->n == 0) return D3GS_OK;
     // a model whose only colour coefficient is the split-off DC term has empty color_sh arrays (sh_stride 0)
     if (!xyz || !quaternion_xyzw || !scale || !opacity || !radii || !cov2d_vecs || !sh_to_rgb_ne_0 ||
@@ -833,7 +912,8 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
     const int per = wide ? 4 : 1;
     dim3 grid((p->n + kBwdBlock * per - 1) / (kBwdBlock * per)), block(kBwdBlock);
 #define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
-    hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,  \
+    hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p,            \
+                       (int)batch_index, (int)accumulate, inst, xyz,                                                   \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
                        touched,                                                                                        \
                        (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, dxyz, dquaternion_xyzw, dscale,      \

@@ -64,6 +64,10 @@ class GaussianSplatOpContext:
     # instance rendering: the view's camera in every instance frame ([I, 12] float32) and the int32 ids
     instance_cameras: torch.Tensor | None = None
     instance_ids: torch.Tensor | None = None
+    # camera bundle rendered in one pass (render.py:314-326): B cameras, every per-gaussian array above has
+    # B * N rows (item b * N + g), tile ids and ranges cover B * tiles; the [B, 16] camera table on the device
+    batch_size: int = 1
+    batch_cameras: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -161,6 +165,7 @@ class GaussianSplatOp:
         self.stage_events: dict[str, list] | None = None
         self.last_num_rendered = 0
         self.last_forward_fused = False
+        self.rebin_count = 0        # views that outgrew the pair buffers sized from the previous view
         # The SH colours are only read by the blend, so they are computed on a second stream beside the
         # latency-bound sort stages.  Set to False for a single-stream forward (the fused preprocess).
         self.overlap_sh_colors = True
@@ -170,6 +175,8 @@ class GaussianSplatOp:
         self.fused_binning = True
         # training: the model-gradient arrays are allocated with the forward pass and cleared by its blend kernel
         self.clear_gradients_early = True
+        # a CameraBundle of several cameras goes through the kernels in one pass (False: camera by camera)
+        self.bundle_in_one_pass = True
         self._pair_capacity = 0
         # Pinned host words the kernels report into (the pair count; the two sorts' status on the launch-by-launch
         # path).  One set per op: an op serves one forward at a time -- two forwards of the same op that overlap
@@ -246,7 +253,10 @@ class GaussianSplatOp:
             pp = np.array([intrinsic[0, 2], intrinsic[1, 2]], np.float32)
             c2w_T = np.ascontiguousarray(np.asarray(cameras.pose.to_world)[:3].T).astype(np.float32)
         elif isinstance(cameras, CameraBundle):
-            assert cameras.cam2world_T.shape[0] == 1, "one camera per kernel pass"
+            if cameras.cam2world_T.shape[0] != 1:
+                # several cameras: the kernels read them from the device table (see batch_table); nothing is
+                # brought to the host
+                return None, None, None, cameras.image_shape_wh
             fpp = cameras.focal_xy_ppoint[0].detach().cpu().numpy().astype(np.float32)
             focal, pp = fpp[:2], fpp[2:]
             c2w_T = cameras.cam2world_T[0].detach().cpu().numpy().astype(np.float32).reshape(4, 3)
@@ -290,8 +300,20 @@ class GaussianSplatOp:
             return None
         return C.byref(_capi.Instances(ids.data_ptr(), table.data_ptr(), int(table.shape[0])))
 
-    def make_params(self, model: GaussianModelOriginBase, cameras, training: bool) -> _capi.Params:
-        """Scalars the reference bakes into kernel source (render.py:198-230, 333-358)."""
+    @staticmethod
+    def batch_table(cameras: "CameraBundle", device) -> torch.Tensor:
+        """The cameras of a bundle as the [B, 16] float32 device table the kernels read (render.py:316-323 loads
+        the same values from cam2world_T [B, 4, 3] and focal_xy_ppoint [B, 4]): rows 0-2 of cam2world_T, its row 3
+        (the centre), focal x, y, principal point x, y.  Built on the device; nothing is read back."""
+        c2w = cameras.cam2world_T.detach().to(device=device, dtype=torch.float32).reshape(-1, 4, 3)
+        fpp = cameras.focal_xy_ppoint.detach().to(device=device, dtype=torch.float32).reshape(-1, 4)
+        assert c2w.shape[0] == fpp.shape[0], "cam2world_T and focal_xy_ppoint must hold one row per camera"
+        return torch.cat([c2w[:, :3, :].reshape(-1, 9), c2w[:, 3, :], fpp], dim=1).contiguous()
+
+    def make_params(self, model: GaussianModelOriginBase, cameras, training: bool, batch_cameras=None) -> _capi.Params:
+        """Scalars the reference bakes into kernel source (render.py:198-230, 333-358).  With ``batch_cameras``
+        (the [B, 16] device table of a bundle of B > 1 cameras) the per-camera fields stay zero: the kernels take
+        them from the table."""
         c = self._cfg
         focal, pp, c2w_T, (width, height) = self._camera_arrays(cameras)
         P = _capi.Params()
@@ -303,11 +325,18 @@ class GaussianSplatOp:
         P.has_sh_base = int(model.color_sh_base is not None)
         P.filter_algo = int(c.early_filter_algo)
         P.training = int(bool(training))
-        P.fx, P.fy, P.cx, P.cy = float(focal[0]), float(focal[1]), float(pp[0]), float(pp[1])
-        tan_fov = np.float32(0.5) * np.array([width, height], np.float32) / focal
-        P.tan_fovx, P.tan_fovy = float(tan_fov[0]), float(tan_fov[1])
-        P.w2c[:] = [float(v) for v in c2w_T[:3].reshape(-1)]
-        P.cam_center[:] = [float(v) for v in c2w_T[3]]
+        if batch_cameras is not None:
+            assert focal is None and batch_cameras.dtype == torch.float32 and batch_cameras.is_contiguous() \
+                and batch_cameras.shape[1] == _capi.BATCH_CAMERA_FLOATS
+            P.batch_size = int(batch_cameras.shape[0])
+            P.batch_cameras = batch_cameras.data_ptr()
+        else:
+            assert focal is not None, "a bundle of several cameras needs its device table (batch_table)"
+            P.fx, P.fy, P.cx, P.cy = float(focal[0]), float(focal[1]), float(pp[0]), float(pp[1])
+            tan_fov = np.float32(0.5) * np.array([width, height], np.float32) / focal
+            P.tan_fovx, P.tan_fovy = float(tan_fov[0]), float(tan_fov[1])
+            P.w2c[:] = [float(v) for v in c2w_T[:3].reshape(-1)]
+            P.cam_center[:] = [float(v) for v in c2w_T[3]]
         P.z_near, P.z_far, P.eps = float(c.near), float(c.far), float(c.eps)
         P.radii_eigen_eps = float(c.cov2d_radii_eigen_eps)
         P.clamp_factor = float(c.projected_clamp_factor)
@@ -347,7 +376,8 @@ class GaussianSplatOp:
                 custom_features=None, mask=None, prep_user_inputs=None):
         """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
         assert model.act_applied, "model must be activated before render"
-        if isinstance(cameras, CameraBundle) and len(cameras) != 1:
+        batch = len(cameras) if isinstance(cameras, CameraBundle) else 1
+        if batch != 1 and not self._bundle_in_one_pass(batch, instance2world_T, custom_features):
             return self._forward_bundle(model, cameras, training, instance2world_T, custom_features, mask,
                                         prep_user_inputs)
         if prep_user_inputs:
@@ -358,20 +388,24 @@ class GaussianSplatOp:
             assert custom_features.is_cuda and custom_features.dtype == torch.float32 and custom_features.ndim == 2 \
                 and custom_features.shape[0] == len(model), "custom_features must be a float32 cuda tensor [N, F]"
         if mask is not None:
-            # True rejects the gaussian (render.py:306-308)
-            assert mask.is_cuda and mask.dtype in (torch.bool, torch.uint8) and mask.numel() == len(model) \
+            # True rejects the gaussian (render.py:306-308); one entry per (camera, gaussian)
+            assert mask.is_cuda and mask.dtype in (torch.bool, torch.uint8) and mask.numel() == batch * len(model) \
                 and mask.is_contiguous(), "mask must be a contiguous bool/uint8 cuda tensor with one entry per gaussian"
             if mask.dtype == torch.bool:
                 mask = mask.view(torch.uint8)
         L = self._lib
-        P = self.make_params(model, cameras, training)
+        dev = model.xyz.device
+        batch_cams = self.batch_table(cameras, dev) if batch > 1 else None
+        P = self.make_params(model, cameras, training, batch_cams)
         inst_ids = inst_cams = None
         if instance2world_T is not None:
             inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
         inst = self._instances_arg(inst_ids, inst_cams)
-        n, dev = P.n, model.xyz.device
+        # n: render items = gaussians x cameras (item b * N + g is gaussian g seen by camera b); everything the
+        # preprocess writes has one row per item, the tile ids carry the camera
+        n = P.n * batch
         width, height = P.width, P.height
-        num_tiles = P.tiles_x * P.tiles_y
+        num_tiles = P.tiles_x * P.tiles_y * batch
         s = self._stream()
         f32, i32 = torch.float32, torch.int32
 
@@ -420,6 +454,7 @@ class GaussianSplatOp:
                 pool_floats = self._grad_pool_floats(model) if self.clear_gradients_early else 0
                 mark_floats = (n + 15) // 16 * 4          # n bytes, in whole 16-byte units
                 grad_clear = torch.empty(rec_floats + pool_floats + mark_floats, dtype=f32, device=dev)
+                # (bundle: one record per render item, one set of model gradient arrays)
                 grad_records = grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
                 grad_pool = grad_clear[rec_floats:rec_floats + pool_floats] if pool_floats else None
                 grad_touched = grad_clear[rec_floats + pool_floats:].view(torch.uint8)[:n]
@@ -555,12 +590,12 @@ class GaussianSplatOp:
                 count_ready = torch.cuda.Event()
                 count_ready.record()
 
-        final_T = torch.empty((1, height, width), dtype=f32, device=dev)
-        n_contrib = torch.empty((1, height, width), dtype=i32, device=dev)
+        final_T = torch.empty((batch, height, width), dtype=f32, device=dev)
+        n_contrib = torch.empty((batch, height, width), dtype=i32, device=dev)
         channels = 4 if self._cfg.render_rgba else 3       # what the kernels write
-        color_shape = (1, channels, height, width) if self._cfg.use_nchw else (1, height, width, channels)
+        color_shape = (batch, channels, height, width) if self._cfg.use_nchw else (batch, height, width, channels)
         out_color = torch.empty(color_shape, dtype=f32, device=dev)
-        out_depth = torch.empty((1, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
+        out_depth = torch.empty((batch, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
         # disable_builtin_rgb: the caller's colour image is the alpha channel alone, or has no channel
         # (config_def.py:152-157)
         out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color[..., 3:] if no_rgb else out_color,
@@ -568,7 +603,7 @@ class GaussianSplatOp:
 
         def _empty_result():
             if custom_features is not None:
-                out.custom_features = torch.zeros((1, height, width, custom_features.shape[1]), dtype=f32, device=dev)
+                out.custom_features = torch.zeros((batch, height, width, custom_features.shape[1]), dtype=f32, device=dev)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             # the reference returns uninitialised buffers here (render.py:706-729); fill with the
@@ -628,7 +663,8 @@ class GaussianSplatOp:
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
                 tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
                 grad_touched=grad_touched,
-                kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids)
+                kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids,
+                batch_size=batch, batch_cameras=batch_cams)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
@@ -658,6 +694,7 @@ class GaussianSplatOp:
         if num_rendered == 0:
             return _empty_result()
         if ctx is None or num_rendered > capacity:
+            self.rebin_count += int(ctx is not None)
             ctx, tile_keys_sorted = _bin_and_blend(num_rendered, False)
         if pair_sort_done[0] is not None:
             # everything is enqueued; the host only waits for the pair sort's status word, the blend runs on
@@ -672,11 +709,21 @@ class GaussianSplatOp:
             ctx = None
         return out, ctx
 
+    def _bundle_in_one_pass(self, batch, instance2world_T, custom_features) -> bool:
+        """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
+        does (render.py:314-326, 787, 809, 1515-1522), unless it uses an option whose host code here is written
+        per camera: instance poses, custom feature channels, disable_builtin_rgb, the 32-bit sort (whose 14 tile
+        bits a bundle soon outgrows), or the fused single-stream preprocess.  Those bundles are rendered camera by
+        camera (_forward_bundle)."""
+        c = self._cfg
+        return bool(self.bundle_in_one_pass and batch > 1 and instance2world_T is None and custom_features is None
+                    and not c.disable_builtin_rgb and not c.enable_32bit_sort and self.overlap_sh_colors)
+
     def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
                         prep_user_inputs):
-        """A bundle of B cameras (render.py:314-326, 787, 1515-1522 index one launch by batch): rendered
-        here as B single-camera passes over the shared model.  Outputs are stacked along the batch
-        axis; radii and the mask are flat [B * N] as in the reference."""
+        """A bundle of B cameras rendered as B single-camera passes over the shared model (the fallback for the
+        options _bundle_in_one_pass lists).  Outputs are stacked along the batch axis; radii and the mask
+        are flat [B * N] as in the reference."""
         B, n = len(cameras), len(model)
         assert B > 0, "empty camera bundle"
         if mask is not None:
@@ -798,7 +845,7 @@ class GaussianSplatOp:
             assert _cameras is not None, "camera needed to rebuild kernel parameters"
             P = self.make_params(model, _cameras, training)
         s = self._stream()
-        n, dev = P.n, ctx.uvs.device
+        n, dev = P.n * ctx.batch_size, ctx.uvs.device        # render items
         color = ctx.kernel_color if ctx.kernel_color is not None else out.color
         if grad is None:
             clear, ctx.grad_clear = ctx.grad_clear, None
@@ -848,9 +895,10 @@ class GaussianSplatOp:
         if isinstance(ctx, GaussianSplatOpBatchContext):
             return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
         L = self._lib
-        P = self.make_params(model, cameras, True)
+        P = self.make_params(model, cameras, True, ctx.batch_cameras)
         s = self._stream()
         n, dev = P.n, model.xyz.device
+        B = ctx.batch_size
         with self._stage("blend_bwd"):
             g = self.rasterize_forward_backward(model, ctx, out, grad, training=True,
                                                 render_depth=self._cfg.render_depth, _params=P)
@@ -872,18 +920,23 @@ class GaussianSplatOp:
             if inst_cams is None and instance2world_T is not None:
                 inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
             inst = self._instances_arg(inst_ids, inst_cams)
-            _capi.check(L.d3gs_preprocess_bwd(
-                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
-                _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs),
-                _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), _capi.ptr(g.touched),
-                int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity),
-                _capi.ptr(dsh), _capi.ptr(dsh_base), inst, s),
-                "d3gs_preprocess_bwd")
+            # One launch per camera (the reference loops over the batch inside its kernel, render.py:2972-2989):
+            # camera b works on its own rows of the per-item arrays, the first call stores, the others add.
+            rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
+            for b in range(B):
+                _capi.check(L.d3gs_preprocess_bwd_camera(
+                    C.byref(P), b, int(b > 0), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),
+                    _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh),
+                    _capi.ptr(rows(ctx.radii, b)), _capi.ptr(rows(ctx.cov2d_vecs, b)),
+                    _capi.ptr(rows(ctx.sh_to_rgb_ne_0, b)), _capi.ptr(rows(g.records, b)), _capi.ptr(rows(g.touched, b)),
+                    int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat),
+                    _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), inst, s),
+                    "d3gs_preprocess_bwd")
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,
                                          color_sh=dsh, color_sh_base=dsh_base)
         self.last_raster_grads = g
         if return_uv_grad:
-            return grad_model, g.duv.unsqueeze(0), dcustom
+            return grad_model, g.duv.reshape(B, n, 2), dcustom
         return grad_model, None, dcustom
 
 

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 25
+#define D3GS_ABI_VERSION 26
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -91,7 +91,21 @@ typedef struct d3gs_params {
                                      of the float bits (render.py:767-770, 853-854): gaussians of a tile that fall into
                                      the same depth step are blended in index order.  At most 2^14 tiles. */
     float depth_32bit_prec;       /* config_def.py:91, default 0.001 */
+    /* Camera bundle (render.py:129-150, 314-326): batch_size = B > 1 renders B cameras of one image size in one
+     * pass over B * n "render items", item i = b * n + g being gaussian g seen by camera b.  The model arrays keep
+     * n rows; everything K1 writes (and the reject mask it reads) has B * n rows; tile ids carry the camera,
+     * b * tiles_x * tiles_y + y * tiles_x + x (render.py:787, 809), so the sort and the range table cover
+     * B * tiles_x * tiles_y tiles; images are [B, H, W, C].  The cameras come from device memory: batch_cameras
+     * [B][16] = rows 0-2 of cam2world_T (9 floats, the layout of w2c), its row 3 (the centre), focal x, y and
+     * principal point x, y; the fields w2c, cam_center, fx, fy, cx, cy, tan_fovx, tan_fovy above are then not read
+     * (render.py:316-323 loads the same from its [B,4,3] and [B,4] tensors).  batch_size 0 or 1: one camera, the
+     * fields above. */
+    int32_t batch_size;
+    int32_t reserved0;
+    const float* batch_cameras;
 } d3gs_params;
+
+#define D3GS_BATCH_CAMERA_FLOATS 16
 
 int d3gs_abi_version(void);
 const char* d3gs_last_error_string(void);
@@ -336,6 +350,20 @@ int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* qua
                         int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw, float* dscale,
                         float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                         d3gs_stream_t stream);
+
+/* K9 for one camera of a bundle (render.py:2972-2989, 3180-3219 loop over the batch inside the kernel): with
+ * p->batch_size = B > 1 the call works on camera batch_index, taken from p->batch_cameras, and every per-item
+ * array (radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched) points at that camera's n rows.  accumulate != 0
+ * adds to the six gradient arrays instead of storing (gaussians without work are left alone): the gradient of a
+ * bundle is B calls, the first storing (or adding to cleared arrays), the others accumulating.  With
+ * batch_size <= 1, batch_index 0 and accumulate 0 this is d3gs_preprocess_bwd. */
+int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,
+                               const float* quaternion_xyzw, const float* scale, const float* opacity,
+                               const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                               const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
+                               int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
+                               float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
+                               const d3gs_instances* instances, d3gs_stream_t stream);
 
 #ifdef __cplusplus
 }
