@@ -126,6 +126,9 @@ def main():
                     help="number of distinct camera poses the steps cycle through (1 = the configuration's own view every "
                          "step, the headline; K > 1 orbits K seeded poses about the scene so that the pair count changes "
                          "from step to step, as in a training loop with a new camera every step)")
+    ap.add_argument("--backward-algo", type=str, default="DEFAULT",
+                    help="rasterize_backward_algo: DEFAULT (lanes = pixels, wave reduction) or PER_GAUSSIAN (lanes = "
+                         "gaussians over the forward's bucket snapshots); the headline is DEFAULT")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--late-gradient-clear", action="store_true",
                     help="let the preprocess backward write the zero gradients itself instead of clearing the arrays "
@@ -150,7 +153,7 @@ def main():
         print(json.dumps({"calibration": "torch.mul(x, 1.0, out=y)", "read_bytes": x.numel() * 4,
                           "write_bytes": y.numel() * 4, "launches": 5}))
         return
-    from d3gs_research_amd.config_def import EarlyFilterAlgo
+    from d3gs_research_amd.config_def import EarlyFilterAlgo, RasterizeBackwardAlgo
     from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
     from d3gs_research_amd.synthetic import gen_scene, scene_config, scene_model
 
@@ -158,7 +161,7 @@ def main():
     scene = gen_scene(args.config)
     cam = scene.camera()
     cams = [cam] + orbit_cameras(scene, args.views - 1)
-    op = GaussianSplatOp(scene_config(scene, filt))
+    op = GaussianSplatOp(scene_config(scene, filt, rasterize_backward_algo=RasterizeBackwardAlgo[args.backward_algo]))
     op.clear_gradients_early = not args.late_gradient_clear
     model = scene_model(scene, "cuda:0")
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
@@ -287,7 +290,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"config {args.config}: {scene.name}", "gaussians": N, "sh_degree": scene.sh_degree,
-                   "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name, "pairs_M": int(M),
+                   "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name,
+                   "rasterize_backward_algo": args.backward_algo, "pairs_M": int(M),
                    "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists,
                    "gaussians_with_gradient": active, "views": views_info},
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),

@@ -15,9 +15,10 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
+BUCKET_SIZE = 64          # D3GS_BUCKET_SIZE
 ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
 COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP = -1, -2
 SCAN_NOALLOC_MAX_N = 1 << 24   # D3GS_SCAN_NOALLOC_MAX_N
@@ -78,6 +79,9 @@ _SIGNATURES = {
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),
     "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
+    "d3gs_bucket_offsets": (C.c_int, [_VP, C.c_int32, _VP, _VP]),
+    "d3gs_blend_fwd_snapshots": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [_VP, C.c_size_t] + [_VP] * 3),
+    "d3gs_blend_bwd_per_gaussian": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
     "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 10 + [C.c_int32, C.c_int32] + [_VP] * 6 +
                             [C.POINTER(Instances), _VP]),
     "d3gs_preprocess_bwd_camera": (C.c_int, [C.POINTER(Params), C.c_int32, C.c_int32] + [_VP] * 10 +

@@ -26,6 +26,8 @@
 
 namespace d3gs {
 
+constexpr int kBucket = D3GS_BUCKET_SIZE;   // list entries per bucket of the per-gaussian backward: one per lane of a wavefront
+
 struct __attribute__((aligned(16))) StagedGaussian {
     float x, y, thr, pad;   // pixel-space centre, cull threshold
     float ha, nb, hc, o;    // pre-scaled conic (-a/2, -b, -c/2) and opacity
@@ -215,7 +217,9 @@ __device__ __forceinline__ TilePlace place_tile(const d3gs_params& P, int tile) 
 
 // kDepth: blend the camera-space depth as one more channel (render.py:1532-1539, 1915-1919).
 // kRgba: fourth colour channel, the sum of the blend weights (render.py:1899-1906).
-template <bool kDepth, bool kRgba>
+// kSnap: besides the image, store every pixel's running state (T and the colour accumulated so far) at the start
+// of each bucket of kBucket list entries, for the per-gaussian backward (render.py:1744-1759).
+template <bool kDepth, bool kRgba, bool kSnap>
 __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, const int32_t* __restrict__ ranges,
                                                             const int32_t* __restrict__ idx_sorted,
                                                             const float* __restrict__ uvs,
@@ -226,7 +230,9 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                                                             float* __restrict__ color, float* __restrict__ final_T,
                                                             int32_t* __restrict__ n_contrib,
                                                             float* __restrict__ final_depth,
-                                                            uint4* __restrict__ clear_vec, size_t clear_count) {
+                                                            uint4* __restrict__ clear_vec, size_t clear_count,
+                                                            const int32_t* __restrict__ bucket_offsets,
+                                                            float4* __restrict__ snap) {
     // Optional service to the backward pass: this kernel hardly uses the memory pipes, so it clears the
     // caller's accumulator arrays (16-byte units, spread over all workgroups) on the side.
     if (clear_vec) {
@@ -280,6 +286,13 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         __syncthreads();
         if (__all(pxf != pxf)) continue;
         for (int chunk = 0; chunk < 4; ++chunk) {
+            if constexpr (kSnap) {
+                // state of this wavefront's pixels in front of list entry round * 256 + chunk * 64 (a wavefront
+                // whose pixels have all finished skips this: no gaussian from here on contributes to them)
+                if (round * kBlock + chunk * kBucket < len)
+                    snap[((size_t)bucket_offsets[tile] + round * (kBlock / kBucket) + chunk) * kBlock + tid] =
+                        make_float4(T, acc0, acc1, acc2);
+            }
             unsigned long long m = uniform_u64(s_mask[wave][chunk]);
             while (m) {
                 const int j = chunk * 64 + __builtin_ctzll(m);
@@ -547,6 +560,232 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// Per-gaussian backward (render.py:2319-2776; config rasterize_backward_algo = PER_GAUSSIAN): the second
+// algorithm for the same gradient.  Lanes are gaussians, not pixels: a wavefront takes one bucket of kBucket
+// consecutive entries of a tile's list, every lane keeps its gaussian's nine sums in registers, and the pixels
+// of the tile pass through the lanes one after the other, lane l handing a pixel's running state (T and the
+// colour still behind) to lane l + 1 with a one-lane wave shift -- the order of the list -- so that no sum ever
+// crosses lanes and each (tile, gaussian) ends in one line-wide atomic.  The state a pixel has in front of the
+// bucket comes from the snapshots the forward pass stored (blend_fwd_kernel<.., kSnap>).  Only pixels that are
+// still open at the bucket's start (their last contributor lies in or behind it) are passed through.
+// The reference runs one 32-lane warp per bucket of 32; here a bucket is the 64 lanes of a wavefront and a
+// workgroup (one per tile, longest lists first) deals its buckets to its four wavefronts.
+// ---------------------------------------------------------------------------
+template <int kCtrl>
+__device__ __forceinline__ float dpp_shift_in(float fresh, float v) {
+    // lanes 1..63 take v of the lane below; lane 0, which has no lane below, keeps `fresh`
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fresh), __float_as_int(v), kCtrl, 0xF, 0xF, false));
+}
+constexpr int kDppWaveShr1 = 0x138;
+
+__global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
+    const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
+    const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
+    const int32_t* __restrict__ tile_order, const float* __restrict__ final_T, const int32_t* __restrict__ n_contrib,
+    const float* __restrict__ color, const float* __restrict__ drgb, const float* __restrict__ dT,
+    const int32_t* __restrict__ bucket_offsets, const float4* __restrict__ snap, float* __restrict__ grad_records,
+    uint8_t* __restrict__ touched) {
+    constexpr int kWaves = kBlock / 64;
+    __shared__ float4 s_pix_grad[kBlock];    // per pixel: drgb (3), -dT * final_T
+    __shared__ float4 s_pix_final[kBlock];   // per pixel: final colour (3), contributor (int bits)
+    __shared__ float4 s_snap[kWaves][kBlock];            // the bucket's snapshots: T, colour in front of the bucket
+    __shared__ unsigned short s_open[kWaves][kBlock];    // pixels still open at the bucket's start
+    __shared__ float s_out[kWaves][kBucket][D3GS_GRAD_RECORD_FLOATS + 1];
+    __shared__ int s_gid[kWaves][kBucket];
+    __shared__ int s_wmax[kWaves];
+
+    const int ntiles = P.tiles_x * P.tiles_y * batch_count(P);
+    const int items = item_count(P);
+    const int tile = tile_for_block(blockIdx.x, tile_order);
+    if (tile < 0 || tile >= ntiles) return;
+    const TilePlace place = place_tile(P, tile);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float tile_x0 = (float)(place.tx * kTile), tile_y0 = (float)(place.ty * kTile);
+    const int r0 = ranges[2 * tile], r1 = ranges[2 * tile + 1];
+    const int len = r1 - r0;
+    if (len <= 0) return;
+
+    {   // pixel tid of the tile, in the forward kernel's thread order (the snapshots are stored in that order)
+        const int px = place.tx * kTile + (wave & 1) * 8 + (lane & 7);
+        const int py = place.ty * kTile + (wave >> 1) * 8 + (lane >> 3);
+        const bool inside = px < P.width && py < P.height;
+        int contributor = 0;
+        float4 pg = make_float4(0.0f, 0.0f, 0.0f, 0.0f), pf = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (inside) {
+            const size_t pid = (size_t)py * P.width + px;
+            const size_t gpid = (size_t)place.batch * P.width * P.height + pid;
+            contributor = min(n_contrib[gpid] + 1, len);
+            pg = make_float4(drgb[color_index(P, place.batch, pid, 0, 3)], drgb[color_index(P, place.batch, pid, 1, 3)],
+                             drgb[color_index(P, place.batch, pid, 2, 3)], (-dT[gpid]) * final_T[gpid]);
+            pf = make_float4(color[color_index(P, place.batch, pid, 0, 3)], color[color_index(P, place.batch, pid, 1, 3)],
+                             color[color_index(P, place.batch, pid, 2, 3)], 0.0f);
+        }
+        pf.w = __int_as_float(contributor);
+        s_pix_grad[tid] = pg;
+        s_pix_final[tid] = pf;
+        const int wmax = wave_max_i32(contributor);
+        if (lane == 0) s_wmax[wave] = wmax;
+    }
+    __syncthreads();
+    const int block_todo = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
+    const int nbuckets = (block_todo + kBucket - 1) / kBucket;
+    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+
+    for (int bucket = wave; bucket < nbuckets; bucket += kWaves) {      // wave-uniform
+        const int bstart = bucket * kBucket;
+        // the bucket's snapshots, and the list of pixels still open at its start
+        const float4* sb = snap + ((size_t)bucket_offsets[tile] + bucket) * kBlock;
+        int cnt = 0;
+#pragma unroll
+        for (int q = 0; q < kBlock / 64; ++q) {
+            const int p = q * 64 + lane;
+            const bool open = __float_as_int(s_pix_final[p].w) > bstart;
+            // a snapshot of a finished pixel may never have been written: it is not read, and not staged
+            s_snap[wave][p] = open ? sb[p] : make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+            const unsigned long long bal = __ballot(open);
+            if (open) s_open[wave][cnt + __popcll(bal & lt_mask)] = (unsigned short)p;
+            cnt += __popcll(bal);
+        }
+        cnt = __builtin_amdgcn_readfirstlane(cnt);
+        // this lane's gaussian
+        const int li = bstart + lane;
+        int gid = -1;
+        StagedGaussian sg = StagedGaussian{0.0f, 0.0f, __builtin_inff(), 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
+        if (li < len) {
+            const int g = idx_sorted[r0 + li];
+            if ((unsigned)g < (unsigned)items) {   // a corrupt index list must not become a wild read or write
+                gid = g;
+                stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &sg);
+                c0 = rgb_g[3 * g];
+                c1 = rgb_g[3 * g + 1];
+                c2 = rgb_g[3 * g + 2];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();    // the wavefront's own LDS writes above are read below
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, a4 = 0.0f, a5 = 0.0f, a6 = 0.0f, a7 = 0.0f, a8 = 0.0f;
+        float T = 1.0f, rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f;
+        const int steps = cnt > 0 ? cnt + kBucket - 1 : 0;
+        for (int j = 0; j < steps; ++j) {
+            // lane 0 takes up open pixel j with the state it has in front of the bucket; every other lane takes
+            // over the pixel its lower neighbour has just finished with
+            const int q = j < cnt ? s_open[wave][j] : 0;     // wave-uniform
+            const float4 sn = s_snap[wave][q];
+            const float4 fin = s_pix_final[q];
+            const bool fresh = j < cnt;
+            T = dpp_shift_in<kDppWaveShr1>(fresh ? sn.x : 1.0f, T);
+            rr0 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.x - sn.y : 0.0f, rr0);
+            rr1 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.y - sn.z : 0.0f, rr1);
+            rr2 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.z - sn.w : 0.0f, rr2);
+            const int k = j - lane;                        // which open pixel this lane holds now
+            const bool holding = k >= 0 && k < cnt;
+            const int p = holding ? s_open[wave][k] : 0;
+            const float4 pg = s_pix_grad[p];
+            const int contributor = __float_as_int(s_pix_final[p].w);
+            const float pxf = tile_x0 + (float)(((p >> 6) & 1) * 8 + (p & 7));
+            const float pyf = tile_y0 + (float)((p >> 7) * 8 + ((p >> 3) & 7));
+            const float dx = sg.x - pxf, dy = sg.y - pyf;
+            const float power = blend_power(sg, dx, dy);
+            // the forward's exact sequence decides which pixels the gaussian contributed to
+            const bool cand = holding && li < contributor && power >= sg.thr && power <= 0.0f;
+            const float G0 = det_expf_inrange(cand ? power : 0.0f);
+            const float alpha0 = fminf(0.99f, sg.o * G0);
+            const bool valid = cand && alpha0 >= P.alpha_eps;
+            const float G = valid ? G0 : 0.0f, alpha = valid ? alpha0 : 0.0f;
+            const float one_m = 1.0f - alpha;
+            const float w = alpha * T;
+            T = T * one_m;
+            rr0 = __builtin_fmaf(-w, c0, rr0);
+            rr1 = __builtin_fmaf(-w, c1, rr1);
+            rr2 = __builtin_fmaf(-w, c2, rr2);
+            float dl = pg.w;
+            dl = __builtin_fmaf(pg.z, __builtin_fmaf(T, c2, -rr2), dl);
+            dl = __builtin_fmaf(pg.y, __builtin_fmaf(T, c1, -rr1), dl);
+            dl = __builtin_fmaf(pg.x, __builtin_fmaf(T, c0, -rr0), dl);
+            const float dL_dalpha = dl * __builtin_amdgcn_rcpf(one_m);
+            const float g5 = dL_dalpha * G;
+            const float qv = sg.o * g5;
+            const float g0 = qv * dx, g1 = qv * dy;
+            a0 += g0;
+            a1 += g1;
+            a2 += g0 * dx;
+            a3 += g0 * dy;
+            a4 += g1 * dy;
+            a5 += g5;
+            a6 += w * pg.x;
+            a7 += w * pg.y;
+            a8 += w * pg.z;
+        }
+        // moments -> (duv, dconic) with a = -2 ha, b = -nb, c = -2 hc, as the default kernel's flush does
+        float* row = s_out[wave][lane];
+        row[0] = __builtin_fmaf(sg.nb, a1, (2.0f * sg.ha) * a0);
+        row[1] = __builtin_fmaf(sg.nb, a0, (2.0f * sg.hc) * a1);
+        row[2] = -0.5f * a2;
+        row[3] = -a3;
+        row[4] = -0.5f * a4;
+        row[5] = a5;
+        row[6] = a6;
+        row[7] = a7;
+        row[8] = a8;
+#pragma unroll
+        for (int c = 9; c < D3GS_GRAD_RECORD_FLOATS; ++c) row[c] = 0.0f;
+        s_gid[wave][lane] = gid;
+        __builtin_amdgcn_wave_barrier();
+        // sixteen lanes add one gaussian's record: one line-wide atomic per (tile, gaussian)
+        const int slot_k = lane & 15;
+#pragma unroll
+        for (int r = 0; r < kBucket / 4; ++r) {
+            const int gl = r * 4 + (lane >> 4);
+            const int id = s_gid[wave][gl];
+            const float v = id >= 0 ? s_out[wave][gl][slot_k] : 0.0f;
+            if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * id + slot_k, v);
+            if (touched) {
+                const unsigned long long nz = __ballot(v != 0.0f);
+                if (slot_k == 0 && ((nz >> (lane & 48)) & 0xFFFFull)) touched[id] = 1;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();    // the next bucket overwrites this wavefront's tables
+    }
+}
+
+// Exclusive prefix sum of the tiles' bucket counts ceil(list length / kBucket) (render.py:940-950): where each
+// tile's snapshots start.  One workgroup; out[num_tiles] is the total.
+__global__ __launch_bounds__(1024) void bucket_offsets_kernel(const int32_t* __restrict__ ranges, int num_tiles,
+                                                              int32_t* __restrict__ out) {
+    __shared__ int s_wave[16];
+    __shared__ int s_carry;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < num_tiles; base += 1024) {
+        const int t = base + tid;
+        int c = 0;
+        if (t < num_tiles) c = (max(ranges[2 * t + 1] - ranges[2 * t], 0) + kBucket - 1) / kBucket;
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        int before = s_carry, total = 0;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            const int v = s_wave[w];
+            if (w < wave) before += v;
+            total += v;
+        }
+        if (t < num_tiles) out[t] = before + incl - c;
+        __syncthreads();
+        if (tid == 0) s_carry += total;
+        __syncthreads();
+    }
+    if (tid == 0) out[num_tiles] = s_carry;
+}
+
 }  // namespace d3gs
 
 using namespace d3gs;
@@ -557,6 +796,22 @@ static int finish_launch(const char* who) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("%s: launch failed: %s", who, hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
+}
+
+static int launch_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                            const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
+                            const int32_t* tile_order, float* color, float* final_T, int32_t* n_contrib,
+                            float* final_depth, void* clear_ptr, size_t clear_bytes, const int32_t* bucket_offsets,
+                            float4* snap, d3gs_stream_t stream) {
+#define D3GS_LAUNCH_FWD(D, A, S)                                                                                    \
+    hipLaunchKernelGGL((blend_fwd_kernel<D, A, S>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,  \
+                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
+                       color, final_T, n_contrib, final_depth, (uint4*)clear_ptr, clear_bytes / 16, bucket_offsets, snap)
+    if (snap) D3GS_LAUNCH_FWD(false, false, true);
+    else if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true, false); else D3GS_LAUNCH_FWD(true, false, false); }
+    else                      { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true, false); else D3GS_LAUNCH_FWD(false, false, false); }
+#undef D3GS_LAUNCH_FWD
+    return finish_launch("d3gs_blend_fwd");
 }
 
 extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
@@ -575,14 +830,34 @@ extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_rang
         set_error("d3gs_blend_fwd: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-#define D3GS_LAUNCH_FWD(D, A)                                                                                       \
-    hipLaunchKernelGGL((blend_fwd_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,     \
-                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
-                       color, final_T, n_contrib, final_depth, (uint4*)clear_ptr, clear_bytes / 16)
-    if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true); else D3GS_LAUNCH_FWD(true, false); }
-    else                 { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true); else D3GS_LAUNCH_FWD(false, false); }
-#undef D3GS_LAUNCH_FWD
-    return finish_launch("d3gs_blend_fwd");
+    return launch_blend_fwd(p, workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,
+                            color, final_T, n_contrib, final_depth, clear_ptr, clear_bytes, nullptr, nullptr, stream);
+}
+
+extern "C" int d3gs_blend_fwd_snapshots(const d3gs_params* p, const int32_t* workload_ranges,
+                                        const int32_t* gaussian_idx_sorted, const float* uvs, const float* conic_opacity,
+                                        const float* rgb_gaussian, const int32_t* tile_order, float* color,
+                                        float* final_T, int32_t* n_contrib, void* clear_ptr, size_t clear_bytes,
+                                        const int32_t* bucket_offsets, float* snapshots, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_blend_fwd_snapshots");
+    if (rc) return rc;
+    if (p->render_depth || p->render_rgba) {
+        set_error("d3gs_blend_fwd_snapshots: the per-gaussian backward covers the colour channels only "
+                  "(no render_depth / render_rgba)");
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    if (clear_ptr && ((((uintptr_t)clear_ptr) | clear_bytes) & 15u)) {
+        set_error("d3gs_blend_fwd_snapshots: clear_ptr / clear_bytes must be multiples of 16");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib ||
+        !bucket_offsets || !snapshots || (((uintptr_t)snapshots) & 15u)) {
+        set_error("d3gs_blend_fwd_snapshots: NULL buffer (snapshots must be 16-byte aligned)");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    return launch_blend_fwd(p, workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, nullptr, tile_order,
+                            color, final_T, n_contrib, nullptr, clear_ptr, clear_bytes, bucket_offsets, (float4*)snapshots,
+                            stream);
 }
 
 extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
@@ -606,4 +881,38 @@ extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_rang
     else                 { if (p->render_rgba) D3GS_LAUNCH_BWD(false, true); else D3GS_LAUNCH_BWD(false, false); }
 #undef D3GS_LAUNCH_BWD
     return finish_launch("d3gs_blend_bwd");
+}
+
+extern "C" int d3gs_bucket_offsets(const int32_t* workload_ranges, int32_t num_tiles, int32_t* bucket_offsets,
+                                   d3gs_stream_t stream) {
+    if (num_tiles < 0 || !bucket_offsets || (num_tiles > 0 && !workload_ranges)) {
+        set_error("d3gs_bucket_offsets: bad argument");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(bucket_offsets_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, workload_ranges, (int)num_tiles,
+                       bucket_offsets);
+    return finish_launch("d3gs_bucket_offsets");
+}
+
+extern "C" int d3gs_blend_bwd_per_gaussian(const d3gs_params* p, const int32_t* workload_ranges,
+                                           const int32_t* gaussian_idx_sorted, const float* uvs, const float* conic_opacity,
+                                           const float* rgb_gaussian, const int32_t* tile_order, const float* final_T,
+                                           const int32_t* n_contrib, const float* color, const float* drgb, const float* dT,
+                                           const int32_t* bucket_offsets, const float* snapshots, float* grad_records,
+                                           uint8_t* touched, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_blend_bwd_per_gaussian");
+    if (rc) return rc;
+    if (p->render_depth || p->render_rgba || p->use_nchw) {
+        set_error("d3gs_blend_bwd_per_gaussian: colour channels in [H,W,3] only (no render_depth / render_rgba / use_nchw)");
+        return D3GS_ERR_UNSUPPORTED;
+    }
+    if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb || !dT ||
+        !bucket_offsets || !snapshots || !grad_records || (((uintptr_t)snapshots) & 15u)) {
+        set_error("d3gs_blend_bwd_per_gaussian: NULL buffer (snapshots must be 16-byte aligned)");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(blend_bwd_per_gaussian_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,
+                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, final_T,
+                       n_contrib, color, drgb, dT, bucket_offsets, (const float4*)snapshots, grad_records, touched);
+    return finish_launch("d3gs_blend_bwd_per_gaussian");
 }

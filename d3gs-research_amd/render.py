@@ -23,7 +23,7 @@ import torch
 
 from . import _capi
 from .camera import BasicPinholeCamera
-from .config_def import GaussianSplatConfig
+from .config_def import GaussianSplatConfig, RasterizeBackwardAlgo
 from .model import GaussianModelOriginBase, GaussianModelOriginFused
 
 
@@ -44,7 +44,10 @@ class GaussianSplatOpContext:
     depths: torch.Tensor
     cov2d_vecs: torch.Tensor | None = None
     sh_to_rgb_ne_0: torch.Tensor | None = None
-    per_gaussian_snap: None = None
+    # rasterize_backward_algo = PER_GAUSSIAN (render.py:44-55, 940-962): (bucket_offsets [tiles + 1] int32,
+    # snapshots [buckets, 256, 4] float32), the running state of every pixel in front of each bucket of 64 list
+    # entries, stored by the forward blend for the per-gaussian backward
+    per_gaussian_snap: tuple | None = None
     # not in the reference: tile ids by descending list length, the blend kernels' launch order
     tile_order: torch.Tensor | None = None
     # not in the reference: the backward's [N, 16] gradient records, cleared by the forward blend kernel
@@ -197,15 +200,17 @@ class GaussianSplatOp:
             "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
             # builtin colours off: the kernels blend zeros in their place (render.py:262, 662, 1898-1931)
             "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
+            # the per-gaussian backward (render.py:2319-2776) is built for the colour channels in [H,W,3]
+            "rasterize_backward_algo = PER_GAUSSIAN with render_depth / render_rgba / use_nchw / disable_builtin_rgb":
+                c.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN
+                and (c.render_depth or c.render_rgba or c.use_nchw or c.disable_builtin_rgb),
             # Accepted without a code path of their own, because they change how the reference computes and not
             # what: move_opacity_in_grad_to_prep (render.py:1973-1990, 2995-3003) takes the factors opacity, -1/2
             # and -1 out of the per-pixel gradient terms and applies them once per gaussian -- the same gradient up
             # to rounding; the blend backward here applies the conic factors once per tile and gaussian in any
             # case, and taking the opacity out as well measured no gain; use_int64_tile_touched (render.py:657-660)
             # widens the tile counters for views beyond 2^31 pairs, while this build stops at 2^30 pairs per
-            # camera with an error; rasterize_backward_algo = PER_GAUSSIAN is accepted: the reference's second backward
-            # (render.py:2319-2776) computes the same gradient with fewer atomics per gaussian, which the one
-            # backward kernel here already has (one record-wide atomic per tile and gaussian)
+            # camera with an error
         }
         bad = [k for k, v in unsupported.items() if v]
         if bad:
@@ -657,9 +662,18 @@ class GaussianSplatOp:
                     _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
                                                        _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
                                 "d3gs_tile_ranges_u32")
+            snap = None
+            if training and self._cfg.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN:
+                # K8 (render.py:940-962): where each tile's buckets start.  The bucket total stays on the device:
+                # ceil(len / 64) summed over the tiles is at most pairs / 64 + tiles, which sizes the snapshots.
+                bucket_offsets = torch.empty(num_tiles + 1, dtype=i32, device=dev)
+                _capi.check(L.d3gs_bucket_offsets(_capi.ptr(workload_ranges), num_tiles, _capi.ptr(bucket_offsets), s),
+                            "d3gs_bucket_offsets")
+                max_buckets = capacity // _capi.BUCKET_SIZE + num_tiles + 1
+                snap = (bucket_offsets, torch.empty((max_buckets, 256, 4), dtype=f32, device=dev))
             ctx = GaussianSplatOpContext(
                 conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
-                gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges,
+                gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges, per_gaussian_snap=snap,
                 image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
                 tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
                 grad_touched=grad_touched,
@@ -849,6 +863,15 @@ class GaussianSplatOp:
         color = ctx.kernel_color if ctx.kernel_color is not None else out.color
         if grad is None:
             clear, ctx.grad_clear = ctx.grad_clear, None
+            if ctx.per_gaussian_snap is not None:      # the forward also stores the pixels' state per bucket
+                bucket_offsets, snapshots = ctx.per_gaussian_snap
+                _capi.check(L.d3gs_blend_fwd_snapshots(
+                    C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                    _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order),
+                    _capi.ptr(color), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(clear),
+                    0 if clear is None else clear.numel() * 4, _capi.ptr(bucket_offsets), _capi.ptr(snapshots), s),
+                    "d3gs_blend_fwd_snapshots")
+                return None
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
@@ -874,12 +897,21 @@ class GaussianSplatOp:
         if rec is None:     # a second backward over this context: fresh records, work found from the records
             rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
             touched = None
-        _capi.check(L.d3gs_blend_bwd(
-            C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-            _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
-            _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
-            _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec),
-            _capi.ptr(touched), s), "d3gs_blend_bwd")
+        if ctx.per_gaussian_snap is not None:      # rasterize_backward_algo = PER_GAUSSIAN (render.py:2319-2776)
+            bucket_offsets, snapshots = ctx.per_gaussian_snap
+            _capi.check(L.d3gs_blend_bwd_per_gaussian(
+                C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
+                _capi.ptr(out.n_contrib), _capi.ptr(color), _capi.ptr(drgb), _capi.ptr(grad.dT),
+                _capi.ptr(bucket_offsets), _capi.ptr(snapshots), _capi.ptr(rec), _capi.ptr(touched), s),
+                "d3gs_blend_bwd_per_gaussian")
+        else:
+            _capi.check(L.d3gs_blend_bwd(
+                C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
+                _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
+                _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec),
+                _capi.ptr(touched), s), "d3gs_blend_bwd")
         res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
                                       dz=rec[:, 9] if render_depth else None, records=rec, touched=touched)
         return res

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 26
+#define D3GS_ABI_VERSION 27
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -331,6 +331,32 @@ int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const i
                    const int32_t* tile_order, const float* final_T, const int32_t* n_contrib, const float* color,
                    const float* final_depth, const float* drgb, const float* dT, const float* ddepth,
                    float* grad_records, uint8_t* touched, d3gs_stream_t stream);
+
+/* The per-gaussian backward, config rasterize_backward_algo = PER_GAUSSIAN (config_def.py:72-74, 149-151;
+ * render.py:940-962, 1577-1583, 1744-1759, 2319-2776): a second algorithm for K7's gradient in which lanes are
+ * gaussians and pixels pass through them, so that no sum crosses lanes.  Three calls:
+ *   d3gs_bucket_offsets (K8, replaces kernel_1d("prepare_bucket_...") + cumsum_, render.py:941-950):
+ *     bucket_offsets[t] = sum over tiles before t of ceil(list length / D3GS_BUCKET_SIZE), [num_tiles + 1] int32,
+ *     the last entry the total; no host read-back is needed: ceil(M / D3GS_BUCKET_SIZE) + num_tiles bounds the total;
+ *   d3gs_blend_fwd_snapshots: d3gs_blend_fwd (colour channels, [H,W,3]) that also stores every pixel's running
+ *     state in front of each bucket: snapshots [total buckets][256][4] float32 (T, accumulated r, g, b; pixel order
+ *     of the kernel's threads), the reference's T_snap / color_snap (render.py:958-959, 1744-1759).  Same image
+ *     bit for bit;
+ *   d3gs_blend_bwd_per_gaussian: the backward over those snapshots; arguments as d3gs_blend_bwd.  One wavefront per
+ *     bucket of 64 list entries (the reference: one 32-lane warp per 32), one workgroup per tile.
+ * The gradient is the complete one, as d3gs_blend_bwd's, up to the order of the float32 sums. */
+#define D3GS_BUCKET_SIZE 64
+int d3gs_bucket_offsets(const int32_t* workload_ranges, int32_t num_tiles, int32_t* bucket_offsets, d3gs_stream_t stream);
+int d3gs_blend_fwd_snapshots(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                             const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                             const int32_t* tile_order, float* color, float* final_T, int32_t* n_contrib,
+                             void* clear_ptr, size_t clear_bytes, const int32_t* bucket_offsets, float* snapshots,
+                             d3gs_stream_t stream);
+int d3gs_blend_bwd_per_gaussian(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                                const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
+                                const int32_t* tile_order, const float* final_T, const int32_t* n_contrib,
+                                const float* color, const float* drgb, const float* dT, const int32_t* bucket_offsets,
+                                const float* snapshots, float* grad_records, uint8_t* touched, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from K7's records (duv, dconic, dopacity, dcolor

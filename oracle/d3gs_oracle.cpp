@@ -708,7 +708,13 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                    const int32_t* n_contrib, const float* color, const float* final_depth, const float* drgb,
                    const float* dT, const float* ddepth, double* duv, double* dconic, double* dopacity,
                    double* dcolor, double* dz /* [N], used when render_depth */,
-                   double* absmass /* [N,10] sum of |terms|, may be NULL */) {
+                   double* absmass /* [N,10] sum of |terms|, may be NULL */,
+                   double* statemass /* [N,6], may be NULL: how strongly duv (2), dconic (3) and dopacity depend on
+                                        the rounding of a pixel's running colour state: the sum over pixels of
+                                        |d term / d dl| * sum_ch |drgb_ch| * |final colour_ch|.  A backward that
+                                        rebuilds "the colour still behind" from sums rounded at the magnitude of the
+                                        final colour (the per-gaussian algorithm's snapshots, render.py:2601)
+                                        differs from this sequence by a few ulp of that magnitude per pixel. */) {
     const int W = P->width, H = P->height;
     const int ntiles = P->tiles_x * P->tiles_y;
     const int NV = 10;
@@ -720,6 +726,7 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
         if (len <= 0) continue;
         std::vector<double> acc((size_t)len * NV, 0.0);
         std::vector<double> mass((size_t)len * NV, 0.0);
+        std::vector<double> smass(statemass ? (size_t)len * 6 : 0, 0.0);
         for (int ly = 0; ly < 16; ++ly)
             for (int lx = 0; lx < 16; ++lx) {
                 int px = tx * 16 + lx, py = ty * 16 + ly;
@@ -787,6 +794,17 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                         a9[k] += (double)term[k];
                         m9[k] += fabs((double)term[k]);
                     }
+                    if (statemass) {
+                        double state = 0.0;
+                        for (int ch = 0; ch < 3; ++ch)
+                            state += fabs((double)dr[ch]) * fabs((double)color[color_index(P, pid, ch)]);
+                        const double per_dl = fabs((double)G / (double)one_m) * state;     // d gop / d dl, times state
+                        const double geom[6] = {fabs((double)co[3] * dx), fabs((double)co[3] * dy),
+                                                fabs((double)co[3] * dx * dx), fabs((double)co[3] * dx * dy),
+                                                fabs((double)co[3] * dy * dy), 1.0};
+                        double* s6 = smass.data() + (size_t)j * 6;
+                        for (int k = 0; k < 6; ++k) s6[k] += per_dl * geom[k];
+                    }
                 }
             }
         // moments -> (duv, dconic) per (tile, gaussian); the magnitudes follow the same map with absolute values
@@ -805,6 +823,14 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
             Ms[1] = fabs(c) * M2 + fabs(b) * M1;
             Ms[2] = 0.5 * Ms[2];
             Ms[4] = 0.5 * Ms[4];
+            if (statemass) {
+                double* Q = smass.data() + (size_t)j * 6;
+                const double Q1 = Q[0], Q2 = Q[1];
+                Q[0] = fabs(a) * Q1 + fabs(b) * Q2;
+                Q[1] = fabs(c) * Q2 + fabs(b) * Q1;
+                Q[2] = 0.5 * Q[2];
+                Q[4] = 0.5 * Q[4];
+            }
         }
         for (int j = 0; j < len; ++j) {
             int g = idx_sorted[r0 + j];
@@ -822,6 +848,10 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                 if (absmass) {
 #pragma omp atomic
                     absmass[NV * (size_t)g + k] += mass[(size_t)j * NV + k];
+                }
+                if (statemass && k < 6) {
+#pragma omp atomic
+                    statemass[6 * (size_t)g + k] += smass[(size_t)j * 6 + k];
                 }
             }
         }

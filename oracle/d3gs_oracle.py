@@ -243,15 +243,19 @@ def blend_bwd(P, ranges, idx_sorted, uvs, conic_opacity, rgb, final_T, n_contrib
     dcol = np.zeros((n, 3), np.float64)
     dz = np.zeros(n, np.float64) if P.render_depth else None
     mass = np.zeros((n, 10), np.float64)
+    statemass = np.zeros((n, 6), np.float64)
     drgb, dT, ddepth = _f32(drgb), _f32(dT), _f32(ddepth)
     assert drgb.shape == _color_shape(P)
     assert not P.render_depth or (depths is not None and final_depth is not None and ddepth is not None)
     lib().orc_blend_bwd(C.byref(P), _p(ranges), _p(idx_sorted), _p(uvs), _p(conic_opacity), _p(rgb), _p(depths),
                         _p(final_T), _p(n_contrib), _p(color), _p(final_depth), _p(drgb), _p(dT), _p(ddepth),
-                        _p(duv), _p(dconic), _p(dop), _p(dcol), _p(dz), _p(mass))
+                        _p(duv), _p(dconic), _p(dop), _p(dcol), _p(dz), _p(mass), _p(statemass))
     # absmass[:, k]: sum of |per-pixel terms| behind each of the ten gradient values (the scale that
     # bounds reordering error): columns duv(2), dconic(3), dopacity(1), dcolor(3), dz(1)
-    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol, dz=dz, absmass=mass)
+    # statemass[:, k]: for duv(2), dconic(3), dopacity(1), the sum over pixels of |d term / d dl| times
+    # sum_ch |drgb| |final colour|: the scale of the error a backward makes whose per-pixel colour state is rebuilt
+    # from sums rounded at the magnitude of the final colour (the per-gaussian algorithm)
+    return dict(duv=duv, dconic=dconic, dopacity=dop, dcolor=dcol, dz=dz, absmass=mass, statemass=statemass)
 
 
 def preprocess_bwd(P, xyz, quat, scale, opacity, sh, radii, cov2d, ne0, duv, dconic, dopacity, dcolor, dz=None,

@@ -46,7 +46,7 @@ def per_gaussian_rel_err(a, b):
     return (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
 
 
-def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11):
+def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11, state_ulps=0.0):
     """What rounding noise in the blend backward's sums does to the preprocess backward, measured on the
     oracle.  A float32 sum of the per-pixel terms, in whatever order, carries an error of the order of
     2^-24 * sum|terms| ("absmass", which the oracle returns next to its float64 sums).  The oracle's own
@@ -55,12 +55,14 @@ def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11):
     spread beyond the input noise is the conditioning of the chain rule itself (near-degenerate projected
     covariances: gradients that are small differences of large terms)."""
     rng = np.random.default_rng(seed)
-    eps = ulps * 2.0 ** -24
-    m = g_ref["absmass"]
-    noisy = {"duv": g_ref["duv"] + rng.standard_normal(g_ref["duv"].shape) * eps * m[:, 0:2],
-             "dconic": g_ref["dconic"] + rng.standard_normal(g_ref["dconic"].shape) * eps * m[:, 2:5],
-             "dopacity": g_ref["dopacity"] + rng.standard_normal(g_ref["dopacity"].shape) * eps * m[:, 5],
-             "dcolor": g_ref["dcolor"] + rng.standard_normal(g_ref["dcolor"].shape) * eps * m[:, 6:9]}
+    # state_ulps: on top of that, noise of state_ulps * 2^-24 * statemass in duv / dconic / dopacity, for a
+    # backward whose per-pixel colour state is rounded differently from the oracle's (the per-gaussian algorithm)
+    m = (ulps * 2.0 ** -24) * g_ref["absmass"][:, :9].copy()
+    m[:, :6] += (state_ulps * 2.0 ** -24) * g_ref["statemass"]
+    noisy = {"duv": g_ref["duv"] + rng.standard_normal(g_ref["duv"].shape) * m[:, 0:2],
+             "dconic": g_ref["dconic"] + rng.standard_normal(g_ref["dconic"].shape) * m[:, 2:5],
+             "dopacity": g_ref["dopacity"] + rng.standard_normal(g_ref["dopacity"].shape) * m[:, 5],
+             "dcolor": g_ref["dcolor"] + rng.standard_normal(g_ref["dcolor"].shape) * m[:, 6:9]}
     pert = O.preprocess_bwd(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
                             ref["radii"], ref["cov2d_vecs"], ref["sh_to_rgb_ne_0"],
                             *(noisy[k].astype(np.float32) for k in ("duv", "dconic", "dopacity", "dcolor")))

@@ -98,3 +98,30 @@ def test_extra_channels_layouts_and_inference_depth(oracle):
     seen = full["T"] < 1
     assert np.allclose(inf["depth"][seen], want_depth[seen], rtol=1e-6, atol=0)
     assert (inf["depth"][~seen] == 0).all() or np.isnan(inf["depth"][~seen]).all()
+
+
+def test_statemass_bounds_the_effect_of_rounding_the_colour_state(oracle):
+    """`statemass` (the bar of the per-gaussian backward's test) is the sensitivity of duv / dconic / dopacity to
+    the pixels' running colour state: moving the final colour the backward starts from by one float32 ulp-scale
+    step per pixel and channel (which only shifts that state, every alpha and T stays the same) must move each
+    value by no more than 2^-24 * statemass, and does move some by a good part of it."""
+    O = oracle
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    P, ref = oracle_forward(O, scene, 1)
+    args = (P, ref["workload_ranges"], ref["gaussian_idx_sorted"], ref["uvs"], ref["conic_opacity"], ref["rgb_gaussian"],
+            ref["T"], ref["n_contrib"])
+    g0 = O.blend_bwd(*args, ref["color"], scene.drgb[0], scene.dT[0])
+    rng = np.random.default_rng(5)
+    step = (2.0 ** -24) * np.abs(ref["color"].astype(np.float64)) * rng.choice([-1.0, 1.0], size=ref["color"].shape)
+    moved = (ref["color"].astype(np.float64) + step).astype(np.float32)
+    moved_by = np.abs(moved.astype(np.float64) - ref["color"])          # what float32 made of the step
+    assert moved_by.max() <= 2.0 ** -23 * np.abs(ref["color"]).max()
+    g1 = O.blend_bwd(*args, moved, scene.drgb[0], scene.dT[0])
+    assert np.array_equal(g0["dcolor"], g1["dcolor"])                   # w * drgb does not see the colour state
+    got = np.concatenate([g1[k].reshape(scene.n, -1) - g0[k].reshape(scene.n, -1) for k in ("duv", "dconic", "dopacity")], 1)
+    # float32 rounds the step to 0, 1 or 2 ulp of the colour: bound with 2^-22 instead of 2^-24, plus the float32
+    # rounding of the terms themselves
+    bound = 2.0 ** -22 * g0["statemass"] + 1e-5 * g0["absmass"][:, :6] + 1e-30
+    assert (np.abs(got) <= bound).all()
+    live = g0["statemass"] > 0
+    assert live.any() and np.quantile((np.abs(got) / (2.0 ** -24 * g0["statemass"] + 1e-300))[live], 0.9) > 0.05
