@@ -89,10 +89,24 @@ __device__ __forceinline__ void apply_instance(d3gs_params& P, const InstanceVie
     }
 }
 
+// Sparse mode (config sparse_mode; render.py:234-238, 478-500, 622-640): everything downstream of K1 works on the
+// accepted render items only, stored compactly.  The reference counts them in a first launch of K1 and lets a
+// second launch take slots from an atomic counter, in whatever order the hardware reaches it; here the first
+// launch (valid_out) writes one flag per item, a scan of the flags gives every accepted item its slot in ascending
+// item order (slot_scan, inclusive), and the second launch writes its outputs there, which keeps the render
+// identical to the dense one bit for bit (ties in the sort go by slot, slots ascend with the item index).
+struct SparseView {
+    int32_t* valid_out;          // first launch: [items] 1 = accepted; nothing else is written
+    const int32_t* slot_scan;    // second launch: [items] inclusive scan of the flags
+    int32_t* gaussian_ids;       // second launch: [accepted] gaussian of each slot (sparse_gaussian_id)
+    int32_t* batch_ids;          // second launch: [accepted] camera of each slot (sparse_batch_id)
+};
+
 // kWithSh = false leaves the SH colour to sh_colors_kernel: no LDS, twice the resident wavefronts.
-template <bool kWithSh, bool kInstances>
+template <bool kWithSh, bool kInstances, bool kSparse = false>
 __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
-    const d3gs_params P0, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const d3gs_params P0, const InstanceView inst, const SparseView sparse, const float* __restrict__ xyz,
+    const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const float* __restrict__ sh_base, const uint8_t* __restrict__ invalid_mask, float* __restrict__ depths,
     int32_t* __restrict__ radii, float* __restrict__ uvs, float* __restrict__ conic_opacity,
@@ -199,6 +213,12 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         int area = (rmaxx - rminx) * (rmaxy - rminy);
         valid = (det > 0.0f) && area != 0 && (op > P.alpha_eps);
     }
+    if constexpr (kSparse) {
+        if (sparse.valid_out) {      // first launch: which items are accepted (wave-uniform branch)
+            if (in_range) sparse.valid_out[i] = valid ? 1 : 0;
+            return;
+        }
+    }
     {
         TileWalkIn g{u, v, radius, con0, con1, con2, op};
         TileWalk walk = {};
@@ -224,7 +244,15 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     }
     if (!valid) z = u = v = con0 = con1 = con2 = op = a = b = c = radius = 0.0f;
     if (!in_range) return;
-
+    int out_i = i;          // row of the outputs
+    if constexpr (kSparse) {
+        if (!valid) return;     // rejected items have no slot
+        out_i = sparse.slot_scan[i] - 1;
+        sparse.gaussian_ids[out_i] = g;
+        sparse.batch_ids[out_i] = batch;
+    }
+    {
+    const int i = out_i;
     depths[i] = z;
     if (depth_sort_keys) depth_sort_keys[i] = depth_sort_key(P, z);
     radii[i] = (int)radius;
@@ -246,6 +274,40 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
         rgb_out[3 * i + 2] = rgb[2];
         if (ne0_out) ne0_out[i] = (uint8_t)ne0;
     }
+    }
+}
+
+// SH colours of sparse mode's compact items: slot s holds gaussian ids[s] seen by camera batch_ids[s].  One
+// thread per slot reads its gaussian's SH row from global memory (the rows of consecutive slots are not
+// neighbours, so there is nothing to stage); same operations as sh_colors_kernel.
+__global__ __launch_bounds__(kPrepBlock) void sh_colors_sparse_kernel(
+    const d3gs_params P0, const int32_t* __restrict__ ids, const int32_t* __restrict__ batch_ids, const int count,
+    const float* __restrict__ xyz, const float* __restrict__ sh, const float* __restrict__ sh_base,
+    const int32_t* __restrict__ radii, float* __restrict__ rgb_out, uint8_t* __restrict__ ne0_out) {
+    const int slot = blockIdx.x * kPrepBlock + threadIdx.x;
+    if (slot >= count) return;
+    const int g = ids[slot];
+    d3gs_params P = P0;
+    if (P0.batch_size > 1) apply_batch_camera(P, batch_ids[slot]);
+    float rgb[3] = {0.0f, 0.0f, 0.0f};
+    uint32_t ne0 = 0;
+    if (radii[slot] > 0 && (unsigned)g < (unsigned)P0.n) {
+        float d[3] = {xyz[3 * g] - P.cam_center[0], xyz[3 * g + 1] - P.cam_center[1], xyz[3 * g + 2] - P.cam_center[2]};
+        float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
+        float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
+        const float* shp = sh + (size_t)g * P.sh_stride * 3;
+        const float* base = P.has_sh_base ? sh_base + 3 * g : shp;
+        const float* rest = P.has_sh_base ? shp : shp + 3;
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch) rgb[ch] = sh_channel(P.sh_degree, dx, dy, dz, base[ch], rest, ch);
+        ne0 = ((rgb[0] < 0.0f) << 2) | ((rgb[1] < 0.0f) << 1) | (rgb[2] < 0.0f);
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch) rgb[ch] = fmaxf(rgb[ch], 0.0f);
+    }
+    rgb_out[3 * slot + 0] = rgb[0];
+    rgb_out[3 * slot + 1] = rgb[1];
+    rgb_out[3 * slot + 2] = rgb[2];
+    if (ne0_out) ne0_out[slot] = (uint8_t)ne0;
 }
 
 // SH colour of the gaussians the preprocess kernel accepted (radii > 0), the part of K1 that
@@ -307,19 +369,20 @@ struct BwdInputs {
     float4 q, ra, rb, rc;      // quaternion; the blend backward's record: duv(2) dconic(3) dopacity dcolor(3) dz
     uint32_t ne0;
 };
-__device__ __forceinline__ BwdInputs load_bwd_inputs(const int i, const float* __restrict__ xyz,
+// i: row of the per-item arrays (cov2d, ne0, records); m: row of the model arrays (the same unless sparse)
+__device__ __forceinline__ BwdInputs load_bwd_inputs(const int i, const int m, const float* __restrict__ xyz,
                                                      const float* __restrict__ quat, const float* __restrict__ scale,
                                                      const float* __restrict__ opacity, const float* __restrict__ cov2d,
                                                      const uint8_t* __restrict__ ne0, const float4* __restrict__ rec4) {
     BwdInputs in;
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
-        in.xyz[k] = xyz[3 * i + k];
-        in.s[k] = scale[3 * i + k];
+        in.xyz[k] = xyz[3 * m + k];
+        in.s[k] = scale[3 * m + k];
         in.cov[k] = cov2d[3 * i + k];
     }
-    in.opacity = opacity[i];
-    in.q = *reinterpret_cast<const float4*>(quat + 4 * i);
+    in.opacity = opacity[m];
+    in.q = *reinterpret_cast<const float4*>(quat + 4 * m);
     in.ra = rec4[4 * (size_t)i];
     in.rb = rec4[4 * (size_t)i + 1];
     in.rc = rec4[4 * (size_t)i + 2];
@@ -592,12 +655,15 @@ static inline int bwd_rows_per_pass(int sh_stride) {
 // first + list[0 .. cnt)
 template <bool kToLds>
 __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float* lds, const unsigned short* list, int cnt,
-                                              int first, int rowlen, int stride, bool accumulate = false) {
+                                              int first, int rowlen, int stride, bool accumulate = false,
+                                              const int32_t* __restrict__ origin = nullptr) {
+    // origin (sparse mode, reads of the model's rows): row first + list[r] of the items is row origin[..] of `global`
+    auto row_of = [&](int r) { const int i = first + list[r]; return (size_t)(origin ? origin[i] : i); };
     if ((rowlen & 3) == 0 && ((uintptr_t)global & 15u) == 0) {
         const int per_row = rowlen >> 2;
         for (int q = threadIdx.x; q < cnt * per_row; q += kBwdBlock) {
             const int r = q / per_row, c = (q - r * per_row) * 4;
-            float4* gp = reinterpret_cast<float4*>(global + (size_t)(first + list[r]) * rowlen + c);
+            float4* gp = reinterpret_cast<float4*>(global + row_of(r) * rowlen + c);
             float* lp = lds + r * stride + c;
             if (kToLds) {
                 const float4 t = *gp;
@@ -612,7 +678,7 @@ __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float*
     } else {
         for (int e = threadIdx.x; e < cnt * rowlen; e += kBwdBlock) {
             const int r = e / rowlen, c = e - r * rowlen;
-            float* gp = global + (size_t)(first + list[r]) * rowlen + c;
+            float* gp = global + row_of(r) * rowlen + c;
             if (kToLds) lds[r * stride + c] = *gp;
             else *gp = accumulate ? *gp + lds[r * stride + c] : lds[r * stride + c];
         }
@@ -630,7 +696,7 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
     const float* __restrict__ grad_records, const uint8_t* __restrict__ touched, const int sh_mask_compat,
-    const int outputs_are_zero, const int rows_per_pass,
+    const int outputs_are_zero, const int rows_per_pass, const int32_t* __restrict__ origin,
     float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
     float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
@@ -717,8 +783,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         const int cnt = min(rows_per_pass, nactive - base);
         const int g = first + s_list[base + min(tid, cnt - 1)];
         BwdInputs in = {};
-        if (tid < cnt) in = load_bwd_inputs(g, xyz, quat, scale, opacity, cov2d, ne0, rec4);
-        bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride);
+        if (tid < cnt) in = load_bwd_inputs(g, origin ? origin[g] : g, xyz, quat, scale, opacity, cov2d, ne0, rec4);
+        bwd_rows_copy<true>(const_cast<float*>(sh), s_rows, s_list + base, cnt, first, rowlen, stride, false, origin);
         __syncthreads();
         if (tid < cnt) {
             d3gs_params Pg = P;
@@ -821,9 +887,10 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     }
     dim3 grid((item_count(*p) + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
     const size_t lds_bytes = with_sh ? (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float) : 0;
+    const SparseView dense = {nullptr, nullptr, nullptr, nullptr};
 #define D3GS_LAUNCH_K1(SH, INST)                                                                                      \
-    hipLaunchKernelGGL((preprocess_fwd_kernel<SH, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, xyz,   \
-                       quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs,     \
+    hipLaunchKernelGGL((preprocess_fwd_kernel<SH, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p, inst, dense, \
+                       xyz, quaternion_xyzw, scale, opacity, color_sh, color_sh_base, invalid_mask, depths, radii, uvs, \
                        conic_opacity, tiles_touched, rgb_gaussian, cov2d_vecs, sh_to_rgb_ne_0,                         \
                        (unsigned long long*)tile_masks, depth_sort_keys)
     if (with_sh) { if (inst.ids) D3GS_LAUNCH_K1(true, true); else D3GS_LAUNCH_K1(true, false); }
@@ -831,6 +898,60 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
 #undef D3GS_LAUNCH_K1
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_fwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
+                                          const float* scale, const float* opacity, const uint8_t* invalid_mask,
+                                          int32_t* valid_flags, const int32_t* slot_scan, int32_t* sparse_gaussian_ids,
+                                          int32_t* sparse_batch_ids, float* depths, int32_t* radii, float* uvs,
+                                          float* conic_opacity, int32_t* tiles_touched, float* cov2d_vecs,
+                                          uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_preprocess_fwd_sparse");
+    if (rc) return rc;
+    if (p->n == 0) return D3GS_OK;
+    if (!xyz || !quaternion_xyzw || !scale || !opacity) {
+        set_error("d3gs_preprocess_fwd_sparse: NULL model buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const bool first = valid_flags != nullptr;
+    if (first == (slot_scan != nullptr) ||
+        (!first && (!sparse_gaussian_ids || !sparse_batch_ids || !depths || !radii || !uvs || !conic_opacity ||
+                    !tiles_touched))) {
+        set_error("d3gs_preprocess_fwd_sparse: give valid_flags alone (first call), or slot_scan with the id and output "
+                  "buffers (second call)");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    const InstanceView inst = {nullptr, nullptr, 0};
+    const SparseView sparse = {valid_flags, slot_scan, sparse_gaussian_ids, sparse_batch_ids};
+    dim3 grid((item_count(*p) + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
+    hipLaunchKernelGGL((preprocess_fwd_kernel<false, true, true>), grid, block, 0, (hipStream_t)stream, *p, inst, sparse,
+                       xyz, quaternion_xyzw, scale, opacity, (const float*)nullptr, (const float*)nullptr, invalid_mask,
+                       depths, radii, uvs, conic_opacity, tiles_touched, (float*)nullptr, cov2d_vecs, (uint8_t*)nullptr,
+                       (unsigned long long*)tile_masks, depth_sort_keys);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_preprocess_fwd_sparse: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
+    return D3GS_OK;
+}
+
+extern "C" int d3gs_sh_colors_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids,
+                                     const int32_t* sparse_batch_ids, int32_t count, const float* xyz,
+                                     const float* color_sh, const float* color_sh_base, const int32_t* radii,
+                                     float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+    int rc = check_params(p, "d3gs_sh_colors_sparse");
+    if (rc) return rc;
+    if (count < 0) { set_error("d3gs_sh_colors_sparse: count < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
+    if (count == 0) return D3GS_OK;
+    if (!sparse_gaussian_ids || !sparse_batch_ids || !xyz || (!color_sh && p->sh_stride > 0) || !radii || !rgb_gaussian ||
+        (p->has_sh_base && !color_sh_base)) {
+        set_error("d3gs_sh_colors_sparse: NULL buffer");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    hipLaunchKernelGGL(sh_colors_sparse_kernel, dim3((count + kPrepBlock - 1) / kPrepBlock), dim3(kPrepBlock), 0,
+                       (hipStream_t)stream, *p, sparse_gaussian_ids, sparse_batch_ids, (int)count, xyz, color_sh,
+                       color_sh_base, radii, rgb_gaussian, sh_to_rgb_ne_0);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { set_error("d3gs_sh_colors_sparse: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
 }
 
@@ -881,6 +1002,31 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
                                       dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base, instances, stream);
 }
 
+static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t accumulate,
+                               const int32_t* origin, const float* xyz, const float* quaternion_xyzw,
+                               const float* scale, const float* opacity, const float* color_sh, const int32_t* radii,
+                               const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0, const float* grad_records,
+                               const uint8_t* touched, int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
+                               float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
+                               float* dcolor_sh_base, const d3gs_instances* instances, d3gs_stream_t stream);
+
+extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids, const float* xyz,
+                                          const float* quaternion_xyzw, const float* scale, const float* opacity,
+                                          const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                                          const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
+                                          int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
+                                          float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
+                                          float* dcolor_sh_base, d3gs_stream_t stream) {
+    if (!sparse_gaussian_ids && p && p->n > 0) {
+        set_error("d3gs_preprocess_bwd_sparse: sparse_gaussian_ids is NULL");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    return preprocess_bwd_impl("d3gs_preprocess_bwd_sparse", p, 0, 0, sparse_gaussian_ids, xyz, quaternion_xyzw, scale,
+                               opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
+                               outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
+                               nullptr, stream);
+}
+
 extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,
                                           const float* quaternion_xyzw, const float* scale, const float* opacity,
                                           const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
@@ -889,7 +1035,23 @@ extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_in
                                           float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
                                           float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                                           d3gs_stream_t stream) {
-    int rc = check_params(p, "d3gs_preprocess_bwd");
+    return preprocess_bwd_impl("d3gs_preprocess_bwd", p, batch_index, accumulate, nullptr, xyz, quaternion_xyzw, scale,
+                               opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
+                               outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
+                               instances, stream);
+}
+
+// origin (sparse mode): p->n compact items, item i being row origin[i] of the model arrays; gradients are written per
+// item.
+static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t accumulate,
+                               const int32_t* origin, const float* xyz,
+                               const float* quaternion_xyzw, const float* scale, const float* opacity,
+                               const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                               const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
+                               int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
+                               float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
+                               const d3gs_instances* instances, d3gs_stream_t stream) {
+    int rc = check_params(p, who);
     if (rc) return rc;
     if (batch_index < 0 || batch_index >= batch_count(*p)) {
         set_error("d3gs_preprocess_bwd_camera: batch_index %d outside the bundle of %d", batch_index, batch_count(*p));
@@ -916,7 +1078,8 @@ extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_in
                        (int)batch_index, (int)accumulate, inst, xyz,                                                   \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
                        touched,                                                                                        \
-                       (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, dxyz, dquaternion_xyzw, dscale,      \
+                       (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, origin, dxyz, dquaternion_xyzw,      \
+                       dscale,                                                                                         \
                        dopacity_out,                                                                                   \
                        dcolor_sh, dcolor_sh_base)
     if (wide) { if (inst.ids) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }

@@ -71,6 +71,9 @@ class GaussianSplatOpContext:
     # B * N rows (item b * N + g), tile ids and ranges cover B * tiles; the [B, 16] camera table on the device
     batch_size: int = 1
     batch_cameras: torch.Tensor | None = None
+    # sparse mode (render.py:234-238, 478-500): every per-gaussian array above has one row per ACCEPTED gaussian;
+    # the gaussian of each row (int32 [V], ascending)
+    sparse_gaussian_ids: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -197,7 +200,12 @@ class GaussianSplatOp:
             # the reference stores 1/z in the buffer it also sorts by (render.py:582, 773), which blends
             # back to front: not reproduced
             "render_inv_depth": c.render_inv_depth,
-            "transmittance_is_double": c.transmittance_is_double, "sparse_mode": c.sparse_mode,
+            "transmittance_is_double": c.transmittance_is_double,
+            # sparse mode is built for the plain colour path (the reference itself excludes custom features there,
+            # render.py:238)
+            "sparse_mode with disable_builtin_rgb / PER_GAUSSIAN":
+                c.sparse_mode and (c.disable_builtin_rgb
+                                   or c.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN),
             # builtin colours off: the kernels blend zeros in their place (render.py:262, 662, 1898-1931)
             "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
             # the per-gaussian backward (render.py:2319-2776) is built for the colour channels in [H,W,3]
@@ -413,6 +421,42 @@ class GaussianSplatOp:
         num_tiles = P.tiles_x * P.tiles_y * batch
         s = self._stream()
         f32, i32 = torch.float32, torch.int32
+        if self._count_host is None:
+            self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+            self._sort_status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+        # Sparse mode (render.py:234-238, 478-500, 622-640): a first pass of the preprocess flags the accepted
+        # gaussians, a scan gives each its row, and from here on n is their number V: every buffer below has V rows
+        # and the kernels after the preprocess see a scene of V gaussians.  The count has to reach the host before
+        # anything can be sized (the reference reads it back the same way, render.py:636).
+        sparse = bool(self._cfg.sparse_mode)
+        Pd = P            # what the kernels behind the preprocess are given
+        sparse_scan = sparse_gaussian_ids = sparse_batch_ids = None
+        if sparse:
+            assert custom_features is None, "custom_features must not be provided in sparse mode"    # render.py:238
+            if instance2world_T is not None:
+                raise NotImplementedError("sparse_mode with instance poses is not supported")
+            flags = torch.empty(n, dtype=i32, device=dev)
+            _capi.check(L.d3gs_preprocess_fwd_sparse(
+                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+                _capi.ptr(model.opacity), _capi.ptr(mask), _capi.ptr(flags), *([None] * 11), s),
+                "d3gs_preprocess_fwd_sparse (flags)")
+            sparse_scan = torch.empty(n, dtype=i32, device=dev)
+            ws_bytes = C.c_size_t(0)
+            _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
+            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
+            total_valid = torch.empty(1, dtype=torch.int64, device=dev)
+            _capi.check(L.d3gs_scan_gathered(_capi.ptr(flags), n, None, n, _capi.ptr(sparse_scan), _capi.ptr(ws),
+                                             ws.numel(), 0, _capi.ptr(total_valid),
+                                             C.c_void_p(self._count_host.data_ptr()), s), "d3gs_scan_gathered (flags)")
+            torch.cuda.current_stream().synchronize()
+            num_valid = int(self._count_host[0])
+            if num_valid < 0:
+                raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
+            n_items, n = n, num_valid
+            Pd = _capi.Params.from_buffer_copy(P)
+            Pd.n, Pd.batch_size, Pd.batch_cameras = n, 0, None
+            sparse_gaussian_ids = torch.empty(n, dtype=i32, device=dev)
+            sparse_batch_ids = torch.empty(n, dtype=i32, device=dev)
 
         def _sort_ws_bytes(count, begin_bit, end_bit):
             nbytes = C.c_size_t(0)
@@ -425,6 +469,23 @@ class GaussianSplatOp:
         # scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later
         tile_bits = L.d3gs_higher_msb(num_tiles)
         depth_bits = L.d3gs_depth_key_bits(C.byref(P))      # the depth sort's key width: 27 bits for the default planes
+        if sparse and n == 0:      # nothing accepted: the empty render, without touching zero-row buffers
+            self.last_num_rendered = 0
+            empty = GaussianSplatOutput(
+                custom_features=None, T=torch.ones((batch, height, width), dtype=f32, device=dev),
+                color=torch.zeros((batch, 4 if self._cfg.render_rgba else 3, height, width) if self._cfg.use_nchw else
+                                  (batch, height, width, 4 if self._cfg.render_rgba else 3), dtype=f32, device=dev),
+                depth=torch.zeros((batch, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None,
+                n_contrib=torch.zeros((batch, height, width), dtype=i32, device=dev),
+                radii=torch.zeros(0, dtype=i32, device=dev), sparse_gaussian_ids=sparse_gaussian_ids,
+                sparse_batch_ids=sparse_batch_ids)
+            if not training:
+                bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=dev).clamp(0, 1)
+                if self._cfg.use_nchw:
+                    empty.color[:, :3] = bg.view(1, 3, 1, 1)
+                else:
+                    empty.color[..., :3] = bg
+            return empty, None
         spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
         align = lambda v: (v + 255) // 256 * 256
         scan_ws_bytes = C.c_size_t(0)
@@ -458,6 +519,8 @@ class GaussianSplatOp:
                 rec_floats = n * _capi.GRAD_RECORD_FLOATS
                 pool_floats = self._grad_pool_floats(model) if self.clear_gradients_early else 0
                 mark_floats = (n + 15) // 16 * 4          # n bytes, in whole 16-byte units
+                if sparse:      # sparse gradients: one row per accepted gaussian (render.py:2918)
+                    pool_floats = self._grad_pool_floats(model, n) if self.clear_gradients_early else 0
                 grad_clear = torch.empty(rec_floats + pool_floats + mark_floats, dtype=f32, device=dev)
                 # (bundle: one record per render item, one set of model gradient arrays)
                 grad_records = grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
@@ -471,14 +534,25 @@ class GaussianSplatOp:
                 rgb_gaussian.zero_()
                 if ne0 is not None:
                     ne0.zero_()
-            _capi.check(L.d3gs_preprocess_fwd(
-                C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
-                _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
-                _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                _capi.ptr(tiles_touched), None if (overlap or no_rgb) else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
-                None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), inst, s),
-                "d3gs_preprocess_fwd")
+            if sparse:       # second pass: the accepted gaussians' outputs, row by row in ascending order
+                overlap = True      # (the colours always come from their own kernel here)
+                _capi.check(L.d3gs_preprocess_fwd_sparse(
+                    C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+                    _capi.ptr(model.opacity), _capi.ptr(mask), None, _capi.ptr(sparse_scan),
+                    _capi.ptr(sparse_gaussian_ids), _capi.ptr(sparse_batch_ids), _capi.ptr(depths), _capi.ptr(radii),
+                    _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(tiles_touched), _capi.ptr(cov2d_vecs),
+                    _capi.ptr(tile_masks), _capi.ptr(depth_keys), s), "d3gs_preprocess_fwd_sparse")
+            else:
+                _capi.check(L.d3gs_preprocess_fwd(
+                    C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
+                    _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
+                    _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                    _capi.ptr(tiles_touched), None if (overlap or no_rgb) else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
+                    None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), inst, s),
+                    "d3gs_preprocess_fwd")
         sh_done = None
+        if overlap and (self._side_stream is None or self._side_stream.device != dev):
+            self._side_stream = torch.cuda.Stream(device=dev)   # default priority
         if overlap:
             main = torch.cuda.current_stream()
             side = self._side_stream
@@ -486,7 +560,12 @@ class GaussianSplatOp:
             ta = torch.cuda.Event(enable_timing=True) if (self.stage_events is not None and not no_rgb) else None
             if ta is not None:
                 ta.record(side)
-            if not no_rgb:
+            if sparse:
+                _capi.check(L.d3gs_sh_colors_sparse(
+                    C.byref(P), _capi.ptr(sparse_gaussian_ids), _capi.ptr(sparse_batch_ids), n, _capi.ptr(model.xyz),
+                    _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base), _capi.ptr(radii), _capi.ptr(rgb_gaussian),
+                    _capi.ptr(ne0), C.c_void_p(side.cuda_stream)), "d3gs_sh_colors_sparse")
+            elif not no_rgb:
                 _capi.check(L.d3gs_sh_colors(
                     C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                     _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), inst, C.c_void_p(side.cuda_stream)),
@@ -557,7 +636,7 @@ class GaussianSplatOp:
             total = torch.empty(1, dtype=torch.int64, device=dev)
             order_in_b, pairs_in_b = C.c_int(0), C.c_int(0)
             _capi.check(L.d3gs_bin_pairs(
-                C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(depths),
+                C.byref(Pd), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(depths),
                 _capi.ptr(tiles_touched), _capi.ptr(tile_masks), _capi.ptr(depth_keys), at(o_keys_b), at(o_ord_a),
                 at(o_ord_b), _capi.ptr(zero_ws_n), zero_ws_n.numel(), at(o_offs), _capi.ptr(zero_scan_ws),
                 zero_scan_ws.numel(), _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), cap, at(o_tk_a),
@@ -604,7 +683,8 @@ class GaussianSplatOp:
         # disable_builtin_rgb: the caller's colour image is the alpha channel alone, or has no channel
         # (config_def.py:152-157)
         out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color[..., 3:] if no_rgb else out_color,
-                                  depth=out_depth, n_contrib=n_contrib, radii=radii)
+                                  depth=out_depth, n_contrib=n_contrib, radii=radii,
+                                  sparse_gaussian_ids=sparse_gaussian_ids, sparse_batch_ids=sparse_batch_ids)
 
         def _empty_result():
             if custom_features is not None:
@@ -642,7 +722,7 @@ class GaussianSplatOp:
                 with self._stage("make_keys"):
                     tile_keys = torch.empty(capacity, dtype=i32, device=dev)
                     gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
-                    _capi.check(L.d3gs_make_keys(C.byref(P), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
+                    _capi.check(L.d3gs_make_keys(C.byref(Pd), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                                                  _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
                                                  _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
                                                  _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
@@ -678,12 +758,12 @@ class GaussianSplatOp:
                 tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
                 grad_touched=grad_touched,
                 kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids,
-                batch_size=batch, batch_cameras=batch_cams)
+                batch_size=batch, batch_cameras=batch_cams, sparse_gaussian_ids=sparse_gaussian_ids)
             if sh_done is not None:
                 torch.cuda.current_stream().wait_event(sh_done)
             with self._stage("blend_fwd"):
                 self.rasterize_forward_backward(model, ctx, out, training=training,
-                                                render_depth=self._cfg.render_depth, _params=P)
+                                                render_depth=self._cfg.render_depth, _params=Pd)
             return ctx, tile_keys_sorted
 
         # The reference reads the pair count back before it can size the key buffers (render.py:695),
@@ -731,7 +811,8 @@ class GaussianSplatOp:
         camera (_forward_bundle)."""
         c = self._cfg
         return bool(self.bundle_in_one_pass and batch > 1 and instance2world_T is None and custom_features is None
-                    and not c.disable_builtin_rgb and not c.enable_32bit_sort and self.overlap_sh_colors)
+                    and not c.disable_builtin_rgb and not c.enable_32bit_sort and self.overlap_sh_colors
+                    and not c.sparse_mode)
 
     def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
                         prep_user_inputs):
@@ -758,6 +839,9 @@ class GaussianSplatOp:
                                   T=cat("T"), color=cat("color"),
                                   depth=cat("depth") if outs[0].depth is not None else None,
                                   n_contrib=cat("n_contrib"), radii=cat("radii"))
+        if self._cfg.sparse_mode:       # rows of camera 0, then camera 1, ... (render.py:494: sparse_batch_id)
+            out.sparse_gaussian_ids = cat("sparse_gaussian_ids")
+            out.sparse_batch_ids = torch.cat([torch.full_like(o.sparse_gaussian_ids, b) for b, o in enumerate(outs)], 0)
         if not training:
             return out, None
         return out, GaussianSplatOpBatchContext(per_camera=ctxs, cameras=cams, image_shape_wh=cameras.image_shape_wh)
@@ -767,24 +851,26 @@ class GaussianSplatOp:
 
     # ------------------------------------------------------- gradient pool
     @staticmethod
-    def _grad_fields(model):
+    def _grad_fields(model, rows=None):
+        """(name, shape) of the gradient arrays: the model's own shapes, or `rows` rows of them (sparse mode)."""
         fields = [("xyz", model.xyz), ("quaternion_xyzw", model.quaternion_xyzw), ("scale", model.scale),
                   ("opacity", model.opacity), ("color_sh", model.color_sh)]
         if model.color_sh_base is not None:
             fields.append(("color_sh_base", model.color_sh_base))
-        return fields
+        return [(name, tuple(t.shape) if rows is None else (rows,) + tuple(t.shape[1:])) for name, t in fields]
 
     @classmethod
-    def _grad_pool_floats(cls, model) -> int:
-        return sum((t.numel() + 63) // 64 * 64 for _, t in cls._grad_fields(model))
+    def _grad_pool_floats(cls, model, rows=None) -> int:
+        return sum((int(np.prod(shape)) + 63) // 64 * 64 for _, shape in cls._grad_fields(model, rows))
 
     @classmethod
-    def _grad_views(cls, model, pool):
+    def _grad_views(cls, model, pool, rows=None):
         """The model-shaped gradient tensors as 256-byte aligned slices of one allocation."""
         views, off = {}, 0
-        for name, t in cls._grad_fields(model):
-            views[name] = pool[off:off + t.numel()].view(t.shape)
-            off += (t.numel() + 63) // 64 * 64
+        for name, shape in cls._grad_fields(model, rows):
+            numel = int(np.prod(shape))
+            views[name] = pool[off:off + numel].view(shape)
+            off += (numel + 63) // 64 * 64
         return views
 
     # ------------------------------------------------------- custom features
@@ -929,6 +1015,9 @@ class GaussianSplatOp:
         L = self._lib
         P = self.make_params(model, cameras, True, ctx.batch_cameras)
         s = self._stream()
+        sparse_ids = ctx.sparse_gaussian_ids
+        if sparse_ids is not None:      # the kernels see a scene of the V accepted gaussians
+            P.n = int(sparse_ids.numel())
         n, dev = P.n, model.xyz.device
         B = ctx.batch_size
         with self._stage("blend_bwd"):
@@ -941,10 +1030,11 @@ class GaussianSplatOp:
             dcustom = self._backward_custom_features(P, ctx, out, dfeat_img.contiguous(), g.records, g.touched)
         with self._stage("preprocess_bwd"):
             pool, ctx.grad_pool = ctx.grad_pool, None
-            prezeroed = pool is not None and pool.numel() == self._grad_pool_floats(model)
+            grad_rows = None if sparse_ids is None else n     # sparse mode: one gradient row per accepted gaussian
+            prezeroed = pool is not None and pool.numel() == self._grad_pool_floats(model, grad_rows)
             if not prezeroed:
-                pool = torch.empty(self._grad_pool_floats(model), dtype=torch.float32, device=dev)
-            gv = self._grad_views(model, pool)
+                pool = torch.empty(self._grad_pool_floats(model, grad_rows), dtype=torch.float32, device=dev)
+            gv = self._grad_views(model, pool, grad_rows)
             dxyz, dquat, dscale, dopacity, dsh = (gv[k] for k in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh"))
             dsh_base = gv.get("color_sh_base")
             # the cameras of the forward pass; a context from a pass without instances takes the argument
@@ -954,8 +1044,17 @@ class GaussianSplatOp:
             inst = self._instances_arg(inst_ids, inst_cams)
             # One launch per camera (the reference loops over the batch inside its kernel, render.py:2972-2989):
             # camera b works on its own rows of the per-item arrays, the first call stores, the others add.
+            if sparse_ids is not None:
+                # sparse gradient (render.py:2918, 3185-3213): row i belongs to gaussian sparse_gaussian_ids[i]
+                _capi.check(L.d3gs_preprocess_bwd_sparse(
+                    C.byref(P), _capi.ptr(sparse_ids), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),
+                    _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii),
+                    _capi.ptr(ctx.cov2d_vecs), _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), _capi.ptr(g.touched),
+                    int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat),
+                    _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), s),
+                    "d3gs_preprocess_bwd_sparse")
             rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
-            for b in range(B):
+            for b in range(B if sparse_ids is None else 0):
                 _capi.check(L.d3gs_preprocess_bwd_camera(
                     C.byref(P), b, int(b > 0), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),
                     _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh),
@@ -972,8 +1071,49 @@ class GaussianSplatOp:
         return grad_model, None, dcustom
 
 
+def _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad):
+    """Sparse-mode bundle (render.py:2864-2903): each camera has its own accepted gaussians; the gradient rows of a
+    gaussian seen by several cameras are merged.  The reference deduplicates the ids with a hash table
+    (insert, collect, query); here they are sorted and made unique, which also fixes the row order: the result has
+    one row per distinct accepted gaussian, ascending, and ``op.last_sparse_unique_ids`` names them."""
+    parts, duvs, offs = [], [], 0
+    for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
+        if ctx_b is None:
+            continue
+        v = int(ctx_b.sparse_gaussian_ids.numel())
+        sl = slice(offs, offs + v)
+        offs += v
+        g_b = GaussianSplatGradients(drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
+                                     ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous())
+        out_b = out.select_batch(b)
+        out_b.radii = out.radii[sl]
+        gm, duv, _ = op.backward(model, cam_b, ctx_b, out_b, g_b, return_uv_grad=True)
+        parts.append((ctx_b.sparse_gaussian_ids, gm))
+        duvs.append(duv[0])
+    dev = model.xyz.device
+    if not parts:
+        op.last_sparse_unique_ids = torch.zeros(0, dtype=torch.int32, device=dev)
+        zeros = {k: torch.zeros((0,) + tuple(v.shape[1:]), dtype=v.dtype, device=dev)
+                 for k, v in model.get_proxy_field_dict().items()}
+        return dataclasses.replace(model, **zeros), None, None
+    all_ids = torch.cat([ids for ids, _ in parts], 0)
+    unique, inverse = torch.unique(all_ids, sorted=True, return_inverse=True)
+    op.last_sparse_unique_ids = unique.to(torch.int32)
+    merged = {}
+    for name in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh", "color_sh_base"):
+        if getattr(model, name) is None:
+            continue
+        rows = torch.cat([getattr(gm, name) for _, gm in parts], 0)
+        merged[name] = torch.zeros((unique.numel(),) + tuple(rows.shape[1:]), dtype=rows.dtype, device=dev)
+        merged[name].index_add_(0, inverse, rows)
+    # duv: one row per accepted (camera, gaussian), cameras one after the other, as out.sparse_gaussian_ids
+    return dataclasses.replace(model, **merged), (torch.cat(duvs, 0).unsqueeze(0) if return_uv_grad else None), None
+
+
 def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
     """Per-camera backward passes; the model gradients add up over the cameras, duv stays per camera."""
+    if op._cfg.sparse_mode:
+        return _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad)
     total, duvs, dcustom = None, [], None
     n = len(model)
     for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):

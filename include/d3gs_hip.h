@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 27
+#define D3GS_ABI_VERSION 28
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -390,6 +390,38 @@ int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_
                                int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
                                float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
                                const d3gs_instances* instances, d3gs_stream_t stream);
+
+/* Sparse mode (config sparse_mode, config_def.py:119; render.py:234-238, 478-500, 622-640, 753, 2857-2866,
+ * 3185-3213): everything after K1 works on the accepted render items only, stored compactly -- for scenes of which
+ * a view sees a small part.  The reference counts the accepted items with a first launch of K1
+ * (block_reduce + atomicAdd, render.py:480-486), reads the count back, and lets a second launch take slots from an
+ * atomic counter (render.py:490-495).  Here:
+ *   1. d3gs_preprocess_fwd_sparse with valid_flags [items] (slot_scan = NULL): 1 where the item is accepted;
+ *   2. the caller scans the flags (d3gs_scan_gathered with index = NULL; its total is the accepted count V, which the
+ *      caller needs on the host to size the compact buffers, as the reference does);
+ *   3. d3gs_preprocess_fwd_sparse with slot_scan (valid_flags = NULL): outputs [V] in ascending item order,
+ *      sparse_gaussian_ids [V] and sparse_batch_ids [V] say which gaussian and camera each slot holds (the
+ *      reference's sparse_gaussian_id / sparse_batch_id; its slot order is whatever the atomic gives);
+ *   4. d3gs_sh_colors_sparse for the colours, then the binning and blend entry points with params whose n = V
+ *      (they only index per-item arrays), then
+ *   5. d3gs_preprocess_bwd_sparse: K9 over the V items; gradients are written per item, [V] rows (the rows of the
+ *      model arrays are found through sparse_gaussian_ids), as the reference's sparse gradient (render.py:2918).
+ * The render is the dense one bit for bit: slots ascend with the item index, so ties in the sort fall the same way. */
+int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
+                               const float* opacity, const uint8_t* invalid_mask, int32_t* valid_flags,
+                               const int32_t* slot_scan, int32_t* sparse_gaussian_ids, int32_t* sparse_batch_ids,
+                               float* depths, int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
+                               float* cov2d_vecs, uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream);
+int d3gs_sh_colors_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids, const int32_t* sparse_batch_ids,
+                          int32_t count, const float* xyz, const float* color_sh, const float* color_sh_base,
+                          const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
+int d3gs_preprocess_bwd_sparse(const d3gs_params* p /* n = V */, const int32_t* sparse_gaussian_ids, const float* xyz,
+                               const float* quaternion_xyzw, const float* scale, const float* opacity,
+                               const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
+                               const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
+                               int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
+                               float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
+                               d3gs_stream_t stream);
 
 #ifdef __cplusplus
 }
