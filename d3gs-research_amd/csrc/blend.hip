@@ -195,6 +195,14 @@ __device__ __forceinline__ void select2_or_zero(unsigned long long mask, float a
         : "v"(a0), "v"(b0), "s"(mask));
 }
 
+// measure_atomic_add_count: the wavefront's flush instruction issues one line-wide request per group of sixteen
+// lanes that holds a non-zero value (nz: ballot of the lanes with one)
+__device__ __forceinline__ void count_requests(uint32_t* counter, unsigned long long nz) {
+    const uint32_t n = (uint32_t)((nz & 0xFFFFull) != 0) + (uint32_t)(((nz >> 16) & 0xFFFFull) != 0) +
+                       (uint32_t)(((nz >> 32) & 0xFFFFull) != 0) + (uint32_t)((nz >> 48) != 0);
+    if (n) atomicAdd(counter, n);
+}
+
 // Index of channel ch of pixel pid (= y * W + x) of image `batch` in the colour images: [B,H,W,C] or, with
 // use_nchw, [B,C,H,W].
 __device__ __forceinline__ size_t color_index(const d3gs_params& P, int batch, size_t pid, int ch, int channels) {
@@ -552,9 +560,10 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * gid + slot_k, v);
             // one byte per gaussian that received anything: the preprocess backward finds its work in this
             // dense array instead of reading every record
-            if (touched) {
+            if (touched || P.atomic_add_count) {
                 const unsigned long long nz = __ballot(v != 0.0f);
-                if (slot_k == 0 && ((nz >> (tid & 48)) & 0xFFFFull)) touched[gid] = 1;
+                if (touched && slot_k == 0 && ((nz >> (tid & 48)) & 0xFFFFull)) touched[gid] = 1;
+                if (P.atomic_add_count && lane == 0) count_requests(P.atomic_add_count, nz);
             }
         }
     }
@@ -741,9 +750,10 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
             const int id = s_gid[wave][gl];
             const float v = id >= 0 ? s_out[wave][gl][slot_k] : 0.0f;
             if (v != 0.0f) unsafeAtomicAdd(grad_records + (size_t)D3GS_GRAD_RECORD_FLOATS * id + slot_k, v);
-            if (touched) {
+            if (touched || P.atomic_add_count) {
                 const unsigned long long nz = __ballot(v != 0.0f);
-                if (slot_k == 0 && ((nz >> (lane & 48)) & 0xFFFFull)) touched[id] = 1;
+                if (touched && slot_k == 0 && ((nz >> (lane & 48)) & 0xFFFFull)) touched[id] = 1;
+                if (P.atomic_add_count && lane == 0) count_requests(P.atomic_add_count, nz);
             }
         }
         __builtin_amdgcn_wave_barrier();    // the next bucket overwrites this wavefront's tables

@@ -980,6 +980,11 @@ class GaussianSplatOp:
         # and dz are strided views of it
         rec, ctx.grad_records = ctx.grad_records, None
         touched, ctx.grad_touched = ctx.grad_touched, None
+        counter = None
+        if self._cfg.measure_atomic_add_count:     # config_def.py:134; render.py:2310-2311
+            counter = torch.zeros(1, dtype=torch.int32, device=dev)
+            P = _capi.Params.from_buffer_copy(P)
+            P.atomic_add_count = counter.data_ptr()
         if rec is None:     # a second backward over this context: fresh records, work found from the records
             rec = torch.zeros((n, _capi.GRAD_RECORD_FLOATS), dtype=torch.float32, device=dev)
             touched = None
@@ -998,6 +1003,11 @@ class GaussianSplatOp:
                 _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
                 _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth), _capi.ptr(rec),
                 _capi.ptr(touched), s), "d3gs_blend_bwd")
+        if counter is not None:
+            # global atomic requests of this blend backward (one per (tile, gaussian) with a non-zero sum); the
+            # reference prints its count the same way
+            self.last_atomic_add_count = int(counter.item())
+            print(f"atomic add count: {self.last_atomic_add_count}")
         res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
                                       dz=rec[:, 9] if render_depth else None, records=rec, touched=touched)
         return res

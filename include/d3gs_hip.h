@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 28
+#define D3GS_ABI_VERSION 29
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -103,6 +103,11 @@ typedef struct d3gs_params {
     int32_t batch_size;
     int32_t reserved0;
     const float* batch_cameras;
+    /* measure_atomic_add_count (config_def.py:134; render.py:1451-1453, 2145-2148, 2310-2311): when not NULL, the
+     * blend backward kernels add to this device counter the number of global atomic requests they issue (one
+     * line-wide request per (tile, gaussian) whose sums are not all zero; the reference counts its per-value
+     * atomicAdd calls).  The caller zeroes it. */
+    uint32_t* atomic_add_count;
 } d3gs_params;
 
 #define D3GS_BATCH_CAMERA_FLOATS 16

@@ -206,3 +206,33 @@ def test_runs_on_the_callers_stream():
         assert torch.equal(ctx2.gaussian_idx_sorted, ctx.gaussian_idx_sorted)
         assert torch.allclose(gm2.xyz, gm.xyz, rtol=1e-3, atol=1e-5 * float(gm.xyz.abs().max()))
     torch.cuda.synchronize()
+
+
+def test_atomic_add_count(capsys):
+    """measure_atomic_add_count (config_def.py:134): the blend backward reports its global atomic requests, one
+    line-wide request per (tile, gaussian) with a non-zero sum: at least one per gaussian that received a
+    gradient, at most one per list entry in front of a tile's last contributor."""
+    import torch
+    from d3gs_research_amd.config_def import RasterizeBackwardAlgo
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    model = torch_model(scene)
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    counts = {}
+    for algo in (RasterizeBackwardAlgo.DEFAULT, RasterizeBackwardAlgo.PER_GAUSSIAN):
+        op = GaussianSplatOp(op_config(scene, 4, measure_atomic_add_count=True, rasterize_backward_algo=algo))
+        out, ctx = op.forward(model, scene.camera(), training=True)
+        op.backward(model, scene.camera(), ctx, out, grads)
+        assert f"atomic add count: {op.last_atomic_add_count}" in capsys.readouterr().out
+        ranges = ctx.workload_ranges.cpu().numpy()
+        nc = out.n_contrib[0].cpu().numpy()
+        walked = 0
+        for t, (r0, r1) in enumerate(ranges):
+            if r1 > r0:
+                ty, tx = divmod(t, (scene.width + 15) // 16)
+                walked += min(int(nc[ty * 16:ty * 16 + 16, tx * 16:tx * 16 + 16].max()) + 1, r1 - r0)
+        touched = int((op.last_raster_grads.records != 0).any(dim=1).sum())
+        assert touched <= op.last_atomic_add_count <= walked, (touched, op.last_atomic_add_count, walked)
+        counts[algo] = op.last_atomic_add_count
+    # both algorithms flush once per (tile, gaussian): the counts agree up to sums that cancel to zero in one of them
+    assert abs(counts[RasterizeBackwardAlgo.DEFAULT] - counts[RasterizeBackwardAlgo.PER_GAUSSIAN]) <= 0.001 * max(counts.values())
