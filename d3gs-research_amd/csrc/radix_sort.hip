@@ -28,10 +28,12 @@
 
 namespace d3gs {
 
-constexpr int kOsThreads = 512;
-constexpr int kOsWaves = kOsThreads / 64;
-constexpr int kOsItems = 8;
-constexpr int kOsTile = kOsThreads * kOsItems;  // 4096 pairs per workgroup
+constexpr int kOsTile = 4096;  // pairs per workgroup
+// Threads per workgroup of a pass: one thread owns one digit, so 9-bit digits take 512 threads (8 keys per thread);
+// 7- and 8-bit digits run 256 threads with 16 keys each: half the wavefronts per workgroup lets six workgroups
+// instead of four share a CU, which covers the 1500 tiles of a 6M-pair sort in one round of workgroups instead of
+// one and a half (pair sort of the benchmark view: 0.121 -> 0.111 ms; with 2048-pair tiles it was slower).
+template <int kBits> constexpr int os_threads() { return kBits > 8 ? 512 : 256; }
 // Digits are 7, 8 or 9 bits wide: the narrowest width that reaches the fewest passes.  9 saves a pass on 18 or 27
 // key bits (the depth keys of the gaussians); 7 costs none on 9 to 14 bits (the tile ids of an image of up to
 // 16384 tiles) and makes the ranking one ballot shorter and a digit's run in the output twice as long.
@@ -47,7 +49,10 @@ constexpr uint32_t kFlagAggregate = 1u << 30;
 constexpr uint32_t kFlagPrefix = 2u << 30;
 constexpr uint32_t kValueMask = (1u << 30) - 1u;
 constexpr int kSpinLimit = 1 << 22;
-constexpr int kLookWindow = 16;  // predecessor tiles polled per look-back step
+// predecessor tiles polled per look-back step: 4 measured faster than 8, 16, 32 or 64 (0.121 -> 0.112 ms on 6M
+// pairs, 0.075 -> 0.071 ms on 1M keys): the polls of a step are issued by every digit's thread, and what a wider
+// window saves in steps it costs in loads that come back "not published yet"
+constexpr int kLookWindow = 4;
 
 struct SortWorkspace {
     uint32_t* hist;     // [passes][radix] digit totals of the whole input
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __rest
 }
 
 template <typename Key, int kBits>
-__global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restrict__ keys_in,
+__global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key* __restrict__ keys_in,
                                                               const int32_t* __restrict__ vals_in,
                                                               Key* __restrict__ keys_out,
                                                               int32_t* __restrict__ vals_out, long long m,
@@ -139,6 +144,7 @@ __global__ __launch_bounds__(kOsThreads) void os_pass_kernel(const Key* __restri
                                                               uint32_t* __restrict__ status,
                                                               uint32_t* __restrict__ error) {
     constexpr int kRadix = 1 << kBits;
+    constexpr int kOsThreads = os_threads<kBits>(), kOsWaves = kOsThreads / 64, kOsItems = kOsTile / kOsThreads;
     static_assert(kRadix <= kOsThreads && kRadix <= kOsMaxRadix, "one thread owns one digit");
     __shared__ int wave_cnt[kOsWaves][kRadix];  // running, then exclusive-over-waves, per-wave digit counts
     __shared__ int digit_out[kRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
@@ -407,7 +413,8 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         const uint32_t mask = (1u << nb) - 1u;
         const uint32_t* pass_hist = ws.hist + (size_t)p * radix;
         uint32_t* pass_status = ws.status + (size_t)p * ntiles * radix;
-        hipLaunchKernelGGL(pass_kernel, dim3(ntiles), dim3(kOsThreads), 0, s, kin, vin, kout, vout, (long long)m,
+        hipLaunchKernelGGL(pass_kernel, dim3(ntiles), dim3(digit == 9 ? os_threads<9>() : os_threads<8>()), 0, s, kin, vin,
+                           kout, vout, (long long)m,
                            (const long long*)m_device, bit, mask, ntiles, pass_hist, pass_status, ws.error);
         std::swap(kin, kout);
         vin = vout;
