@@ -159,8 +159,28 @@ __device__ __forceinline__ uint32_t stage_gaussian(const d3gs_params& P, int g, 
     const bool in_x = xy.x + hx >= tile_x0 && xy.x - hx <= tile_x0 + 15.0f;
     const bool in_y = xy.y + hy >= tile_y0 && xy.y - hy <= tile_y0 + 15.0f;
     if (!(in_x && in_y)) return 0u;
-    return (uint32_t)(left && top) | ((uint32_t)(right && top) << 1) | ((uint32_t)(left && bottom) << 2) |
-           ((uint32_t)(right && bottom) << 3);
+    const uint32_t box = (uint32_t)(left && top) | ((uint32_t)(right && top) << 1) | ((uint32_t)(left && bottom) << 2) |
+                         ((uint32_t)(right && bottom) << 3);
+    // The ellipse itself against each patch: the minimum of Q = a dx^2 + 2 b dx dy + c dy^2 over the patch's
+    // pixel-centre rectangle.  Q is convex with its minimum at the centre, so over a rectangle it is attained
+    // on the vertical line nearest to the centre in x or on the horizontal line nearest in y, each time at the
+    // clamped one-dimensional minimiser; both candidates are points of the rectangle, so the smaller of the two
+    // is the minimum.  A misplaced minimiser raises Q only in second order; the evaluation error of Q is
+    // covered by widening R once more by 2 err.  A patch is dropped only on "minimum > R" (a NaN keeps it).
+    const float R2 = R + 2.0f * err;
+    const float slope_y = -co.y / co.z, slope_x = -co.y / co.x;  // dy* = slope_y dx on a vertical line, dx* = slope_x dy
+    const float lx = tile_x0 - xy.x, ly = tile_y0 - xy.y;
+    auto reaches = [&](float x_lo, float y_lo) {
+        const float x_hi = x_lo + 7.0f, y_hi = y_lo + 7.0f;
+        const float dxn = __builtin_amdgcn_fmed3f(0.0f, x_lo, x_hi), dyn = __builtin_amdgcn_fmed3f(0.0f, y_lo, y_hi);
+        const float dys = __builtin_amdgcn_fmed3f(slope_y * dxn, y_lo, y_hi);
+        const float dxs = __builtin_amdgcn_fmed3f(slope_x * dyn, x_lo, x_hi);
+        const float q1 = co.x * dxn * dxn + 2.0f * co.y * dxn * dys + co.z * dys * dys;
+        const float q2 = co.x * dxs * dxs + 2.0f * co.y * dxs * dyn + co.z * dyn * dyn;
+        return !(q1 > R2) || !(q2 > R2);
+    };
+    return box & ((uint32_t)reaches(lx, ly) | ((uint32_t)reaches(lx + 8.0f, ly) << 1) |
+                  ((uint32_t)reaches(lx, ly + 8.0f) << 2) | ((uint32_t)reaches(lx + 8.0f, ly + 8.0f) << 3));
 }
 
 // Publishes the four per-patch ballots of this staging wavefront's 64 gaussians.
