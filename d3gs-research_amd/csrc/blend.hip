@@ -28,10 +28,22 @@ namespace d3gs {
 
 constexpr int kBucket = D3GS_BUCKET_SIZE;   // list entries per bucket of the per-gaussian backward: one per lane of a wavefront
 
+// One staged gaussian: everything a visit reads sits in one 48-byte LDS record, so a visit forms one LDS
+// address (the reads differ in their immediate offsets only).
 struct __attribute__((aligned(16))) StagedGaussian {
-    float x, y, thr, pad;   // pixel-space centre, cull threshold
-    float ha, nb, hc, o;    // pre-scaled conic (-a/2, -b, -c/2) and opacity
+    float x, y, thr, o;         // pixel-space centre, cull threshold, opacity
+    float ha, nb, hc, depth;    // pre-scaled conic (-a/2, -b, -c/2); camera-space depth (depth channel only)
+    float r, g, b, pad;         // colour
 };
+
+// Staged gaussian j of a wave-uniform index: the record's byte offset is formed once, in a vector register that
+// every read of the visit then shares (written out because the compiler re-forms a scalar-to-vector move for
+// each read instead of keeping it).
+__device__ __forceinline__ const StagedGaussian& staged_at(const StagedGaussian* base, int j) {
+    uint32_t off;
+    asm("v_mov_b32 %0, %1" : "=v"(off) : "s"(j * (int)sizeof(StagedGaussian)));
+    return *reinterpret_cast<const StagedGaussian*>(reinterpret_cast<const char*>(base) + off);
+}
 
 // power = -1/2 (a dx^2 + c dy^2) - b dx dy (render.py:1765-1767) as a fixed sequence of three
 // multiplies and two fused multiply-adds; a CPU evaluating the same sequence gets the same bits.
@@ -81,6 +93,8 @@ __device__ __forceinline__ int reduce_slot(int lane) {
     return -1;
 }
 
+// kTen = false: v9 is the constant zero and the one instruction that only moves it is left out.
+template <bool kTen>
 __device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
                                                float v7, float v8, float v9) {
     // 16 -> 8 and 8 -> 4 inside each row of 16 lanes, while the most registers are live, with DPP adds whose
@@ -89,26 +103,48 @@ __device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, flo
     // select.  row_ror:8 pairs lane i with i ^ 8 (banks 0,1 | 2,3), row_half_mirror pairs i with 7 - i inside
     // each 8 lanes (banks 0,2 | 1,3).  The block opens and closes with two wait states: a DPP read needs
     // them after a vector write of its source, and so does what follows; the compiler cannot see inside.
-    asm("s_nop 1\n\t"
-        "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %0, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %1, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %2, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %3, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %4, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+    if constexpr (kTen) {
+        asm("s_nop 1\n\t"
+            "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %0, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %1, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %2, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %3, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %4, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
         // now %0..%4 hold (v0|v1), (v2|v3), (v4|v5), (v6|v7), (v8|v9) in lanes (bit 3 clear | set)
-        "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
-        "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
-        "v_add_f32_dpp %4, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %1, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
-        "v_add_f32_dpp %3, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
-        "s_nop 1"
-        : "+v"(v1), "+v"(v3), "+v"(v5), "+v"(v7), "+v"(v9)
-        : "v"(v0), "v"(v2), "v"(v4), "v"(v6), "v"(v8));
+            "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %4, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %3, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "s_nop 1"
+            : "+v"(v1), "+v"(v3), "+v"(v5), "+v"(v7), "+v"(v9)
+            : "v"(v0), "v"(v2), "v"(v4), "v"(v6), "v"(v8));
+    } else {
+        asm("s_nop 1\n\t"
+            "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %0, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %1, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %2, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %3, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %4, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        // now %0..%4 hold (v0|v1), (v2|v3), (v4|v5), (v6|v7), (v8|v9) in lanes (bit 3 clear | set)
+            "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %3, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %4, %4, %4 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %3, %2, %2 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "s_nop 1"
+            : "+v"(v1), "+v"(v3), "+v"(v5), "+v"(v7), "+v"(v9)
+            : "v"(v0), "v"(v2), "v"(v4), "v"(v6), "v"(v8));
+    }
     // v3: v0 v1 | v2 v3 by (bit 3, bit 2) of the lane; v7: v4 .. v7 likewise; v9: v8 | v9 by bit 3
     // 64 -> 32: rows 0,1 keep the first register, rows 2,3 the second
     const float e0 = swap_add32(v3, v7), e1 = swap_add32(v9, 0.0f);
@@ -129,19 +165,24 @@ __device__ __forceinline__ int wave_max_i32(int v) {
 // Stages one gaussian and returns a 4-bit mask: bit q set when the gaussian may reach a pixel of
 // the tile's 8x8 patch q (q & 1 = right half, q >> 1 = lower half).  Conservative by construction.
 __device__ __forceinline__ uint32_t stage_gaussian(const d3gs_params& P, int g, const float* __restrict__ uvs,
-                                                   const float* __restrict__ conic_opacity, float tile_x0,
-                                                   float tile_y0, StagedGaussian* dst) {
+                                                   const float* __restrict__ conic_opacity,
+                                                   const float* __restrict__ rgb_g, const float* __restrict__ depths,
+                                                   float tile_x0, float tile_y0, StagedGaussian* dst) {
     const float2 xy = *reinterpret_cast<const float2*>(uvs + 2 * g);
     const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * g);
     StagedGaussian s;
     s.x = xy.x;
     s.y = xy.y;
     s.thr = __logf(P.alpha_eps / co.w) - 1.0e-3f;
-    s.pad = 0.0f;
+    s.o = co.w;
     s.ha = -0.5f * co.x;  // exact scalings: power = (ha dx) dx + (hc dy) dy + (nb dx) dy
     s.nb = -co.y;
     s.hc = -0.5f * co.z;
-    s.o = co.w;
+    s.depth = depths ? depths[g] : 0.0f;
+    s.r = rgb_g[3 * g];
+    s.g = rgb_g[3 * g + 1];
+    s.b = rgb_g[3 * g + 2];
+    s.pad = 0.0f;
     *dst = s;
     // Level set {power >= thr}: a dx^2 + 2 b dx dy + c dy^2 <= R with R = -2 thr.  A pixel of this tile
     // evaluates `power` with an absolute rounding error below err; widening R by 2 err keeps every pixel
@@ -269,7 +310,6 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
             clear_vec[q] = make_uint4(0u, 0u, 0u, 0u);
     }
     __shared__ StagedGaussian s_g[kBlock];
-    __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
     constexpr int kChannels = kRgba ? 4 : 3;
 
@@ -306,8 +346,8 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
         if (src < r1) {
             const int g = idx_sorted[src];
             if ((unsigned)g < (unsigned)items) {  // a corrupt index list must not become a wild read
-                bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
+                bits = stage_gaussian(P, g, uvs, conic_opacity, rgb_g, kDepth ? depths : nullptr, tile_x0, tile_y0,
+                                      &s_g[tid]);
             }
         }
         publish_masks(bits, wave, lane, s_mask);
@@ -325,7 +365,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
             while (m) {
                 const int j = chunk * 64 + __builtin_ctzll(m);
                 m &= m - 1;
-                const StagedGaussian sg = s_g[j];
+                const StagedGaussian& sg = staged_at(s_g, j);
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
                 const float power = blend_power(sg, dx, dy);
                 const bool live = power >= sg.thr;      // false for a finished pixel (NaN)
@@ -346,12 +386,11 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 const float w = use ? alpha * T : 0.0f;
                 T = use ? nextT : T;
                 contributor = use ? round * kBlock + j : contributor;
-                const float4 c = s_rgb[j];
-                acc0 = __builtin_fmaf(w, c.x, acc0);
-                acc1 = __builtin_fmaf(w, c.y, acc1);
-                acc2 = __builtin_fmaf(w, c.z, acc2);
+                acc0 = __builtin_fmaf(w, sg.r, acc0);
+                acc1 = __builtin_fmaf(w, sg.g, acc1);
+                acc2 = __builtin_fmaf(w, sg.b, acc2);
                 if constexpr (kRgba) acc3 = acc3 + w;
-                if constexpr (kDepth) depth_accum = __builtin_fmaf(w, c.w, depth_accum);
+                if constexpr (kDepth) depth_accum = __builtin_fmaf(w, sg.depth, depth_accum);
                 pxf = stop ? __builtin_nanf("") : pxf;
                 // every pixel of the patch finished: both loops end at their next test (one way out of the
                 // loops keeps the scalar control flow short; the scalar unit is shared by the CU's four SIMDs
@@ -399,7 +438,6 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     constexpr int kValues = kDepth ? 10 : 9;
     constexpr int kChannels = kRgba ? 4 : 3;
     __shared__ StagedGaussian s_g[kBlock];
-    __shared__ float4 s_rgb[kBlock];   // w: depth of the gaussian (kDepth)
     __shared__ int s_id[kBlock];
     // one row per value; the odd row stride puts the (up to ten) lanes of one LDS atomic instruction,
     // which address the same gaussian in consecutive rows, into different banks
@@ -469,14 +507,13 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const int g = idx_sorted[src];
             if ((unsigned)g < (unsigned)items) {
                 s_id[tid] = g;
-                bits = stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &s_g[tid]);
-                s_rgb[tid] = make_float4(rgb_g[3 * g], rgb_g[3 * g + 1], rgb_g[3 * g + 2], kDepth ? depths[g] : 0.0f);
+                bits = stage_gaussian(P, g, uvs, conic_opacity, rgb_g, kDepth ? depths : nullptr, tile_x0, tile_y0,
+                                      &s_g[tid]);
             } else {
                 // a corrupt index list must not become a wild read or write: the slot is staged as a gaussian
                 // nobody visits (bits = 0) with finite parameters, and id -1 keeps the flush away from it
                 s_id[tid] = -1;
-                s_g[tid] = StagedGaussian{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-                s_rgb[tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                s_g[tid] = StagedGaussian{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
         publish_masks(bits, wave, lane, s_mask);
@@ -491,8 +528,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
           while (m) {
             const int j = chunk * 64 + __builtin_ctzll(m);
             m &= m - 1;
-            const StagedGaussian sg = s_g[j];
-            const float4 c = s_rgb[j];
+            const StagedGaussian& sg = staged_at(s_g, j);
             const float dx = sg.x - pxf, dy = sg.y - pyf;
             const float power = blend_power(sg, dx, dy);
             // Per-lane conditions as 64-bit lane masks (one compare instruction each, combined with scalar
@@ -519,23 +555,23 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float one_m = 1.0f - alpha;
             const float w = alpha * T;
             T = T * one_m;
-            rr0 = __builtin_fmaf(-w, c.x, rr0);
-            rr1 = __builtin_fmaf(-w, c.y, rr1);
-            rr2 = __builtin_fmaf(-w, c.z, rr2);
+            rr0 = __builtin_fmaf(-w, sg.r, rr0);
+            rr1 = __builtin_fmaf(-w, sg.g, rr1);
+            rr2 = __builtin_fmaf(-w, sg.b, rr2);
             float dl = dT_term;
             float g9 = 0.0f;
             if constexpr (kDepth) {  // render.py:1887-1890, 1948-1950
-                rdep = __builtin_fmaf(-w, c.w, rdep);
-                dl = __builtin_fmaf(ddep, __builtin_fmaf(T, c.w, -rdep), dl);
+                rdep = __builtin_fmaf(-w, sg.depth, rdep);
+                dl = __builtin_fmaf(ddep, __builtin_fmaf(T, sg.depth, -rdep), dl);
                 g9 = w * ddep;       // render.py:1964-1967
             }
             if constexpr (kRgba) {   // the alpha channel blends the constant 1 (render.py:1871-1874, 1926-1931)
                 rr3 = rr3 - w;
                 dl = __builtin_fmaf(dr3, T - rr3, dl);
             }
-            dl = __builtin_fmaf(dr2, __builtin_fmaf(T, c.z, -rr2), dl);
-            dl = __builtin_fmaf(dr1, __builtin_fmaf(T, c.y, -rr1), dl);
-            dl = __builtin_fmaf(dr0, __builtin_fmaf(T, c.x, -rr0), dl);
+            dl = __builtin_fmaf(dr2, __builtin_fmaf(T, sg.b, -rr2), dl);
+            dl = __builtin_fmaf(dr1, __builtin_fmaf(T, sg.g, -rr1), dl);
+            dl = __builtin_fmaf(dr0, __builtin_fmaf(T, sg.r, -rr0), dl);
             // 1 - alpha lies in [0.01, 1): the hardware reciprocal (1 ulp) replaces the 11-instruction IEEE
             // division; the quotient scales every term of this pixel alike, by at most 2 ulp
             const float dL_dalpha = dl * __builtin_amdgcn_rcpf(one_m);
@@ -555,7 +591,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float g7 = w * dr1;
             const float g8 = w * dr2;
             // the wave totals land in different lanes: one LDS atomic instruction adds them all
-            const float total = wave_reduce10(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9);
+            const float total = wave_reduce10<kDepth>(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9);
             if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }
@@ -681,16 +717,16 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
         // this lane's gaussian
         const int li = bstart + lane;
         int gid = -1;
-        StagedGaussian sg = StagedGaussian{0.0f, 0.0f, __builtin_inff(), 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        StagedGaussian sg = StagedGaussian{0.0f, 0.0f, __builtin_inff(), 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
         if (li < len) {
             const int g = idx_sorted[r0 + li];
             if ((unsigned)g < (unsigned)items) {   // a corrupt index list must not become a wild read or write
                 gid = g;
-                stage_gaussian(P, g, uvs, conic_opacity, tile_x0, tile_y0, &sg);
-                c0 = rgb_g[3 * g];
-                c1 = rgb_g[3 * g + 1];
-                c2 = rgb_g[3 * g + 2];
+                stage_gaussian(P, g, uvs, conic_opacity, rgb_g, nullptr, tile_x0, tile_y0, &sg);
+                c0 = sg.r;
+                c1 = sg.g;
+                c2 = sg.b;
             }
         }
         __builtin_amdgcn_wave_barrier();    // the wavefront's own LDS writes above are read below
