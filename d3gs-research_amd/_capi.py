@@ -21,6 +21,7 @@ BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
 BUCKET_SIZE = 64          # D3GS_BUCKET_SIZE
 ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
 COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP = -1, -2
+MAX_PAIRS = (1 << 31) - 1024     # D3GS_MAX_PAIRS
 SCAN_NOALLOC_MAX_N = 1 << 24   # D3GS_SCAN_NOALLOC_MAX_N
 
 

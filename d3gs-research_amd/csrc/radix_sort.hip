@@ -19,9 +19,9 @@
 // contiguous segments.
 //
 // Look-back protocol: a workgroup's tile is its id, and workgroups are dispatched in
-// id order, so a workgroup only ever waits on tiles that started before it.  A status word carries a
-// 30-bit count and two flag bits (aggregate of this tile / inclusive prefix up
-// to this tile); words are read and written with relaxed device-scope atomics.
+// id order, so a workgroup only ever waits on tiles that started before it.  A status word is 0 (not
+// published), bit 30 + this tile's count of the digit (at most kOsTile), or bit 31 + the 31-bit inclusive
+// prefix up to this tile; words are read and written with relaxed device-scope atomics.
 // Polling is bounded: past the limit the workgroup raises an error flag and
 // stops waiting, so the grid always drains.
 #include "device_math.h"
@@ -45,9 +45,10 @@ static inline int os_digit_bits(int begin_bit, int end_bit) {
         if ((bits + d - 1) / d == fewest) return d;
     return 9;
 }
-constexpr uint32_t kFlagAggregate = 1u << 30;
-constexpr uint32_t kFlagPrefix = 2u << 30;
-constexpr uint32_t kValueMask = (1u << 30) - 1u;
+constexpr uint32_t kFlagAggregate = 1u << 30;               // + a tile's own count, below 2^30
+constexpr uint32_t kFlagPrefix = 1u << 31;                  // + an inclusive prefix, below 2^31
+constexpr uint32_t kAggregateMask = kFlagAggregate - 1u, kPrefixMask = kFlagPrefix - 1u;
+constexpr long long kOsMaxPairs = D3GS_MAX_PAIRS;           // positions and counts stay inside 31 bits
 constexpr int kSpinLimit = 1 << 22;
 // predecessor tiles polled per look-back step: 4 measured faster than 8, 16, 32 or 64 (0.121 -> 0.112 ms on 6M
 // pairs, 0.075 -> 0.071 ms on 1M keys): the polls of a step are issued by every digit's thread, and what a wider
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
     constexpr int kOsThreads = os_threads<kBits>(), kOsWaves = kOsThreads / 64, kOsItems = kOsTile / kOsThreads;
     static_assert(kRadix <= kOsThreads && kRadix <= kOsMaxRadix, "one thread owns one digit");
     __shared__ int wave_cnt[kOsWaves][kRadix];  // running, then exclusive-over-waves, per-wave digit counts
-    __shared__ int digit_out[kRadix];  // global position of tile-local sorted index 0, per digit (m < 2^30)
+    __shared__ int digit_out[kRadix];  // global position of tile-local sorted index 0, per digit (m < 2^31)
     __shared__ Key s_keys[kOsTile];
     __shared__ uint16_t s_src[kOsTile];  // tile-local input index of the pair at each sorted position
     __shared__ int s_scan[kOsWaves];
@@ -233,15 +234,14 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
 #pragma unroll
                 for (int i = 0; i < kLookWindow; ++i) {
                     if (consumed != kLookWindow) continue;
-                    const uint32_t flag = s[i] & ~kValueMask;
-                    if (flag == 0u) {
+                    if (s[i] == 0u) {
                         consumed = i;  // not published yet: poll again from this tile
+                    } else if (s[i] & kFlagPrefix) {
+                        prev += s[i] & kPrefixMask;
+                        finished = true;
+                        consumed = i + 1;
                     } else {
-                        prev += s[i] & kValueMask;
-                        if (flag == kFlagPrefix) {
-                            finished = true;
-                            consumed = i + 1;
-                        }
+                        prev += s[i] & kAggregateMask;
                     }
                 }
                 t -= consumed;
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
                 }
             }
         }
-        __hip_atomic_store(my_status, kFlagPrefix | ((prev + total) & kValueMask), __ATOMIC_RELAXED,
+        __hip_atomic_store(my_status, kFlagPrefix | ((prev + total) & kPrefixMask), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
         digit_out[tid] = excl_global + (int)prev - excl_local;
         int running = excl_local;
@@ -373,7 +373,7 @@ static int sort_pairs_impl(const char* who, int key_bits, Key* keys_a, Key* keys
         set_error("%s: bad argument (m=%lld bits=[%d,%d))", who, (long long)m, begin_bit, end_bit);
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    if (m >= (1ll << 30)) { set_error("%s: m >= 2^30 is not supported", who); return D3GS_ERR_UNSUPPORTED; }
+    if (m > kOsMaxPairs) { set_error("%s: more than 2^31 - 1024 pairs are not supported", who); return D3GS_ERR_UNSUPPORTED; }
     *result_in_b_host = 0;
     if (m == 0 || begin_bit == end_bit) return D3GS_OK;
     if (!keys_a || !keys_b || !vals_a || !vals_b || !workspace) {

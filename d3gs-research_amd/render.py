@@ -217,8 +217,8 @@ class GaussianSplatOp:
             # and -1 out of the per-pixel gradient terms and applies them once per gaussian -- the same gradient up
             # to rounding; the blend backward here applies the conic factors once per tile and gaussian in any
             # case, and taking the opacity out as well measured no gain; use_int64_tile_touched (render.py:657-660)
-            # widens the tile counters for views beyond 2^31 pairs, while this build stops at 2^30 pairs per
-            # camera with an error
+            # widens the tile counters, while the reference's sort takes an int count all the same; this build
+            # keeps 31-bit list positions and raises beyond 2^31 - 1024 pairs per call
         }
         bad = [k for k, v in unsupported.items() if v]
         if bad:
@@ -783,8 +783,12 @@ class GaussianSplatOp:
             raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
         if not fused:
             _check_sort_status(0, "depth order")
+        if num_rendered > _capi.MAX_PAIRS:
+            raise RuntimeError(f"GaussianSplatOp: {num_rendered} (tile, gaussian) pairs in one call; list positions are "
+                               f"31-bit, at most {_capi.MAX_PAIRS} pairs (render fewer cameras per bundle, or use a "
+                               "tighter early_filter_algo)")
         self.last_num_rendered = num_rendered
-        self._pair_capacity = num_rendered + num_rendered // 4 + 4096
+        self._pair_capacity = min(num_rendered + num_rendered // 4 + 4096, _capi.MAX_PAIRS)
         if num_rendered == 0:
             return _empty_result()
         if ctx is None or num_rendered > capacity:

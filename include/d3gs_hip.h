@@ -44,6 +44,10 @@ extern "C" {
  * the count when a kernel's bounded wait on an earlier workgroup ran out; the lists are then not valid. */
 #define D3GS_COUNT_SCAN_GAVE_UP (-1)
 #define D3GS_COUNT_SORT_GAVE_UP (-2)
+/* Most (tile, gaussian) pairs of one call: list positions are 31-bit (int32 offsets, tile ranges and sort
+ * prefixes, like the reference's, whose CUB sort takes an int count, devsort.py:96-129).  A sort of more is
+ * refused with D3GS_ERR_UNSUPPORTED; the scans still return the true int64 total, so a caller sees it. */
+#define D3GS_MAX_PAIRS ((1ll << 31) - 1024)
 
 /* EarlyFilterAlgo, d3sim/algos/d3gs/config_def.py:59-70 */
 #define D3GS_FILTER_NONE 0
@@ -231,7 +235,7 @@ int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t* index, int
  * (devsort.py:38-129; call site render.py:846-887).  Stable LSD radix sort of
  * (uint64 key, int32 value) pairs on key bits [begin_bit, end_bit), ping-ponging
  * between the a and b buffers.  *result_in_b_host (host int) tells which pair of
- * buffers holds the result, like the reference's (key_swap, value_swap). */
+ * buffers holds the result, like the reference's (key_swap, value_swap).  m <= D3GS_MAX_PAIRS. */
 int d3gs_sort_workspace_bytes(int64_t m, int begin_bit, int end_bit, size_t* bytes_out_host);
 int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
                     size_t workspace_bytes, int64_t m, int begin_bit, int end_bit, int* result_in_b_host,

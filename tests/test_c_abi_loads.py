@@ -70,7 +70,7 @@ def test_error_codes_without_compute():
     assert L.d3gs_sort_workspace_bytes(1000, 0, 65, C.byref(n)) == -1
     assert L.d3gs_sort_workspace_bytes(1000, 0, 45, C.byref(n)) == 0 and n.value > 0
     in_b = C.c_int(7)
-    assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 1 << 30, 0, 45, C.byref(in_b), None) == -2   # unsupported size
+    assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 1 << 31, 0, 45, C.byref(in_b), None) == -2   # unsupported size
     assert L.d3gs_sort_pairs(None, None, None, None, None, 0, 0, 0, 45, C.byref(in_b), None) == 0 and in_b.value == 0
 
 
