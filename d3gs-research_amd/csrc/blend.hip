@@ -503,7 +503,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         __syncthreads();  // previous round's flush has read s_grad / s_id
         const int src = r0 + round * kBlock + tid;
         uint32_t bits = 0;
-        if (src < r1) {
+        if (src < r1 && round * kBlock + tid < block_todo) {    // entries behind the tile's last contributor: not staged
             const int g = idx_sorted[src];
             if ((unsigned)g < (unsigned)items) {
                 s_id[tid] = g;
