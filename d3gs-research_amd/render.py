@@ -398,8 +398,10 @@ class GaussianSplatOp:
         self._check_model(model)
         if custom_features is not None:
             assert not self.is_nchw, "custom feat don't support nchw, set use_nchw=False in config."   # render.py:246
+            # one row per (camera, gaussian), camera by camera (render.py:245)
             assert custom_features.is_cuda and custom_features.dtype == torch.float32 and custom_features.ndim == 2 \
-                and custom_features.shape[0] == len(model), "custom_features must be a float32 cuda tensor [N, F]"
+                and custom_features.shape[0] == batch * len(model) and custom_features.is_contiguous(), \
+                "custom_features must be a contiguous float32 cuda tensor [B * N, F]"
         if mask is not None:
             # True rejects the gaussian (render.py:306-308); one entry per (camera, gaussian)
             assert mask.is_cuda and mask.dtype in (torch.bool, torch.uint8) and mask.numel() == batch * len(model) \
@@ -810,13 +812,11 @@ class GaussianSplatOp:
     def _bundle_in_one_pass(self, batch, instance2world_T, custom_features) -> bool:
         """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
         does (render.py:314-326, 787, 809, 1515-1522), unless it uses an option whose host code here is written
-        per camera: instance poses, custom feature channels, disable_builtin_rgb, the 32-bit sort (whose 14 tile
-        bits a bundle soon outgrows), or the fused single-stream preprocess.  Those bundles are rendered camera by
-        camera (_forward_bundle)."""
+        per camera: instance poses, the 32-bit sort (whose 14 tile bits a bundle soon outgrows), sparse mode, or
+        the fused single-stream preprocess.  Those bundles are rendered camera by camera (_forward_bundle)."""
         c = self._cfg
-        return bool(self.bundle_in_one_pass and batch > 1 and instance2world_T is None and custom_features is None
-                    and not c.disable_builtin_rgb and not c.enable_32bit_sort and self.overlap_sh_colors
-                    and not c.sparse_mode)
+        return bool(self.bundle_in_one_pass and batch > 1 and instance2world_T is None
+                    and not c.enable_32bit_sort and self.overlap_sh_colors and not c.sparse_mode)
 
     def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
                         prep_user_inputs):
@@ -828,10 +828,13 @@ class GaussianSplatOp:
         if mask is not None:
             assert mask.numel() == B * n, "mask must have one entry per (camera, gaussian)"
             mask = mask.reshape(B, n)
+        if custom_features is not None:      # one row per (camera, gaussian) (render.py:245)
+            assert custom_features.ndim == 2 and custom_features.shape[0] == B * n, "custom_features must be [B * N, F]"
         outs, ctxs, cams, rendered = [], [], [], 0
         for b in range(B):
             cam_b = cameras.select(b)
-            out_b, ctx_b = self.forward(model, cam_b, training, instance2world_T, custom_features,
+            out_b, ctx_b = self.forward(model, cam_b, training, instance2world_T,
+                                        None if custom_features is None else custom_features[b * n:(b + 1) * n],
                                         None if mask is None else mask[b].contiguous(), prep_user_inputs)
             outs.append(out_b)
             ctxs.append(ctx_b)
@@ -900,33 +903,33 @@ class GaussianSplatOp:
     def _blend_custom_features(self, P, ctx, out, feat):
         L, s = self._lib, self._stream()
         Q = self._feature_params(P)
-        H, W = out.T.shape[1], out.T.shape[2]
-        res = torch.empty((1, H, W, feat.shape[1]), dtype=torch.float32, device=feat.device)
+        B, H, W = out.T.shape        # a bundle in one pass: B images, feature rows of the B * N render items
+        res = torch.empty((B, H, W, feat.shape[1]), dtype=torch.float32, device=feat.device)
         T2, nc2 = torch.empty_like(out.T), torch.empty_like(out.n_contrib)
         for k, w, tri in self._feature_triples(feat.detach()):
-            img = torch.empty((H, W, 3), dtype=torch.float32, device=feat.device)
+            img = torch.empty((B, H, W, 3), dtype=torch.float32, device=feat.device)
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
                 _capi.ptr(ctx.conic_opacity), _capi.ptr(tri), None, _capi.ptr(ctx.tile_order), _capi.ptr(img),
                 _capi.ptr(T2), _capi.ptr(nc2), None, None, 0, s), "d3gs_blend_fwd (custom features)")
-            res[0, :, :, k:k + w] = img[:, :, :w]
+            res[..., k:k + w] = img[..., :w]
         return res
 
     def _backward_custom_features(self, P, ctx, out, dfeat_img, rec, touched=None):
-        """Adds the feature channels' share to rec[:, 0:6] and returns dcustom_features [N, F]; gaussians that
-        receive anything are marked in ``touched`` as in the colour pass."""
+        """Adds the feature channels' share to rec[:, 0:6] and returns dcustom_features, one row per render item
+        like the features; gaussians that receive anything are marked in ``touched`` as in the colour pass."""
         L, s = self._lib, self._stream()
         Q = self._feature_params(P)
         feat = ctx.custom_features.detach()
         n, F = feat.shape
-        H, W = out.T.shape[1], out.T.shape[2]
+        B, H, W = out.T.shape
         dfeat = torch.empty((n, F), dtype=torch.float32, device=feat.device)
         zero_dT = torch.zeros_like(out.T)
         for k, w, tri in self._feature_triples(feat):
-            img = torch.zeros((H, W, 3), dtype=torch.float32, device=feat.device)
-            img[:, :, :w] = out.custom_features[0, :, :, k:k + w]
-            dimg = torch.zeros((H, W, 3), dtype=torch.float32, device=feat.device)
-            dimg[:, :, :w] = dfeat_img[0, :, :, k:k + w]
+            img = torch.zeros((B, H, W, 3), dtype=torch.float32, device=feat.device)
+            img[..., :w] = out.custom_features[..., k:k + w]
+            dimg = torch.zeros((B, H, W, 3), dtype=torch.float32, device=feat.device)
+            dimg[..., :w] = dfeat_img[..., k:k + w]
             rec_k = torch.zeros_like(rec)
             _capi.check(L.d3gs_blend_bwd(
                 C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
@@ -1128,11 +1131,13 @@ def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
     """Per-camera backward passes; the model gradients add up over the cameras, duv stays per camera."""
     if op._cfg.sparse_mode:
         return _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad)
-    total, duvs, dcustom = None, [], None
+    total, duvs, dcfs = None, [], []
     n = len(model)
     for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
         if ctx_b is None:       # nothing was rendered for this camera: zero gradient
             duvs.append(torch.zeros((1, n, 2), dtype=torch.float32, device=model.xyz.device))
+            if out.custom_features is not None:
+                dcfs.append(torch.zeros((n, out.custom_features.shape[-1]), dtype=torch.float32, device=model.xyz.device))
             continue
         g_b = GaussianSplatGradients(
             drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
@@ -1141,7 +1146,7 @@ def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
         gm, duv, dcf = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True)
         duvs.append(duv)
         if dcf is not None:
-            dcustom = dcf if dcustom is None else dcustom + dcf
+            dcfs.append(dcf)
         if total is None:
             total = gm
         else:
@@ -1152,7 +1157,8 @@ def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
     if total is None:
         zeros = {k: torch.zeros_like(v) for k, v in model.get_proxy_field_dict().items()}
         total = dataclasses.replace(model, **zeros)
-    return total, (torch.cat(duvs, 0) if return_uv_grad else None), dcustom
+    # feature gradients: rows of camera 0, then camera 1, ..., like the features themselves
+    return total, (torch.cat(duvs, 0) if return_uv_grad else None), (torch.cat(dcfs, 0) if dcfs else None)
 
 
 class _RasterizeGaussians(torch.autograd.Function):

@@ -151,3 +151,51 @@ def test_bundle_through_autograd_entry_point():
     assert duv is not None and tuple(duv.shape) == (len(cams), scene.n, 2) and float(duv.abs().max()) > 0
     for k in g_single:
         assert float((g_bundle[k] - g_single[k]).abs().max()) <= 1e-4 * float(g_single[k].abs().max()), k
+
+
+@pytest.mark.parametrize("one_pass,no_rgb", [(True, False), (False, False), (True, True)])
+def test_bundle_with_custom_features(one_pass, no_rgb):
+    """Custom feature channels of a bundle have one row per (camera, gaussian), camera by camera (render.py:245),
+    and so has their gradient; disable_builtin_rgb leaves the alpha channel as the colour image.  In one pass and
+    camera by camera, against single-camera renders of each camera's rows."""
+    import torch
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(250, 190))
+    cams = _cameras(scene)
+    B, n, F = len(cams), scene.n, 5
+    op = GaussianSplatOp(op_config(scene, 4, disable_builtin_rgb=no_rgb, render_rgba=no_rgb))
+    op.bundle_in_one_pass = one_pass
+    model = torch_model(scene)
+    bundle = CameraBundle.from_pinhole_cams(cams)
+    rng = np.random.default_rng(21)
+    feat = torch.from_numpy(rng.standard_normal((B * n, F)).astype(np.float32)).cuda()
+    out, ctx = op.forward(model, bundle, training=True, custom_features=feat)
+    assert tuple(out.custom_features.shape) == (B, scene.height, scene.width, F)
+    assert tuple(out.color.shape) == (B, scene.height, scene.width, 1 if no_rgb else 3)
+    drgb = torch.from_numpy(rng.standard_normal(out.color.shape).astype(np.float32)).cuda()
+    dT = torch.from_numpy(rng.standard_normal(out.T.shape).astype(np.float32)).cuda()
+    dfi = torch.from_numpy(rng.standard_normal(out.custom_features.shape).astype(np.float32)).cuda()
+    gm, duv, dcf = op.backward(model, bundle, ctx, out,
+                               GaussianSplatGradients(drgb=drgb, dT=dT, dcustom_features=dfi), return_uv_grad=True)
+    assert tuple(dcf.shape) == (B * n, F) and tuple(duv.shape) == (B, n, 2)
+    want = {k: torch.zeros_like(v, dtype=torch.float64) for k, v in model.get_proxy_field_dict().items()}
+    for b, cam in enumerate(cams):
+        rows = slice(b * n, (b + 1) * n)
+        o1, c1 = op.forward(model, cam, training=True, custom_features=feat[rows].contiguous())
+        assert torch.equal(o1.color[0], out.color[b]) and torch.equal(o1.T[0], out.T[b])
+        assert torch.equal(o1.custom_features[0], out.custom_features[b])
+        g1 = GaussianSplatGradients(drgb=drgb[b:b + 1].contiguous(), dT=dT[b:b + 1].contiguous(),
+                                    dcustom_features=dfi[b:b + 1].contiguous())
+        gm1, duv1, dcf1 = op.backward(model, cam, c1, o1, g1, return_uv_grad=True)
+        # two runs of the same backward add their float32 terms in different orders
+        assert float((dcf1 - dcf[rows]).abs().max()) <= 1e-4 * float(dcf1.abs().max())
+        assert float((duv1[0] - duv[b]).abs().max()) <= 1e-4 * float(duv1.abs().max())
+        for k in want:
+            want[k] += getattr(gm1, k).double()
+    for k, w in want.items():
+        err = (getattr(gm, k).double() - w).abs().reshape(-1)
+        top = float(w.abs().max())
+        if no_rgb and k == "color_sh":
+            assert top == 0.0 and float(err.max()) == 0.0      # no SH colours: no gradient reaches the coefficients
+            continue
+        assert float(torch.quantile(err, 0.999)) <= 1e-4 * top and float(err.max()) <= 1e-3 * top, k
