@@ -73,15 +73,15 @@ __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src
 // world-to-camera rotation (row major) followed by the camera centre; the others keep the view's camera.
 struct InstanceView {
     const int32_t* ids;     // [N], may be NULL
-    const float* cameras;   // [count][12]
+    const float* cameras;   // [count][12]; for a bundle of B cameras B such tables, camera by camera
     int count;
 };
 
-__device__ __forceinline__ void apply_instance(d3gs_params& P, const InstanceView& inst, int i) {
+__device__ __forceinline__ void apply_instance(d3gs_params& P, const InstanceView& inst, int i, int batch = 0) {
     if (!inst.ids) return;
     const int id = inst.ids[i];
     if (id >= 0 && id < inst.count) {
-        const float* m = inst.cameras + 12 * (size_t)id;
+        const float* m = inst.cameras + 12 * ((size_t)batch * inst.count + id);
 #pragma unroll
         for (int k = 0; k < 9; ++k) P.w2c[k] = m[k];
 #pragma unroll
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
             g = i - batch * P0.n;
             apply_batch_camera(P, batch);
         }
-        if (inst.ids) apply_instance(P, inst, g);
+        if (inst.ids) apply_instance(P, inst, g, batch);
     }
 
     bool valid = true;
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
         d3gs_params P = P0;
         if constexpr (kInstances) {
             if (P0.batch_size > 1) apply_batch_camera(P, batch);
-            if (inst.ids) apply_instance(P, inst, g);
+            if (inst.ids) apply_instance(P, inst, g, batch);
         }
         float rgb[3] = {0.0f, 0.0f, 0.0f};
         uint32_t ne0 = 0;
@@ -880,9 +880,8 @@ extern "C" int d3gs_preprocess_fwd(const d3gs_params* p, const float* xyz, const
     InstanceView inst;
     if (!instance_view(instances, &inst, "d3gs_preprocess_fwd")) return D3GS_ERR_INVALID_ARGUMENT;
     const bool bundle = p->batch_size > 1;
-    if (bundle && (with_sh || inst.ids)) {
-        set_error("d3gs_preprocess_fwd: a camera bundle takes its colours from d3gs_sh_colors (rgb_gaussian = NULL) "
-                  "and no instance table");
+    if (bundle && with_sh) {
+        set_error("d3gs_preprocess_fwd: a camera bundle takes its colours from d3gs_sh_colors (rgb_gaussian = NULL)");
         return D3GS_ERR_UNSUPPORTED;
     }
     dim3 grid((item_count(*p) + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
@@ -967,10 +966,6 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
     }
     InstanceView inst;
     if (!instance_view(instances, &inst, "d3gs_sh_colors")) return D3GS_ERR_INVALID_ARGUMENT;
-    if (p->batch_size > 1 && inst.ids) {
-        set_error("d3gs_sh_colors: a camera bundle takes no instance table");
-        return D3GS_ERR_UNSUPPORTED;
-    }
     const int chunks = ((p->n + kPrepBlock - 1) / kPrepBlock) * batch_count(*p);
     dim3 grid(chunks < kShColorBlocks ? chunks : kShColorBlocks), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);

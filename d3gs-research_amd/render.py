@@ -284,7 +284,8 @@ class GaussianSplatOp:
         cam2instance = world2instance o cam2world per gaussian inside its kernels; here it is done once per
         instance, in float64 on the device, and the kernels read a [I, 12] float32 table: the world-to-camera
         rotation in the instance frame (row major) and the camera centre in the instance frame.
-        Returns ``(instance_ids int32 [N], instance_cameras float32 [I, 12])``."""
+        Returns ``(instance_ids int32 [N], instance_cameras float32 [I, 12])``; for a bundle of B > 1 cameras
+        the table has B * I rows, the I rows of camera 0 first (each camera with the poses of its own frame)."""
         assert model.instance_id is not None, "instance_id must be provided in model when render with instance"
         T = instance2world_T
         if T.ndim == 4:      # [num_frame, num_instance, 4, 3]
@@ -297,21 +298,40 @@ class GaussianSplatOp:
         assert T.ndim == 3 and tuple(T.shape[1:]) == (4, 3), \
             "instance2world_T must be [num_frame, num_instance, 4, 3] (or [num_instance, 4, 3] for one frame)"
         dev = model.xyz.device
+        ids = model.instance_id.detach().to(device=dev, dtype=torch.int32).contiguous()
+        assert ids.numel() == len(model), "instance_id must hold one id per gaussian"
+        if isinstance(cameras, CameraBundle) and len(cameras) > 1:
+            Tall = instance2world_T
+            if Tall.ndim == 4:
+                assert cameras.frame_ids is not None, "frame_ids must be provided when render with instance"
+                Tall = Tall[cameras.frame_ids.to(device=Tall.device, dtype=torch.long)]      # [B, I, 4, 3]
+            else:
+                Tall = Tall.unsqueeze(0).expand(len(cameras), -1, -1, -1)
+            assert Tall.ndim == 4 and tuple(Tall.shape[2:]) == (4, 3), "instance2world_T must be [num_frame, num_instance, 4, 3]"
+            Tall = Tall.detach().to(device=dev, dtype=torch.float64)
+            cw = cameras.cam2world_T.detach().to(device=dev, dtype=torch.float32).reshape(-1, 4, 3).to(torch.float64)
+            rot_T = Tall[:, :, :3, :]                                              # [B, I, 3, 3]
+            w2c = cw[:, None, :3, :] @ rot_T.transpose(2, 3)
+            centre = rot_T @ (cw[:, None, 3, :] - Tall[:, :, 3, :]).unsqueeze(-1)
+            table = torch.cat([w2c.reshape(-1, 9), centre.reshape(-1, 3)], 1).to(torch.float32).contiguous()
+            return ids, table
         T = T.detach().to(device=dev, dtype=torch.float64)
         cw = torch.from_numpy(self._camera_arrays(cameras)[2].astype(np.float64)).to(dev)
         rot_T = T[:, :3, :]                                   # R_i^T: world -> instance
         w2c = cw[:3] @ rot_T.transpose(1, 2)                  # R_c^T R_i
         centre = rot_T @ (cw[3] - T[:, 3, :]).unsqueeze(-1)   # R_i^T (c - t_i)
         table = torch.cat([w2c.reshape(-1, 9), centre.reshape(-1, 3)], 1).to(torch.float32).contiguous()
-        ids = model.instance_id.detach().to(device=dev, dtype=torch.int32).contiguous()
-        assert ids.numel() == len(model), "instance_id must hold one id per gaussian"
         return ids, table
 
     @staticmethod
-    def _instances_arg(ids, table):
+    def _instances_arg(ids, table, batch=1, camera=None):
+        """The kernels' instance argument; `table` holds `batch` tables one after the other, of which `camera`
+        selects one (the preprocess backward runs camera by camera)."""
         if table is None:
             return None
-        return C.byref(_capi.Instances(ids.data_ptr(), table.data_ptr(), int(table.shape[0])))
+        count = int(table.shape[0]) // batch
+        first = 0 if camera is None else camera * count
+        return C.byref(_capi.Instances(ids.data_ptr(), table.data_ptr() + 48 * first, count))
 
     @staticmethod
     def batch_table(cameras: "CameraBundle", device) -> torch.Tensor:
@@ -415,7 +435,7 @@ class GaussianSplatOp:
         inst_ids = inst_cams = None
         if instance2world_T is not None:
             inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
-        inst = self._instances_arg(inst_ids, inst_cams)
+        inst = self._instances_arg(inst_ids, inst_cams, batch)
         # n: render items = gaussians x cameras (item b * N + g is gaussian g seen by camera b); everything the
         # preprocess writes has one row per item, the tile ids carry the camera
         n = P.n * batch
@@ -812,11 +832,11 @@ class GaussianSplatOp:
     def _bundle_in_one_pass(self, batch, instance2world_T, custom_features) -> bool:
         """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
         does (render.py:314-326, 787, 809, 1515-1522), unless it uses an option whose host code here is written
-        per camera: instance poses, the 32-bit sort (whose 14 tile bits a bundle soon outgrows), sparse mode, or
-        the fused single-stream preprocess.  Those bundles are rendered camera by camera (_forward_bundle)."""
+        per camera: the 32-bit sort (whose 14 tile bits a bundle soon outgrows), sparse mode, or the fused
+        single-stream preprocess.  Those bundles are rendered camera by camera (_forward_bundle)."""
         c = self._cfg
-        return bool(self.bundle_in_one_pass and batch > 1 and instance2world_T is None
-                    and not c.enable_32bit_sort and self.overlap_sh_colors and not c.sparse_mode)
+        return bool(self.bundle_in_one_pass and batch > 1 and not c.enable_32bit_sort and self.overlap_sh_colors
+                    and not c.sparse_mode)
 
     def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
                         prep_user_inputs):
@@ -1058,7 +1078,6 @@ class GaussianSplatOp:
             inst_ids, inst_cams = ctx.instance_ids, ctx.instance_cameras
             if inst_cams is None and instance2world_T is not None:
                 inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
-            inst = self._instances_arg(inst_ids, inst_cams)
             # One launch per camera (the reference loops over the batch inside its kernel, render.py:2972-2989):
             # camera b works on its own rows of the per-item arrays, the first call stores, the others add.
             if sparse_ids is not None:
@@ -1072,6 +1091,7 @@ class GaussianSplatOp:
                     "d3gs_preprocess_bwd_sparse")
             rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
             for b in range(B if sparse_ids is None else 0):
+                inst = self._instances_arg(inst_ids, inst_cams, B, b)      # the instance poses as camera b sees them
                 _capi.check(L.d3gs_preprocess_bwd_camera(
                     C.byref(P), b, int(b > 0), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),
                     _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh),

@@ -137,7 +137,9 @@ int d3gs_depth_key_bits(const d3gs_params* p);
  * camera.  Passed by pointer to K1, the SH colours and K9; NULL, or instance_ids == NULL, means no instances. */
 typedef struct d3gs_instances {
     const int32_t* instance_ids;     /* [N] device */
-    const float* instance_cameras;   /* [num_instances][12] device */
+    const float* instance_cameras;   /* [num_instances][12] device; with d3gs_params.batch_size = B > 1 one such
+                                      * table per camera, [B][num_instances][12] (d3gs_preprocess_bwd_camera takes
+                                      * the table of its camera alone) */
     int32_t num_instances;
 } d3gs_instances;
 
@@ -391,7 +393,8 @@ int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* qua
  * array (radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched) points at that camera's n rows.  accumulate != 0
  * adds to the six gradient arrays instead of storing (gaussians without work are left alone): the gradient of a
  * bundle is B calls, the first storing (or adding to cleared arrays), the others accumulating.  With
- * batch_size <= 1, batch_index 0 and accumulate 0 this is d3gs_preprocess_bwd. */
+ * batch_size <= 1, batch_index 0 and accumulate 0 this is d3gs_preprocess_bwd.  `instances` is the table of this
+ * camera alone ([num_instances][12], the batch_index-th of the B tables K1 was given). */
 int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,
                                const float* quaternion_xyzw, const float* scale, const float* opacity,
                                const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
