@@ -67,6 +67,24 @@ def committed_traffic_bytes(stage, config_id):
     return None
 
 
+def committed_valu_instructions(stage, config_id):
+    """Vector-ALU wave instructions per launch of `stage`'s kernel from the committed rocprofv3 --pmc summary
+    (SQ_INSTS_VALU), or None when none is committed for this configuration."""
+    kernel = {"blend_fwd": "blend_fwd_kernel", "blend_bwd": "blend_bwd_kernel", "preprocess": "preprocess_fwd_kernel",
+              "preprocess_bwd": "preprocess_bwd_kernel", "make_keys": "make_keys_kernel"}.get(stage)
+    path = os.path.join(ROOT, "profiles", f"config{config_id}_blend_valu_issue.txt")
+    if kernel is None or not os.path.exists(path):
+        return None
+    for line in open(path):
+        f = line.split()
+        if len(f) == 10 and f[0] == kernel:
+            try:
+                return float(f[2])
+            except ValueError:
+                return None
+    return None
+
+
 def hbm_copy_probe(torch, nbytes=1 << 30, reps=10):
     """GB/s (bytes read + bytes written) of a 1 GiB device-to-device copy, HIP events, best of `reps`."""
     src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
@@ -241,6 +259,15 @@ def main():
                 "pair_evals_per_s": round(256.0 * M / (stages[dom]["ms"] * 1e-3), 1),
                 # what a plain device-to-device copy reaches on this box (read + written bytes per second)
                 "measured_copy_gbs": copy_gbs, "frac_of_measured_copy": round(achieved / copy_gbs, 5)}
+    # The blend kernels are bound by vector-instruction issue, not by HBM: next to the HBM fraction asked for, the
+    # rate at which the dominant kernel retires vector instructions (count from the committed counter summary, time
+    # from this run) against 256 CUs x 4 SIMDs x 2.4 GHz / 4 cycles per wave64 instruction.  Plain FP32 operations
+    # issue in half that time on this chip, so the ratio can exceed 1; its ceiling for this kernel's mix is about 1.3.
+    valu = committed_valu_instructions(dom, args.config)
+    if valu is not None:
+        rate = valu / (stages[dom]["ms"] * 1e-3)
+        roofline["valu"] = {"wave_instructions_per_launch": valu, "per_s": round(rate, 1),
+                            "vs_4_cycle_issue": round(rate / (256 * 4 * 2.4e9 / 4), 3)}
     # tile list lengths of the last view (the blend kernels' work is their sum and their skew)
     _, last_ctx = op.forward(model, cam, training=True)
     lens = (last_ctx.workload_ranges[:, 1] - last_ctx.workload_ranges[:, 0]).to(torch.float64)
