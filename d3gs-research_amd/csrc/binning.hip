@@ -662,10 +662,6 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
     if (p->n == 0 || m == 0) return D3GS_OK;
-    if (p->batch_size > 1 && p->enable_32bit_sort) {
-        set_error("d3gs_make_keys: a camera bundle with enable_32bit_sort is not supported");
-        return D3GS_ERR_UNSUPPORTED;
-    }
     if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
         !gaussian_idx) {
         set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");

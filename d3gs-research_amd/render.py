@@ -385,7 +385,7 @@ class GaussianSplatOp:
         P.use_nchw, P.enable_anti_aliasing = int(c.use_nchw), int(c.enable_anti_aliasing)
         P.enable_32bit_sort, P.depth_32bit_prec = int(c.enable_32bit_sort), float(c.depth_32bit_prec)
         if c.enable_32bit_sort:
-            assert P.tiles_x * P.tiles_y < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
+            assert P.tiles_x * P.tiles_y * max(P.batch_size, 1) < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
         return P
 
     @staticmethod
@@ -410,7 +410,7 @@ class GaussianSplatOp:
         """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
         assert model.act_applied, "model must be activated before render"
         batch = len(cameras) if isinstance(cameras, CameraBundle) else 1
-        if batch != 1 and not self._bundle_in_one_pass(batch, instance2world_T, custom_features):
+        if batch != 1 and not self._bundle_in_one_pass(batch, cameras):
             return self._forward_bundle(model, cameras, training, instance2world_T, custom_features, mask,
                                         prep_user_inputs)
         if prep_user_inputs:
@@ -829,14 +829,19 @@ class GaussianSplatOp:
             ctx = None
         return out, ctx
 
-    def _bundle_in_one_pass(self, batch, instance2world_T, custom_features) -> bool:
+    def _bundle_in_one_pass(self, batch, cameras) -> bool:
         """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
         does (render.py:314-326, 787, 809, 1515-1522), unless it uses an option whose host code here is written
-        per camera: the 32-bit sort (whose 14 tile bits a bundle soon outgrows), sparse mode, or the fused
-        single-stream preprocess.  Those bundles are rendered camera by camera (_forward_bundle)."""
+        per camera (sparse mode, the fused single-stream preprocess), or the 32-bit sort when the bundle's tiles
+        outgrow its 14 tile bits (the reference asserts there, render.py:227-228).  Those bundles are rendered camera
+        by camera (_forward_bundle)."""
         c = self._cfg
-        return bool(self.bundle_in_one_pass and batch > 1 and not c.enable_32bit_sort and self.overlap_sh_colors
-                    and not c.sparse_mode)
+        if not (self.bundle_in_one_pass and batch > 1 and self.overlap_sh_colors and not c.sparse_mode):
+            return False
+        if c.enable_32bit_sort:
+            width, height = cameras.image_shape_wh
+            return batch * div_up(width, 16) * div_up(height, 16) < 2 ** 14
+        return True
 
     def _forward_bundle(self, model, cameras: "CameraBundle", training, instance2world_T, custom_features, mask,
                         prep_user_inputs):

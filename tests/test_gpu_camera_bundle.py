@@ -25,16 +25,19 @@ def _cameras(scene):
 
 # one_pass: the bundle goes through the kernels as B * N render items with the camera in the tile id (the
 # reference's way, render.py:314-326, 787, 809); otherwise camera by camera (the fallback some options take)
-@pytest.mark.parametrize("depth,one_pass,nchw", [(False, True, False), (True, True, False), (False, False, False),
-                                                 (True, False, False), (True, True, True)])
-def test_bundle_equals_single_cameras(oracle, depth, one_pass, nchw):
+@pytest.mark.parametrize("depth,one_pass,nchw,sort32", [(False, True, False, False), (True, True, False, False),
+                                                        (False, False, False, False), (True, False, False, False),
+                                                        (True, True, True, False), (False, True, False, True)])
+def test_bundle_equals_single_cameras(oracle, depth, one_pass, nchw, sort32):
     import torch
     from d3gs_research_amd.render import (CameraBundle, GaussianSplatGradients, GaussianSplatOp,
                                           GaussianSplatOpBatchContext, GaussianSplatOpContext)
     scene = gen_scene(1, n=20000, wh=(250, 190))
     cams = _cameras(scene)
     B, n = len(cams), scene.n
-    op = GaussianSplatOp(op_config(scene, 4, render_depth=depth, use_nchw=nchw, render_rgba=nchw))
+    # sort32: the lighter sort key, 14 bits of tile over 18 bits of depth steps; 3 x 192 tiles fit its tile bits
+    op = GaussianSplatOp(op_config(scene, 4, render_depth=depth, use_nchw=nchw, render_rgba=nchw,
+                                   enable_32bit_sort=sort32, depth_32bit_prec=0.01))
     op.bundle_in_one_pass = one_pass
     model = torch_model(scene)
     bundle = CameraBundle.from_pinhole_cams(cams)
@@ -77,7 +80,7 @@ def test_bundle_equals_single_cameras(oracle, depth, one_pass, nchw):
             # gaussian ids by b * N (render item ids), ranges by the pairs of the cameras before
             m_b = op.last_num_rendered
             seg = slice(pairs_before, pairs_before + m_b)
-            assert torch.equal(bundle_keys[seg], op._last_keys_sorted + ((b * tiles) << 32))
+            assert torch.equal(bundle_keys[seg], op._last_keys_sorted + ((b * tiles) << (18 if sort32 else 32)))
             assert torch.equal(bundle_idx[seg], c1.gaussian_idx_sorted + b * n)
             r1 = c1.workload_ranges
             want_r = torch.where((r1[:, 1] > r1[:, 0]).unsqueeze(1), r1 + pairs_before, torch.zeros_like(r1))
@@ -105,7 +108,7 @@ def test_bundle_equals_single_cameras(oracle, depth, one_pass, nchw):
 
     # one oracle check of the second camera, so that the per-camera parameters are known to be that camera's
     cam = cams[1]
-    P = oracle_params(oracle, scene, 4)
+    P = oracle_params(oracle, scene, 4, enable_32bit_sort=sort32, depth_32bit_prec=0.01)
     P.fx, P.fy, P.cx, P.cy = [float(v) for v in (*cam.focal_length, *cam.principal_point)]
     P.tan_fovx = float(np.float32(0.5) * np.float32(scene.width) / np.float32(P.fx))
     P.tan_fovy = float(np.float32(0.5) * np.float32(scene.height) / np.float32(P.fy))
