@@ -196,7 +196,7 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
         // The pair sort's kernels (7- and 8-bit digits, many rounds of tiles) form the rank here, one register per
         // key: left alone the compiler keeps the masked ballot (two registers) and `before` alive instead and
         // counts the bits after the look-back, 114 registers instead of 84, which costs a wavefront per SIMD.  The
-        // depth sort's (9 bits, one round of tiles, bound by latency) is better off with the count deferred.
+        // depth sort's (9 bits, one round of tiles, bound by latency) gains nothing from it.
         if constexpr (kBits < 9) asm volatile("" : "+v"(rank[k]));
     }
     __syncthreads();
