@@ -41,9 +41,15 @@ __device__ __forceinline__ float det_expf(float x) {
     return __builtin_ldexpf(e, (int)kf);
 }
 
-// Same, for arguments already known to lie in [-86, 88] and not NaN.
+// exp of the blend kernels: arguments known to lie in [-80, 80] and not NaN (a power that passed the cull
+// threshold).  The same polynomial as det_expf with a cheaper range reduction, fixed like the rest of the
+// sequence: k = round(x log2 e) comes out of one fused multiply-add with 1.5 * 2^23 (the sum's low mantissa bits
+// are k), the reduced argument uses t - 1.5 * 2^23 = k, and 2^k is applied by adding k to the exponent field
+// (the result stays normal in this range).  Two full-rate operations and an integer add in place of a multiply, a
+// round, a convert and an ldexp, which issue at half rate.
 __device__ __forceinline__ float det_expf_inrange(float x) {
-    float kf = __builtin_rintf(x * 1.44269504088896341f);
+    const float t = __builtin_fmaf(x, 1.44269504088896341f, 12582912.0f);
+    const float kf = t - 12582912.0f;
     float r = __builtin_fmaf(kf, -0.693359375f, x);
     r = __builtin_fmaf(kf, 2.12194440e-4f, r);
     float z = r * r;
@@ -54,7 +60,7 @@ __device__ __forceinline__ float det_expf_inrange(float x) {
     p = __builtin_fmaf(p, r, 1.6666665459e-1f);
     p = __builtin_fmaf(p, r, 5.0000001201e-1f);
     float e = __builtin_fmaf(p, z, r) + 1.0f;
-    return __builtin_ldexpf(e, (int)kf);
+    return __uint_as_float(__float_as_uint(e) + (__float_as_uint(t) << 23));
 }
 
 __device__ __forceinline__ float det_logf(float x) {

@@ -20,6 +20,7 @@
 // Pinning status (what independent evidence checks each function; see
 // tests/test_oracle_*.py):
 //   orc_expf / orc_logf          : against float64 libm, <= 1.5 ulp
+//   orc_expf_blend               : the same, over the range the blend evaluates it in
 //   orc_preprocess_fwd           : float64 closed forms (pinhole, R S S^T R^T via
 //                                  scipy Rotation, EWA J W S W^T J^T, 2x2 inverse,
 //                                  eigen radius), SH against a float64 restatement
@@ -103,6 +104,27 @@ ORC_API float orc_expf(float x) {
     if (x < -86.0f) return 0.0f;
     if (x > 88.0f) return INFINITY;
     float kf = rintf(x * 1.44269504088896341f);
+    float r = fmaf(kf, -0.693359375f, x);
+    r = fmaf(kf, 2.12194440e-4f, r);
+    float z = r * r;
+    float p = 1.9875691500e-4f;
+    p = fmaf(p, r, 1.3981999507e-3f);
+    p = fmaf(p, r, 8.3334519073e-3f);
+    p = fmaf(p, r, 4.1665795894e-2f);
+    p = fmaf(p, r, 1.6666665459e-1f);
+    p = fmaf(p, r, 5.0000001201e-1f);
+    float e = fmaf(p, z, r) + 1.0f;
+    return ldexpf(e, (int)kf);
+}
+
+// exp as the blend kernels evaluate it (device_math.h: det_expf_inrange): orc_expf's polynomial with a range
+// reduction that costs the GPU less -- k from one fused multiply-add with 1.5 * 2^23 instead of a multiply and
+// a round (the two differ only where x log2 e is within a rounding of a half-integer, and then by which of two
+// equally good k is taken).  Below -80, where the kernels never evaluate it, the plain function.
+ORC_API float orc_expf_blend(float x) {
+    if (!(x == x) || x < -80.0f || x > 80.0f) return orc_expf(x);
+    const float t = fmaf(x, 1.44269504088896341f, 12582912.0f);
+    const float kf = t - 12582912.0f;
     float r = fmaf(kf, -0.693359375f, x);
     r = fmaf(kf, 2.12194440e-4f, r);
     float z = r * r;
@@ -661,7 +683,7 @@ ORC_API void orc_blend_fwd(const orc_params* P, const int32_t* ranges, const int
                     float dx = uvs[2 * g] - pxf, dy = uvs[2 * g + 1] - pyf;
                     const float* co = conic_opacity + 4 * g;
                     float power = blend_power(co, dx, dy);
-                    float G = orc_expf(power);
+                    float G = orc_expf_blend(power);
                     float alpha = fminf(0.99f, co[3] * G);
                     if (alpha < P->alpha_eps) continue;
                     float nextT = T * (1.0f - alpha);
@@ -750,7 +772,7 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     float dx = uvs[2 * g] - pxf, dy = uvs[2 * g + 1] - pyf;
                     const float* co = conic_opacity + 4 * g;
                     float power = blend_power(co, dx, dy);
-                    float G = orc_expf(power);
+                    float G = orc_expf_blend(power);
                     float alpha = fminf(0.99f, co[3] * G);
                     bool valid = power <= 0.0f && alpha >= P->alpha_eps;
                     if (!valid) continue;

@@ -55,6 +55,8 @@ def lib():
         _lib = C.CDLL(_LIB_PATH)
         _lib.orc_expf.restype = C.c_float
         _lib.orc_expf.argtypes = [C.c_float]
+        _lib.orc_expf_blend.restype = C.c_float
+        _lib.orc_expf_blend.argtypes = [C.c_float]
         _lib.orc_logf.restype = C.c_float
         _lib.orc_logf.argtypes = [C.c_float]
         _lib.orc_scan.restype = C.c_int64
@@ -120,6 +122,12 @@ def params_for_scene(scene, filter_algo, training=True, **over) -> OracleParams:
 def expf(x):
     L = lib()
     return np.array([L.orc_expf(float(v)) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
+def expf_blend(x):
+    """exp as the blend evaluates it (orc_expf_blend)."""
+    L = lib()
+    return np.array([L.orc_expf_blend(float(v)) for v in np.asarray(x, np.float32).ravel()], np.float32)
 
 
 def logf(x):

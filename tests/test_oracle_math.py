@@ -20,6 +20,21 @@ def test_expf_within_1p5_ulp(oracle):
     assert oracle.expf([0.0])[0] == 1.0
 
 
+def test_blend_expf_within_1p5_ulp(oracle):
+    """The blend's exp takes its k = round(x log2 e) from one fused multiply-add with 1.5 * 2^23: same accuracy
+    bound as the plain function over the range it is evaluated in, the same value wherever both pick the same k."""
+    rng = np.random.default_rng(2)
+    x = np.concatenate([np.linspace(-79.9, 79.9, 20001), rng.uniform(-6, 0, 40000), [0.0, -0.0, -1e-8,
+                        # half-integers of x log2 e, where the two range reductions may pick different k
+                        *(np.float32((k + 0.5) / 1.44269504088896341) for k in range(-9, 2))]]).astype(np.float32)
+    got = oracle.expf_blend(x)
+    assert _ulp_err(got, np.exp(x.astype(np.float64))).max() <= 1.5
+    plain = oracle.expf(x)
+    assert (got == plain).mean() > 0.999 and oracle.expf_blend([0.0])[0] == 1.0
+    # outside the range the kernels evaluate it in: the plain function
+    assert oracle.expf_blend([-86.5])[0] == 0.0 and np.isnan(oracle.expf_blend([np.nan])[0])
+
+
 def test_logf_within_1p5_ulp(oracle):
     rng = np.random.default_rng(1)
     x = np.concatenate([np.exp(rng.uniform(-80, 80, 20000)), rng.uniform(1 / 300, 1.0, 20000), [1.0, 0.5, 2.0]]).astype(np.float32)
