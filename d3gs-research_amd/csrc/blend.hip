@@ -147,13 +147,24 @@ __device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, flo
     }
     // v3: v0 v1 | v2 v3 by (bit 3, bit 2) of the lane; v7: v4 .. v7 likewise; v9: v8 | v9 by bit 3
     // 64 -> 32: rows 0,1 keep the first register, rows 2,3 the second
-    const float e0 = swap_add32(v3, v7), e1 = swap_add32(v9, 0.0f);
+    // (v9's partner only feeds rows 2 and 3 of e1, which end in row 3 of the result, where no slot lives: any
+    // register does, and an unset one costs no move)
+    float unset;
+    asm volatile("" : "=v"(unset));
+    const float e0 = swap_add32(v3, v7), e1 = swap_add32(v9, unset);
     // 32 -> 16: rows 0,2 keep e0, rows 1,3 keep e1
     float y = swap_add16(e0, e1);
-    // 4 -> 1 inside each quad
-    y = y + dpp_f<0x4E>(y);
-    y = y + dpp_f<0xB1>(y);
-    return y;
+    // 4 -> 1 inside each quad: two DPP adds (written out: the compiler forms a zero "old" operand for the second
+    // one and splits it into a move, a DPP move and an add); a DPP read needs two wait states after the vector
+    // write of its source
+    float total;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"
+        : "=&v"(total)
+        : "v"(y));
+    return total;
 }
 
 __device__ __forceinline__ int wave_max_i32(int v) {
