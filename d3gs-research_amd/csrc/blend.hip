@@ -93,10 +93,14 @@ __device__ __forceinline__ int reduce_slot(int lane) {
     return -1;
 }
 
-// kTen = false: v9 is the constant zero and the one instruction that only moves it is left out.
+// kTen = false: there is no tenth value.  Its slot's lanes (bit 3 of the lane set, in the register that carries
+// v8) only ever combine with each other and end in a lane whose slot nobody reads, so they need no defined
+// content: the register starts unset (no move to form a zero) and the instruction that would add the tenth
+// value's halves is left out.
 template <bool kTen>
 __device__ __forceinline__ float wave_reduce10(float v0, float v1, float v2, float v3, float v4, float v5, float v6,
                                                float v7, float v8, float v9) {
+    if constexpr (!kTen) asm volatile("" : "=v"(v9));
     // 16 -> 8 and 8 -> 4 inside each row of 16 lanes, while the most registers are live, with DPP adds whose
     // bank mask writes only one half of the lanes: "b += b[partner]" on the lanes that keep b, then
     // "b = a + a[partner]" on the lanes that keep a, merges a pair of registers in two instructions and no
