@@ -258,7 +258,7 @@ __device__ __forceinline__ unsigned long long uniform_u64(unsigned long long v) 
 }
 
 // Predicate codes of __builtin_amdgcn_fcmpf / __builtin_amdgcn_sicmp (LLVM's CmpInst::Predicate).
-constexpr int kFcmpOge = 3, kFcmpOle = 5, kIcmpSlt = 40;
+constexpr int kFcmpOgt = 2, kFcmpOge = 3, kFcmpOlt = 4, kFcmpOle = 5, kIcmpSlt = 40;
 
 // a = mask ? a0 : 0 and b = mask ? b0 : 0 for a lane mask held in a scalar register pair.  The compiler has no
 // cheap way from a 64-bit integer back to a per-lane predicate, hence the instruction is written out; the
@@ -269,6 +269,24 @@ __device__ __forceinline__ void select2_or_zero(unsigned long long mask, float a
         "v_cndmask_b32_e64 %1, 0, %3, %4"
         : "=&v"(a), "=&v"(b)
         : "v"(a0), "v"(b0), "s"(mask));
+}
+
+// r = mask ? if_set : if_clear, and r = mask ? if_set : 0, for a lane mask held in a scalar register pair (the same
+// reason as above: conditions that are combined as 64-bit masks with scalar instructions come back as selects)
+__device__ __forceinline__ float select_by_mask(unsigned long long mask, float if_set, float if_clear) {
+    float r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    return r;
+}
+__device__ __forceinline__ int select_by_mask(unsigned long long mask, int if_set, int if_clear) {
+    int r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    return r;
+}
+__device__ __forceinline__ float select_or_zero(unsigned long long mask, float if_set) {
+    float r;
+    asm("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(r) : "v"(if_set), "s"(mask));
+    return r;
 }
 
 // measure_atomic_add_count: the wavefront's flush instruction issues one line-wide request per group of sixteen
@@ -383,8 +401,12 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 const StagedGaussian& sg = staged_at(s_g, j);
                 const float dx = sg.x - pxf, dy = sg.y - pyf;
                 const float power = blend_power(sg, dx, dy);
-                const bool live = power >= sg.thr;      // false for a finished pixel (NaN)
-                if (!__any(live)) continue;
+                // Per-lane conditions as 64-bit lane masks: one compare each, combined with scalar instructions
+                // and applied with selects that take the mask from a scalar pair (as booleans the compiler formed
+                // "any lane stops?" by a select into a vector register and a second compare, and both senses of
+                // the transmittance test).  Ordered compares: a NaN fails them as it fails the C operators.
+                const unsigned long long live_m = __builtin_amdgcn_fcmpf(power, sg.thr, kFcmpOge);   // a finished pixel: NaN
+                if (live_m == 0ull) continue;
                 // From here on every lane runs the same instructions and the outcome is applied with
                 // selects (w = 0 leaves the accumulators untouched): far fewer scalar mask operations
                 // than nested per-lane branches.  exp of a lane that is not live may be garbage; it is
@@ -393,24 +415,24 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 // fminf(0.99, .) gives 0.99 in every case, as it does for the guarded exp's inf
                 const float G = det_expf_inrange(power);
                 const float alpha = fminf(0.99f, sg.o * G);
-                const bool hit = live && alpha >= P.alpha_eps;
+                const unsigned long long hit_m = live_m & __builtin_amdgcn_fcmpf(alpha, P.alpha_eps, kFcmpOge);
                 const float nextT = T * (1.0f - alpha);
-                const bool should_done = nextT < P.transmittance_eps;
-                const bool stop = hit && should_done;                      // render.py:1781-1792
-                const bool use = hit && !should_done && !(power > 0.0f);
-                const float w = use ? alpha * T : 0.0f;
-                T = use ? nextT : T;
-                contributor = use ? round * kBlock + j : contributor;
+                const unsigned long long done_m = __builtin_amdgcn_fcmpf(nextT, P.transmittance_eps, kFcmpOlt);
+                const unsigned long long stop_m = hit_m & done_m;                      // render.py:1781-1792
+                const unsigned long long use_m = hit_m & ~done_m & ~__builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOgt);
+                const float w = select_or_zero(use_m, alpha * T);
+                T = select_by_mask(use_m, nextT, T);
+                contributor = select_by_mask(use_m, round * kBlock + j, contributor);
                 acc0 = __builtin_fmaf(w, sg.r, acc0);
                 acc1 = __builtin_fmaf(w, sg.g, acc1);
                 acc2 = __builtin_fmaf(w, sg.b, acc2);
                 if constexpr (kRgba) acc3 = acc3 + w;
                 if constexpr (kDepth) depth_accum = __builtin_fmaf(w, sg.depth, depth_accum);
-                pxf = stop ? __builtin_nanf("") : pxf;
+                pxf = select_by_mask(stop_m, __builtin_nanf(""), pxf);
                 // every pixel of the patch finished: both loops end at their next test (one way out of the
                 // loops keeps the scalar control flow short; the scalar unit is shared by the CU's four SIMDs
                 // and this kernel issues two scalar instructions for every three vector ones)
-                if (__any(stop) && __all(pxf != pxf)) {
+                if (stop_m != 0ull && __all(pxf != pxf)) {
                     m = 0ull;
                     chunk = 4;
                 }
