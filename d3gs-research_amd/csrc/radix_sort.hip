@@ -45,6 +45,9 @@ static inline int os_digit_bits(int begin_bit, int end_bit) {
         if ((bits + d - 1) / d == fewest) return d;
     return 9;
 }
+constexpr int kPeersAndAgree = 0x90;  // v_bitop3 truth table of a & ~(b ^ c): rows (a,b,c) = (1,0,0) and (1,1,1)
+constexpr int kIcmpSlt = 40;                                  // "signed less than"
+constexpr int kIcmpNe = 33;                                   // LLVM integer predicate "not equal", for lane-mask compares
 constexpr uint32_t kFlagAggregate = 1u << 30;               // + a tile's own count, below 2^30
 constexpr uint32_t kFlagPrefix = 1u << 31;                  // + an inclusive prefix, below 2^31
 constexpr uint32_t kAggregateMask = kFlagAggregate - 1u, kPrefixMask = kFlagPrefix - 1u;
@@ -177,16 +180,25 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
         const bool in = idx < m;
         key[k] = in ? keys_in[idx] : (Key)~(Key)0;
     }
+    // pairs of the input from this lane's first one on, as far as it matters (a tile holds fewer than 2^16)
+    const int left = (int)min(m - (tile_begin + wave_begin + lane), (long long)kOsTile);
 #pragma unroll
     for (int k = 0; k < kOsItems; ++k) {
-        const bool in = tile_begin + wave_begin + k * 64 + lane < m;
+        const bool in = k * 64 < left;
         const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
-        uint64_t peers = __ballot(in);
+        // lanes whose digit equals this lane's: per bit, the lanes that agree with this lane on it.  The bit is
+        // extracted as 0 / -1, which serves as the ballot's operand and as the mask that turns the ballot
+        // into "agrees with me" (one three-input bit operation per half).
+        const uint64_t live = __builtin_amdgcn_sicmp(k * 64, left, kIcmpSlt);
+        uint32_t peers_lo = (uint32_t)live, peers_hi = (uint32_t)(live >> 32);
 #pragma unroll
         for (int b = 0; b < kBits; ++b) {
-            const uint64_t bal = __ballot((d >> b) & 1u);
-            peers &= ((d >> b) & 1u) ? bal : ~bal;
+            const int set = __builtin_amdgcn_sbfe((int)d, b, 1);
+            const uint64_t bal = __builtin_amdgcn_sicmp(set, 0, kIcmpNe);
+            peers_lo = __builtin_amdgcn_bitop3_b32(peers_lo, (uint32_t)set, (uint32_t)bal, kPeersAndAgree);
+            peers_hi = __builtin_amdgcn_bitop3_b32(peers_hi, (uint32_t)set, (uint32_t)(bal >> 32), kPeersAndAgree);
         }
+        const uint64_t peers = ((uint64_t)peers_hi << 32) | peers_lo;
         int before = 0;
         if (in) before = wave_cnt[wave][d];
         __builtin_amdgcn_wave_barrier();
@@ -283,18 +295,35 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
         }
     }
     __syncthreads();
-    // consecutive threads write consecutive sorted positions: equal-digit runs leave as contiguous segments
+    // consecutive threads write consecutive sorted positions: equal-digit runs leave as contiguous segments.
+    // All of a thread's values are fetched before the first is stored (positions past the count read the tile's
+    // first pair instead and store nothing), so the gathers' latencies overlap instead of adding up.
     const int count = (int)min((long long)kOsTile, m - tile_begin);
+    Key sorted_key[kOsItems];
+    int32_t sorted_val[kOsItems];
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const int i = k * kOsThreads + tid;
+        const int ii = i < count ? i : 0;
+        sorted_key[k] = s_keys[ii];
+        sorted_val[k] = (int32_t)s_src[ii];
+    }
+    // without an input value array the values are the pairs' own indices
+    if (vals_in) {
+#pragma unroll
+        for (int k = 0; k < kOsItems; ++k) sorted_val[k] = vals_in[tile_begin + sorted_val[k]];
+    } else {
+#pragma unroll
+        for (int k = 0; k < kOsItems; ++k) sorted_val[k] += (int32_t)tile_begin;
+    }
 #pragma unroll
     for (int k = 0; k < kOsItems; ++k) {
         const int i = k * kOsThreads + tid;
         if (i < count) {
-            const Key kk = s_keys[i];
-            const uint32_t d = (uint32_t)(kk >> shift) & mask;
+            const uint32_t d = (uint32_t)(sorted_key[k] >> shift) & mask;
             const long long pos = (long long)digit_out[d] + i;
-            keys_out[pos] = kk;
-            // without an input value array the values are the pairs' own indices
-            vals_out[pos] = vals_in ? vals_in[tile_begin + s_src[i]] : (int32_t)(tile_begin + s_src[i]);
+            keys_out[pos] = sorted_key[k];
+            vals_out[pos] = sorted_val[k];
         }
     }
 }
