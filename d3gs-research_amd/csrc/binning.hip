@@ -327,12 +327,10 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
         const float4 co = *reinterpret_cast<const float4*>(conic_opacity + 4 * i);
         TileWalkIn g{uv.x, uv.y, (float)radii[i], co.x, co.y, co.z, co.w};
         walk = tile_walk_setup(P, g);
-        // camera b of a bundle owns the tile rows from b * tiles_y on (render.py:787, 809); the shift moves the
-        // 3-sigma rect and the candidate rect together, so the per-tile decisions are the single camera's
+        // camera b of a bundle owns the tile rows from b * tiles_y on (render.py:787, 809); the per-tile test works
+        // in candidate-rect coordinates, so moving the rect's origin leaves the single camera's decisions as they are
         const int shift = P.batch_size > 1 ? (i / P.n) * P.tiles_y : 0;
         walk.bminy += shift;
-        walk.rminy += shift;
-        walk.rmaxy += shift;
     }
     wave_tile_emit<Key>(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
 }

@@ -12,6 +12,7 @@
 #include <stdint.h>
 
 #include "../../include/d3gs_hip.h"
+#include <type_traits>
 
 namespace d3gs {
 
@@ -190,6 +191,7 @@ struct TileWalkIn {
 
 struct TileWalk {
     int rminx, rminy, rmaxx, rmaxy;  // 3-sigma tile rect
+    int lx0, ly0, lx1, ly1;          // the same rect in candidate-rect coordinates (what the per-tile test compares)
     int bminx, bminy, bw, bh;        // candidate rect (origin, size); the 3-sigma rect when no filter
     float uo, vo, bx, by;            // centre relative to the candidate rect origin, AABB half extents
     float ow, oh, os, oc;            // OBB: axis radii r1, r2 (ow, oh) and sin, cos; ELLIPSE: conic a, b, c and the bound
@@ -268,6 +270,9 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
         w.bminy = w.rminy;
         w.bw = w.rmaxx - w.rminx;
         w.bh = w.rmaxy - w.rminy;
+        w.lx0 = w.ly0 = 0;
+        w.lx1 = w.bw;
+        w.ly1 = w.bh;
         return w;
     }
     // half extents of the exact alpha >= alpha_eps ellipse (gs3d.py:710-742)
@@ -291,6 +296,10 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
     w.bh = max(bmaxy - w.bminy, 0);
     w.uo = g.u - (float)w.bminx * 16.0f;
     w.vo = g.v - (float)w.bminy * 16.0f;
+    w.lx0 = w.rminx - w.bminx;
+    w.lx1 = w.rmaxx - w.bminx;
+    w.ly0 = w.rminy - w.bminy;
+    w.ly1 = w.rmaxy - w.bminy;
     if (P.filter_algo == D3GS_FILTER_OBB || P.filter_algo == D3GS_FILTER_OBB_DFVT) {
         // oriented bounding box of the ellipse x^T Q x = 1, Q = -conic / bound (gs3d.py:761-791, 981-987)
         float eA = (-g.conic0) / bound, eC = (-g.conic2) / bound, eB = (-g.conic1) / bound;
@@ -321,41 +330,63 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
     return w;
 }
 
-// Is candidate tile (lx, ly) — coordinates relative to the candidate rect origin — kept?
-__device__ __forceinline__ bool tile_keep(const int filter_algo, const TileWalk& w, int lx, int ly) {
-    if (filter_algo == D3GS_FILTER_NONE) return true;
+// Is candidate tile (lx, ly) — coordinates relative to the candidate rect origin — kept?  The filter is a template
+// argument: the walks below run their loops once per filter instead of choosing the test anew for every tile.
+template <int kFilter>
+__device__ __forceinline__ bool tile_keep(const TileWalk& w, int lx, int ly) {
+    if constexpr (kFilter == D3GS_FILTER_NONE) return true;
     const float px0 = (float)(lx * 16), py0 = (float)(ly * 16);
-    const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
     bool keep;
-    if (filter_algo == D3GS_FILTER_AABB) {
+    if constexpr (kFilter == D3GS_FILTER_AABB) {
+        const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
         const bool xo = (w.uo - w.bx) <= px1 && (w.uo + w.bx) >= px0;
         const bool yo = (w.vo - w.by) <= py1 && (w.vo + w.by) >= py0;
         keep = xo && yo;
-    } else if (filter_algo == D3GS_FILTER_ELLIPSE) {
+    } else if constexpr (kFilter == D3GS_FILTER_ELLIPSE) {
+        const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
         keep = ellipse_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
     } else {
         const ObbAxes ax{w.ow, w.oh, w.or3, w.or4, w.os, w.oc};
         keep = obb_overlaps_tile(px0, py0, ax, w.uo, w.vo);
     }
-    const int x = lx + w.bminx, y = ly + w.bminy;
-    return keep && x >= w.rminx && x < w.rmaxx && y >= w.rminy && y < w.rmaxy;
+    return keep && lx >= w.lx0 && lx < w.lx1 && ly >= w.ly0 && ly < w.ly1;      // inside the 3-sigma rect
+}
+
+// Runs f(std::integral_constant<int, filter>) for the filter named at run time (OBB_DFVT is computed as OBB).
+template <class F>
+__device__ __forceinline__ void with_filter(const int filter_algo, F&& f) {
+    switch (filter_algo) {
+        case D3GS_FILTER_NONE: f(std::integral_constant<int, D3GS_FILTER_NONE>{}); break;
+        case D3GS_FILTER_AABB: f(std::integral_constant<int, D3GS_FILTER_AABB>{}); break;
+        case D3GS_FILTER_ELLIPSE: f(std::integral_constant<int, D3GS_FILTER_ELLIPSE>{}); break;
+        default: f(std::integral_constant<int, D3GS_FILTER_OBB>{}); break;
+    }
 }
 
 __device__ __forceinline__ int bcast_i(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
 __device__ __forceinline__ float bcast_f(float v, int src) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
 }
+template <int kFilter>
 __device__ __forceinline__ TileWalk bcast_walk(const TileWalk& w, int src) {
-    TileWalk r;
-    r.rminx = bcast_i(w.rminx, src); r.rminy = bcast_i(w.rminy, src);
-    r.rmaxx = bcast_i(w.rmaxx, src); r.rmaxy = bcast_i(w.rmaxy, src);
+    TileWalk r = {};      // (fields the filter's test does not read stay zero)
+    r.lx0 = bcast_i(w.lx0, src); r.ly0 = bcast_i(w.ly0, src);
+    r.lx1 = bcast_i(w.lx1, src); r.ly1 = bcast_i(w.ly1, src);
     r.bminx = bcast_i(w.bminx, src); r.bminy = bcast_i(w.bminy, src);
     r.bw = bcast_i(w.bw, src); r.bh = bcast_i(w.bh, src);
-    r.uo = bcast_f(w.uo, src); r.vo = bcast_f(w.vo, src);
-    r.bx = bcast_f(w.bx, src); r.by = bcast_f(w.by, src);
-    r.ow = bcast_f(w.ow, src); r.oh = bcast_f(w.oh, src);
-    r.os = bcast_f(w.os, src); r.oc = bcast_f(w.oc, src);
-    r.or3 = bcast_f(w.or3, src); r.or4 = bcast_f(w.or4, src);
+    if constexpr (kFilter != D3GS_FILTER_NONE) {
+        r.uo = bcast_f(w.uo, src); r.vo = bcast_f(w.vo, src);
+    }
+    if constexpr (kFilter == D3GS_FILTER_AABB) {
+        r.bx = bcast_f(w.bx, src); r.by = bcast_f(w.by, src);
+    }
+    if constexpr (kFilter == D3GS_FILTER_ELLIPSE || kFilter == D3GS_FILTER_OBB) {
+        r.ow = bcast_f(w.ow, src); r.oh = bcast_f(w.oh, src);
+        r.os = bcast_f(w.os, src); r.oc = bcast_f(w.oc, src);
+    }
+    if constexpr (kFilter == D3GS_FILTER_OBB) {
+        r.or3 = bcast_f(w.or3, src); r.or4 = bcast_f(w.or4, src);
+    }
     return r;
 }
 
@@ -374,12 +405,13 @@ __device__ __forceinline__ unsigned long long tile_mask_meta(const TileWalk& w, 
 // Number of kept tiles of this lane's gaussian.  Must be called by all 64 lanes of a wavefront
 // (lanes without a gaussian pass active = false).  `mask` receives the kept-tile bit mask when the
 // candidate rect has at most 64 tiles (`has_mask`).
-__device__ __forceinline__ int wave_tile_count(const int filter_algo, bool active, const TileWalk& w,
-                                               unsigned long long& mask, bool& has_mask) {
+template <int kFilter>
+__device__ __forceinline__ int wave_tile_count_with(bool active, const TileWalk& w, unsigned long long& mask,
+                                                    bool& has_mask) {
     const int area = active ? w.bw * w.bh : 0;
     has_mask = active && area <= 64 && w.bw <= 64;
     mask = 0ull;
-    if (filter_algo == D3GS_FILTER_NONE) {
+    if constexpr (kFilter == D3GS_FILTER_NONE) {
         if (has_mask) mask = area == 64 ? ~0ull : (1ull << area) - 1ull;
         return area;
     }
@@ -387,20 +419,22 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
     const bool big = area > kSmallWalk;
     const float my_inv_bw = 1.0f / (float)w.bw;
     if (!big) {
+        static_assert(kSmallWalk <= 32, "the kept tiles of a small walk are collected in one 32-bit word");
+        uint32_t kept = 0;
         int lx = 0, ly = 0;
         for (int t = 0; t < area; ++t) {
-            const bool k = tile_keep(filter_algo, w, lx, ly);
-            count += k ? 1 : 0;
-            mask |= k ? (1ull << t) : 0ull;
+            kept |= (tile_keep<kFilter>(w, lx, ly) ? 1u : 0u) << t;
             if (++lx == w.bw) { lx = 0; ++ly; }
         }
+        count = __popc(kept);
+        mask = kept;
     }
     const int lane = threadIdx.x & 63;
     unsigned long long todo = __ballot(big);
     while (todo) {
         const int src = __builtin_ctzll(todo);
         todo &= todo - 1;
-        const TileWalk ws = bcast_walk(w, src);
+        const TileWalk ws = bcast_walk<kFilter>(w, src);
         const int a = ws.bw * ws.bh;
         int c = 0;
         unsigned long long first = 0ull;
@@ -412,7 +446,7 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
             bool k = false;
             if (t < a) {
                 const int ly = (int)(((float)t + 0.5f) * inv_bw);
-                k = tile_keep(filter_algo, ws, t - ly * ws.bw, ly);
+                k = tile_keep<kFilter>(ws, t - ly * ws.bw, ly);
             }
             const unsigned long long b = __ballot(k);
             if (base == 0) first = b;
@@ -423,6 +457,15 @@ __device__ __forceinline__ int wave_tile_count(const int filter_algo, bool activ
             mask = first;   // the whole rect when it has at most 64 tiles
         }
     }
+    return count;
+}
+
+__device__ __forceinline__ int wave_tile_count(const int filter_algo, bool active, const TileWalk& w,
+                                               unsigned long long& mask, bool& has_mask) {
+    int count = 0;
+    with_filter(filter_algo, [&](auto filter) {
+        count = wave_tile_count_with<decltype(filter)::value>(active, w, mask, has_mask);
+    });
     return count;
 }
 
@@ -453,8 +496,8 @@ __device__ __forceinline__ Key make_pair_key(uint64_t tile, uint32_t depth_bits)
 }
 
 // Key: uint64_t for (tile << 32) | depth bits, uint32_t for the tile id alone.
-template <typename Key>
-__device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool active, const TileWalk& w, int tiles_x,
+template <typename Key, int kFilter>
+__device__ __forceinline__ void wave_tile_emit_with(bool active, const TileWalk& w, int tiles_x,
                                                uint32_t depth_bits, int value, long long off, long long end,
                                                Key* __restrict__ keys, int32_t* __restrict__ vals) {
     const int area = active ? w.bw * w.bh : 0;
@@ -462,7 +505,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
     if (!big) {
         int lx = 0, ly = 0;
         for (int t = 0; t < area; ++t, lx = (lx + 1 == w.bw ? 0 : lx + 1), ly += (lx == 0)) {
-            if (tile_keep(filter_algo, w, lx, ly)) {
+            if (tile_keep<kFilter>(w, lx, ly)) {
                 if (off < end) {
                     const uint64_t tile = (uint64_t)(uint32_t)((ly + w.bminy) * tiles_x + lx + w.bminx);
                     keys[off] = make_pair_key<Key>(tile, depth_bits);
@@ -479,7 +522,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
     while (todo) {
         const int src = __builtin_ctzll(todo);
         todo &= todo - 1;
-        const TileWalk ws = bcast_walk(w, src);
+        const TileWalk ws = bcast_walk<kFilter>(w, src);
         const uint32_t dbits = (uint32_t)bcast_i((int)depth_bits, src);
         const int val = bcast_i(value, src);
         long long o = ((long long)bcast_i((int)(off >> 32), src) << 32) | (uint32_t)bcast_i((int)off, src);
@@ -493,7 +536,7 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
             if (t < a) {
                 ly = (int)(((float)t + 0.5f) * inv_bw);
                 lx = t - ly * ws.bw;
-                k = tile_keep(filter_algo, ws, lx, ly);
+                k = tile_keep<kFilter>(ws, lx, ly);
             }
             const unsigned long long b = __ballot(k);
             if (k) {
@@ -507,6 +550,15 @@ __device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool activ
             o += __popcll(b);
         }
     }
+}
+
+template <typename Key>
+__device__ __forceinline__ void wave_tile_emit(const int filter_algo, bool active, const TileWalk& w, int tiles_x,
+                                               uint32_t depth_bits, int value, long long off, long long end,
+                                               Key* __restrict__ keys, int32_t* __restrict__ vals) {
+    with_filter(filter_algo, [&](auto filter) {
+        wave_tile_emit_with<Key, decltype(filter)::value>(active, w, tiles_x, depth_bits, value, off, end, keys, vals);
+    });
 }
 
 constexpr float kShC0 = 0.28209479177387814f;
