@@ -218,11 +218,10 @@ __device__ __forceinline__ ObbAxes obb_axes(float w, float h, float s, float c) 
 }
 __device__ __forceinline__ bool obb_overlaps_tile(float bx0, float by0, const ObbAxes& a, float cu, float cv) {
     const float lx = (bx0 + 8.0f) - cu, ly = (by0 + 8.0f) - cv;   // (bx1 + bx0) / 2 is exactly bx0 + 8
-    if (a.r1 <= fabsf(lx)) return false;
-    if (a.r2 <= fabsf(ly)) return false;
-    if (a.r3 <= fabsf(lx * a.c + ly * a.s)) return false;
-    if (a.r4 <= fabsf(lx * (-a.s) + ly * a.c)) return false;
-    return true;
+    // all four axes, no early way out: in a wavefront some lane nearly always needs every one of them
+    const bool s1 = a.r1 <= fabsf(lx), s2 = a.r2 <= fabsf(ly);
+    const bool s3 = a.r3 <= fabsf(lx * a.c + ly * a.s), s4 = a.r4 <= fabsf(lx * (-a.s) + ly * a.c);
+    return !(s1 | s2 | s3 | s4);
 }
 
 // Where the level set {conic form = -bound} crosses a horizontal (axis = 1) or vertical (axis = 0)
@@ -333,23 +332,43 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
 // Is candidate tile (lx, ly) — coordinates relative to the candidate rect origin — kept?  The filter is a template
 // argument: the walks below run their loops once per filter instead of choosing the test anew for every tile.
 template <int kFilter>
-__device__ __forceinline__ bool tile_keep(const TileWalk& w, int lx, int ly) {
+__device__ __forceinline__ bool tile_test(const TileWalk& w, float px0, float py0) {
     if constexpr (kFilter == D3GS_FILTER_NONE) return true;
-    const float px0 = (float)(lx * 16), py0 = (float)(ly * 16);
-    bool keep;
     if constexpr (kFilter == D3GS_FILTER_AABB) {
         const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
         const bool xo = (w.uo - w.bx) <= px1 && (w.uo + w.bx) >= px0;
         const bool yo = (w.vo - w.by) <= py1 && (w.vo + w.by) >= py0;
-        keep = xo && yo;
+        return xo && yo;
     } else if constexpr (kFilter == D3GS_FILTER_ELLIPSE) {
         const float px1 = px0 + 16.0f, py1 = py0 + 16.0f;
-        keep = ellipse_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
+        return ellipse_overlaps_box(px0, py0, px1, py1, w.ow, w.oh, w.os, w.oc, w.uo, w.vo);
     } else {
         const ObbAxes ax{w.ow, w.oh, w.or3, w.or4, w.os, w.oc};
-        keep = obb_overlaps_tile(px0, py0, ax, w.uo, w.vo);
+        return obb_overlaps_tile(px0, py0, ax, w.uo, w.vo);
     }
+}
+template <int kFilter>
+__device__ __forceinline__ bool tile_keep(const TileWalk& w, int lx, int ly) {
+    const bool keep = tile_test<kFilter>(w, (float)(lx * 16), (float)(ly * 16));
     return keep && lx >= w.lx0 && lx < w.lx1 && ly >= w.ly0 && ly < w.ly1;      // inside the 3-sigma rect
+}
+
+// A lane's walk over its own small candidate rect, row by row: calls visit(kept) once per candidate tile.  The
+// tile's pixel origin is stepped as a float (multiples of 16, exact), and the 3-sigma rect is compared in the
+// same units, so the loop carries no integer coordinates and converts nothing.
+template <int kFilter, class Visit>
+__device__ __forceinline__ void small_walk(const TileWalk& w, int area, Visit&& visit) {
+    const float x_end = (float)(w.bw * 16);
+    const float fx0 = (float)(w.lx0 * 16), fx1 = (float)(w.lx1 * 16);
+    const float fy0 = (float)(w.ly0 * 16), fy1 = (float)(w.ly1 * 16);
+    float px0 = 0.0f, py0 = 0.0f;
+    for (int t = 0; t < area; ++t) {
+        visit(t, px0, py0, tile_test<kFilter>(w, px0, py0) && px0 >= fx0 && px0 < fx1 && py0 >= fy0 && py0 < fy1);
+        px0 += 16.0f;
+        const bool wrap = px0 == x_end;
+        px0 = wrap ? 0.0f : px0;
+        py0 += wrap ? 16.0f : 0.0f;
+    }
 }
 
 // Runs f(std::integral_constant<int, filter>) for the filter named at run time (OBB_DFVT is computed as OBB).
@@ -421,11 +440,7 @@ __device__ __forceinline__ int wave_tile_count_with(bool active, const TileWalk&
     if (!big) {
         static_assert(kSmallWalk <= 32, "the kept tiles of a small walk are collected in one 32-bit word");
         uint32_t kept = 0;
-        int lx = 0, ly = 0;
-        for (int t = 0; t < area; ++t) {
-            kept |= (tile_keep<kFilter>(w, lx, ly) ? 1u : 0u) << t;
-            if (++lx == w.bw) { lx = 0; ++ly; }
-        }
+        small_walk<kFilter>(w, area, [&](int t, float, float, bool k) { kept |= (k ? 1u : 0u) << t; });
         count = __popc(kept);
         mask = kept;
     }
@@ -503,17 +518,17 @@ __device__ __forceinline__ void wave_tile_emit_with(bool active, const TileWalk&
     const int area = active ? w.bw * w.bh : 0;
     const bool big = area > kSmallWalk;
     if (!big) {
-        int lx = 0, ly = 0;
-        for (int t = 0; t < area; ++t, lx = (lx + 1 == w.bw ? 0 : lx + 1), ly += (lx == 0)) {
-            if (tile_keep<kFilter>(w, lx, ly)) {
+        small_walk<kFilter>(w, area, [&](int, float px0, float py0, bool k) {
+            if (k) {
                 if (off < end) {
+                    const int lx = (int)px0 >> 4, ly = (int)py0 >> 4;
                     const uint64_t tile = (uint64_t)(uint32_t)((ly + w.bminy) * tiles_x + lx + w.bminx);
                     keys[off] = make_pair_key<Key>(tile, depth_bits);
                     vals[off] = value;
                 }
                 ++off;
             }
-        }
+        });
     }
     const int lane = threadIdx.x & 63;
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
