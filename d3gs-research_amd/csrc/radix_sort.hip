@@ -229,6 +229,52 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
     // where each digit starts in the whole output, and inside this tile
     const int excl_global = os_block_excl_scan<kOsWaves>(owner ? (int)hist[tid] : 0, s_scan);
     const int excl_local = os_block_excl_scan<kOsWaves>((int)total, s_scan);
+    if (owner) {    // where each wavefront's keys of the digit start inside the tile
+        int running = excl_local;
+#pragma unroll
+        for (int w = 0; w < kOsWaves; ++w) {
+            wave_cnt[w][tid] = running;
+            running += c[w];
+        }
+    }
+    __syncthreads();
+
+    // Place every pair at its tile-local sorted position, read the sorted keys back and request the values: none
+    // of this needs the earlier tiles, so the values' round trip through memory runs while the look-back below
+    // makes its own.
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const int local = wave_begin + k * 64 + lane;
+        if (tile_begin + local < m) {
+            const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
+            const int pos = wave_cnt[wave][d] + rank[k];
+            s_keys[pos] = key[k];
+            s_src[pos] = (uint16_t)local;
+        }
+    }
+    __syncthreads();
+    // consecutive threads take consecutive sorted positions: equal-digit runs leave as contiguous segments.
+    // All of a thread's values are fetched before the first is stored (positions past the count read the tile's
+    // first pair instead and store nothing), so the gathers' latencies overlap instead of adding up.
+    const int count = (int)min((long long)kOsTile, m - tile_begin);
+    Key sorted_key[kOsItems];
+    int32_t sorted_val[kOsItems];
+#pragma unroll
+    for (int k = 0; k < kOsItems; ++k) {
+        const int i = k * kOsThreads + tid;
+        const int ii = i < count ? i : 0;
+        sorted_key[k] = s_keys[ii];
+        sorted_val[k] = (int32_t)s_src[ii];
+    }
+    // without an input value array the values are the pairs' own indices
+    if (vals_in) {
+#pragma unroll
+        for (int k = 0; k < kOsItems; ++k) sorted_val[k] = vals_in[tile_begin + sorted_val[k]];
+    } else {
+#pragma unroll
+        for (int k = 0; k < kOsItems; ++k) sorted_val[k] += (int32_t)tile_begin;
+    }
+
     if (owner) {
         // digits of earlier tiles: walk back until a tile that already knows its inclusive prefix.
         // kLookWindow predecessors are polled per step with independent loads, so the serial depth of
@@ -274,48 +320,8 @@ __global__ __launch_bounds__(os_threads<kBits>()) void os_pass_kernel(const Key*
         __hip_atomic_store(my_status, kFlagPrefix | ((prev + total) & kPrefixMask), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
         digit_out[tid] = excl_global + (int)prev - excl_local;
-        int running = excl_local;
-#pragma unroll
-        for (int w = 0; w < kOsWaves; ++w) {
-            wave_cnt[w][tid] = running;
-            running += c[w];
-        }
     }
     __syncthreads();
-
-    // place every pair at its tile-local sorted position
-#pragma unroll
-    for (int k = 0; k < kOsItems; ++k) {
-        const int local = wave_begin + k * 64 + lane;
-        if (tile_begin + local < m) {
-            const uint32_t d = (uint32_t)(key[k] >> shift) & mask;
-            const int pos = wave_cnt[wave][d] + rank[k];
-            s_keys[pos] = key[k];
-            s_src[pos] = (uint16_t)local;
-        }
-    }
-    __syncthreads();
-    // consecutive threads write consecutive sorted positions: equal-digit runs leave as contiguous segments.
-    // All of a thread's values are fetched before the first is stored (positions past the count read the tile's
-    // first pair instead and store nothing), so the gathers' latencies overlap instead of adding up.
-    const int count = (int)min((long long)kOsTile, m - tile_begin);
-    Key sorted_key[kOsItems];
-    int32_t sorted_val[kOsItems];
-#pragma unroll
-    for (int k = 0; k < kOsItems; ++k) {
-        const int i = k * kOsThreads + tid;
-        const int ii = i < count ? i : 0;
-        sorted_key[k] = s_keys[ii];
-        sorted_val[k] = (int32_t)s_src[ii];
-    }
-    // without an input value array the values are the pairs' own indices
-    if (vals_in) {
-#pragma unroll
-        for (int k = 0; k < kOsItems; ++k) sorted_val[k] = vals_in[tile_begin + sorted_val[k]];
-    } else {
-#pragma unroll
-        for (int k = 0; k < kOsItems; ++k) sorted_val[k] += (int32_t)tile_begin;
-    }
 #pragma unroll
     for (int k = 0; k < kOsItems; ++k) {
         const int i = k * kOsThreads + tid;
