@@ -119,8 +119,27 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __rest
             atomicAdd(&mine[p * kRadix + ((uint32_t)(key >> bit) & ((1u << nb) - 1u))], 1u);
         }
     };
-    // four independent loads in flight per thread: with one, a workgroup per CU waits a memory round trip per key
+    // Independent loads in flight per thread: with one, a workgroup per CU waits a memory round trip per key.  The
+    // body of the input goes in 16-byte loads, two in flight (the bytes a CU has under way set its rate here);
+    // the last few keys, and an input that is not 16-byte aligned, go one key at a time, four in flight.
     long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x;
+    if constexpr (sizeof(Key) == 4) {
+        if ((reinterpret_cast<uintptr_t>(keys) & 15u) == 0) {
+            const uint4* quads = reinterpret_cast<const uint4*>(keys);
+            const long long nq = m / 4;
+            long long q = i;
+            for (; q + stride < nq; q += 2 * stride) {
+                const uint4 a = quads[q], b = quads[q + stride];
+                count(a.x); count(a.y); count(a.z); count(a.w);
+                count(b.x); count(b.y); count(b.z); count(b.w);
+            }
+            for (; q < nq; q += stride) {
+                const uint4 a = quads[q];
+                count(a.x); count(a.y); count(a.z); count(a.w);
+            }
+            i += nq * 4;      // the up to three keys behind the last whole quad
+        }
+    }
     for (; i + 3 * stride < m; i += 4 * stride) {
         const Key k0 = keys[i], k1 = keys[i + stride], k2 = keys[i + 2 * stride], k3 = keys[i + 3 * stride];
         count(k0);
