@@ -408,7 +408,8 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
 // thread keeps its tiles' lengths in registers and takes its place inside a bucket from the counting atomic's
 // return value, so the lists are read once and every tile costs one LDS atomic).  Order inside a bucket is
 // arbitrary: the result only steers scheduling.
-constexpr int kOrderThreads = 1024, kOrderBuckets = 1024, kOrderPerThread = 8;
+constexpr int kOrderThreads = 1024, kOrderBuckets = 1024;
+constexpr int kOrderPerThread = 8, kOrderPerThreadLarge = 32;    // 8 192 tiles (1080p has 8 160), 32 768 (4K has 32 400)
 
 __device__ __forceinline__ int order_wave_max(int v) {
 #pragma unroll
@@ -438,6 +439,7 @@ __device__ __forceinline__ void fold_sort_errors(const BinStatus& st) {
 
 __global__ void bin_status_kernel(BinStatus st) { fold_sort_errors(st); }
 
+template <int kPerThread>
 __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t* __restrict__ work, int num_tiles,
                                                                    int32_t* __restrict__ order, BinStatus st) {
     if (threadIdx.x == 0) fold_sort_errors(st);
@@ -448,13 +450,13 @@ __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t
     const int2* ranges = reinterpret_cast<const int2*>(work);
     auto amount_of = [&](int t) { const int2 r = ranges[t]; return max(r.y - r.x, 0); };
     auto bucket_of = [&](int a, float scale) { return kOrderBuckets - 1 - min(kOrderBuckets - 1, (int)((float)a * scale)); };
-    const bool in_registers = num_tiles <= kOrderThreads * kOrderPerThread;   // else the lists are read three times
+    const bool in_registers = num_tiles <= kOrderThreads * kPerThread;   // else the lists are read three times
 
-    int amount[kOrderPerThread];
+    int amount[kPerThread];
     int mx = 0;
     if (in_registers) {
 #pragma unroll
-        for (int k = 0; k < kOrderPerThread; ++k) {
+        for (int k = 0; k < kPerThread; ++k) {
             const int t = k * kOrderThreads + tid;
             amount[k] = t < num_tiles ? amount_of(t) : 0;
             mx = max(mx, amount[k]);
@@ -471,10 +473,10 @@ __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t
     for (int w = 0; w < kOrderThreads / 64; ++w) mx = max(mx, s_max[w]);
     const float scale = (float)kOrderBuckets / ((float)mx + 1.0f);
 
-    int bucket[kOrderPerThread], rank[kOrderPerThread];
+    int bucket[kPerThread], rank[kPerThread];
     if (in_registers) {
 #pragma unroll
-        for (int k = 0; k < kOrderPerThread; ++k) {
+        for (int k = 0; k < kPerThread; ++k) {
             bucket[k] = bucket_of(amount[k], scale);
             rank[k] = (k * kOrderThreads + tid < num_tiles) ? atomicAdd(&s_bin[bucket[k]], 1) : 0;
         }
@@ -498,7 +500,7 @@ __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t
     __syncthreads();
     if (in_registers) {
 #pragma unroll
-        for (int k = 0; k < kOrderPerThread; ++k) {
+        for (int k = 0; k < kPerThread; ++k) {
             const int t = k * kOrderThreads + tid;
             if (t < num_tiles) order[s_bin[bucket[k]] + rank[k]] = t;
         }
@@ -722,9 +724,14 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
                            dim3((unsigned)((m + (long long)kBlock * kRangeItems - 1) / ((long long)kBlock * kRangeItems))), dim3(kBlock), 0,
                            (hipStream_t)stream, keys_sorted, (long long)m, (const long long*)m_device, workload_ranges,
                            (int)num_tiles);
-    if (tile_order && num_tiles > 0)
-        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(kOrderThreads), 0, (hipStream_t)stream, workload_ranges,
-                           (int)num_tiles, tile_order, status);
+    if (tile_order && num_tiles > 0) {
+        if (num_tiles <= kOrderThreads * kOrderPerThread)
+            hipLaunchKernelGGL(tile_order_kernel<kOrderPerThread>, dim3(1), dim3(kOrderThreads), 0, (hipStream_t)stream,
+                               workload_ranges, (int)num_tiles, tile_order, status);
+        else
+            hipLaunchKernelGGL(tile_order_kernel<kOrderPerThreadLarge>, dim3(1), dim3(kOrderThreads), 0,
+                               (hipStream_t)stream, workload_ranges, (int)num_tiles, tile_order, status);
+    }
     else if (report)
         hipLaunchKernelGGL(bin_status_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, status);
     hipError_t e = hipGetLastError();
