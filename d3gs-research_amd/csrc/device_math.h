@@ -329,8 +329,9 @@ __device__ __forceinline__ TileWalk tile_walk_setup(const d3gs_params& P, const 
     return w;
 }
 
-// Is candidate tile (lx, ly) — coordinates relative to the candidate rect origin — kept?  The filter is a template
-// argument: the walks below run their loops once per filter instead of choosing the test anew for every tile.
+// Does the filter keep the candidate tile whose pixel origin, relative to the candidate rect's, is (px0, py0)?
+// The filter is a template argument: the walks below run their loops once per filter instead of choosing the
+// test anew for every tile.  tile_keep() adds the 3-sigma rect for a tile given by its coordinates (lx, ly).
 template <int kFilter>
 __device__ __forceinline__ bool tile_test(const TileWalk& w, float px0, float py0) {
     if constexpr (kFilter == D3GS_FILTER_NONE) return true;
@@ -353,7 +354,8 @@ __device__ __forceinline__ bool tile_keep(const TileWalk& w, int lx, int ly) {
     return keep && lx >= w.lx0 && lx < w.lx1 && ly >= w.ly0 && ly < w.ly1;      // inside the 3-sigma rect
 }
 
-// A lane's walk over its own small candidate rect, row by row: calls visit(kept) once per candidate tile.  The
+// A lane's walk over its own small candidate rect, row by row: calls visit(t, px0, py0, kept) once per candidate
+// tile t.  The
 // tile's pixel origin is stepped as a float (multiples of 16, exact), and the 3-sigma rect is compared in the
 // same units, so the loop carries no integer coordinates and converts nothing.
 template <int kFilter, class Visit>
