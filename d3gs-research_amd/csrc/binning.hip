@@ -130,18 +130,22 @@ __global__ __launch_bounds__(kGatherScanBlock) void scan_gather_lookback_kernel(
     // other) in front of the launch.
     const int chunk = blockIdx.x;
     const int base = chunk * kGatherScanChunk + threadIdx.x * kGatherScanItems;
-    int v[kGatherScanItems];
+    // every index first, then every gather: two trips to memory, not one per item after the other (positions past
+    // the end take position 0's index and count nothing)
+    int v[kGatherScanItems], at[kGatherScanItems];
+#pragma unroll
+    for (int k = 0; k < kGatherScanItems; ++k) {
+        const int j = base + k < n ? base + k : 0;
+        at[k] = index ? index[j] : j;
+    }
     int s = 0;
 #pragma unroll
     for (int k = 0; k < kGatherScanItems; ++k) {
-        const int j = base + k;
-        int x = 0;
-        if (j < n) {
-            const int i = index ? index[j] : j;
-            if ((unsigned)i < (unsigned)src_n) x = src[i];   // a corrupt index must not become a wild read
-        }
-        v[k] = x;
-        s += x;
+        // a corrupt index must not become a wild read
+        const bool ok = (unsigned)at[k] < (unsigned)src_n;      // (false throughout for an empty source)
+        const int x = src_n > 0 ? src[ok ? at[k] : 0] : 0;
+        v[k] = (ok && base + k < n) ? x : 0;
+        s += v[k];
     }
     // exclusive scan of s over the workgroup
     const int wlane = threadIdx.x & 63, wave = threadIdx.x >> 6;
