@@ -273,17 +273,23 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     const bool sane = (unsigned)i < (unsigned)items;
     i = sane ? i : 0;
     const long long end = offsets[j];
-    long long off = !in_range ? end : (j == 0 ? 0 : offsets[j - 1]);   // lanes past the end: an empty range at the total
+    // requested with the loads above, whether it is needed or not (the empty statement keeps the compiler from
+    // moving the load behind the test of the lane, where it would wait for a round trip of its own)
+    const int before = offsets[j > 0 ? j - 1 : 0];
+    asm volatile("" : : "v"(before));
+    long long off = !in_range ? end : (j == 0 ? 0 : before);   // lanes past the end: an empty range at the total
     // a gaussian with no tiles has an empty slot range; a caller that passed a smaller buffer than
     // the scan total must never be written past
     const bool active = in_range && sane && end > off && end <= m;
     const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : reference_depth_bits(P, depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
     unsigned long long kept = 0ull, meta = 0ull;
-    if (tile_masks && active) {     // both words in one 16-byte load: one round trip, not two dependent ones
+    // both words in one 16-byte load, and requested as soon as the gaussian is known: whether the lane has pairs to
+    // emit is known a round trip earlier than it is needed here
+    if (tile_masks && in_range && sane) {
         const ulonglong2 rec = *reinterpret_cast<const ulonglong2*>(tile_masks + 2 * (size_t)i);
-        kept = rec.x;
-        meta = rec.y;
+        kept = active ? rec.x : 0ull;
+        meta = active ? rec.y : 0ull;
     }
     const bool has_mask = (meta & kTileMaskHas) != 0;
     const bool walk_again = active && !has_mask;
@@ -376,6 +382,7 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
     if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the key buffer
     const long long i0 = ((long long)blockIdx.x * kBlock + threadIdx.x) * kRangeItems;
     if (i0 >= m) return;
+    const Key before = keys[i0 > 0 ? i0 - 1 : 0];     // (requested together with the thread's own keys)
     Key k[kRangeItems];
     if (i0 + kRangeItems <= m) {
         if constexpr (sizeof(Key) == 4) {
@@ -389,7 +396,7 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
 #pragma unroll
         for (int j = 0; j < kRangeItems; ++j) k[j] = i0 + j < m ? keys[i0 + j] : (Key)0;
     }
-    uint32_t tp = i0 > 0 ? key_tile<Key>(keys[i0 - 1]) : 0u;
+    uint32_t tp = i0 > 0 ? key_tile<Key>(before) : 0u;
 #pragma unroll
     for (int j = 0; j < kRangeItems; ++j) {
         const long long i = i0 + j;
@@ -460,9 +467,10 @@ __global__ __launch_bounds__(kOrderThreads) void tile_order_kernel(const int32_t
     int mx = 0;
     if (in_registers) {
 #pragma unroll
-        for (int k = 0; k < kPerThread; ++k) {
-            const int t = k * kOrderThreads + tid;
-            amount[k] = t < num_tiles ? amount_of(t) : 0;
+        for (int k = 0; k < kPerThread; ++k) {      // (tiles past the end read the last tile: loads without a
+            const int t = k * kOrderThreads + tid;  // condition are issued together, conditional ones one by one)
+            const int a = amount_of(min(t, num_tiles - 1));
+            amount[k] = t < num_tiles ? a : 0;
             mx = max(mx, amount[k]);
         }
     } else {
