@@ -661,6 +661,43 @@ __device__ __forceinline__ void bwd_rows_copy(float* __restrict__ global, float*
     auto row_of = [&](int r) { const int i = first + list[r]; return (size_t)(origin ? origin[i] : i); };
     if ((rowlen & 3) == 0 && ((uintptr_t)global & 15u) == 0) {
         const int per_row = rowlen >> 2;
+        if constexpr (kToLds) {
+            // Rows in: four 16-byte loads of a thread are requested before the first is stored to LDS.  One at a
+            // time, each would wait for its own trip to memory (the row's position comes out of LDS, and the
+            // compiler does not move that read ahead of the stores before it).  Elements past the end read
+            // element 0 and store nothing.
+            constexpr int kAhead = 4;
+            const int total = cnt * per_row;
+            for (int q0 = threadIdx.x; q0 < total; q0 += kBwdBlock * kAhead) {
+                float4 t[kAhead];
+                int at[kAhead], col[kAhead];
+                size_t row[kAhead];
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u) {
+                    const int q = q0 + u * kBwdBlock;
+                    const int qq = q < total ? q : 0;
+                    const int r = qq / per_row;
+                    col[u] = (qq - r * per_row) * 4;
+                    at[u] = q < total ? r * stride + col[u] : -1;
+                    row[u] = (size_t)(first + list[r]);
+                }
+                if (origin) {
+#pragma unroll
+                    for (int u = 0; u < kAhead; ++u) row[u] = (size_t)origin[row[u]];
+                }
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u)
+                    t[u] = *reinterpret_cast<const float4*>(global + row[u] * rowlen + col[u]);
+#pragma unroll
+                for (int u = 0; u < kAhead; ++u) {
+                    if (at[u] >= 0) {
+                        float* lp = lds + at[u];
+                        lp[0] = t[u].x; lp[1] = t[u].y; lp[2] = t[u].z; lp[3] = t[u].w;
+                    }
+                }
+            }
+            return;
+        }
         for (int q = threadIdx.x; q < cnt * per_row; q += kBwdBlock) {
             const int r = q / per_row, c = (q - r * per_row) * 4;
             float4* gp = reinterpret_cast<float4*>(global + row_of(r) * rowlen + c);
@@ -717,24 +754,34 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     unsigned long long mates[kPer];
     // all radii first, then all records: two round trips to memory instead of two per gaussian.  With the blend
     // backward's `touched` bytes a gaussian it did not mark counts as culled, and its record is never read.
+    // (Every load below is unconditional: one behind a per-lane condition is issued and waited for on its own, one
+    // after the other.  Lanes past the end read the block's last gaussian, gaussians without a mark the block's
+    // first record, and what they read is dropped.)
     int rad[kPer];
+    unsigned char mark[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
-        const int local = k * kBwdBlock + tid;
-        rad[k] = local < nrows ? radii[(size_t)first + local] : 0;
-        if (touched && local < nrows && !touched[(size_t)first + local]) rad[k] = 0;
+        rad[k] = radii[(size_t)first + min(k * kBwdBlock + tid, nrows - 1)];
+        mark[k] = 1;
     }
+    if (touched) {
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) mark[k] = touched[(size_t)first + min(k * kBwdBlock + tid, nrows - 1)];
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k)
+        if (k * kBwdBlock + tid >= nrows || !mark[k]) rad[k] = 0;
     float4 ra[kPer], rb[kPer], rc[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
-        const size_t i = (size_t)first + k * kBwdBlock + tid;
-        ra[k] = rb[k] = rc[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (rad[k] != 0) {
-            ra[k] = rec4[4 * i];
-            rb[k] = rec4[4 * i + 1];
-            rc[k] = rec4[4 * i + 2];
-        }
+        const size_t i = rad[k] != 0 ? (size_t)first + k * kBwdBlock + tid : (size_t)first;
+        ra[k] = rec4[4 * i];
+        rb[k] = rec4[4 * i + 1];
+        rc[k] = rec4[4 * i + 2];
     }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k)
+        if (rad[k] == 0) ra[k] = rb[k] = rc[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
         const int local = k * kBwdBlock + tid;
