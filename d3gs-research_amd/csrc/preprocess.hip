@@ -43,28 +43,35 @@ constexpr int kShColorBlocks = 512;   // two workgroups per CU for the SH colour
 // Rows of `rowlen` floats per gaussian move from global memory into LDS with consecutive threads on
 // consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
 // different cache line in every lane).  LDS rows are padded to an odd stride: conflict-free per-thread access.
+// kAhead 16-byte loads of a thread are requested before the first is stored: one at a time, each waits for its own
+// trip to memory, and a kernel that runs one wavefront per SIMD has nothing else to do meanwhile.
+template <int kAhead>
 __device__ __forceinline__ void rows_global_to_lds(const float* __restrict__ src, float* lds, int nrows, int rowlen,
                                                    int stride) {
     const int total = nrows * rowlen;
     const float inv = 1.0f / (float)rowlen;
-    const bool vec = ((uintptr_t)src & 15u) == 0;
-    for (int e4 = threadIdx.x * 4; e4 < total; e4 += kPrepBlock * 4) {
-        float v[4];
-        if (vec && e4 + 3 < total) {
-            const float4 t = *reinterpret_cast<const float4*>(src + e4);
-            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-        } else {
+    auto place = [&](int e, float v) {
+        const int g = (int)(((float)e + 0.5f) * inv);
+        lds[g * stride + (e - g * rowlen)] = v;
+    };
+    if ((((uintptr_t)src & 15u) == 0) && (total & 3) == 0) {
+        for (int e0 = threadIdx.x * 4; e0 < total; e0 += kPrepBlock * 4 * kAhead) {
+            float4 t[kAhead];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) v[c] = e4 + c < total ? src[e4 + c] : 0.0f;
-        }
+            for (int u = 0; u < kAhead; ++u) {      // (elements past the end read element 0 and store nothing)
+                const int e4 = e0 + u * kPrepBlock * 4;
+                t[u] = *reinterpret_cast<const float4*>(src + (e4 < total ? e4 : 0));
+            }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int e = e4 + c;
-            if (e < total) {
-                const int g = (int)(((float)e + 0.5f) * inv);
-                lds[g * stride + (e - g * rowlen)] = v[c];
+            for (int u = 0; u < kAhead; ++u) {
+                const int e4 = e0 + u * kPrepBlock * 4;
+                if (e4 < total) {
+                    place(e4, t[u].x); place(e4 + 1, t[u].y); place(e4 + 2, t[u].z); place(e4 + 3, t[u].w);
+                }
             }
         }
+    } else {
+        for (int e = threadIdx.x; e < total; e += kPrepBlock) place(e, src[e]);
     }
 }
 
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     const int rowlen = P0.sh_stride * 3, stride = rowlen | 1;
     if constexpr (kWithSh) {
         const int first = blockIdx.x * kPrepBlock;
-        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
+        rows_global_to_lds<4>(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
         __syncthreads();
     }
     // no early return: every lane of the wavefront takes part in the cooperative tile count
@@ -327,9 +334,14 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
         const int batch = chunk / chunks_per_view;
         const int first = (chunk - batch * chunks_per_view) * kPrepBlock;      // first gaussian of the chunk
         __syncthreads();   // the previous chunk's rows have been read
-        rows_global_to_lds(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
-        __syncthreads();
+        // what the thread's own gaussian needs besides its row, requested ahead of the rows (lanes past the end
+        // read the chunk's first gaussian)
         const int g = first + threadIdx.x;
+        const int g_safe = g < P0.n ? g : first;
+        const int radius = radii[batch * P0.n + g_safe];
+        const float centre[3] = {xyz[3 * g_safe], xyz[3 * g_safe + 1], xyz[3 * g_safe + 2]};
+        rows_global_to_lds<12>(sh + (size_t)first * rowlen, s_rows, min(kPrepBlock, P0.n - first), rowlen, stride);
+        __syncthreads();
         if (g >= P0.n) continue;
         const int i = batch * P0.n + g;     // render item
         d3gs_params P = P0;
@@ -339,8 +351,8 @@ __global__ __launch_bounds__(kPrepBlock) void sh_colors_kernel(
         }
         float rgb[3] = {0.0f, 0.0f, 0.0f};
         uint32_t ne0 = 0;
-        if (radii[i] > 0) {
-            float d[3] = {xyz[3 * g] - P.cam_center[0], xyz[3 * g + 1] - P.cam_center[1], xyz[3 * g + 2] - P.cam_center[2]};
+        if (radius > 0) {
+            float d[3] = {centre[0] - P.cam_center[0], centre[1] - P.cam_center[1], centre[2] - P.cam_center[2]};
             float dn = sqrtf((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2]);
             float dx = d[0] / dn, dy = d[1] / dn, dz = d[2] / dn;
             const float* shp = s_rows + threadIdx.x * stride;
