@@ -38,7 +38,7 @@ __device__ __forceinline__ float sh_channel(int degree, float x, float y, float 
 }
 
 constexpr int kPrepBlock = 128;   // gaussians (= threads) per workgroup of the per-gaussian kernels
-constexpr int kShColorBlocks = 512;   // two workgroups per CU for the SH colour kernel
+constexpr int kShColorBlocks = 384;   // fewest workgroups of the SH colour kernel: three on every two CUs
 
 // Rows of `rowlen` floats per gaussian move from global memory into LDS with consecutive threads on
 // consecutive addresses (the per-gaussian rows are 180-192 B apart, so per-thread access would touch a
@@ -1027,10 +1027,13 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
     if (!instance_view(instances, &inst, "d3gs_sh_colors")) return D3GS_ERR_INVALID_ARGUMENT;
     const int chunks = ((p->n + kPrepBlock - 1) / kPrepBlock) * batch_count(*p);
     // A small grid, so that the kernel fills idle slots beside the binning stages it runs next to instead of
-    // displacing them: two workgroups per CU up to 1.5M gaussians, growing to four at 3M so that it still ends
-    // before the pair sort starts (3M gaussians, 1080p: 2.15 -> 2.06 ms per view; six or eight per CU slowed the
-    // depth sort by more than they gained).
-    const int blocks = std::min(2 * kShColorBlocks, std::max(kShColorBlocks, chunks / 24));
+    // displacing them; what it has to do is end before the forward blend starts.  Measured per view: 1M gaussians
+    // 0.837 ms with 512 workgroups, 0.842 with 325 to 384, 0.846 with 768, 0.857 with 1024 (the larger grids slow
+    // the depth sort by more than they gain); 3M gaussians 1.94 ms with 384, 1.96 with 512, 1.97 with 976 (the depth
+    // sort of 3M keys suffers most).  Hence 512 falling to 384 between 1M and 2M gaussians, and growing with the
+    // scene only where 384 could no longer end in time.
+    const int falling = std::min(512, std::max(kShColorBlocks, 768 - chunks / 30));
+    const int blocks = std::min(1024, std::max(falling, chunks / 60));
     dim3 grid(chunks < blocks ? chunks : blocks), block(kPrepBlock);
     const size_t lds_bytes = (size_t)kPrepBlock * ((p->sh_stride * 3) | 1) * sizeof(float);
     if (inst.ids || p->batch_size > 1)
