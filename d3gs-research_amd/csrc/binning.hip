@@ -435,6 +435,9 @@ struct BinStatus {
     const uint32_t* sort_error[2];   // error words of the depth sort and the pair sort (either may be NULL)
     int64_t* total_dev;              // count words to poison (either may be NULL)
     int64_t* total_host;
+    // the host word is written here and only here (the count, or the status in its place), by a store that the
+    // host sees while the stream runs on: a caller polls the word instead of putting an event into the stream
+    bool publish_host;
 };
 
 __device__ __forceinline__ void fold_sort_errors(const BinStatus& st) {
@@ -442,9 +445,12 @@ __device__ __forceinline__ void fold_sort_errors(const BinStatus& st) {
 #pragma unroll
     for (int k = 0; k < 2; ++k)
         if (st.sort_error[k]) err |= __hip_atomic_load(st.sort_error[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (err) {
-        if (st.total_dev) *st.total_dev = D3GS_COUNT_SORT_GAVE_UP;
-        if (st.total_host) *st.total_host = D3GS_COUNT_SORT_GAVE_UP;
+    if (err && st.total_dev) *st.total_dev = D3GS_COUNT_SORT_GAVE_UP;
+    if (st.publish_host) {
+        const long long word = err ? (long long)D3GS_COUNT_SORT_GAVE_UP : (st.total_dev ? *st.total_dev : 0ll);
+        __hip_atomic_store((long long*)st.total_host, word, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    } else if (err && st.total_host) {
+        *st.total_host = D3GS_COUNT_SORT_GAVE_UP;
     }
 }
 
@@ -724,8 +730,9 @@ extern "C" int d3gs_gather_i32(const int32_t* src, int32_t src_n, const int32_t*
 template <typename Key>
 static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, const int64_t* m_device,
                             int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order, d3gs_stream_t stream,
-                            BinStatus status = BinStatus{{nullptr, nullptr}, nullptr, nullptr}) {
-    const bool report = (status.sort_error[0] || status.sort_error[1]) && (status.total_dev || status.total_host);
+                            BinStatus status = BinStatus{{nullptr, nullptr}, nullptr, nullptr, false}) {
+    const bool report = status.publish_host ||
+                        ((status.sort_error[0] || status.sort_error[1]) && (status.total_dev || status.total_host));
     if (m < 0 || num_tiles < 0) { set_error("%s: bad argument", who); return D3GS_ERR_INVALID_ARGUMENT; }
     if ((m > 0 && !keys_sorted) || (num_tiles > 0 && !workload_ranges)) {
         set_error("%s: NULL buffer", who);
@@ -761,10 +768,11 @@ namespace d3gs {
 int tile_ranges_u32_with_status(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
                                 int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
                                 const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
-                                int64_t* total_host, d3gs_stream_t stream) {
+                                int64_t* total_host, bool publish_host, d3gs_stream_t stream) {
     return tile_ranges_impl<uint32_t>("d3gs_bin_pairs (tile ranges)", tile_keys_sorted, m, m_device, workload_ranges,
                                       num_tiles, tile_order, stream,
-                                      BinStatus{{sort_error_a, sort_error_b}, total_dev, total_host});
+                                      BinStatus{{sort_error_a, sort_error_b}, total_dev, total_host,
+                                                publish_host && total_host != nullptr});
 }
 }  // namespace d3gs
 

@@ -611,10 +611,11 @@ void set_error(const char* fmt, ...);
 int check_params(const d3gs_params* p, const char* who);
 // d3gs_tile_ranges_u32 whose last kernel also folds the error words of up to two sort workspaces into the
 // pair-count words: D3GS_COUNT_SORT_GAVE_UP replaces the count when either is set (defined in binning.hip).
+// publish_host: that kernel is the only one to write *total_host, count or status, by a store the host can poll for.
 int tile_ranges_u32_with_status(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
                                 int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
                                 const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
-                                int64_t* total_host, d3gs_stream_t stream);
+                                int64_t* total_host, bool publish_host, d3gs_stream_t stream);
 
 // Depth part of the reference's sort key (render.py:767-775): the float bits (positive floats order like their
 // bit patterns), or with enable_32bit_sort the depth in steps of depth_32bit_prec, truncated to 18 bits.

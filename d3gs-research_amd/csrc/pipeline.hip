@@ -14,7 +14,7 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
                               size_t scan_ws_bytes, int64_t* total_dev, int64_t* total_host, int64_t capacity,
                               uint32_t* tile_keys_a, uint32_t* tile_keys_b, int32_t* idx_a, int32_t* idx_b,
                               void* pair_sort_ws, size_t pair_sort_ws_bytes, int32_t* workload_ranges,
-                              int32_t* tile_order, int32_t workspaces_are_zero, int32_t* order_in_b,
+                              int32_t* tile_order, int32_t flags, int32_t* order_in_b,
                               int32_t* pairs_in_b, d3gs_stream_t stream) {
     if (!p || !order_in_b || !pairs_in_b || !total_dev || capacity < 0) {
         set_error("d3gs_bin_pairs: bad argument");
@@ -22,15 +22,18 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
     }
     const int32_t n = item_count(*p);                               // render items: gaussians x cameras of a bundle
     const int32_t num_tiles = p->tiles_x * p->tiles_y * batch_count(*p);
+    const int32_t workspaces_are_zero = flags & D3GS_BIN_WORKSPACES_ARE_ZERO;
+    const bool host_word_at_end = (flags & D3GS_BIN_HOST_COUNT_AT_END) != 0;
     int rc = d3gs_sort_pairs_u32(depth_keys_a, depth_keys_b, order_a, order_b, depth_sort_ws, depth_sort_ws_bytes, n,
                                  nullptr, /*values_are_indices=*/1, workspaces_are_zero, 0,
                                  d3gs_depth_key_bits(p), order_in_b, stream);
     if (rc) return rc;
     const uint32_t* depth_keys_sorted = *order_in_b ? depth_keys_b : depth_keys_a;
     const int32_t* order = *order_in_b ? order_b : order_a;
-    // the pair count also goes to the host word, written by the scan itself; nothing here waits for it
+    // the pair count also goes to the host word, written by the scan itself (or, with D3GS_BIN_HOST_COUNT_AT_END, by
+    // the last kernel of the call only); nothing here waits for it
     rc = d3gs_scan_gathered(tiles_touched, n, order, n, offsets, scan_ws, scan_ws_bytes, workspaces_are_zero, total_dev,
-                            total_host, stream);
+                            host_word_at_end ? nullptr : total_host, stream);
     if (rc) return rc;
     rc = d3gs_make_keys(p, radii, uvs, conic_opacity, depths, offsets, order, depth_keys_sorted, tile_masks, nullptr,
                         tile_keys_a, idx_a, capacity, stream);
@@ -46,5 +49,6 @@ extern "C" int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const 
     const uint32_t* e_depth = n > 0 && depth_sort_ws ? (const uint32_t*)((const char*)depth_sort_ws + err_depth) : nullptr;
     const uint32_t* e_pairs = capacity > 0 && pair_sort_ws ? (const uint32_t*)((const char*)pair_sort_ws + err_pairs) : nullptr;
     return tile_ranges_u32_with_status(*pairs_in_b ? tile_keys_b : tile_keys_a, capacity, total_dev, workload_ranges,
-                                       num_tiles, tile_order, e_depth, e_pairs, total_dev, total_host, stream);
+                                       num_tiles, tile_order, e_depth, e_pairs, total_dev, total_host, host_word_at_end,
+                                       stream);
 }

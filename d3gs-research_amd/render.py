@@ -17,6 +17,7 @@ import contextlib
 import copy
 import ctypes as C
 import dataclasses
+import time
 
 import numpy as np
 import torch
@@ -183,6 +184,10 @@ class GaussianSplatOp:
         self.clear_gradients_early = True
         # a CameraBundle of several cameras goes through the kernels in one pass (False: camera by camera)
         self.bundle_in_one_pass = True
+        # the one-call binning writes the pair count to its pinned host word with a store the host can see while
+        # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
+        # forward blend back by the few microseconds the stream takes to process the marker
+        self.poll_pair_count = True
         self._pair_capacity = 0
         # Pinned host words the kernels report into (the pair count; the two sorts' status on the launch-by-launch
         # path).  One set per op: an op serves one forward at a time -- two forwards of the same op that overlap
@@ -445,6 +450,7 @@ class GaussianSplatOp:
         f32, i32 = torch.float32, torch.int32
         if self._count_host is None:
             self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+            self._count_np = self._count_host.numpy()      # the same word, read without a tensor operation
             self._sort_status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
         # Sparse mode (render.py:234-238, 478-500, 622-640): a first pass of the preprocess flags the accepted
         # gaussians, a scan gives each its row, and from here on n is their number V: every buffer below has V rows
@@ -657,15 +663,21 @@ class GaussianSplatOp:
             at = lambda off: C.c_void_p(base + 4 * off)
             total = torch.empty(1, dtype=torch.int64, device=dev)
             order_in_b, pairs_in_b = C.c_int(0), C.c_int(0)
+            polled = bool(self.poll_pair_count and n > 0)
+            if polled:
+                self._count_np[0] = _capi.COUNT_PENDING
             _capi.check(L.d3gs_bin_pairs(
                 C.byref(Pd), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(depths),
                 _capi.ptr(tiles_touched), _capi.ptr(tile_masks), _capi.ptr(depth_keys), at(o_keys_b), at(o_ord_a),
                 at(o_ord_b), _capi.ptr(zero_ws_n), zero_ws_n.numel(), at(o_offs), _capi.ptr(zero_scan_ws),
                 zero_scan_ws.numel(), _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), cap, at(o_tk_a),
                 at(o_tk_b), at(o_ix_a), at(o_ix_b), _capi.ptr(zero_ws_m), zero_ws_m.numel(), _capi.ptr(zero_ranges),
-                at(o_order), 1, C.byref(order_in_b), C.byref(pairs_in_b), s), "d3gs_bin_pairs")
-            count_ready = torch.cuda.Event()
-            count_ready.record()
+                at(o_order), _capi.BIN_WORKSPACES_ARE_ZERO | (_capi.BIN_HOST_COUNT_AT_END if polled else 0),
+                C.byref(order_in_b), C.byref(pairs_in_b), s), "d3gs_bin_pairs")
+            count_ready = None
+            if not polled:
+                count_ready = torch.cuda.Event()
+                count_ready.record()
             # what a second, exactly sized binning of this view would start from
             depth_keys_sorted = pool[o_keys_b:o_keys_b + n] if order_in_b.value else depth_keys
             gaussian_order = pool[o_ord_b:o_ord_b + n] if order_in_b.value else pool[o_ord_a:o_ord_a + n]
@@ -796,7 +808,17 @@ class GaussianSplatOp:
         ctx = None
         if capacity > 0:
             ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
-        count_ready.synchronize()
+        if count_ready is not None:
+            count_ready.synchronize()
+        else:
+            # the binning's last kernel stores the count (or a status) over the marker put there before the call
+            give_up = time.perf_counter() + 0.02
+            while int(self._count_np[0]) == _capi.COUNT_PENDING:
+                if time.perf_counter() > give_up:       # a very large view, or a store the host does not see
+                    torch.cuda.current_stream().synchronize()
+                    if int(self._count_np[0]) == _capi.COUNT_PENDING:
+                        raise RuntimeError("d3gs_bin_pairs: the pair count never reached the host")
+                    break
         num_rendered = int(self._count_host[0])
         if num_rendered == _capi.COUNT_SORT_GAVE_UP:
             raise RuntimeError("d3gs_bin_pairs: a sort workgroup's bounded wait on an earlier tile ran out; "

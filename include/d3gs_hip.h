@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 29
+#define D3GS_ABI_VERSION 30
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -44,6 +44,8 @@ extern "C" {
  * the count when a kernel's bounded wait on an earlier workgroup ran out; the lists are then not valid. */
 #define D3GS_COUNT_SCAN_GAVE_UP (-1)
 #define D3GS_COUNT_SORT_GAVE_UP (-2)
+/* not written by the library: what a caller that polls the host word of d3gs_bin_pairs puts there beforehand */
+#define D3GS_COUNT_PENDING (-3)
 /* Most (tile, gaussian) pairs of one call: list positions are 31-bit (int32 offsets, tile ranges and sort
  * prefixes, like the reference's, whose CUB sort takes an int count, devsort.py:96-129).  A sort of more is
  * refused with D3GS_ERR_UNSUPPORTED; the scans still return the true int64 total, so a caller sees it. */
@@ -291,8 +293,14 @@ int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int6
  * D3GS_COUNT_SORT_GAVE_UP, so a caller that checks the count for a negative value never takes a mis-sorted list
  * for a result.  Workspace sizes as for the single calls
  * (d3gs_sort_workspace_bytes(n, 0, d3gs_depth_key_bits(p)), d3gs_scan_gathered_workspace_bytes(n),
- * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))); workspaces_are_zero != 0 says the caller has
- * cleared all three.  workload_ranges must be zero on entry. */
+ * d3gs_sort_workspace_bytes(capacity, 0, d3gs_higher_msb(tiles))).  flags: D3GS_BIN_WORKSPACES_ARE_ZERO says the
+ * caller has cleared all three.  With D3GS_BIN_HOST_COUNT_AT_END *total_host is written once, by the last kernel
+ * of the call (it needs tile_order != NULL or a workspace to run), with the count or the status in its place, as
+ * a system-scope release store: a caller that sets the word to D3GS_COUNT_PENDING before the call can poll it
+ * from the host while the stream runs on, where waiting on an event would put a marker into the stream ahead of
+ * the kernels that follow.  workload_ranges must be zero on entry. */
+#define D3GS_BIN_WORKSPACES_ARE_ZERO 1
+#define D3GS_BIN_HOST_COUNT_AT_END 2
 int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                    const float* depths, const int32_t* tiles_touched, const uint64_t* tile_masks,
                    uint32_t* depth_keys_a, uint32_t* depth_keys_b, int32_t* order_a, int32_t* order_b,
@@ -300,7 +308,7 @@ int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs,
                    size_t scan_ws_bytes, int64_t* total_dev, int64_t* total_host, int64_t capacity,
                    uint32_t* tile_keys_a, uint32_t* tile_keys_b, int32_t* idx_a, int32_t* idx_b, void* pair_sort_ws,
                    size_t pair_sort_ws_bytes, int32_t* workload_ranges, int32_t* tile_order,
-                   int32_t workspaces_are_zero, int32_t* order_in_b, int32_t* pairs_in_b, d3gs_stream_t stream);
+                   int32_t flags, int32_t* order_in_b, int32_t* pairs_in_b, d3gs_stream_t stream);
 
 /* K6 — replaces kernel_raw("rasterize_False_...") at render.py:1434-1464, 2304-2309.
  * color [H,W,C] (or [C,H,W] when p->use_nchw), C = 3 + p->render_rgba; final_T [H,W], n_contrib [H,W].

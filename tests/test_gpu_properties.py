@@ -104,10 +104,11 @@ def test_forward_is_deterministic_and_backward_is_linear():
         assert med <= 1e-5 and p99 <= 2e-3, f"{name}: additivity per-gaussian median {med:.2e} p99 {p99:.2e}"
 
 
-@pytest.mark.parametrize("fused", [True, False])
-def test_pair_buffers_sized_from_the_previous_view(oracle, fused):
+@pytest.mark.parametrize("fused,polled", [(True, True), (True, False), (False, False)])
+def test_pair_buffers_sized_from_the_previous_view(oracle, fused, polled):
     """The operator sizes the pair buffers of a view from the previous view's count (no host wait
-    before binning) and, with `fused_binning`, enqueues the whole binning through d3gs_bin_pairs.  A view
+    before binning) and, with `fused_binning`, enqueues the whole binning through d3gs_bin_pairs, whose
+    pair count the host either polls for in pinned memory (`poll_pair_count`) or waits for on an event.  A view
     that fits, one that outgrows the buffers (binned again), an empty one and the unspeculative path must
     all equal the oracle, and the backward pass must run from the context either path leaves."""
     import torch
@@ -116,7 +117,8 @@ def test_pair_buffers_sized_from_the_previous_view(oracle, fused):
     small, big = gen_scene(1, n=5000, wh=(250, 190), with_grad=False), gen_scene(1, n=40000, wh=(250, 190), with_grad=False)
     op = GaussianSplatOp(op_config(small, DFVT))
     op.fused_binning = fused
-    print(f"speculative pair buffers, fused_binning={fused}", flush=True)
+    op.poll_pair_count = polled
+    print(f"speculative pair buffers, fused_binning={fused}, poll_pair_count={polled}", flush=True)
     refs = {id(sc): oracle_forward(oracle, sc, DFVT)[1] for sc in (small, big)}
     seq = [small, small, big, big, small]          # exact, fits, outgrown, fits, fits with large head room
     for k, sc in enumerate(seq):
@@ -160,6 +162,7 @@ def test_every_optional_acceleration_off_gives_the_same_result():
     fast = GaussianSplatOp(op_config(scene, DFVT))
     plain = GaussianSplatOp(op_config(scene, DFVT))
     plain.overlap_sh_colors = plain.fused_binning = plain.speculative_pair_buffers = plain.clear_gradients_early = False
+    plain.poll_pair_count = False
     g = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
     for view in range(3):
         res = []
