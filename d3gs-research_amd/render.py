@@ -816,6 +816,7 @@ class GaussianSplatOp:
             while int(self._count_np[0]) == _capi.COUNT_PENDING:
                 if time.perf_counter() > give_up:       # a very large view, or a store the host does not see
                     torch.cuda.current_stream().synchronize()
+                    self.poll_pair_count = False        # later views wait on an event again
                     if int(self._count_np[0]) == _capi.COUNT_PENDING:
                         raise RuntimeError("d3gs_bin_pairs: the pair count never reached the host")
                     break
