@@ -17,6 +17,7 @@ import contextlib
 import copy
 import ctypes as C
 import dataclasses
+import math
 import time
 
 import numpy as np
@@ -262,6 +263,11 @@ class GaussianSplatOp:
 
     @staticmethod
     def _stream():
+        """The current stream's handle.  (torch.cuda.current_stream() builds a Stream object, some 10 us of host
+        time a call, which a view of a small scene notices: its host code is what bounds it.)"""
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if raw is not None:
+            return C.c_void_p(raw(torch.cuda.current_device()))
         return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def _camera_arrays(self, cameras):
@@ -793,8 +799,10 @@ class GaussianSplatOp:
                 grad_touched=grad_touched,
                 kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids,
                 batch_size=batch, batch_cameras=batch_cams, sparse_gaussian_ids=sparse_gaussian_ids)
+            # the view's kernel parameters, for a backward pass over the same model and cameras
+            ctx._forward_params = (P, model, cameras, bool(training))
             if sh_done is not None:
-                torch.cuda.current_stream().wait_event(sh_done)
+                main.wait_event(sh_done)      # (the stream object of the fork: forward runs on one stream)
             with self._stage("blend_fwd"):
                 self.rasterize_forward_backward(model, ctx, out, training=training,
                                                 render_depth=self._cfg.render_depth, _params=Pd)
@@ -916,14 +924,14 @@ class GaussianSplatOp:
 
     @classmethod
     def _grad_pool_floats(cls, model, rows=None) -> int:
-        return sum((int(np.prod(shape)) + 63) // 64 * 64 for _, shape in cls._grad_fields(model, rows))
+        return sum((math.prod(shape) + 63) // 64 * 64 for _, shape in cls._grad_fields(model, rows))
 
     @classmethod
     def _grad_views(cls, model, pool, rows=None):
         """The model-shaped gradient tensors as 256-byte aligned slices of one allocation."""
         views, off = {}, 0
         for name, shape in cls._grad_fields(model, rows):
-            numel = int(np.prod(shape))
+            numel = math.prod(shape)
             views[name] = pool[off:off + numel].view(shape)
             off += (numel + 63) // 64 * 64
         return views
@@ -1078,7 +1086,11 @@ class GaussianSplatOp:
         if isinstance(ctx, GaussianSplatOpBatchContext):
             return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
         L = self._lib
-        P = self.make_params(model, cameras, True, ctx.batch_cameras)
+        kept = getattr(ctx, "_forward_params", None)
+        if kept is not None and kept[1] is model and kept[2] is cameras and kept[3]:
+            P = _capi.Params.from_buffer_copy(kept[0])      # (a copy: sparse mode edits n below)
+        else:
+            P = self.make_params(model, cameras, True, ctx.batch_cameras)
         s = self._stream()
         sparse_ids = ctx.sparse_gaussian_ids
         if sparse_ids is not None:      # the kernels see a scene of the V accepted gaussians
