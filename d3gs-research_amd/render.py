@@ -654,9 +654,6 @@ class GaussianSplatOp:
         fused = bool(self.fused_binning and spec_capacity > 0 and self.stage_events is None)
         self.last_forward_fused = fused      # which of the two binning paths this view took (tests look at it)
         fused_result = None
-        if self._count_host is None:
-            self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
-            self._sort_status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
         if fused:
             cap = spec_capacity
             up = lambda v: (v + 63) // 64 * 64          # 256-byte aligned slices of one int32 allocation
