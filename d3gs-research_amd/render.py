@@ -189,6 +189,7 @@ class GaussianSplatOp:
         # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
         # forward blend back by the few microseconds the stream takes to process the marker
         self.poll_pair_count = True
+        self._poll_timeouts = 0     # consecutive views whose count did not arrive within the polling time
         self._pair_capacity = 0
         # Pinned host words the kernels report into (the pair count; the two sorts' status on the launch-by-launch
         # path).  One set per op: an op serves one forward at a time -- two forwards of the same op that overlap
@@ -821,10 +822,14 @@ class GaussianSplatOp:
             while int(self._count_np[0]) == _capi.COUNT_PENDING:
                 if time.perf_counter() > give_up:       # a very large view, or a store the host does not see
                     torch.cuda.current_stream().synchronize()
-                    self.poll_pair_count = False        # later views wait on an event again
+                    self._poll_timeouts += 1
+                    if self._poll_timeouts >= 3:        # not one slow view: later views wait on an event again
+                        self.poll_pair_count = False
                     if int(self._count_np[0]) == _capi.COUNT_PENDING:
                         raise RuntimeError("d3gs_bin_pairs: the pair count never reached the host")
                     break
+            else:
+                self._poll_timeouts = 0
         num_rendered = int(self._count_host[0])
         if num_rendered == _capi.COUNT_SORT_GAVE_UP:
             raise RuntimeError("d3gs_bin_pairs: a sort workgroup's bounded wait on an earlier tile ran out; "
