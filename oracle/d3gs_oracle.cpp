@@ -25,7 +25,13 @@
 //                                  scipy Rotation, EWA J W S W^T J^T, 2x2 inverse,
 //                                  eigen radius), SH against a float64 restatement
 //                                  of the in-tree Inria eval_sh table
-//   tile filters NONE/AABB/OBB   : brute-force per-pixel losslessness + subset chain
+//   tile filters NONE/AABB/OBB   : from both sides: brute-force per-pixel losslessness and the
+//                                  subset chain bound them from below; from above, AABB must equal
+//                                  the tiles meeting the float64 box u +- sqrt(L Sigma_ii) and OBB the
+//                                  tiles meeting the oriented rectangle built with numpy eigh and an
+//                                  independent separating-axis test (tiles within 1e-3 of a boundary
+//                                  skipped); ELLIPSE inside OBB; an isotropic conic (NaN axis) keeps
+//                                  every candidate tile
 //   OBB_DFVT                     : implemented as the OBB tile set (the author's
 //                                  stated invariant, render.py:1051-1072); the
 //                                  third-party cumm OBBCornersGridOverlap::inc_step

@@ -209,3 +209,165 @@ def test_32bit_sort_depth_steps_wrap_at_18_bits(oracle):
     assert (steps[ref["radii"] > 0] >= 2 ** 18).any()
     got = (ref["keys"] & np.uint64(0x3FFFF)).astype(np.uint32)
     assert np.array_equal(got, (steps & np.uint32(0x3FFFF))[ref["vals"]])
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# AABB and OBB tile sets pinned from both sides: an independent float64 construction of the level set's bounding
+# boxes (closed forms of the inverse conic, numpy.linalg.eigh) and a numpy separating-axis test decide every tile
+# of the 3-sigma rect; the oracle must keep exactly those.  A filter that is too tight AND one that is too loose
+# (a full width where the reference halves it, a wrong level) both fail here.
+# ---------------------------------------------------------------------------------------------------------------
+_TWO_SIDED_SCENES = [lambda: gen_scene(0, n=1500), lambda: gen_scene(2, n=4000, wh=(640, 360)),
+                     lambda: gen_scene(4, n=3000, wh=(480, 270))]
+
+
+def _rect_tiles(lo, hi):
+    ys, xs = np.meshgrid(np.arange(lo[1], hi[1]), np.arange(lo[0], hi[0]), indexing="ij")
+    return xs.ravel(), ys.ravel()
+
+
+def _three_sigma_rect(u, v, r, tiles_x, tiles_y):
+    """render.py:472-473."""
+    lim = np.array([tiles_x, tiles_y])
+    lo = np.clip(np.trunc((np.array([u, v]) - r) / 16), 0, lim).astype(int)
+    hi = np.clip(np.trunc((np.array([u, v]) + r + 15) / 16), 0, lim).astype(int)
+    return lo, hi
+
+
+def _level_and_extents(co):
+    """The level L of {q <= L} <=> {alpha >= 1/255} (render.py:1019-1028) and the half extents of the level
+    set's axis-aligned bounding box, sqrt(L * Sigma_ii) with Sigma the inverse of the conic matrix."""
+    a, b, c, o = co
+    level = -2.0 * np.log((1 / 255.0) / o)
+    sigma = np.linalg.inv(np.array([[a, b], [b, c]]))
+    return level, np.sqrt(level * sigma[0, 0]), np.sqrt(level * sigma[1, 1])
+
+
+def _near_integer(x, tol=1e-4):
+    return abs(x - np.round(x)) < tol
+
+
+def _candidate_rect(u, v, ex, ey, tiles_x, tiles_y):
+    """gs3d.py:968-989 / render.py:1300-1310: tiles [trunc((c - e)/16), ceil((c + e)/16)) of the level set's
+    bounding box, clamped to the grid.  None when float32 could round an end to the other side of a tile edge."""
+    ends = [(u - ex) / 16, (v - ey) / 16, (u + ex) / 16, (v + ey) / 16]
+    if any(_near_integer(e) for e in ends):
+        return None
+    lim = np.array([tiles_x, tiles_y])
+    lo = np.clip(np.trunc(ends[:2]), 0, lim).astype(int)
+    hi = np.clip(np.ceil(ends[2:]), 0, lim).astype(int)
+    return lo, hi
+
+
+@pytest.mark.parametrize("make", _TWO_SIDED_SCENES)
+def test_aabb_filter_is_exactly_the_level_set_bounding_box(oracle, make):
+    """gs3d.py:710-742, 968-989; render.py:1300-1310: AABB keeps a tile of the 3-sigma rect iff its closed box
+    [16x, 16x+16] x [16y, 16y+16] meets [u - ex, u + ex] x [v - ey, v + ey]."""
+    scene = make()
+    ref = oracle_forward(oracle, scene, AABB)[1]
+    sets = _tile_sets(ref, scene.n)
+    tiles_x, tiles_y = (scene.width + 15) // 16, (scene.height + 15) // 16
+    uv, co = ref["uvs"].astype(np.float64), ref["conic_opacity"].astype(np.float64)
+    decided = dropped = 0
+    for g in np.flatnonzero(ref["radii"] > 0):
+        u, v = uv[g]
+        level, ex, ey = _level_and_extents(co[g])
+        lo, hi = _three_sigma_rect(u, v, float(ref["radii"][g]), tiles_x, tiles_y)
+        xs, ys = _rect_tiles(lo, hi)
+        # signed gaps between the two intervals on each axis: overlap iff both <= 0
+        gx = np.maximum(16.0 * xs - (u + ex), (u - ex) - (16.0 * xs + 16))
+        gy = np.maximum(16.0 * ys - (v + ey), (v - ey) - (16.0 * ys + 16))
+        gap = np.maximum(gx, gy)
+        sure = np.abs(gap) > 1e-3 * max(ex, ey, 1.0)
+        # gaps a hair away on the OTHER axis can flip the decision too
+        sure &= (np.abs(gx) > 1e-3 * max(ex, 1.0)) & (np.abs(gy) > 1e-3 * max(ey, 1.0))
+        want = {int(t) for t in (ys * tiles_x + xs)[sure & (gap < 0)]}
+        unsure = {int(t) for t in (ys * tiles_x + xs)[~sure]}
+        got = sets[g]
+        assert got - unsure == want, (g, sorted(got - unsure), sorted(want))
+        decided += int(sure.sum())
+        dropped += int((sure & (gap > 0)).sum())
+    assert decided > 3000 and dropped > 100
+
+
+def _obb_gaps(co, u, v, xs, ys):
+    """Separating-axis gaps (positive = separated on that axis) between the closed tile boxes and the oriented
+    bounding rectangle of {q <= L}: centre (u, v), axes = eigenvectors of the conic matrix (numpy.linalg.eigh),
+    half lengths sqrt(L / eigenvalue).  Returns [tiles, 4]."""
+    a, b, c, o = co
+    level = -2.0 * np.log((1 / 255.0) / o)
+    lam, vec = np.linalg.eigh(np.array([[a, b], [b, c]]))
+    half = np.sqrt(level / lam)                            # half lengths along vec[:, 0], vec[:, 1]
+    d = np.stack([16.0 * xs + 8 - u, 16.0 * ys + 8 - v], 1)   # box centres relative to the rectangle's centre
+    axes = np.array([[1.0, 0.0], [0.0, 1.0], vec[:, 0], vec[:, 1]])
+    box_r = 8.0 * np.abs(axes).sum(1)                      # projected half extent of a 16 x 16 box
+    rect_r = np.abs(axes @ vec) @ half                     # ... of the rectangle
+    return np.abs(d @ axes.T) - (box_r + rect_r)[None, :]
+
+
+@pytest.mark.parametrize("make", _TWO_SIDED_SCENES)
+def test_obb_filter_is_exactly_the_oriented_bounding_rectangle(oracle, make):
+    """gs3d.py:745-791, 981-987, 1254-1322; render.py:1300-1310: OBB keeps a tile of (candidate rect of the
+    level set's bounding box) n (3-sigma rect) iff its closed box meets the oriented bounding rectangle of the
+    level set.  ELLIPSE keeps a subset of it."""
+    scene = make()
+    ref = oracle_forward(oracle, scene, OBB)[1]
+    sets = _tile_sets(ref, scene.n)
+    sets_ell = _tile_sets(oracle_forward(oracle, scene, ELLIPSE)[1], scene.n)
+    sets_aabb = _tile_sets(oracle_forward(oracle, scene, AABB)[1], scene.n)
+    tiles_x, tiles_y = (scene.width + 15) // 16, (scene.height + 15) // 16
+    uv, co = ref["uvs"].astype(np.float64), ref["conic_opacity"].astype(np.float64)
+    decided = dropped = tighter_than_aabb = 0
+    for g in np.flatnonzero(ref["radii"] > 0):
+        assert sets_ell[g] <= sets[g], g                    # the ellipse lies inside its oriented rectangle
+        u, v = uv[g]
+        a, b, c, _ = co[g]
+        if abs(b) < 1e-6 * max(a, c) and abs(a - c) < 1e-6 * max(a, c):
+            continue                                        # isotropic: no axis (own test below)
+        level, ex, ey = _level_and_extents(co[g])
+        cand = _candidate_rect(u, v, ex, ey, tiles_x, tiles_y)
+        if cand is None:
+            continue
+        lo3, hi3 = _three_sigma_rect(u, v, float(ref["radii"][g]), tiles_x, tiles_y)
+        lo, hi = np.maximum(cand[0], lo3), np.minimum(cand[1], hi3)
+        assert all((t % tiles_x >= lo[0]) and (t % tiles_x < hi[0]) and (t // tiles_x >= lo[1]) and
+                   (t // tiles_x < hi[1]) for t in sets[g]), g
+        if (hi <= lo).any():
+            assert not sets[g]
+            continue
+        xs, ys = _rect_tiles(lo, hi)
+        gaps = _obb_gaps(co[g], u, v, xs, ys)
+        scale = max(np.sqrt(level / min(np.linalg.eigvalsh(np.array([[a, b], [b, c]])))), 8.0)
+        sure = (np.abs(gaps) > 1e-3 * scale).all(1)
+        meets = (gaps < 0).all(1)
+        ids = ys * tiles_x + xs
+        want = {int(t) for t in ids[sure & meets]}
+        unsure = {int(t) for t in ids[~sure]}
+        assert sets[g] - unsure == want, (g, sorted(sets[g] - unsure), sorted(want))
+        decided += int(sure.sum())
+        dropped += int((sure & ~meets).sum())
+        tighter_than_aabb += len(sets_aabb[g] - sets[g])
+    assert decided > 3000 and dropped > 100 and tighter_than_aabb > 50
+
+
+def test_obb_without_an_axis_keeps_every_candidate_tile(oracle):
+    """An isotropic conic has no major axis: the reference normalises a zero vector (gs3d.py:761-791), sine and
+    cosine are NaN, every `<=` of the separating-axis test (gs3d.py:1254-1322) is false and every tile of the
+    candidate rect is kept, the corner tiles the circle does not reach included.  An on-axis isotropic gaussian
+    seen by a camera with fx == fy projects to such a conic."""
+    import dataclasses
+    base = gen_scene(0, n=4)
+    xyz = np.array([[0, 0, 3.0], [0, 0, 5.0], [0.4, -0.3, 4.0], [0, 0, 2.0]], np.float32)
+    scale = np.log(np.array([[0.4] * 3, [0.72] * 3, [0.5, 0.04, 0.1], [0.2] * 3], np.float32))
+    quat = np.array([[0, 0, 0, 1.0]] * 4, np.float32)
+    quat[2] = [0, 0, np.sin(np.pi / 8), np.cos(np.pi / 8)]      # long axis along the image diagonal
+    scene = dataclasses.replace(base, xyz=xyz, scale=scale, quaternion_xyzw=quat,
+                                opacity=np.full(4, 3.0, np.float32))
+    refs = {f: oracle_forward(oracle, scene, f)[1] for f in (AABB, ELLIPSE, OBB, DFVT)}
+    sets = {f: _tile_sets(refs[f], 4) for f in refs}
+    co = refs[OBB]["conic_opacity"]
+    for g in (0, 1, 3):
+        assert co[g, 0] == co[g, 2] and co[g, 1] == 0 and refs[OBB]["radii"][g] > 0
+        assert sets[OBB][g] == sets[AABB][g] == sets[DFVT][g]
+        assert len(sets[OBB][g] - sets[ELLIPSE][g]) >= 2, g     # corners of the box the circle leaves out
+    assert sets[OBB][2] < sets[AABB][2]      # the anisotropic one is still filtered
