@@ -279,8 +279,9 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     asm volatile("" : : "v"(before));
     long long off = !in_range ? end : (j == 0 ? 0 : before);   // lanes past the end: an empty range at the total
     // a gaussian with no tiles has an empty slot range; a caller that passed a smaller buffer than
-    // the scan total must never be written past
-    const bool active = in_range && sane && end > off && end <= m;
+    // the scan total must never be written past, and offsets that wrapped (a view with more than 2^31 - 1 pairs
+    // has negative 32-bit prefix sums) must not be written in front of the buffer either
+    const bool active = in_range && sane && off >= 0 && end > off && end <= m;
     const uint32_t dbits = ordered_depth_keys ? ordered_depth_keys[j] : reference_depth_bits(P, depths[i]);
     // the preprocess kernel's record of the kept tiles, when it was asked to write one
     unsigned long long kept = 0ull, meta = 0ull;
@@ -297,7 +298,8 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
     // coalesced segments: consecutive lanes write consecutive slots, stepping over the runs of the (few, large)
     // gaussians that are walked again below.  Each packed element carries the lane it came from, which gives its
     // slot: the lane's first slot plus the element's place in the lane's run.
-    const int my_cnt = (active && has_mask) ? (int)(end - off) : 0;
+    // a mask names at most 64 tiles; the bound keeps the wave's packed total small whatever the offsets hold
+    const int my_cnt = (active && has_mask) ? (int)min(end - off, 64ll) : 0;
     int incl = my_cnt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
