@@ -46,14 +46,23 @@ def per_gaussian_rel_err(a, b):
     return (np.linalg.norm(a - b, axis=1) / (rn + 1e-6 * rn.max()))[rn > 0]
 
 
-def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11, state_ulps=0.0):
+def rel_err_summary(e):
+    """(median, 99th percentile, maximum, share of gaussians beyond 1e-4) of per-gaussian relative errors."""
+    if e.size == 0:
+        return 0.0, 0.0, 0.0, 0.0
+    med, p99 = np.quantile(e, [0.5, 0.99])
+    return float(med), float(p99), float(e.max()), float((e > 1e-4).mean())
+
+
+def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11, state_ulps=0.0, tail=False):
     """What rounding noise in the blend backward's sums does to the preprocess backward, measured on the
     oracle.  A float32 sum of the per-pixel terms, in whatever order, carries an error of the order of
     2^-24 * sum|terms| ("absmass", which the oracle returns next to its float64 sums).  The oracle's own
     preprocess backward is run again on the screen-space gradients perturbed by N(0, 1) * ulps * 2^-24 * absmass;
     returned: {gradient name: (median, 99th percentile)} of the per-gaussian relative error it induces.  The
     spread beyond the input noise is the conditioning of the chain rule itself (near-degenerate projected
-    covariances: gradients that are small differences of large terms)."""
+    covariances: gradients that are small differences of large terms).  With tail=True each entry is
+    (median, 99th percentile, maximum, share of gaussians beyond 1e-4) instead."""
     rng = np.random.default_rng(seed)
     # state_ulps: on top of that, noise of state_ulps * 2^-24 * statemass in duv / dconic / dopacity, for a
     # backward whose per-pixel colour state is rounded differently from the oracle's (the per-gaussian algorithm)
@@ -66,5 +75,7 @@ def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11, state_ul
     pert = O.preprocess_bwd(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
                             ref["radii"], ref["cov2d_vecs"], ref["sh_to_rgb_ne_0"],
                             *(noisy[k].astype(np.float32) for k in ("duv", "dconic", "dopacity", "dcolor")))
-    return {k: tuple(np.quantile(per_gaussian_rel_err(pert[k], pb_ref[k]), [0.5, 0.99]))
-            for k in ("dxyz", "dquat", "dscale", "dopacity", "dsh")}
+    names = ("dxyz", "dquat", "dscale", "dopacity", "dsh")
+    if tail:
+        return {k: rel_err_summary(per_gaussian_rel_err(pert[k], pb_ref[k])) for k in names}
+    return {k: tuple(np.quantile(per_gaussian_rel_err(pert[k], pb_ref[k]), [0.5, 0.99])) for k in names}

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from helpers import (gen_scene, grad_close, k9_noise_spread, op_config, oracle_forward, per_gaussian_rel_err,
-                     torch_model)
+                     rel_err_summary, torch_model)
 
 pytestmark = pytest.mark.gpu
 
@@ -153,16 +153,25 @@ def test_backward_parity(oracle, cfg_id, n, wh, filt, views):
     # covariances.  The bar is what the oracle's own preprocess backward does with such noise on this very
     # scene (k9_noise_spread: inputs perturbed by N(0,1) * 2 * 2^-24 * sum|terms|): the per-gaussian relative
     # error's median and 99th percentile must stay within twice the spread that noise induces.
-    spread = k9_noise_spread(oracle, P, scene, ref, g_ref, pb_ref)
+    # The tail is recorded as well: the largest per-gaussian relative error and the share of gaussians beyond an
+    # elementwise 1e-4, for the GPU chain and for the noise model; the GPU's share must not exceed twice the model's
+    # (plus five gaussians, for shares of a handful).
+    spread = k9_noise_spread(oracle, P, scene, ref, g_ref, pb_ref, tail=True)
     for name, got in (("dxyz", gm.xyz), ("dquat", gm.quaternion_xyzw), ("dscale", gm.scale),
                       ("dopacity", gm.opacity), ("dsh", gm.color_sh)):
         a = cpu(got).astype(np.float64).reshape(scene.n, -1)
         b = pb_ref[name].astype(np.float64).reshape(scene.n, -1)
-        med, p99 = np.quantile(per_gaussian_rel_err(a, b), [0.5, 0.99])
-        m_med, m_p99 = spread[name]
+        e = per_gaussian_rel_err(a, b)
+        med, p99, worst, share = rel_err_summary(e)
+        m_med, m_p99, m_worst, m_share = spread[name]
+        print(f"  chain tail cfg={cfg_id} n={scene.n} {name}: gpu median {med:.2e} p99 {p99:.2e} max {worst:.2e} "
+              f"beyond-1e-4 {share:.2e} | noise model median {m_med:.2e} p99 {m_p99:.2e} max {m_worst:.2e} "
+              f"beyond-1e-4 {m_share:.2e}", flush=True)
         assert med <= 2 * m_med and p99 <= 2 * m_p99, \
             f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}; noise model {m_med:.2e} {m_p99:.2e}"
         assert med <= 1e-5 and p99 <= 2e-3
+        assert share * e.size <= 2 * m_share * e.size + 5, \
+            f"{name}: {share * e.size:.0f} gaussians beyond 1e-4, the noise model has {m_share * e.size:.0f}"
         assert not (np.abs(a[np.linalg.norm(b, axis=1) == 0]) > 0).any(), \
             f"{name}: gradient on a gaussian the oracle leaves at zero"
 

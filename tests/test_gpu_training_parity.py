@@ -1,0 +1,195 @@
+"""The callers either side of the rasterizer, compared with the oracle's chain (not just for their properties):
+
+* one ``Trainer.train_step`` (d3sim/algos/d3gs/train.py:162-177: render with a gradient holder, L1 + D-SSIM,
+  ``loss.backward()``, Adam step, densification statistics from the holder's gradient,
+  origin/strategy.py:75-122).  The image must be the oracle's bit for bit; the loss gradient torch forms in
+  float32 on the GPU must agree with the same loss evaluated in float64 on the oracle's image; and the model
+  gradients the optimizer receives must be the oracle's blend backward + preprocess backward of that gradient, to
+  the bars of ``test_gpu_parity.test_backward_parity``; the holder's gradient must be the oracle's ``duv``.
+* an Inria-layout point cloud (tools.py:20-62) written by the test itself, loaded with ``load_3dgs_origin_model``
+  and rendered: image bit-identical to the oracle on the arrays the file holds.
+"""
+import numpy as np
+import pytest
+
+from helpers import (gen_scene, grad_close, k9_noise_spread, op_config, oracle_forward, oracle_params,
+                     per_gaussian_rel_err, torch_model)
+
+pytestmark = pytest.mark.gpu
+
+DFVT = 4
+
+
+def _target_image(oracle, scene, filt):
+    """A plausible ground-truth picture: the same gaussians with other colours and opacities, clamped to [0, 1]."""
+    import dataclasses
+    other = dataclasses.replace(scene, color_sh=(scene.color_sh * np.float32(0.7) + np.float32(0.05)).astype(np.float32),
+                                opacity=(scene.opacity - np.float32(0.3)).astype(np.float32))
+    return np.clip(oracle_forward(oracle, other, filt)[1]["color"], 0.0, 1.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("cfg_id,n,wh", [(1, 20000, (256, 256)), (2, 60000, (480, 270))])
+def test_train_step_gradients_match_the_oracle_chain(oracle, cfg_id, n, wh):
+    import torch
+    from d3gs_research_amd import config_def, train
+    from d3gs_research_amd.render import GaussianSplatOp
+
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    print(f"train step parity cfg={cfg_id} n={scene.n} wh={wh}", flush=True)
+    cam = scene.camera()
+    gt = _target_image(oracle, scene, DFVT)                                   # [H, W, 3]
+    gt_nchw = torch.from_numpy(np.ascontiguousarray(gt.transpose(2, 0, 1)[None])).cuda()
+
+    model = torch_model(scene)
+    cfg = config_def.Train()
+    trainer = train.Trainer(model, GaussianSplatOp(op_config(scene, DFVT)), cfg, scene_scale=2.0)
+
+    # taps on the step, none of which changes what it computes: the image handed to the loss keeps its gradient,
+    # the optimizer's gradients are copied before Adam consumes them, the densification update shows its input
+    seen = {}
+    real_loss, real_step, real_update = train.photometric_loss, trainer.optim.step, trainer.strategy.update
+
+    def loss_tap(color_nchw, gt_image, lam):
+        color_nchw.retain_grad()
+        seen["color_nchw"] = color_nchw
+        return real_loss(color_nchw, gt_image, lam)
+
+    def step_tap(*a, **k):
+        for group in trainer.optim.param_groups:
+            seen[group["name"]] = group["params"][0].grad.detach().clone()
+        return real_step(*a, **k)
+
+    def update_tap(state, out, duv):
+        seen["holder_grad"] = duv.detach().clone()
+        return real_update(state, out, duv)
+
+    train.photometric_loss, trainer.optim.step, trainer.strategy.update = loss_tap, step_tap, update_tap
+    try:
+        before = {k: v.detach().clone() for k, v in model.get_proxy_field_dict().items()}
+        res = trainer.train_step(cam, gt_nchw)
+    finally:
+        train.photometric_loss = real_loss
+    torch.cuda.synchronize()
+    cpu = lambda t: t.detach().cpu().numpy()
+
+    # ---- forward: the step's image is the oracle's
+    P, ref = oracle_forward(oracle, scene, DFVT)
+    assert np.array_equal(cpu(res.output.color)[0].view(np.uint32), ref["color"].view(np.uint32))
+
+    # ---- the loss and its gradient: float32 on the GPU against float64 on the oracle's image
+    img64 = torch.tensor(ref["color"], dtype=torch.float64).permute(2, 0, 1)[None].contiguous().requires_grad_(True)
+    loss64 = train.photometric_loss(img64, torch.tensor(gt, dtype=torch.float64).permute(2, 0, 1)[None].contiguous(),
+                                    cfg.lambda_dssim)
+    loss64.backward()
+    dimg64 = img64.grad[0].permute(1, 2, 0).numpy()                            # [H, W, 3]
+    assert abs(res.loss - float(loss64.detach())) <= 1e-5 * float(loss64.detach())
+    dimg_gpu = cpu(seen["color_nchw"].grad)[0].transpose(1, 2, 0)
+    # torch's float32 SSIM (variances formed as E[x^2] - mu^2 out of 11 x 11 convolutions) against float64: each value
+    # within 1e-4 relative plus 1e-4 of the largest (measured: 77 of 196 608 values beyond 3e-5 of the largest, none
+    # beyond 7e-5)
+    ok, worst, nbad = grad_close(dimg_gpu, dimg64, rel=1e-4, abs_frac=1e-4)
+    print(f"  loss {res.loss:.6f} (float64 {float(loss64.detach()):.6f}); dL/dimage worst {worst:.2f}x of its bar", flush=True)
+    assert ok, f"dL/dimage: {nbad} pixels outside tolerance (worst {worst:.2f}x)"
+
+    # ---- backward, link by link on identical inputs: the oracle's K7 + K9 of the very gradient the GPU used
+    drgb = np.ascontiguousarray(dimg_gpu, np.float32)
+    dT = np.zeros((scene.height, scene.width), np.float32)
+    g_ref, pb_ref = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                    scene.color_sh, drgb, dT)
+    holder = cpu(seen["holder_grad"]).astype(np.float64)
+    assert holder.shape == (1, scene.n, 2)
+    excess = np.abs(holder[0] - g_ref["duv"]) - (1e-4 * g_ref["absmass"][:, 0:2] + 1e-30)
+    assert (excess <= 0).all(), f"holder gradient: {int((excess > 0).sum())} values beyond 1e-4 * sum|terms|"
+    ok, worst, nbad = grad_close(holder[0], g_ref["duv"])
+    assert ok, f"holder gradient vs oracle duv: {nbad} outside tolerance (worst {worst:.2f}x)"
+
+    spread = k9_noise_spread(oracle, P, scene, ref, g_ref, pb_ref)
+    for name, key in (("dxyz", "xyz"), ("dquat", "quaternion_xyzw"), ("dscale", "scale"), ("dopacity", "opacity"),
+                      ("dsh", "color_sh")):
+        a = cpu(seen[key]).astype(np.float64).reshape(scene.n, -1)
+        b = pb_ref[name].astype(np.float64).reshape(scene.n, -1)
+        med, p99 = np.quantile(per_gaussian_rel_err(a, b), [0.5, 0.99])
+        m_med, m_p99 = spread[name]
+        print(f"  {name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e} (noise model {m_med:.2e} {m_p99:.2e})",
+              flush=True)
+        assert med <= 2 * m_med and p99 <= 2 * m_p99, \
+            f"{name}: per-gaussian relative error median {med:.2e} p99 {p99:.2e}; noise model {m_med:.2e} {m_p99:.2e}"
+        assert med <= 1e-5 and p99 <= 2e-3
+        assert not (np.abs(a[np.linalg.norm(b, axis=1) == 0]) > 0).any(), f"{name}: gradient where the oracle has none"
+
+    # ---- end to end: float64 loss gradient through the oracle against what the optimizer received
+    g64, pb64 = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity,
+                                scene.color_sh, np.ascontiguousarray(dimg64, np.float32), dT)
+    for name, key in (("dxyz", "xyz"), ("dscale", "scale"), ("dopacity", "opacity"), ("dsh", "color_sh")):
+        a = cpu(seen[key]).astype(np.float64).reshape(scene.n, -1)
+        b = pb64[name].astype(np.float64).reshape(scene.n, -1)
+        med = float(np.median(per_gaussian_rel_err(a, b)))
+        print(f"  {name}: end to end (float64 loss on the CPU) median relative error {med:.2e}", flush=True)
+        assert med <= 1e-4
+
+    # ---- and the step was taken: Adam moved every parameter that has a gradient, the statistics saw the view
+    moved = {k: float((getattr(model, k).detach() - before[k]).abs().max()) for k in before}
+    assert all(v > 0 for v in moved.values()), moved
+    seen_view = cpu(res.output.radii).reshape(-1) > 0
+    assert np.array_equal(cpu(trainer.state.count) > 0, seen_view)
+    want_len = np.linalg.norm(holder[0] * np.array([0.5 * scene.width, 0.5 * scene.height]), axis=-1) * seen_view
+    assert np.allclose(cpu(trainer.state.duv_ndc_length), want_len, rtol=1e-5, atol=1e-12)
+
+
+NAMES = ["x", "y", "z", "nx", "ny", "nz"] + [f"f_dc_{i}" for i in range(3)] + [f"f_rest_{i}" for i in range(45)] + \
+        ["opacity"] + [f"scale_{i}" for i in range(3)] + [f"rot_{i}" for i in range(4)]
+
+
+@pytest.mark.parametrize("split,fused", [(True, True), (False, True), (True, False)])
+def test_inria_point_cloud_renders_like_the_oracle(oracle, tmp_path, split, fused):
+    """The file is written here property by property in the Inria order (origin/data/scene/gaussian_model.py:177-208:
+    f_rest channel-major, rotation w x y z, raw log-scale and logit); what `load_3dgs_origin_model` makes of it
+    must render to the oracle's image of the scene's own arrays, bit for bit."""
+    import torch
+    from d3gs_research_amd import tools
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(1, n=30000, wh=(320, 240))
+    n = scene.n
+    col = {"x": scene.xyz[:, 0], "y": scene.xyz[:, 1], "z": scene.xyz[:, 2], "opacity": scene.opacity}
+    for k in ("nx", "ny", "nz"):
+        col[k] = np.zeros(n, np.float32)
+    for c in range(3):
+        col[f"f_dc_{c}"] = scene.color_sh[:, 0, c]
+        col[f"scale_{c}"] = scene.scale[:, c]
+        for k in range(15):
+            col[f"f_rest_{c * 15 + k}"] = scene.color_sh[:, k + 1, c]
+    for i, src in enumerate((3, 0, 1, 2)):                      # file order w, x, y, z
+        col[f"rot_{i}"] = scene.quaternion_xyzw[:, src]
+    table = np.stack([col[name] for name in NAMES], axis=1).astype("<f4")
+    path = str(tmp_path / "point_cloud.ply")
+    with open(path, "wb") as f:
+        f.write(("ply\nformat binary_little_endian 1.0\nelement vertex %d\n" % n +
+                 "".join(f"property float {name}\n" for name in NAMES) + "end_header\n").encode())
+        f.write(table.tobytes())
+
+    model = tools.load_3dgs_origin_model(path, fused=fused, split=split, device="cuda")
+    assert len(model) == n and model.cur_sh_degree == 3 and (model.color_sh_base is not None) == split
+    op = GaussianSplatOp(op_config(scene, DFVT))
+    cpu = lambda t: t.detach().cpu().numpy()
+    if fused:
+        P = oracle_params(oracle, scene, DFVT, training=False)
+        quat, scale, opacity = scene.quaternion_xyzw, scene.scale, scene.opacity
+        render_model = model.create_model_with_act()            # raw tensors: the kernels apply the activations
+    else:                                                       # torch applies the activations, the kernels see the results
+        render_model = model.create_model_with_act()
+        P = oracle_params(oracle, scene, DFVT, training=False)
+        P.fused_activation = 0
+        quat, scale, opacity = cpu(render_model.quaternion_xyzw), cpu(render_model.scale), cpu(render_model.opacity)
+    if split:
+        P.has_sh_base, P.sh_stride = 1, 15
+        ref = oracle.forward(P, scene.xyz, quat, scale, opacity, np.ascontiguousarray(scene.color_sh[:, 1:]),
+                             sh_base=np.ascontiguousarray(scene.color_sh[:, 0]))
+    else:
+        ref = oracle.forward(P, scene.xyz, quat, scale, opacity, scene.color_sh)
+    with torch.no_grad():
+        out, _ = op.forward(render_model, scene.camera(), training=False)
+    torch.cuda.synchronize()
+    assert ref["num_rendered"] > 100000
+    assert np.array_equal(cpu(out.radii), ref["radii"])
+    assert np.array_equal(cpu(out.color)[0].view(np.uint32), ref["color"].view(np.uint32))
+    assert np.array_equal(cpu(out.T)[0].view(np.uint32), ref["T"].view(np.uint32))
