@@ -47,6 +47,26 @@ __device__ __forceinline__ const StagedGaussian& staged_at(const StagedGaussian*
     return *reinterpret_cast<const StagedGaussian*>(reinterpret_cast<const char*>(base) + off);
 }
 
+// Timing-only builds (csrc/Makefile, target timing-variants; never what the tests or the operator load): they
+// price two parts of a visit by leaving them out, at the cost of wrong results.
+//   D3GS_TIMING_ONLY_HW_EXP        exp as v_mul + v_exp_f32 (the hardware's rounding, which no CPU reproduces)
+//   D3GS_TIMING_ONLY_NO_REDUCTION  the backward's ten per-lane terms are formed and kept alive, the wave reduction
+//                                  is left out (the LDS atomic adds one lane's value)
+//   D3GS_TIMING_ONLY_NO_VISITS     backward only (it walks as far as the forward's n_contrib says, so the forward
+//                                  stays exact): no gaussian is visited; what is left is the prologue, the staging
+//                                  rounds with their barriers and the flush
+//   D3GS_TIMING_ONLY_LDS_PAD=bytes backward only, results unchanged: extra LDS per workgroup, so that fewer
+//                                  workgroups share a compute unit (7 fit as built; 8192 more leave 5, 16384 leave 4)
+//   D3GS_TIMING_ONLY_POWER_ONLY    backward only: every visit ends behind its first test (mask walk, record read,
+//                                  power, compares)
+__device__ __forceinline__ float blend_expf(float power) {
+#ifdef D3GS_TIMING_ONLY_HW_EXP
+    return __builtin_amdgcn_exp2f(power * 1.44269504088896341f);
+#else
+    return det_expf_inrange(power);
+#endif
+}
+
 // power = -1/2 (a dx^2 + c dy^2) - b dx dy (render.py:1765-1767) as a fixed sequence of three
 // multiplies and two fused multiply-adds; a CPU evaluating the same sequence gets the same bits.
 __device__ __forceinline__ float blend_power(const StagedGaussian& g, float dx, float dy) {
@@ -415,7 +435,7 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
                 // never selected.
                 // no overflow guard: beyond exp's range the product o * G is inf, huge or NaN, and
                 // fminf(0.99, .) gives 0.99 in every case, as it does for the guarded exp's inf
-                const float G = det_expf_inrange(power);
+                const float G = blend_expf(power);
                 const float alpha = fminf(0.99f, sg.o * G);
                 const unsigned long long hit_m = live_m & __builtin_amdgcn_fcmpf(alpha, P.alpha_eps, kFcmpOge);
                 const float nextT = T * (1.0f - alpha);
@@ -483,6 +503,11 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     __shared__ float s_grad[kValues][kBlock + 1];
     __shared__ int s_wmax[4];
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
+#ifdef D3GS_TIMING_ONLY_LDS_PAD
+    // fewer workgroups fit a compute unit: how the duration follows the number of resident wavefronts
+    __shared__ int s_pad[D3GS_TIMING_ONLY_LDS_PAD / 4];
+    if (P.n < 0) s_pad[threadIdx.x] = blockIdx.x;
+#endif
 
     const int ntiles = P.tiles_x * P.tiles_y * batch_count(P);
     const int items = item_count(P);
@@ -563,6 +588,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
         for (int chunk = 0; chunk < 4 && chunk * 64 < cnt; ++chunk) {
           unsigned long long m = uniform_u64(s_mask[wave][chunk]);
           if (cnt - chunk * 64 < 64) m &= (1ull << (cnt - chunk * 64)) - 1ull;
+#ifdef D3GS_TIMING_ONLY_NO_VISITS
+          m = 0ull;
+#endif
           if (!m) continue;
           while (m) {
             const int j = chunk * 64 + __builtin_ctzll(m);
@@ -572,9 +600,15 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float power = blend_power(sg, dx, dy);
             // Per-lane conditions as 64-bit lane masks (one compare instruction each, combined with scalar
             // instructions; ordered compares, a NaN fails them as it fails the C operators they stand for).
+#ifdef D3GS_TIMING_ONLY_POWER_ONLY
+            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBlock + j, contributor, kIcmpSlt) &
+                                              __builtin_amdgcn_fcmpf(power, 1.0e30f, kFcmpOge) &
+                                              __builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOle);
+#else
             const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBlock + j, contributor, kIcmpSlt) &
                                               __builtin_amdgcn_fcmpf(power, sg.thr, kFcmpOge) &
                                               __builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOle);
+#endif
             if (cand_m == 0) continue;
             // power, exp and alpha repeat the forward's exact sequence: they decide which pixels the
             // gaussian contributed to.  From here on every lane runs the same instructions: a lane the
@@ -582,7 +616,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             // (T, colour behind) untouched and makes all of its terms exact zeros, so no lane masking
             // or zero-filling is needed.  (exp of a non-candidate lane's power may be garbage; it is
             // discarded by the select.)
-            const float G0 = det_expf_inrange(power);   // candidates have power in [thr, 0]
+            const float G0 = blend_expf(power);   // candidates have power in [thr, 0]
             const float alpha0 = fminf(0.99f, sg.o * G0);
             const unsigned long long valid_m = cand_m & __builtin_amdgcn_fcmpf(alpha0, P.alpha_eps, kFcmpOge);
             if (valid_m == 0) continue;
@@ -630,7 +664,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             const float g7 = w * dr1;
             const float g8 = w * dr2;
             // the wave totals land in different lanes: one LDS atomic instruction adds them all
+#ifdef D3GS_TIMING_ONLY_NO_REDUCTION
+            asm volatile("" : : "v"(g0), "v"(g1), "v"(g2), "v"(g3), "v"(g4), "v"(g5), "v"(g6), "v"(g7), "v"(g8), "v"(g9));
+            const float total = g5;
+#else
             const float total = wave_reduce10<kDepth>(g0, g1, g2, g3, g4, g5, g6, g7, g8, g9);
+#endif
             if (slot >= 0) atomicAdd(&s_grad[slot][j], total);
           }
         }

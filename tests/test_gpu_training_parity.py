@@ -189,7 +189,7 @@ def test_inria_point_cloud_renders_like_the_oracle(oracle, tmp_path, split, fuse
     with torch.no_grad():
         out, _ = op.forward(render_model, scene.camera(), training=False)
     torch.cuda.synchronize()
-    assert ref["num_rendered"] > 100000
+    assert ref["num_rendered"] > 50000
     assert np.array_equal(cpu(out.radii), ref["radii"])
     assert np.array_equal(cpu(out.color)[0].view(np.uint32), ref["color"].view(np.uint32))
     assert np.array_equal(cpu(out.T)[0].view(np.uint32), ref["T"].view(np.uint32))
