@@ -167,6 +167,9 @@ def main():
     ap.add_argument("--late-gradient-clear", action="store_true",
                     help="let the preprocess backward write the zero gradients itself instead of clearing the arrays "
                          "beside the forward pass (for comparison)")
+    ap.add_argument("--op-set", action="append", default=[], metavar="ATTR=0|1",
+                    help="set a boolean switch of the operator for an A/B run, e.g. "
+                         "overlap_sh_colors=0, poll_pair_count=0, fused_binning=0 (repeatable); the headline runs with the defaults")
     ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="only run a plain 256 MiB -> 256 MiB elementwise copy 5 times (reference reading for "
@@ -197,6 +200,10 @@ def main():
     cams = [cam] + orbit_cameras(scene, args.views - 1)
     op = GaussianSplatOp(scene_config(scene, filt, rasterize_backward_algo=RasterizeBackwardAlgo[args.backward_algo]))
     op.clear_gradients_early = not args.late_gradient_clear
+    for item in args.op_set:
+        name, _, value = item.partition("=")
+        assert hasattr(op, name) and isinstance(getattr(op, name), bool), f"--op-set: the operator has no switch {name!r}"
+        setattr(op, name, bool(int(value)))
     model = scene_model(scene, "cuda:0")
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
 
@@ -378,7 +385,8 @@ def main():
                    "image": f"{scene.width}x{scene.height}", "early_filter_algo": filt.name,
                    "rasterize_backward_algo": args.backward_algo, "pairs_M": int(M),
                    "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists,
-                   "gaussians_with_gradient": active, "views": views_info},
+                   "gaussians_with_gradient": active, "views": views_info,
+                   **({"op_set": args.op_set} if args.op_set else {})},
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
         "gpu_stage_sum_ms": round(gpu_sum, 4),
         "stages": stages,

@@ -57,6 +57,8 @@ __device__ __forceinline__ const StagedGaussian& staged_at(const StagedGaussian*
 //                                  rounds with their barriers and the flush
 //   D3GS_TIMING_ONLY_LDS_PAD=bytes backward only, results unchanged: extra LDS per workgroup, so that fewer
 //                                  workgroups share a compute unit (7 fit as built; 8192 more leave 5, 16384 leave 4)
+//   D3GS_TIMING_ONLY_NO_FLUSH      backward only: a round ends behind its visits (no moments -> gradients step, no
+//                                  flush of the tile's sums to the records)
 //   D3GS_TIMING_ONLY_POWER_ONLY    backward only: every visit ends behind its first test (mask walk, record read,
 //                                  power, compares)
 __device__ __forceinline__ float blend_expf(float power) {
@@ -674,6 +676,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
           }
         }
         __syncthreads();
+#ifdef D3GS_TIMING_ONLY_NO_FLUSH
+        continue;
+#endif
         const int flush_cnt = min(kBlock, block_todo - round * kBlock);
         if (tid < flush_cnt) {  // moments -> (duv, dconic) of gaussian tid, with a = -2 ha, b = -nb, c = -2 hc
             const StagedGaussian sg = s_g[tid];
