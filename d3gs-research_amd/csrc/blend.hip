@@ -230,8 +230,10 @@ __device__ __forceinline__ uint32_t stage_gaussian(const d3gs_params& P, int g, 
     const float err = 1.0e-6f * (co.x * X * X + co.z * Y * Y + 2.0f * fabsf(co.y) * X * Y);
     const float R = -2.0f * s.thr + 2.0f * err + 1.0e-3f;
     const float D = co.x * co.z - co.y * co.y;
-    // ill-conditioned conic (or not positive definite in float): no box, visit everywhere
-    if (!(D > 1.0e-4f * co.x * co.z) || !(R > 0.0f)) return 0xFu;
+    // ill-conditioned conic, or one that is not positive definite (a caller of the C ABI may hand over any conic;
+    // the box and the per-patch minimum below assume an ellipse): no cull, every patch visits it and the exact
+    // per-pixel sequence decides
+    if (!(co.x > 0.0f) || !(co.z > 0.0f) || !(D > 1.0e-4f * co.x * co.z) || !(R > 0.0f)) return 0xFu;
     const float hx = 1.01f * __fsqrt_rn(R * co.z / D) + 0.01f;
     const float hy = 1.01f * __fsqrt_rn(R * co.x / D) + 0.01f;
     const bool left = xy.x - hx <= tile_x0 + 7.0f, right = xy.x + hx >= tile_x0 + 8.0f;

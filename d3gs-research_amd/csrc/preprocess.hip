@@ -289,13 +289,15 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
 // neighbours, so there is nothing to stage); same operations as sh_colors_kernel.
 __global__ __launch_bounds__(kPrepBlock) void sh_colors_sparse_kernel(
     const d3gs_params P0, const int32_t* __restrict__ ids, const int32_t* __restrict__ batch_ids, const int count,
-    const float* __restrict__ xyz, const float* __restrict__ sh, const float* __restrict__ sh_base,
-    const int32_t* __restrict__ radii, float* __restrict__ rgb_out, uint8_t* __restrict__ ne0_out) {
+    const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ sh,
+    const float* __restrict__ sh_base, const int32_t* __restrict__ radii, float* __restrict__ rgb_out,
+    uint8_t* __restrict__ ne0_out) {
     const int slot = blockIdx.x * kPrepBlock + threadIdx.x;
     if (slot >= count) return;
     const int g = ids[slot];
     d3gs_params P = P0;
     if (P0.batch_size > 1) apply_batch_camera(P, batch_ids[slot]);
+    if (inst.ids && (unsigned)g < (unsigned)P0.n) apply_instance(P, inst, g, P0.batch_size > 1 ? batch_ids[slot] : 0);
     float rgb[3] = {0.0f, 0.0f, 0.0f};
     uint32_t ne0 = 0;
     if (radii[slot] > 0 && (unsigned)g < (unsigned)P0.n) {
@@ -847,7 +849,7 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         __syncthreads();
         if (tid < cnt) {
             d3gs_params Pg = P;
-            if constexpr (kInstances) apply_instance(Pg, inst, g);
+            if constexpr (kInstances) apply_instance(Pg, inst, origin ? origin[g] : g);      // ids are per model row
             preprocess_bwd_one(Pg, g, in, sh_mask_compat, accumulate != 0, dxyz, dquat, dscale, dopacity_out,
                                s_rows + tid * stride, dsh_base);
         }
@@ -964,7 +966,8 @@ extern "C" int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz
                                           int32_t* valid_flags, const int32_t* slot_scan, int32_t* sparse_gaussian_ids,
                                           int32_t* sparse_batch_ids, float* depths, int32_t* radii, float* uvs,
                                           float* conic_opacity, int32_t* tiles_touched, float* cov2d_vecs,
-                                          uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream) {
+                                          uint64_t* tile_masks, uint32_t* depth_sort_keys,
+                                          const d3gs_instances* instances, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_preprocess_fwd_sparse");
     if (rc) return rc;
     if (p->n == 0) return D3GS_OK;
@@ -980,7 +983,8 @@ extern "C" int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz
                   "buffers (second call)");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    const InstanceView inst = {nullptr, nullptr, 0};
+    InstanceView inst;
+    if (!instance_view(instances, &inst, "d3gs_preprocess_fwd_sparse")) return D3GS_ERR_INVALID_ARGUMENT;
     const SparseView sparse = {valid_flags, slot_scan, sparse_gaussian_ids, sparse_batch_ids};
     dim3 grid((item_count(*p) + kPrepBlock - 1) / kPrepBlock), block(kPrepBlock);
     hipLaunchKernelGGL((preprocess_fwd_kernel<false, true, true>), grid, block, 0, (hipStream_t)stream, *p, inst, sparse,
@@ -995,7 +999,8 @@ extern "C" int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz
 extern "C" int d3gs_sh_colors_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids,
                                      const int32_t* sparse_batch_ids, int32_t count, const float* xyz,
                                      const float* color_sh, const float* color_sh_base, const int32_t* radii,
-                                     float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream) {
+                                     float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, const d3gs_instances* instances,
+                                     d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_sh_colors_sparse");
     if (rc) return rc;
     if (count < 0) { set_error("d3gs_sh_colors_sparse: count < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
@@ -1005,8 +1010,10 @@ extern "C" int d3gs_sh_colors_sparse(const d3gs_params* p, const int32_t* sparse
         set_error("d3gs_sh_colors_sparse: NULL buffer");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
+    InstanceView inst;
+    if (!instance_view(instances, &inst, "d3gs_sh_colors_sparse")) return D3GS_ERR_INVALID_ARGUMENT;
     hipLaunchKernelGGL(sh_colors_sparse_kernel, dim3((count + kPrepBlock - 1) / kPrepBlock), dim3(kPrepBlock), 0,
-                       (hipStream_t)stream, *p, sparse_gaussian_ids, sparse_batch_ids, (int)count, xyz, color_sh,
+                       (hipStream_t)stream, *p, sparse_gaussian_ids, sparse_batch_ids, (int)count, inst, xyz, color_sh,
                        color_sh_base, radii, rgb_gaussian, sh_to_rgb_ne_0);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_sh_colors_sparse: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
@@ -1078,7 +1085,8 @@ extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* s
                                           const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
                                           int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
                                           float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
-                                          float* dcolor_sh_base, d3gs_stream_t stream) {
+                                          float* dcolor_sh_base, const d3gs_instances* instances,
+                                          d3gs_stream_t stream) {
     if (!sparse_gaussian_ids && p && p->n > 0) {
         set_error("d3gs_preprocess_bwd_sparse: sparse_gaussian_ids is NULL");
         return D3GS_ERR_INVALID_ARGUMENT;
@@ -1086,7 +1094,7 @@ extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* s
     return preprocess_bwd_impl("d3gs_preprocess_bwd_sparse", p, 0, 0, sparse_gaussian_ids, xyz, quaternion_xyzw, scale,
                                opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
                                outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
-                               nullptr, stream);
+                               instances, stream);
 }
 
 extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,

@@ -7,9 +7,11 @@ with ``forward`` (169-1015), ``rasterize_forward_backward`` (1329-2316) and
 text and JIT-compiles it, this module allocates with torch and calls the
 ahead-of-time HIP library through ``_capi`` on torch's current stream.
 
-Scope: one camera per call (batch 1), RGB output in NHWC, early filters NONE /
-AABB / OBB / OBB_DFVT (the latter computed as the OBB tile set), the default
-backward algorithm.  Options outside that scope raise ``NotImplementedError``.
+Scope: single cameras and camera bundles (one pass over B x N render items), every
+early filter (OBB_DFVT computed as the OBB tile set), RGB / RGBA / depth / custom
+feature channels in NHWC or NCHW, instances, sparse mode, both backward algorithms.
+The few options outside that scope (``render_inv_depth``, ``transmittance_is_double``,
+tile sizes other than 16 x 16, ``prep_user_inputs``) raise ``NotImplementedError``.
 """
 from __future__ import annotations
 
@@ -18,7 +20,11 @@ import copy
 import ctypes as C
 import dataclasses
 import math
+import os
 import time
+import types
+import warnings
+import weakref
 
 import numpy as np
 import torch
@@ -31,6 +37,41 @@ from .model import GaussianModelOriginBase, GaussianModelOriginFused
 
 def div_up(a: int, b: int) -> int:
     return (a + b - 1) // b
+
+
+# Parity tests compare the sorted keys with the oracle's; they switch this on (through the environment, before the
+# package is imported) so that an operator keeps the last view's sorted tile keys and indices alive.
+KEEP_SORTED_KEYS = os.environ.get("D3GS_KEEP_SORTED_KEYS", "0") not in ("", "0")
+# How long the host polls the pinned pair-count word before it falls back to synchronising the stream, and the
+# largest view (in pairs the buffers are sized for) whose count is polled at all.
+POLL_SECONDS = 0.02
+POLL_MAX_PAIRS = 1 << 26
+
+
+def poll_host_word(word, pending, seconds, synchronize, clock=time.perf_counter):
+    """Waits until ``word[0]`` (a pinned host word a kernel stores into) no longer holds ``pending``.  Returns
+    "polled" when the store showed up within ``seconds``; otherwise calls ``synchronize()`` (the stream has then run
+    dry) and returns "synced" when the word has changed by then, "never" when it still holds ``pending``."""
+    give_up = clock() + seconds
+    while int(word[0]) == pending:
+        if clock() > give_up:
+            synchronize()
+            return "never" if int(word[0]) == pending else "synced"
+    return "polled"
+
+
+@dataclasses.dataclass
+class _StreamSlot:
+    """What one forward pass at a time needs outside its own buffers, kept per (device, stream): the pinned host
+    words the kernels report into (the pair count; the two sorts' status on the launch-by-launch path), the pair
+    buffer size learnt from the stream's last view, and the side stream of the SH colours.  Two forwards of one
+    operator on two streams use two slots; two host threads on ONE stream would still race."""
+    count_host: torch.Tensor
+    count_np: np.ndarray            # the same word, read without a tensor operation
+    sort_status_host: torch.Tensor
+    pair_capacity: int = 0
+    poll_timeouts: int = 0          # consecutive views whose count did not arrive within the polling time
+    side_stream: torch.cuda.Stream | None = None
 
 
 @dataclasses.dataclass
@@ -85,6 +126,9 @@ class GaussianSplatOpBatchContext:
     per_camera: list
     cameras: list
     image_shape_wh: tuple[int, int]
+    # sparse mode: rows of out.radii / out.sparse_gaussian_ids each camera contributed (also for a camera whose
+    # accepted gaussians ended without a single pair, which has rows but no context)
+    rows_per_camera: list | None = None
 
 
 @dataclasses.dataclass
@@ -189,15 +233,9 @@ class GaussianSplatOp:
         # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
         # forward blend back by the few microseconds the stream takes to process the marker
         self.poll_pair_count = True
-        self._poll_timeouts = 0     # consecutive views whose count did not arrive within the polling time
-        self._pair_capacity = 0
-        # Pinned host words the kernels report into (the pair count; the two sorts' status on the launch-by-launch
-        # path).  One set per op: an op serves one forward at a time -- two forwards of the same op that overlap
-        # (two host threads, or two streams) would race on these words and on _pair_capacity.  Use one op per
-        # stream.
-        self._count_host: torch.Tensor | None = None
-        self._sort_status_host: torch.Tensor | None = None
-        self._side_stream: torch.cuda.Stream | None = None
+        self.recovered_views = 0    # views binned a second time because a look-back of the one-call binning gave up
+        self._slots: dict[tuple[int, int], _StreamSlot] = {}
+        self._last_sorted = None
 
     # ------------------------------------------------------------------ utils
     def _check_supported(self):
@@ -235,6 +273,7 @@ class GaussianSplatOp:
     def _last_keys_sorted(self) -> torch.Tensor:
         """The reference's sorted 64-bit keys, (tile << 32) | depth bits, rebuilt from the last forward's
         sorted tile keys and gaussian indices (parity tests compare them with the oracle's)."""
+        assert self._last_sorted is not None, "set D3GS_KEEP_SORTED_KEYS=1 before importing the package"
         tile_keys, idx, depths = self._last_sorted
         if self._cfg.enable_32bit_sort:     # render.py:767-770, 820: (tile << 18) | depth steps
             steps = (depths / torch.tensor(self._cfg.depth_32bit_prec, dtype=torch.float32, device=depths.device))
@@ -416,10 +455,35 @@ class GaussianSplatOp:
             assert b.is_cuda and b.dtype == torch.float32 and tuple(b.shape) == (n, 3) and b.is_contiguous()
         assert 0 <= model.cur_sh_degree <= min(3, model.color_sh_degree), "cur_sh_degree out of range"
 
+    @staticmethod
+    def _params_signature(model, cameras):
+        """What the kernel parameters of a view depend on, cheap to form: backward() reuses the forward's parameters
+        only while this has not changed (a pose updated in place, a model grown or pruned, a raised SH degree)."""
+        if isinstance(cameras, BasicPinholeCamera):
+            cam = (np.asarray(cameras.intrinsic).tobytes(), np.asarray(cameras.pose.to_world).tobytes(),
+                   tuple(cameras.image_shape_wh))
+        else:
+            cam = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (cameras.cam2world_T, cameras.focal_xy_ppoint)) \
+                + (tuple(cameras.image_shape_wh),)
+        return (len(model), int(model.cur_sh_degree), int(model.color_sh.shape[1]), model.color_sh_base is not None,
+                type(model).__name__, cam)
+
+    def _snapshot_floats(self) -> int:
+        """Floats per pixel and bucket of the per-gaussian backward's snapshots: T and the colour accumulated so far,
+        and with a depth or an alpha channel their sums too (render.py:1744-1759, 2412-2415)."""
+        return 4 + int(bool(self._cfg.render_depth)) + int(bool(self._cfg.render_rgba)) \
+            if (self._cfg.render_depth or self._cfg.render_rgba) else 4
+
     # ---------------------------------------------------------------- forward
     def forward(self, model: GaussianModelOriginBase, cameras, training: bool = False, instance2world_T=None,
                 custom_features=None, mask=None, prep_user_inputs=None):
-        """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``."""
+        """render.py:169-1015.  Returns ``(GaussianSplatOutput, GaussianSplatOpContext | None)``.
+
+        The pass runs in four steps, each a method of its own: ``_start_view`` (arguments, kernel parameters, sparse
+        mode's first pass), ``_preprocess`` (K1 and the colours), ``_order_and_count`` (depth order and pair count, or
+        the whole binning as one library call) and ``_bin_and_blend`` (key expansion .. forward blend); ``forward``
+        strings them together and decides, once the pair count has reached the host, whether the view has to be
+        binned again (buffers outgrown, or a look-back that gave up)."""
         assert model.act_applied, "model must be activated before render"
         batch = len(cameras) if isinstance(cameras, CameraBundle) else 1
         if batch != 1 and not self._bundle_in_one_pass(batch, cameras):
@@ -427,6 +491,84 @@ class GaussianSplatOp:
                                         prep_user_inputs)
         if prep_user_inputs:
             raise NotImplementedError("prep_user_inputs is not supported")
+        v = self._start_view(model, cameras, training, instance2world_T, custom_features, mask, batch)
+        if v.sparse and v.n == 0:      # nothing accepted: the empty render, without touching zero-row buffers
+            self.last_num_rendered = 0
+            self._alloc_outputs(v)
+            return self._empty_result(v)
+        self._alloc_zero_workspaces(v, v.slot.pair_capacity if self.speculative_pair_buffers else 0)
+        self._preprocess(v)
+        self._order_and_count(v)
+        self._alloc_outputs(v)
+
+        # The reference reads the pair count back before it can size the key buffers (render.py:695),
+        # which idles the GPU for a host round trip.  From the second view on the buffers are sized from
+        # the previous count with head room, everything is enqueued at once and the count is read
+        # afterwards; a view that outgrows its buffers is binned again with exact sizes.
+        capacity = v.spec_capacity
+        ctx = None
+        if capacity > 0:
+            ctx, tile_keys_sorted = self._bin_and_blend(v, capacity, True)
+        num_rendered = self._wait_pair_count(v)
+        if num_rendered in (_capi.COUNT_SORT_GAVE_UP, _capi.COUNT_SCAN_GAVE_UP) and v.fused:
+            # A look-back of the one-call binning ran out of its bounded wait (its workgroups rely on being
+            # dispatched in id order): nothing of this binning is used; the view is binned once more, launch by
+            # launch into exactly sized buffers, before anything is raised.
+            self.recovered_views += 1
+            ctx = None
+            self._alloc_zero_workspaces(v, 0)
+            self._preprocess(v)       # (its depth keys were sorted in place by the binning that failed)
+            self._order_and_count(v, stepwise=True)
+            num_rendered = self._wait_pair_count(v)
+        if num_rendered == _capi.COUNT_SORT_GAVE_UP:
+            raise RuntimeError("d3gs_bin_pairs: a sort workgroup's bounded wait on an earlier tile ran out; "
+                               "the tile lists are not sorted")
+        if num_rendered < 0:
+            raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
+        if not v.fused:
+            self._check_sort_status(v, 0, "depth order")
+        if num_rendered > _capi.MAX_PAIRS:
+            raise RuntimeError(f"GaussianSplatOp: {num_rendered} (tile, gaussian) pairs in one call; list positions are "
+                               f"31-bit, at most {_capi.MAX_PAIRS} pairs (render fewer cameras per bundle, or use a "
+                               "tighter early_filter_algo)")
+        self.last_num_rendered = num_rendered
+        v.slot.pair_capacity = min(num_rendered + num_rendered // 4 + 4096, _capi.MAX_PAIRS)
+        if num_rendered == 0:
+            return self._empty_result(v)
+        if ctx is None or num_rendered > capacity:
+            self.rebin_count += int(ctx is not None)
+            ctx, tile_keys_sorted = self._bin_and_blend(v, num_rendered, False)
+        if v.pair_sort_done is not None:
+            # everything is enqueued; the host only waits for the pair sort's status word, the blend runs on
+            v.pair_sort_done.synchronize()
+            self._check_sort_status(v, 1, "tile lists")
+        ctx.gaussian_idx_sorted = ctx.gaussian_idx_sorted[:num_rendered]
+        out = v.out
+        if custom_features is not None:
+            out.custom_features = self._blend_custom_features(v.P, ctx, out, custom_features)
+            ctx.custom_features = custom_features
+        if KEEP_SORTED_KEYS:        # parity tests rebuild the reference's 64-bit keys from these
+            self._last_sorted = (tile_keys_sorted[:num_rendered], ctx.gaussian_idx_sorted, v.depths)
+        if not training:
+            ctx = None
+        return out, ctx
+
+    # -- step 1: arguments, parameters, per-stream state, sparse mode's first pass
+    def _slot(self, dev) -> _StreamSlot:
+        """The host words and hints of the stream this call runs on (one set per device and stream: two forwards of
+        one operator on two streams do not share a word)."""
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        handle = raw(torch.cuda.current_device()) if raw is not None else torch.cuda.current_stream().cuda_stream
+        key = (dev.index if dev.index is not None else torch.cuda.current_device(), int(handle))
+        slot = self._slots.get(key)
+        if slot is None:
+            count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
+            slot = _StreamSlot(count_host=count_host, count_np=count_host.numpy(),
+                               sort_status_host=torch.zeros(2, dtype=torch.int32, pin_memory=True))
+            self._slots[key] = slot
+        return slot
+
+    def _start_view(self, model, cameras, training, instance2world_T, custom_features, mask, batch):
         self._check_model(model)
         if custom_features is not None:
             assert not self.is_nchw, "custom feat don't support nchw, set use_nchw=False in config."   # render.py:246
@@ -441,130 +583,118 @@ class GaussianSplatOp:
             if mask.dtype == torch.bool:
                 mask = mask.view(torch.uint8)
         L = self._lib
-        dev = model.xyz.device
-        batch_cams = self.batch_table(cameras, dev) if batch > 1 else None
-        P = self.make_params(model, cameras, training, batch_cams)
-        inst_ids = inst_cams = None
+        v = types.SimpleNamespace()
+        v.model, v.cameras, v.training, v.batch, v.mask, v.custom_features = model, cameras, bool(training), batch, mask, custom_features
+        v.dev = dev = model.xyz.device
+        v.batch_cams = self.batch_table(cameras, dev) if batch > 1 else None
+        v.P = P = self.make_params(model, cameras, training, v.batch_cams)
+        v.inst_ids = v.inst_cams = None
         if instance2world_T is not None:
-            inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
-        inst = self._instances_arg(inst_ids, inst_cams, batch)
+            v.inst_ids, v.inst_cams = self.instance_table(model, cameras, instance2world_T)
+        v.inst = self._instances_arg(v.inst_ids, v.inst_cams, batch)
         # n: render items = gaussians x cameras (item b * N + g is gaussian g seen by camera b); everything the
         # preprocess writes has one row per item, the tile ids carry the camera
-        n = P.n * batch
-        width, height = P.width, P.height
-        num_tiles = P.tiles_x * P.tiles_y * batch
-        s = self._stream()
-        f32, i32 = torch.float32, torch.int32
-        if self._count_host is None:
-            self._count_host = torch.empty(1, dtype=torch.int64, pin_memory=True)
-            self._count_np = self._count_host.numpy()      # the same word, read without a tensor operation
-            self._sort_status_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+        v.n = P.n * batch
+        v.width, v.height = P.width, P.height
+        v.num_tiles = P.tiles_x * P.tiles_y * batch
+        v.s = self._stream()
+        v.slot = self._slot(dev)
+        v.tile_bits = L.d3gs_higher_msb(v.num_tiles)
+        v.depth_bits = L.d3gs_depth_key_bits(C.byref(P))      # the depth sort's key width: 27 bits for the default planes
+        v.status_pending, v.pair_sort_done, v.pooled_ranges_used = [], None, False
         # Sparse mode (render.py:234-238, 478-500, 622-640): a first pass of the preprocess flags the accepted
         # gaussians, a scan gives each its row, and from here on n is their number V: every buffer below has V rows
         # and the kernels after the preprocess see a scene of V gaussians.  The count has to reach the host before
         # anything can be sized (the reference reads it back the same way, render.py:636).
-        sparse = bool(self._cfg.sparse_mode)
-        Pd = P            # what the kernels behind the preprocess are given
-        sparse_scan = sparse_gaussian_ids = sparse_batch_ids = None
-        if sparse:
+        v.sparse = bool(self._cfg.sparse_mode)
+        v.Pd = P            # what the kernels behind the preprocess are given
+        v.sparse_scan = v.sparse_gaussian_ids = v.sparse_batch_ids = None
+        if v.sparse:
             assert custom_features is None, "custom_features must not be provided in sparse mode"    # render.py:238
-            if instance2world_T is not None:
-                raise NotImplementedError("sparse_mode with instance poses is not supported")
+            n, i32 = v.n, torch.int32
             flags = torch.empty(n, dtype=i32, device=dev)
             _capi.check(L.d3gs_preprocess_fwd_sparse(
                 C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
-                _capi.ptr(model.opacity), _capi.ptr(mask), _capi.ptr(flags), *([None] * 11), s),
+                _capi.ptr(model.opacity), _capi.ptr(mask), _capi.ptr(flags), *([None] * 11), v.inst, v.s),
                 "d3gs_preprocess_fwd_sparse (flags)")
-            sparse_scan = torch.empty(n, dtype=i32, device=dev)
+            v.sparse_scan = torch.empty(n, dtype=i32, device=dev)
             ws_bytes = C.c_size_t(0)
             _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
             ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=dev)
             total_valid = torch.empty(1, dtype=torch.int64, device=dev)
-            _capi.check(L.d3gs_scan_gathered(_capi.ptr(flags), n, None, n, _capi.ptr(sparse_scan), _capi.ptr(ws),
+            _capi.check(L.d3gs_scan_gathered(_capi.ptr(flags), n, None, n, _capi.ptr(v.sparse_scan), _capi.ptr(ws),
                                              ws.numel(), 0, _capi.ptr(total_valid),
-                                             C.c_void_p(self._count_host.data_ptr()), s), "d3gs_scan_gathered (flags)")
+                                             C.c_void_p(v.slot.count_host.data_ptr()), v.s), "d3gs_scan_gathered (flags)")
             torch.cuda.current_stream().synchronize()
-            num_valid = int(self._count_host[0])
+            num_valid = int(v.slot.count_host[0])
             if num_valid < 0:
                 raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
-            n_items, n = n, num_valid
-            Pd = _capi.Params.from_buffer_copy(P)
-            Pd.n, Pd.batch_size, Pd.batch_cameras = n, 0, None
-            sparse_gaussian_ids = torch.empty(n, dtype=i32, device=dev)
-            sparse_batch_ids = torch.empty(n, dtype=i32, device=dev)
+            v.n = num_valid
+            v.Pd = _capi.Params.from_buffer_copy(P)
+            v.Pd.n, v.Pd.batch_size, v.Pd.batch_cameras = num_valid, 0, None
+            v.sparse_gaussian_ids = torch.empty(num_valid, dtype=i32, device=dev)
+            v.sparse_batch_ids = torch.empty(num_valid, dtype=i32, device=dev)
+        return v
 
-        def _sort_ws_bytes(count, begin_bit, end_bit):
-            nbytes = C.c_size_t(0)
-            _capi.check(L.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
-                        "d3gs_sort_workspace_bytes")
-            return nbytes.value
+    def _sort_ws_bytes(self, count, begin_bit, end_bit):
+        nbytes = C.c_size_t(0)
+        _capi.check(self._lib.d3gs_sort_workspace_bytes(count, begin_bit, end_bit, C.byref(nbytes)),
+                    "d3gs_sort_workspace_bytes")
+        return nbytes.value
 
-
-        # every zero-initialised work buffer of the forward pass comes out of one fill (the two sorts' and the
-        # scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later
-        tile_bits = L.d3gs_higher_msb(num_tiles)
-        depth_bits = L.d3gs_depth_key_bits(C.byref(P))      # the depth sort's key width: 27 bits for the default planes
-        if sparse and n == 0:      # nothing accepted: the empty render, without touching zero-row buffers
-            self.last_num_rendered = 0
-            empty = GaussianSplatOutput(
-                custom_features=None, T=torch.ones((batch, height, width), dtype=f32, device=dev),
-                color=torch.zeros((batch, 4 if self._cfg.render_rgba else 3, height, width) if self._cfg.use_nchw else
-                                  (batch, height, width, 4 if self._cfg.render_rgba else 3), dtype=f32, device=dev),
-                depth=torch.zeros((batch, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None,
-                n_contrib=torch.zeros((batch, height, width), dtype=i32, device=dev),
-                radii=torch.zeros(0, dtype=i32, device=dev), sparse_gaussian_ids=sparse_gaussian_ids,
-                sparse_batch_ids=sparse_batch_ids)
-            if not training:
-                bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=dev).clamp(0, 1)
-                if self._cfg.use_nchw:
-                    empty.color[:, :3] = bg.view(1, 3, 1, 1)
-                else:
-                    empty.color[..., :3] = bg
-            return empty, None
-        spec_capacity = self._pair_capacity if self.speculative_pair_buffers else 0
-        align = lambda v: (v + 255) // 256 * 256
+    def _alloc_zero_workspaces(self, v, spec_capacity):
+        """Every zero-initialised work buffer of the forward pass comes out of one fill (the two sorts' and the
+        scan's workspaces, the tile ranges), issued ahead of the preprocess so that nothing waits for it later."""
+        v.spec_capacity = spec_capacity
+        align = lambda x: (x + 255) // 256 * 256
         scan_ws_bytes = C.c_size_t(0)
-        _capi.check(L.d3gs_scan_gathered_workspace_bytes(n, C.byref(scan_ws_bytes)), "d3gs_scan_gathered_workspace_bytes")
-        sizes = [align(_sort_ws_bytes(n, 0, depth_bits)), align(_sort_ws_bytes(spec_capacity, 0, tile_bits)) if spec_capacity else 0,
-                 align(num_tiles * 8), align(scan_ws_bytes.value)]
-        zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=dev)
-        zero_scan_ws = zero_pool[sum(sizes[:3]):]
-        zero_ws_n = zero_pool[:sizes[0]]
-        zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
-        zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + num_tiles * 8].view(torch.int32).view(num_tiles, 2)
+        _capi.check(self._lib.d3gs_scan_gathered_workspace_bytes(v.n, C.byref(scan_ws_bytes)),
+                    "d3gs_scan_gathered_workspace_bytes")
+        sizes = [align(self._sort_ws_bytes(v.n, 0, v.depth_bits)),
+                 align(self._sort_ws_bytes(spec_capacity, 0, v.tile_bits)) if spec_capacity else 0,
+                 align(v.num_tiles * 8), align(scan_ws_bytes.value)]
+        zero_pool = torch.zeros(sum(sizes), dtype=torch.uint8, device=v.dev)
+        v.zero_scan_ws = zero_pool[sum(sizes[:3]):]
+        v.zero_ws_n = zero_pool[:sizes[0]]
+        v.zero_ws_m = zero_pool[sizes[0]:sizes[0] + sizes[1]] if spec_capacity else None
+        v.zero_ranges = zero_pool[sizes[0] + sizes[1]:sizes[0] + sizes[1] + v.num_tiles * 8].view(torch.int32).view(v.num_tiles, 2)
+        v.pooled_ranges_used = False
 
+    # -- step 2: K1 and the colours
+    def _preprocess(self, v):
+        L, P, model, dev, n, s = self._lib, v.P, v.model, v.dev, v.n, v.s
+        f32, i32 = torch.float32, torch.int32
+        training, sparse, mask = v.training, v.sparse, v.mask
         with self._stage("preprocess"):
-            depths = torch.empty(n, dtype=f32, device=dev)
-            radii = torch.empty(n, dtype=i32, device=dev)
-            uvs = torch.empty((n, 2), dtype=f32, device=dev)
-            conic_opacity = torch.empty((n, 4), dtype=f32, device=dev)
-            tiles_touched = torch.empty(n, dtype=i32, device=dev)
-            rgb_gaussian = torch.empty((n, 3), dtype=f32, device=dev)
-            cov2d_vecs = torch.empty((n, 3), dtype=f32, device=dev) if training else None
-            ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
+            v.depths = depths = torch.empty(n, dtype=f32, device=dev)
+            v.radii = radii = torch.empty(n, dtype=i32, device=dev)
+            v.uvs = uvs = torch.empty((n, 2), dtype=f32, device=dev)
+            v.conic_opacity = conic_opacity = torch.empty((n, 4), dtype=f32, device=dev)
+            v.tiles_touched = tiles_touched = torch.empty(n, dtype=i32, device=dev)
+            v.rgb_gaussian = rgb_gaussian = torch.empty((n, 3), dtype=f32, device=dev)
+            v.cov2d_vecs = cov2d_vecs = torch.empty((n, 3), dtype=f32, device=dev) if training else None
+            v.ne0 = ne0 = torch.empty(n, dtype=torch.uint8, device=dev) if training else None
             # kept-tile record per gaussian: key expansion reads it instead of repeating the tile tests
-            tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
-            depth_keys = torch.empty(n, dtype=i32, device=dev)      # float bits of the depths: the depth sort's keys
+            v.tile_masks = tile_masks = torch.empty((n, 2), dtype=torch.int64, device=dev)
+            v.depth_keys = depth_keys = torch.empty(n, dtype=i32, device=dev)      # float bits of the depths: the depth sort's keys
             # The backward's accumulators (one record per gaussian) and, with clear_gradients_early, the model
             # gradient arrays: one allocation that the forward blend kernel clears while it runs (it leaves the
             # memory pipes idle).  Most gaussians of a view end with an all-zero gradient (culled, or never reached
             # before their pixels saturated), which the preprocess backward then need not write.
-            grad_records = grad_pool = grad_clear = grad_touched = None
+            v.grad_records = v.grad_pool = v.grad_clear = v.grad_touched = None
             if training:
                 rec_floats = n * _capi.GRAD_RECORD_FLOATS
                 pool_floats = self._grad_pool_floats(model) if self.clear_gradients_early else 0
                 mark_floats = (n + 15) // 16 * 4          # n bytes, in whole 16-byte units
                 if sparse:      # sparse gradients: one row per accepted gaussian (render.py:2918)
                     pool_floats = self._grad_pool_floats(model, n) if self.clear_gradients_early else 0
-                grad_clear = torch.empty(rec_floats + pool_floats + mark_floats, dtype=f32, device=dev)
+                v.grad_clear = torch.empty(rec_floats + pool_floats + mark_floats, dtype=f32, device=dev)
                 # (bundle: one record per render item, one set of model gradient arrays)
-                grad_records = grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
-                grad_pool = grad_clear[rec_floats:rec_floats + pool_floats] if pool_floats else None
-                grad_touched = grad_clear[rec_floats + pool_floats:].view(torch.uint8)[:n]
+                v.grad_records = v.grad_clear[:rec_floats].view(n, _capi.GRAD_RECORD_FLOATS)
+                v.grad_pool = v.grad_clear[rec_floats:rec_floats + pool_floats] if pool_floats else None
+                v.grad_touched = v.grad_clear[rec_floats + pool_floats:].view(torch.uint8)[:n]
             overlap = bool(self.overlap_sh_colors)
-            no_rgb = bool(self._cfg.disable_builtin_rgb)
-            if overlap and (self._side_stream is None or self._side_stream.device != dev):
-                self._side_stream = torch.cuda.Stream(device=dev)   # default priority
+            v.no_rgb = no_rgb = bool(self._cfg.disable_builtin_rgb)
             if no_rgb:      # no SH evaluation: zero colours, nothing clamped
                 rgb_gaussian.zero_()
                 if ne0 is not None:
@@ -573,294 +703,281 @@ class GaussianSplatOp:
                 overlap = True      # (the colours always come from their own kernel here)
                 _capi.check(L.d3gs_preprocess_fwd_sparse(
                     C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
-                    _capi.ptr(model.opacity), _capi.ptr(mask), None, _capi.ptr(sparse_scan),
-                    _capi.ptr(sparse_gaussian_ids), _capi.ptr(sparse_batch_ids), _capi.ptr(depths), _capi.ptr(radii),
+                    _capi.ptr(model.opacity), _capi.ptr(mask), None, _capi.ptr(v.sparse_scan),
+                    _capi.ptr(v.sparse_gaussian_ids), _capi.ptr(v.sparse_batch_ids), _capi.ptr(depths), _capi.ptr(radii),
                     _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(tiles_touched), _capi.ptr(cov2d_vecs),
-                    _capi.ptr(tile_masks), _capi.ptr(depth_keys), s), "d3gs_preprocess_fwd_sparse")
+                    _capi.ptr(tile_masks), _capi.ptr(depth_keys), v.inst, s), "d3gs_preprocess_fwd_sparse")
             else:
                 _capi.check(L.d3gs_preprocess_fwd(
                     C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw), _capi.ptr(model.scale),
                     _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
                     _capi.ptr(mask), _capi.ptr(depths), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
                     _capi.ptr(tiles_touched), None if (overlap or no_rgb) else _capi.ptr(rgb_gaussian), _capi.ptr(cov2d_vecs),
-                    None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), inst, s),
+                    None if (overlap or no_rgb) else _capi.ptr(ne0), _capi.ptr(tile_masks), _capi.ptr(depth_keys), v.inst, s),
                     "d3gs_preprocess_fwd")
-        sh_done = None
-        if overlap and (self._side_stream is None or self._side_stream.device != dev):
-            self._side_stream = torch.cuda.Stream(device=dev)   # default priority
+        # The SH colours are only read by the blend: they run on a second (default-priority) stream beside the
+        # latency-bound binning stages and are joined in front of the forward blend.
+        v.sh_done = None
         if overlap:
-            main = torch.cuda.current_stream()
-            side = self._side_stream
+            slot = v.slot
+            if slot.side_stream is None or slot.side_stream.device != dev:
+                slot.side_stream = torch.cuda.Stream(device=dev)   # default priority
+            v.main_stream = main = torch.cuda.current_stream()
+            side = slot.side_stream
             side.wait_stream(main)          # radii (and the buffers' allocation) are ready
             ta = torch.cuda.Event(enable_timing=True) if (self.stage_events is not None and not no_rgb) else None
             if ta is not None:
                 ta.record(side)
             if sparse:
                 _capi.check(L.d3gs_sh_colors_sparse(
-                    C.byref(P), _capi.ptr(sparse_gaussian_ids), _capi.ptr(sparse_batch_ids), n, _capi.ptr(model.xyz),
+                    C.byref(P), _capi.ptr(v.sparse_gaussian_ids), _capi.ptr(v.sparse_batch_ids), n, _capi.ptr(model.xyz),
                     _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base), _capi.ptr(radii), _capi.ptr(rgb_gaussian),
-                    _capi.ptr(ne0), C.c_void_p(side.cuda_stream)), "d3gs_sh_colors_sparse")
+                    _capi.ptr(ne0), v.inst, C.c_void_p(side.cuda_stream)), "d3gs_sh_colors_sparse")
             elif not no_rgb:
                 _capi.check(L.d3gs_sh_colors(
                     C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.color_sh), _capi.ptr(model.color_sh_base),
-                    _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), inst, C.c_void_p(side.cuda_stream)),
+                    _capi.ptr(radii), _capi.ptr(rgb_gaussian), _capi.ptr(ne0), v.inst, C.c_void_p(side.cuda_stream)),
                     "d3gs_sh_colors")
             tb = torch.cuda.Event(enable_timing=True) if ta is not None else None
             if tb is not None:
                 tb.record(side)
                 self.stage_events.setdefault("sh_colors", []).append((ta, tb))
-            sh_done = torch.cuda.Event()
-            sh_done.record(side)
+            v.sh_done = torch.cuda.Event()
+            v.sh_done.record(side)
 
-        def _sort(keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None,
-                  status_slot=None):
-            keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
-            nbytes = _sort_ws_bytes(count, begin_bit, end_bit)
-            ws = zero_ws if zero_ws is not None else torch.empty(nbytes, dtype=torch.uint8, device=dev)
-            assert ws.numel() >= nbytes
-            in_b = C.c_int(0)
-            if status_slot is not None:
-                self._sort_status_host[status_slot] = 0
-            if keys_a.dtype == torch.int64:
-                rc = L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                       _capi.ptr(ws), nbytes, count, begin_bit, end_bit, C.byref(in_b), s)
-            else:
-                rc = L.d3gs_sort_pairs_u32(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
-                                           _capi.ptr(ws), nbytes, count, count_dev, int(values_are_indices),
-                                           int(zero_ws is not None), begin_bit, end_bit, C.byref(in_b), s)
-            _capi.check(rc, "d3gs_sort_pairs")
-            if status_slot is not None and count > 0 and end_bit > begin_bit:
-                status_pending.append((ws, nbytes, count, begin_bit, end_bit, status_slot))
-            return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
+    # -- the radix sort of the launch-by-launch path and its status words
+    def _sort(self, v, keys_a, vals_a, count, begin_bit, end_bit, count_dev=None, values_are_indices=False, zero_ws=None,
+              status_slot=None):
+        L, s = self._lib, v.s
+        keys_b, vals_b = torch.empty_like(keys_a), torch.empty_like(vals_a)
+        nbytes = self._sort_ws_bytes(count, begin_bit, end_bit)
+        ws = zero_ws if zero_ws is not None else torch.empty(nbytes, dtype=torch.uint8, device=v.dev)
+        assert ws.numel() >= nbytes
+        in_b = C.c_int(0)
+        if status_slot is not None:
+            v.slot.sort_status_host[status_slot] = 0
+        if keys_a.dtype == torch.int64:
+            rc = L.d3gs_sort_pairs(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
+                                   _capi.ptr(ws), nbytes, count, begin_bit, end_bit, C.byref(in_b), s)
+        else:
+            rc = L.d3gs_sort_pairs_u32(_capi.ptr(keys_a), _capi.ptr(keys_b), _capi.ptr(vals_a), _capi.ptr(vals_b),
+                                       _capi.ptr(ws), nbytes, count, count_dev, int(values_are_indices),
+                                       int(zero_ws is not None), begin_bit, end_bit, C.byref(in_b), s)
+        _capi.check(rc, "d3gs_sort_pairs")
+        if status_slot is not None and count > 0 and end_bit > begin_bit:
+            v.status_pending.append((ws, nbytes, count, begin_bit, end_bit, status_slot))
+        return (keys_b, vals_b) if in_b.value else (keys_a, vals_a)
 
-        status_pending = []
+    def _report_sort_status(self, v):
+        """The error word of every sort issued since the last call (a look-back that gave up) goes to its
+        pinned host word, by a one-thread kernel behind the sort (outside the stage timers)."""
+        while v.status_pending:
+            ws, nbytes, count, begin_bit, end_bit, slot = v.status_pending.pop()
+            _capi.check(self._lib.d3gs_sort_status(_capi.ptr(ws), nbytes, count, begin_bit, end_bit, None,
+                                                   C.c_void_p(v.slot.sort_status_host.data_ptr() + 4 * slot), v.s),
+                        "d3gs_sort_status")
 
-        def _report_sort_status():
-            """The error word of every sort issued since the last call (a look-back that gave up) goes to its
-            pinned host word, by a one-thread kernel behind the sort (outside the stage timers)."""
-            while status_pending:
-                ws, nbytes, count, begin_bit, end_bit, slot = status_pending.pop()
-                _capi.check(L.d3gs_sort_status(_capi.ptr(ws), nbytes, count, begin_bit, end_bit, None,
-                                               C.c_void_p(self._sort_status_host.data_ptr() + 4 * slot), s),
-                            "d3gs_sort_status")
+    @staticmethod
+    def _check_sort_status(v, slot, what):
+        if int(v.slot.sort_status_host[slot]) != 0:
+            raise RuntimeError(f"d3gs_sort_pairs_u32 ({what}): a workgroup's bounded wait on an earlier tile ran "
+                               "out; the list is not sorted")
 
-        def _check_sort_status(slot, what):
-            if int(self._sort_status_host[slot]) != 0:
-                raise RuntimeError(f"d3gs_sort_pairs_u32 ({what}): a workgroup's bounded wait on an earlier tile ran "
-                                   "out; the list is not sorted")
-
-        # With buffers sized from the previous view and no stage timers, the whole binning is one call into the
-        # library (d3gs_bin_pairs): the launches of this phase are short, and issuing them one by one from
-        # Python leaves the GPU idle between them.
-        fused = bool(self.fused_binning and spec_capacity > 0 and self.stage_events is None)
-        self.last_forward_fused = fused      # which of the two binning paths this view took (tests look at it)
-        fused_result = None
-        if fused:
-            cap = spec_capacity
-            up = lambda v: (v + 63) // 64 * 64          # 256-byte aligned slices of one int32 allocation
+    # -- step 3: depth order and pair count (or the whole binning as one call)
+    def _order_and_count(self, v, stepwise=False):
+        """With buffers sized from the previous view and no stage timers, the whole binning is one call into the
+        library (d3gs_bin_pairs): the launches of this phase are short, and issuing them one by one from Python
+        leaves the GPU idle between them.  Otherwise (first view of a stream, stage timers, `stepwise`) the depth
+        sort and the scan are issued here and the rest follows once the pair count is known."""
+        L, dev, n, s = self._lib, v.dev, v.n, v.s
+        i32 = torch.int32
+        v.fused = bool(self.fused_binning and v.spec_capacity > 0 and self.stage_events is None and not stepwise)
+        self.last_forward_fused = v.fused      # which of the two binning paths this view took (tests look at it)
+        v.fused_result = None
+        v.count_ready = None
+        v.polled = False
+        if v.fused:
+            cap = v.spec_capacity
+            up = lambda x: (x + 63) // 64 * 64          # 256-byte aligned slices of one int32 allocation
             o_keys_b, o_ord_a, o_ord_b, o_offs = 0, up(n), 2 * up(n), 3 * up(n)
             o_tk_a = 4 * up(n)
             o_tk_b, o_ix_a, o_ix_b = o_tk_a + up(cap), o_tk_a + 2 * up(cap), o_tk_a + 3 * up(cap)
             o_order = o_tk_a + 4 * up(cap)
-            pool = torch.empty(o_order + up(num_tiles), dtype=i32, device=dev)
+            pool = torch.empty(o_order + up(v.num_tiles), dtype=i32, device=dev)
             base = pool.data_ptr()
             at = lambda off: C.c_void_p(base + 4 * off)
-            total = torch.empty(1, dtype=torch.int64, device=dev)
+            v.total = torch.empty(1, dtype=torch.int64, device=dev)
             order_in_b, pairs_in_b = C.c_int(0), C.c_int(0)
-            polled = bool(self.poll_pair_count and n > 0)
-            if polled:
-                self._count_np[0] = _capi.COUNT_PENDING
+            # Polling gains a few microseconds per view; a view whose binning takes milliseconds (hundreds of millions
+            # of pairs) waits on an event instead, which costs it nothing by comparison and keeps the host thread free.
+            v.polled = bool(self.poll_pair_count and n > 0 and cap <= POLL_MAX_PAIRS)
+            if v.polled:
+                v.slot.count_np[0] = _capi.COUNT_PENDING
             _capi.check(L.d3gs_bin_pairs(
-                C.byref(Pd), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity), _capi.ptr(depths),
-                _capi.ptr(tiles_touched), _capi.ptr(tile_masks), _capi.ptr(depth_keys), at(o_keys_b), at(o_ord_a),
-                at(o_ord_b), _capi.ptr(zero_ws_n), zero_ws_n.numel(), at(o_offs), _capi.ptr(zero_scan_ws),
-                zero_scan_ws.numel(), _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), cap, at(o_tk_a),
-                at(o_tk_b), at(o_ix_a), at(o_ix_b), _capi.ptr(zero_ws_m), zero_ws_m.numel(), _capi.ptr(zero_ranges),
-                at(o_order), _capi.BIN_WORKSPACES_ARE_ZERO | (_capi.BIN_HOST_COUNT_AT_END if polled else 0),
+                C.byref(v.Pd), _capi.ptr(v.radii), _capi.ptr(v.uvs), _capi.ptr(v.conic_opacity), _capi.ptr(v.depths),
+                _capi.ptr(v.tiles_touched), _capi.ptr(v.tile_masks), _capi.ptr(v.depth_keys), at(o_keys_b), at(o_ord_a),
+                at(o_ord_b), _capi.ptr(v.zero_ws_n), v.zero_ws_n.numel(), at(o_offs), _capi.ptr(v.zero_scan_ws),
+                v.zero_scan_ws.numel(), _capi.ptr(v.total), C.c_void_p(v.slot.count_host.data_ptr()), cap, at(o_tk_a),
+                at(o_tk_b), at(o_ix_a), at(o_ix_b), _capi.ptr(v.zero_ws_m), v.zero_ws_m.numel(), _capi.ptr(v.zero_ranges),
+                at(o_order), _capi.BIN_WORKSPACES_ARE_ZERO | (_capi.BIN_HOST_COUNT_AT_END if v.polled else 0),
                 C.byref(order_in_b), C.byref(pairs_in_b), s), "d3gs_bin_pairs")
-            count_ready = None
-            if not polled:
-                count_ready = torch.cuda.Event()
-                count_ready.record()
+            if not v.polled:
+                v.count_ready = torch.cuda.Event()
+                v.count_ready.record()
             # what a second, exactly sized binning of this view would start from
-            depth_keys_sorted = pool[o_keys_b:o_keys_b + n] if order_in_b.value else depth_keys
-            gaussian_order = pool[o_ord_b:o_ord_b + n] if order_in_b.value else pool[o_ord_a:o_ord_a + n]
-            counts_ordered = pool[o_offs:o_offs + n]
+            v.depth_keys_sorted = pool[o_keys_b:o_keys_b + n] if order_in_b.value else v.depth_keys
+            v.gaussian_order = pool[o_ord_b:o_ord_b + n] if order_in_b.value else pool[o_ord_a:o_ord_a + n]
+            v.counts_ordered = pool[o_offs:o_offs + n]
             o_tk, o_ix = (o_tk_b, o_ix_b) if pairs_in_b.value else (o_tk_a, o_ix_a)
-            fused_result = (pool[o_tk:o_tk + cap], pool[o_ix:o_ix + cap], pool[o_order:o_order + num_tiles])
-        else:
-            # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
-            # digits only depend on the gaussian, so the same stable order comes from sorting the N
-            # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
-            # tile digits only: 2 passes over M pairs instead of 6.
-            with self._stage("depth_order"):
-                depth_keys_sorted, gaussian_order = _sort(depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0,
-                                                          depth_bits, values_are_indices=True, zero_ws=zero_ws_n,
-                                                          status_slot=0)
-            _report_sort_status()
+            v.fused_result = (pool[o_tk:o_tk + cap], pool[o_ix:o_ix + cap], pool[o_order:o_order + v.num_tiles])
+            return
+        # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
+        # digits only depend on the gaussian, so the same stable order comes from sorting the N
+        # gaussians by depth first, emitting the pairs in that order and sorting the pairs on the
+        # tile digits only: 2 passes over M pairs instead of 6.
+        with self._stage("depth_order"):
+            v.depth_keys_sorted, v.gaussian_order = self._sort(
+                v, v.depth_keys, torch.empty(n, dtype=i32, device=dev), n, 0, v.depth_bits, values_are_indices=True,
+                zero_ws=v.zero_ws_n, status_slot=0)
+        self._report_sort_status(v)
+        with self._stage("scan"):
+            # tile counts gathered into depth order and scanned in one launch
+            v.counts_ordered = torch.empty(n, dtype=i32, device=dev)
+            v.total = torch.empty(1, dtype=torch.int64, device=dev)
+            _capi.check(L.d3gs_scan_gathered(_capi.ptr(v.tiles_touched), n, _capi.ptr(v.gaussian_order), n,
+                                             _capi.ptr(v.counts_ordered), _capi.ptr(v.zero_scan_ws), v.zero_scan_ws.numel(), 1,
+                                             _capi.ptr(v.total), C.c_void_p(v.slot.count_host.data_ptr()), s),
+                        "d3gs_scan_gathered")
+            # the scan also stores the count to pinned host memory; the host looks at it only after the
+            # rest of the forward pass has been enqueued
+            v.count_ready = torch.cuda.Event()
+            v.count_ready.record()
 
-            with self._stage("scan"):
-                # tile counts gathered into depth order and scanned in one launch
-                counts_ordered = torch.empty(n, dtype=i32, device=dev)
-                total = torch.empty(1, dtype=torch.int64, device=dev)
-                _capi.check(L.d3gs_scan_gathered(_capi.ptr(tiles_touched), n, _capi.ptr(gaussian_order), n,
-                                                 _capi.ptr(counts_ordered), _capi.ptr(zero_scan_ws), zero_scan_ws.numel(), 1,
-                                                 _capi.ptr(total), C.c_void_p(self._count_host.data_ptr()), s),
-                            "d3gs_scan_gathered")
-                # the scan also stores the count to pinned host memory; the host looks at it only after the
-                # rest of the forward pass has been enqueued
-                count_ready = torch.cuda.Event()
-                count_ready.record()
-
-        final_T = torch.empty((batch, height, width), dtype=f32, device=dev)
-        n_contrib = torch.empty((batch, height, width), dtype=i32, device=dev)
-        channels = 4 if self._cfg.render_rgba else 3       # what the kernels write
-        color_shape = (batch, channels, height, width) if self._cfg.use_nchw else (batch, height, width, channels)
-        out_color = torch.empty(color_shape, dtype=f32, device=dev)
-        out_depth = torch.empty((batch, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
-        # disable_builtin_rgb: the caller's colour image is the alpha channel alone, or has no channel
-        # (config_def.py:152-157)
-        out = GaussianSplatOutput(custom_features=None, T=final_T, color=out_color[..., 3:] if no_rgb else out_color,
-                                  depth=out_depth, n_contrib=n_contrib, radii=radii,
-                                  sparse_gaussian_ids=sparse_gaussian_ids, sparse_batch_ids=sparse_batch_ids)
-
-        def _empty_result():
-            if custom_features is not None:
-                out.custom_features = torch.zeros((batch, height, width, custom_features.shape[1]), dtype=f32, device=dev)
-            if sh_done is not None:
-                torch.cuda.current_stream().wait_event(sh_done)
-            # the reference returns uninitialised buffers here (render.py:706-729); fill with the
-            # values an empty scene renders to instead
-            final_T.fill_(1.0)
-            n_contrib.zero_()
-            out_color.zero_()
-            if out_depth is not None:
-                out_depth.zero_()
-            if not training:
-                bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=dev).clamp(0, 1)
-                if self._cfg.use_nchw:
-                    out_color[:, :3] = bg.view(1, 3, 1, 1)
-                else:
-                    out_color[..., :3] = bg
-            return out, None
-
-        pooled_ranges_used = [False]
-        pair_sort_done = [None]      # launch-by-launch path: recorded behind the pair sort's status word
-
-        def _bin_and_blend(capacity: int, count_on_device: bool):
-            """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
-            read the pair count from `total` on the device and nothing here waits for the host."""
-            if fused_result is not None and count_on_device:
-                tile_keys_sorted, gaussian_idx_sorted, tile_order = fused_result
-                workload_ranges = zero_ranges
-                pooled_ranges_used[0] = True
-            else:
-                m_dev = _capi.ptr(total) if count_on_device else None
-                # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
-                with self._stage("make_keys"):
-                    tile_keys = torch.empty(capacity, dtype=i32, device=dev)
-                    gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
-                    _capi.check(L.d3gs_make_keys(C.byref(Pd), _capi.ptr(radii), _capi.ptr(uvs), _capi.ptr(conic_opacity),
-                                                 _capi.ptr(depths), _capi.ptr(counts_ordered), _capi.ptr(gaussian_order),
-                                                 _capi.ptr(depth_keys_sorted), _capi.ptr(tile_masks), None,
-                                                 _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
-                                "d3gs_make_keys")
-                with self._stage("sort"):
-                    tile_keys_sorted, gaussian_idx_sorted = _sort(tile_keys, gaussian_idx, capacity, 0, tile_bits, m_dev,
-                                                                  zero_ws=zero_ws_m if count_on_device else None,
-                                                                  status_slot=1)
-                _report_sort_status()
-                pair_sort_done[0] = torch.cuda.Event()
-                pair_sort_done[0].record()
-                with self._stage("tile_ranges"):
-                    # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
-                    workload_ranges = zero_ranges if not pooled_ranges_used[0] else torch.zeros((num_tiles, 2), dtype=i32, device=dev)
-                    pooled_ranges_used[0] = True
-                    tile_order = torch.empty(num_tiles, dtype=i32, device=dev)
-                    _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
-                                                       _capi.ptr(workload_ranges), num_tiles, _capi.ptr(tile_order), s),
-                                "d3gs_tile_ranges_u32")
-            snap = None
-            if training and self._cfg.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN:
-                # K8 (render.py:940-962): where each tile's buckets start.  The bucket total stays on the device:
-                # ceil(len / 64) summed over the tiles is at most pairs / 64 + tiles, which sizes the snapshots.
-                bucket_offsets = torch.empty(num_tiles + 1, dtype=i32, device=dev)
-                _capi.check(L.d3gs_bucket_offsets(_capi.ptr(workload_ranges), num_tiles, _capi.ptr(bucket_offsets), s),
-                            "d3gs_bucket_offsets")
-                max_buckets = capacity // _capi.BUCKET_SIZE + num_tiles + 1
-                snap = (bucket_offsets, torch.empty((max_buckets, 256, 4), dtype=f32, device=dev))
-            ctx = GaussianSplatOpContext(
-                conic_opacity=conic_opacity, radii=radii, uvs=uvs, rgb_gaussian=rgb_gaussian,
-                gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges, per_gaussian_snap=snap,
-                image_shape_wh=(width, height), cov2d_vecs=cov2d_vecs, sh_to_rgb_ne_0=ne0, depths=depths,
-                tile_order=tile_order, grad_records=grad_records, grad_pool=grad_pool, grad_clear=grad_clear,
-                grad_touched=grad_touched,
-                kernel_color=out_color if no_rgb else None, instance_cameras=inst_cams, instance_ids=inst_ids,
-                batch_size=batch, batch_cameras=batch_cams, sparse_gaussian_ids=sparse_gaussian_ids)
-            # the view's kernel parameters, for a backward pass over the same model and cameras
-            ctx._forward_params = (P, model, cameras, bool(training))
-            if sh_done is not None:
-                main.wait_event(sh_done)      # (the stream object of the fork: forward runs on one stream)
-            with self._stage("blend_fwd"):
-                self.rasterize_forward_backward(model, ctx, out, training=training,
-                                                render_depth=self._cfg.render_depth, _params=Pd)
-            return ctx, tile_keys_sorted
-
-        # The reference reads the pair count back before it can size the key buffers (render.py:695),
-        # which idles the GPU for a host round trip.  From the second view on the buffers are sized from
-        # the previous count with head room, everything is enqueued at once and the count is read
-        # afterwards; a view that outgrows its buffers is binned again with exact sizes.
-        capacity = spec_capacity
-        ctx = None
-        if capacity > 0:
-            ctx, tile_keys_sorted = _bin_and_blend(capacity, True)
-        if count_ready is not None:
-            count_ready.synchronize()
+    def _wait_pair_count(self, v) -> int:
+        """The pair count of the view (or the negative status that replaces it), once it has reached the host."""
+        if v.count_ready is not None:
+            v.count_ready.synchronize()
         else:
             # the binning's last kernel stores the count (or a status) over the marker put there before the call
-            give_up = time.perf_counter() + 0.02
-            while int(self._count_np[0]) == _capi.COUNT_PENDING:
-                if time.perf_counter() > give_up:       # a very large view, or a store the host does not see
-                    torch.cuda.current_stream().synchronize()
-                    self._poll_timeouts += 1
-                    if self._poll_timeouts >= 3:        # not one slow view: later views wait on an event again
-                        self.poll_pair_count = False
-                    if int(self._count_np[0]) == _capi.COUNT_PENDING:
-                        raise RuntimeError("d3gs_bin_pairs: the pair count never reached the host")
-                    break
+            arrived = poll_host_word(v.slot.count_np, _capi.COUNT_PENDING, POLL_SECONDS,
+                                     torch.cuda.current_stream().synchronize)
+            if arrived == "polled":
+                v.slot.poll_timeouts = 0
             else:
-                self._poll_timeouts = 0
-        num_rendered = int(self._count_host[0])
-        if num_rendered == _capi.COUNT_SORT_GAVE_UP:
-            raise RuntimeError("d3gs_bin_pairs: a sort workgroup's bounded wait on an earlier tile ran out; "
-                               "the tile lists are not sorted")
-        if num_rendered < 0:
-            raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
-        if not fused:
-            _check_sort_status(0, "depth order")
-        if num_rendered > _capi.MAX_PAIRS:
-            raise RuntimeError(f"GaussianSplatOp: {num_rendered} (tile, gaussian) pairs in one call; list positions are "
-                               f"31-bit, at most {_capi.MAX_PAIRS} pairs (render fewer cameras per bundle, or use a "
-                               "tighter early_filter_algo)")
-        self.last_num_rendered = num_rendered
-        self._pair_capacity = min(num_rendered + num_rendered // 4 + 4096, _capi.MAX_PAIRS)
-        if num_rendered == 0:
-            return _empty_result()
-        if ctx is None or num_rendered > capacity:
-            self.rebin_count += int(ctx is not None)
-            ctx, tile_keys_sorted = _bin_and_blend(num_rendered, False)
-        if pair_sort_done[0] is not None:
-            # everything is enqueued; the host only waits for the pair sort's status word, the blend runs on
-            pair_sort_done[0].synchronize()
-            _check_sort_status(1, "tile lists")
-        ctx.gaussian_idx_sorted = ctx.gaussian_idx_sorted[:num_rendered]
-        if custom_features is not None:
-            out.custom_features = self._blend_custom_features(P, ctx, out, custom_features)
-            ctx.custom_features = custom_features
-        self._last_sorted = (tile_keys_sorted[:num_rendered], ctx.gaussian_idx_sorted, depths)  # kept for parity tests
-        if not training:
-            ctx = None
-        return out, ctx
+                v.slot.poll_timeouts += 1
+                if v.slot.poll_timeouts >= 3 and self.poll_pair_count:      # not one slow view: wait on an event from now on
+                    self.poll_pair_count = False
+                    warnings.warn("GaussianSplatOp: the pair count did not reach the host within "
+                                  f"{POLL_SECONDS * 1e3:.0f} ms on three views in a row; polling is switched off "
+                                  "for this operator (the host waits on an event instead)")
+                if arrived == "never":
+                    raise RuntimeError("d3gs_bin_pairs: the pair count never reached the host")
+        return int(v.slot.count_host[0])
+
+    # -- step 4: key expansion .. forward blend
+    def _alloc_outputs(self, v):
+        dev, batch, height, width = v.dev, v.batch, v.height, v.width
+        f32, i32 = torch.float32, torch.int32
+        v.final_T = torch.empty((batch, height, width), dtype=f32, device=dev)
+        v.n_contrib = torch.empty((batch, height, width), dtype=i32, device=dev)
+        channels = 4 if self._cfg.render_rgba else 3       # what the kernels write
+        color_shape = (batch, channels, height, width) if self._cfg.use_nchw else (batch, height, width, channels)
+        v.out_color = torch.empty(color_shape, dtype=f32, device=dev)
+        v.out_depth = torch.empty((batch, height, width), dtype=f32, device=dev) if self._cfg.render_depth else None
+        no_rgb = bool(self._cfg.disable_builtin_rgb)
+        # disable_builtin_rgb: the caller's colour image is the alpha channel alone, or has no channel
+        # (config_def.py:152-157)
+        v.out = GaussianSplatOutput(custom_features=None, T=v.final_T, color=v.out_color[..., 3:] if no_rgb else v.out_color,
+                                    depth=v.out_depth, n_contrib=v.n_contrib,
+                                    radii=getattr(v, "radii", None) if v.n else torch.zeros(0, dtype=i32, device=dev),
+                                    sparse_gaussian_ids=v.sparse_gaussian_ids, sparse_batch_ids=v.sparse_batch_ids)
+
+    def _empty_result(self, v):
+        """The render of a view without a single (tile, gaussian) pair.  The reference returns uninitialised buffers
+        here (render.py:706-729); this fills in what an empty scene renders to."""
+        out = v.out
+        if v.custom_features is not None:
+            out.custom_features = torch.zeros((v.batch, v.height, v.width, v.custom_features.shape[1]),
+                                              dtype=torch.float32, device=v.dev)
+        if getattr(v, "sh_done", None) is not None:
+            torch.cuda.current_stream().wait_event(v.sh_done)
+        v.final_T.fill_(1.0)
+        v.n_contrib.zero_()
+        v.out_color.zero_()
+        if v.out_depth is not None:
+            v.out_depth.zero_()
+        if not v.training:
+            bg = torch.tensor(np.asarray(self._cfg.bg_color, np.float32), device=v.dev).clamp(0, 1)
+            if self._cfg.use_nchw:
+                v.out_color[:, :3] = bg.view(1, 3, 1, 1)
+            else:
+                v.out_color[..., :3] = bg
+        return out, None
+
+    def _bin_and_blend(self, v, capacity: int, count_on_device: bool):
+        """Key expansion .. blend for buffers of `capacity` pairs.  With count_on_device the kernels
+        read the pair count from `total` on the device and nothing here waits for the host."""
+        L, dev, s, Pd = self._lib, v.dev, v.s, v.Pd
+        i32 = torch.int32
+        if v.fused_result is not None and count_on_device:
+            tile_keys_sorted, gaussian_idx_sorted, tile_order = v.fused_result
+            workload_ranges = v.zero_ranges
+            v.pooled_ranges_used = True
+        else:
+            m_dev = _capi.ptr(v.total) if count_on_device else None
+            # pairs leave key expansion in depth order, so the pair sort only needs the tile id: 32-bit keys
+            with self._stage("make_keys"):
+                tile_keys = torch.empty(capacity, dtype=i32, device=dev)
+                gaussian_idx = torch.empty(capacity, dtype=i32, device=dev)
+                _capi.check(L.d3gs_make_keys(C.byref(Pd), _capi.ptr(v.radii), _capi.ptr(v.uvs), _capi.ptr(v.conic_opacity),
+                                             _capi.ptr(v.depths), _capi.ptr(v.counts_ordered), _capi.ptr(v.gaussian_order),
+                                             _capi.ptr(v.depth_keys_sorted), _capi.ptr(v.tile_masks), None,
+                                             _capi.ptr(tile_keys), _capi.ptr(gaussian_idx), capacity, s),
+                            "d3gs_make_keys")
+            with self._stage("sort"):
+                tile_keys_sorted, gaussian_idx_sorted = self._sort(
+                    v, tile_keys, gaussian_idx, capacity, 0, v.tile_bits, m_dev,
+                    zero_ws=v.zero_ws_m if count_on_device else None, status_slot=1)
+            self._report_sort_status(v)
+            v.pair_sort_done = torch.cuda.Event()
+            v.pair_sort_done.record()
+            with self._stage("tile_ranges"):
+                # the pooled ranges serve the first binning of this view; a second one starts from fresh zeros
+                workload_ranges = v.zero_ranges if not v.pooled_ranges_used else \
+                    torch.zeros((v.num_tiles, 2), dtype=i32, device=dev)
+                v.pooled_ranges_used = True
+                tile_order = torch.empty(v.num_tiles, dtype=i32, device=dev)
+                _capi.check(L.d3gs_tile_ranges_u32(_capi.ptr(tile_keys_sorted), capacity, m_dev,
+                                                   _capi.ptr(workload_ranges), v.num_tiles, _capi.ptr(tile_order), s),
+                            "d3gs_tile_ranges_u32")
+        snap = None
+        if v.training and self._cfg.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN:
+            # K8 (render.py:940-962): where each tile's buckets start.  The bucket total stays on the device:
+            # ceil(len / 64) summed over the tiles is at most pairs / 64 + tiles, which sizes the snapshots.
+            bucket_offsets = torch.empty(v.num_tiles + 1, dtype=i32, device=dev)
+            _capi.check(L.d3gs_bucket_offsets(_capi.ptr(workload_ranges), v.num_tiles, _capi.ptr(bucket_offsets), s),
+                        "d3gs_bucket_offsets")
+            max_buckets = capacity // _capi.BUCKET_SIZE + v.num_tiles + 1
+            snap = (bucket_offsets, torch.empty((max_buckets, 256, self._snapshot_floats()), dtype=torch.float32, device=dev))
+        ctx = GaussianSplatOpContext(
+            conic_opacity=v.conic_opacity, radii=v.radii, uvs=v.uvs, rgb_gaussian=v.rgb_gaussian,
+            gaussian_idx_sorted=gaussian_idx_sorted, workload_ranges=workload_ranges, per_gaussian_snap=snap,
+            image_shape_wh=(v.width, v.height), cov2d_vecs=v.cov2d_vecs, sh_to_rgb_ne_0=v.ne0, depths=v.depths,
+            tile_order=tile_order, grad_records=v.grad_records, grad_pool=v.grad_pool, grad_clear=v.grad_clear,
+            grad_touched=v.grad_touched,
+            kernel_color=v.out_color if v.no_rgb else None, instance_cameras=v.inst_cams, instance_ids=v.inst_ids,
+            batch_size=v.batch, batch_cameras=v.batch_cams, sparse_gaussian_ids=v.sparse_gaussian_ids)
+        # The view's kernel parameters, for a backward pass over the same model and cameras.  The model and the
+        # cameras are remembered weakly and by what the parameters depend on: backward() rebuilds the parameters
+        # when it is handed other objects, or the same ones changed in place where that can be seen.
+        ctx._forward_params = (_capi.Params.from_buffer_copy(v.P), weakref.ref(v.model), weakref.ref(v.cameras),
+                               bool(v.training), self._params_signature(v.model, v.cameras))
+        if v.sh_done is not None:
+            v.main_stream.wait_event(v.sh_done)      # (the stream object of the fork: forward runs on one stream)
+        with self._stage("blend_fwd"):
+            self.rasterize_forward_backward(v.model, ctx, v.out, training=v.training,
+                                            render_depth=self._cfg.render_depth, _params=Pd)
+        return ctx, tile_keys_sorted
 
     def _bundle_in_one_pass(self, batch, cameras) -> bool:
         """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
@@ -909,10 +1026,48 @@ class GaussianSplatOp:
             out.sparse_batch_ids = torch.cat([torch.full_like(o.sparse_gaussian_ids, b) for b, o in enumerate(outs)], 0)
         if not training:
             return out, None
-        return out, GaussianSplatOpBatchContext(per_camera=ctxs, cameras=cams, image_shape_wh=cameras.image_shape_wh)
+        rows = [int(o.sparse_gaussian_ids.numel()) for o in outs] if self._cfg.sparse_mode else None
+        return out, GaussianSplatOpBatchContext(per_camera=ctxs, cameras=cams, image_shape_wh=cameras.image_shape_wh,
+                                                rows_per_camera=rows)
 
-    def _backward_bundle(self, model, ctx, out, grad, return_uv_grad):
-        return _backward_bundle_impl(self, model, ctx, out, grad, return_uv_grad)
+    # ------------------------------------------------------- sparse bundles: K10
+    def unique_ids(self, ids: torch.Tensor, id_limit: int):
+        """Distinct values of ``ids`` (int32 [R], each in [0, id_limit)) in ascending order, and the rows grouped by
+        value: ``(unique [U], run_rows [R], run_starts [R + 1])`` (render.py:2864-2903 does this with a hash table).
+        One host synchronisation: U sizes the result."""
+        assert ids.is_cuda and ids.dtype == torch.int32 and ids.ndim == 1 and ids.is_contiguous()
+        L, s, dev, R = self._lib, self._stream(), ids.device, int(ids.numel())
+        i32 = torch.int32
+        nbytes = C.c_size_t(0)
+        _capi.check(L.d3gs_unique_ids_workspace_bytes(R, int(id_limit), C.byref(nbytes)), "d3gs_unique_ids_workspace_bytes")
+        ws = torch.empty(max(nbytes.value, 1), dtype=torch.uint8, device=dev)
+        unique = torch.empty(R, dtype=i32, device=dev)
+        inverse, run_rows = torch.empty(R, dtype=i32, device=dev), torch.empty(R, dtype=i32, device=dev)
+        run_starts = torch.empty(R + 1, dtype=i32, device=dev)
+        count_dev = torch.empty(1, dtype=torch.int64, device=dev)
+        slot = self._slot(dev)
+        _capi.check(L.d3gs_unique_ids(_capi.ptr(ids), R, int(id_limit), _capi.ptr(unique), _capi.ptr(inverse),
+                                      _capi.ptr(run_rows), _capi.ptr(run_starts), _capi.ptr(ws), nbytes.value,
+                                      _capi.ptr(count_dev), C.c_void_p(slot.count_host.data_ptr()), s), "d3gs_unique_ids")
+        torch.cuda.current_stream().synchronize()
+        U = int(slot.count_host[0])
+        if U < 0:
+            raise RuntimeError("d3gs_unique_ids: a workgroup's bounded wait on an earlier chunk ran out")
+        self.last_unique_inverse = inverse
+        return unique[:U], run_rows, run_starts
+
+    def merge_rows(self, rows: torch.Tensor, run_rows: torch.Tensor, run_starts: torch.Tensor, n_runs: int):
+        """``merged[u] = sum of rows[r]`` over the rows r of run u (see ``unique_ids``), in run order."""
+        rows = rows.contiguous()
+        R = int(rows.shape[0])
+        width = int(rows.numel() // max(R, 1))
+        merged = torch.empty((n_runs,) + tuple(rows.shape[1:]), dtype=torch.float32, device=rows.device)
+        _capi.check(self._lib.d3gs_merge_rows(_capi.ptr(rows), R, width, _capi.ptr(run_rows), _capi.ptr(run_starts),
+                                              int(n_runs), _capi.ptr(merged), self._stream()), "d3gs_merge_rows")
+        return merged
+
+    def _backward_bundle(self, model, ctx, out, grad, return_uv_grad, instance2world_T=None):
+        return _backward_bundle_impl(self, model, ctx, out, grad, return_uv_grad, instance2world_T)
 
     # ------------------------------------------------------- gradient pool
     @staticmethod
@@ -1072,7 +1227,8 @@ class GaussianSplatOp:
             # global atomic requests of this blend backward (one per (tile, gaussian) with a non-zero sum); the
             # reference prints its count the same way
             self.last_atomic_add_count = int(counter.item())
-            print(f"atomic add count: {self.last_atomic_add_count}")
+            if self._cfg.verbose:
+                print(f"atomic add count: {self.last_atomic_add_count}")
         res = RasterizeGradientOutput(duv=rec[:, 0:2], dconic=rec[:, 2:5], dopacity=rec[:, 5], dcolor=rec[:, 6:9],
                                       dz=rec[:, 9] if render_depth else None, records=rec, touched=touched)
         return res
@@ -1086,10 +1242,11 @@ class GaussianSplatOp:
         if prep_user_inputs:
             raise NotImplementedError("prep_user_inputs is not supported")
         if isinstance(ctx, GaussianSplatOpBatchContext):
-            return self._backward_bundle(model, ctx, out, grad, return_uv_grad)
+            return self._backward_bundle(model, ctx, out, grad, return_uv_grad, instance2world_T)
         L = self._lib
         kept = getattr(ctx, "_forward_params", None)
-        if kept is not None and kept[1] is model and kept[2] is cameras and kept[3]:
+        if kept is not None and kept[1]() is model and kept[2]() is cameras and kept[3] \
+                and kept[4] == self._params_signature(model, cameras):
             P = _capi.Params.from_buffer_copy(kept[0])      # (a copy: sparse mode edits n below)
         else:
             P = self.make_params(model, cameras, True, ctx.batch_cameras)
@@ -1129,8 +1286,8 @@ class GaussianSplatOp:
                     _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh), _capi.ptr(ctx.radii),
                     _capi.ptr(ctx.cov2d_vecs), _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), _capi.ptr(g.touched),
                     int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat),
-                    _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base), s),
-                    "d3gs_preprocess_bwd_sparse")
+                    _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base),
+                    self._instances_arg(inst_ids, inst_cams), s), "d3gs_preprocess_bwd_sparse")
             rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
             for b in range(B if sparse_ids is None else 0):
                 inst = self._instances_arg(inst_ids, inst_cams, B, b)      # the instance poses as camera b sees them
@@ -1150,49 +1307,53 @@ class GaussianSplatOp:
         return grad_model, None, dcustom
 
 
-def _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad):
+def _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad, instance2world_T=None):
     """Sparse-mode bundle (render.py:2864-2903): each camera has its own accepted gaussians; the gradient rows of a
     gaussian seen by several cameras are merged.  The reference deduplicates the ids with a hash table
-    (insert, collect, query); here they are sorted and made unique, which also fixes the row order: the result has
-    one row per distinct accepted gaussian, ascending, and ``op.last_sparse_unique_ids`` names them."""
+    (insert, collect, query); here the library sorts them and numbers the runs of equal ids (d3gs_unique_ids), which
+    also fixes the row order: the result has one row per distinct accepted gaussian, ascending, and
+    ``op.last_sparse_unique_ids`` names them; d3gs_merge_rows adds each gaussian's rows in camera order."""
     parts, duvs, offs = [], [], 0
+    dev = model.xyz.device
     for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
-        if ctx_b is None:
-            continue
-        v = int(ctx_b.sparse_gaussian_ids.numel())
+        # the camera's rows of out.radii / out.sparse_gaussian_ids: it has them even when its accepted gaussians ended
+        # without a single (tile, gaussian) pair, in which case there is no context and its gradients are zero
+        v = ctx.rows_per_camera[b] if ctx.rows_per_camera is not None else \
+            (0 if ctx_b is None else int(ctx_b.sparse_gaussian_ids.numel()))
         sl = slice(offs, offs + v)
         offs += v
+        if ctx_b is None:
+            duvs.append(torch.zeros((v, 2), dtype=torch.float32, device=dev))
+            continue
         g_b = GaussianSplatGradients(drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
                                      ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous())
         out_b = out.select_batch(b)
         out_b.radii = out.radii[sl]
-        gm, duv, _ = op.backward(model, cam_b, ctx_b, out_b, g_b, return_uv_grad=True)
+        gm, duv, _ = op.backward(model, cam_b, ctx_b, out_b, g_b, return_uv_grad=True, instance2world_T=instance2world_T)
         parts.append((ctx_b.sparse_gaussian_ids, gm))
         duvs.append(duv[0])
-    dev = model.xyz.device
     if not parts:
         op.last_sparse_unique_ids = torch.zeros(0, dtype=torch.int32, device=dev)
         zeros = {k: torch.zeros((0,) + tuple(v.shape[1:]), dtype=v.dtype, device=dev)
                  for k, v in model.get_proxy_field_dict().items()}
-        return dataclasses.replace(model, **zeros), None, None
-    all_ids = torch.cat([ids for ids, _ in parts], 0)
-    unique, inverse = torch.unique(all_ids, sorted=True, return_inverse=True)
-    op.last_sparse_unique_ids = unique.to(torch.int32)
+        return dataclasses.replace(model, **zeros), (torch.cat(duvs, 0).unsqueeze(0) if return_uv_grad and duvs else None), None
+    all_ids = torch.cat([ids for ids, _ in parts], 0).to(torch.int32).contiguous()
+    unique, run_rows, run_starts = op.unique_ids(all_ids, len(model))
+    op.last_sparse_unique_ids = unique
     merged = {}
     for name in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh", "color_sh_base"):
         if getattr(model, name) is None:
             continue
         rows = torch.cat([getattr(gm, name) for _, gm in parts], 0)
-        merged[name] = torch.zeros((unique.numel(),) + tuple(rows.shape[1:]), dtype=rows.dtype, device=dev)
-        merged[name].index_add_(0, inverse, rows)
+        merged[name] = op.merge_rows(rows, run_rows, run_starts, int(unique.numel()))
     # duv: one row per accepted (camera, gaussian), cameras one after the other, as out.sparse_gaussian_ids
     return dataclasses.replace(model, **merged), (torch.cat(duvs, 0).unsqueeze(0) if return_uv_grad else None), None
 
 
-def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
+def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad, instance2world_T=None):
     """Per-camera backward passes; the model gradients add up over the cameras, duv stays per camera."""
     if op._cfg.sparse_mode:
-        return _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad)
+        return _backward_bundle_sparse(op, model, ctx, out, grad, return_uv_grad, instance2world_T)
     total, duvs, dcfs = None, [], []
     n = len(model)
     for b, (ctx_b, cam_b) in enumerate(zip(ctx.per_camera, ctx.cameras)):
@@ -1205,7 +1366,8 @@ def _backward_bundle_impl(op, model, ctx, out, grad, return_uv_grad):
             drgb=grad.drgb[b:b + 1].contiguous(), dT=grad.dT[b:b + 1].contiguous(),
             ddepth=None if grad.ddepth is None else grad.ddepth[b:b + 1].contiguous(),
             dcustom_features=None if grad.dcustom_features is None else grad.dcustom_features[b:b + 1].contiguous())
-        gm, duv, dcf = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True)
+        gm, duv, dcf = op.backward(model, cam_b, ctx_b, out.select_batch(b), g_b, return_uv_grad=True,
+                                   instance2world_T=instance2world_T)
         duvs.append(duv)
         if dcf is not None:
             dcfs.append(dcf)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 30
+#define D3GS_ABI_VERSION 31
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -318,7 +318,12 @@ int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs,
  * clear_ptr (may be NULL; no counterpart in the reference): clear_bytes of device memory, both multiples of
  * 16, that the kernel sets to zero while it runs -- meant for the arrays the backward pass accumulates into
  * (grad_records, and the gradient arrays handed to d3gs_preprocess_bwd with outputs_are_zero): the blend is
- * bound by arithmetic and leaves the memory pipes idle, so the clear costs nothing here. */
+ * bound by arithmetic and leaves the memory pipes idle, so the clear costs nothing here.
+ * conic_opacity may hold any conic: the kernels' staging cull (bounding box and per-patch minimum of the quadratic
+ * form) only acts on positive definite ones and leaves the rest to the exact per-pixel sequence.  What is asked
+ * for is that power = -1/2 (a dx^2 + c dy^2) - b dx dy stays below 80 at every pixel of a tile that lists the
+ * gaussian (the blend's exp has no overflow guard); every positive semi-definite conic satisfies it, K1 writes no
+ * other.  The same holds for d3gs_blend_bwd. */
 int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                    const float* uvs, const float* conic_opacity, const float* rgb_gaussian, const float* depths,
                    const int32_t* tile_order /* from d3gs_tile_ranges, or NULL for raster order */, float* color,
@@ -426,22 +431,43 @@ int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_
  *      (they only index per-item arrays), then
  *   5. d3gs_preprocess_bwd_sparse: K9 over the V items; gradients are written per item, [V] rows (the rows of the
  *      model arrays are found through sparse_gaussian_ids), as the reference's sparse gradient (render.py:2918).
- * The render is the dense one bit for bit: slots ascend with the item index, so ties in the sort fall the same way. */
+ * The render is the dense one bit for bit: slots ascend with the item index, so ties in the sort fall the same way.
+ * `instances` (may be NULL) as in the dense entry points: instance ids are per row of the model arrays. */
 int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                                const float* opacity, const uint8_t* invalid_mask, int32_t* valid_flags,
                                const int32_t* slot_scan, int32_t* sparse_gaussian_ids, int32_t* sparse_batch_ids,
                                float* depths, int32_t* radii, float* uvs, float* conic_opacity, int32_t* tiles_touched,
-                               float* cov2d_vecs, uint64_t* tile_masks, uint32_t* depth_sort_keys, d3gs_stream_t stream);
+                               float* cov2d_vecs, uint64_t* tile_masks, uint32_t* depth_sort_keys,
+                               const d3gs_instances* instances, d3gs_stream_t stream);
 int d3gs_sh_colors_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids, const int32_t* sparse_batch_ids,
                           int32_t count, const float* xyz, const float* color_sh, const float* color_sh_base,
-                          const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0, d3gs_stream_t stream);
+                          const int32_t* radii, float* rgb_gaussian, uint8_t* sh_to_rgb_ne_0,
+                          const d3gs_instances* instances, d3gs_stream_t stream);
 int d3gs_preprocess_bwd_sparse(const d3gs_params* p /* n = V */, const int32_t* sparse_gaussian_ids, const float* xyz,
                                const float* quaternion_xyzw, const float* scale, const float* opacity,
                                const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
                                const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
                                int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
                                float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
-                               d3gs_stream_t stream);
+                               const d3gs_instances* instances, d3gs_stream_t stream);
+
+/* K10 -- replaces the hash-table deduplication of a sparse bundle's gradient rows (render.py:2864-2903: insert the
+ * accepted gaussian ids of all cameras, collect the distinct ones, query each row's slot, add the rows with atomics).
+ * d3gs_unique_ids: ids [count] (each in [0, id_limit)) -> the distinct ids in ascending order (unique_ids, the
+ * first *unique_count_dev entries of a [count] buffer), for every input row the index of its id in that list
+ * (inverse [count]), and the rows grouped by id: run_rows [count] lists the input rows sorted by id (rows of equal
+ * id in input order), run_starts [count + 1] where each id's run begins in it (run_starts[unique] = count).
+ * Built from the library's radix sort (value = row) and scan; the count also goes to unique_count_host (pinned
+ * host word, may be NULL) as in d3gs_scan_gathered.  workspace: d3gs_unique_ids_workspace_bytes, 256-byte aligned,
+ * need not be cleared.
+ * d3gs_merge_rows: merged[u][c] = sum of rows[r][c] over the rows r of run u, added in run order by one thread per
+ * (u, c): no atomics, so the sums do not depend on scheduling.  rows [n_rows][width], merged [n_runs][width]. */
+int d3gs_unique_ids_workspace_bytes(int32_t count, int32_t id_limit, size_t* bytes_out_host);
+int d3gs_unique_ids(const int32_t* ids, int32_t count, int32_t id_limit, int32_t* unique_ids, int32_t* inverse,
+                    int32_t* run_rows, int32_t* run_starts, void* workspace, size_t workspace_bytes,
+                    int64_t* unique_count_dev, int64_t* unique_count_host, d3gs_stream_t stream);
+int d3gs_merge_rows(const float* rows, int32_t n_rows, int32_t width, const int32_t* run_rows,
+                    const int32_t* run_starts, int32_t n_runs, float* merged, d3gs_stream_t stream);
 
 #ifdef __cplusplus
 }

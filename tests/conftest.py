@@ -3,6 +3,9 @@ import sys
 
 import pytest
 
+# the operator keeps the last view's sorted keys alive for the parity tests (read when the package is imported)
+os.environ.setdefault("D3GS_KEEP_SORTED_KEYS", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

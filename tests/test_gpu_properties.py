@@ -223,7 +223,7 @@ def test_atomic_add_count(capsys):
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
     counts = {}
     for algo in (RasterizeBackwardAlgo.DEFAULT, RasterizeBackwardAlgo.PER_GAUSSIAN):
-        op = GaussianSplatOp(op_config(scene, 4, measure_atomic_add_count=True, rasterize_backward_algo=algo))
+        op = GaussianSplatOp(op_config(scene, 4, measure_atomic_add_count=True, verbose=True, rasterize_backward_algo=algo))
         out, ctx = op.forward(model, scene.camera(), training=True)
         op.backward(model, scene.camera(), ctx, out, grads)
         assert f"atomic add count: {op.last_atomic_add_count}" in capsys.readouterr().out
@@ -239,3 +239,65 @@ def test_atomic_add_count(capsys):
         counts[algo] = op.last_atomic_add_count
     # both algorithms flush once per (tile, gaussian): the counts agree up to sums that cancel to zero in one of them
     assert abs(counts[RasterizeBackwardAlgo.DEFAULT] - counts[RasterizeBackwardAlgo.PER_GAUSSIAN]) <= 0.001 * max(counts.values())
+
+
+def test_one_operator_on_two_streams():
+    """The host words and buffer hints of an operator are kept per stream: forward + backward issued from two
+    streams in turn (each with a camera of its own, so that their pair counts differ) give what each gives alone."""
+    import torch
+    from d3gs_research_amd.camera import BasicPinholeCamera
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=30000, wh=(320, 240))
+    model = torch_model(scene)
+    tw = np.array(scene.to_world, np.float64)
+    tw[0, 3] += 0.4
+    cams = [scene.camera(), BasicPinholeCamera.from_params(scene.fx * 0.7, scene.fy * 0.7, scene.cx, scene.cy, scene.width,
+                                                          scene.height, tw)]
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    alone = []
+    for cam in cams:
+        op1 = GaussianSplatOp(op_config(scene, 4))
+        for _ in range(2):
+            out, ctx = op1.forward(model, cam, training=True)
+        gm, _, _ = op1.backward(model, cam, ctx, out, grads)
+        torch.cuda.synchronize()
+        alone.append((out.color.clone(), op1.last_num_rendered, gm.xyz.clone()))
+    assert alone[0][1] != alone[1][1]
+    op = GaussianSplatOp(op_config(scene, 4))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    got = [None, None]
+    for view in range(3):
+        for k, (cam, st) in enumerate(zip(cams, streams)):
+            with torch.cuda.stream(st):
+                out, ctx = op.forward(model, cam, training=True)
+                assert op.last_forward_fused == (view > 0) and op.last_num_rendered == alone[k][1]
+                gm, _, _ = op.backward(model, cam, ctx, out, grads)
+                got[k] = (out.color, gm.xyz)
+    torch.cuda.synchronize()
+    assert len(op._slots) == 2
+    for k in range(2):
+        assert torch.equal(got[k][0], alone[k][0])
+        assert torch.allclose(got[k][1], alone[k][2], rtol=1e-3, atol=1e-5 * float(alone[k][2].abs().max()))
+
+
+def test_polling_switches_itself_off_with_a_warning(monkeypatch):
+    """Three views in a row whose pair count does not reach the host within the polling time: the operator waits
+    on an event from then on and says so once."""
+    import torch
+    from d3gs_research_amd import render
+    scene = gen_scene(0)
+    op = render.GaussianSplatOp(op_config(scene, 1))
+    model = torch_model(scene)
+    out0, _ = op.forward(model, scene.camera(), training=True)
+    def slow(word, pending, seconds, synchronize, clock=None):  # every poll times out: the stream has to run dry
+        synchronize()
+        return "never" if int(word[0]) == pending else "synced"
+    monkeypatch.setattr(render, "poll_host_word", slow)
+    with pytest.warns(UserWarning, match="polling is switched off"):
+        for _ in range(3):
+            out, _ = op.forward(model, scene.camera(), training=True)
+            assert torch.equal(out.color, out0.color)
+    assert op.poll_pair_count is False
+    out, _ = op.forward(model, scene.camera(), training=True)
+    assert op.last_forward_fused and torch.equal(out.color, out0.color)

@@ -88,25 +88,57 @@ class _LibWithRaisedSortError:
 
 
 @pytest.mark.parametrize("which", ["depth", "pairs"])
-def test_forward_raises_when_a_sort_gave_up(which):
-    """Second view of an operator (binning as one library call): the raised error word must reach the host as a
-    negative pair count and forward must raise."""
+def test_forward_bins_again_when_a_sort_of_the_one_call_binning_gave_up(which):
+    """Second view of an operator (binning as one library call): the raised error word reaches the host as a
+    negative pair count; forward then bins the view once more, launch by launch into exactly sized buffers, and
+    renders the right image."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=20000, wh=(256, 192))
+    op = GaussianSplatOp(op_config(scene, 1))
+    model = torch_model(scene)
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    out, ctx = op.forward(model, scene.camera(), training=True)       # sizes the pair buffers
+    gm0, _, _ = op.backward(model, scene.camera(), ctx, out, grads)
+    good, good_idx, good_dxyz = out.color.clone(), ctx.gaussian_idx_sorted.clone(), gm0.xyz.clone()
+    real = op._lib
+    op._lib = _LibWithRaisedSortError(real, which)
+    out, ctx = op.forward(model, scene.camera(), training=True)
+    gm, _, _ = op.backward(model, scene.camera(), ctx, out, grads)
+    torch.cuda.synchronize()
+    assert op._lib.calls == 1 and op.recovered_views == 1 and not op.last_forward_fused
+    assert torch.equal(out.color, good) and torch.equal(ctx.gaussian_idx_sorted, good_idx)
+    assert torch.allclose(gm.xyz, good_dxyz, rtol=1e-3, atol=1e-5 * float(good_dxyz.abs().max()))
+    op._lib = real
+    out, ctx = op.forward(model, scene.camera(), training=True)       # and the next view takes the one-call path again
+    assert op.last_forward_fused and op.recovered_views == 1 and torch.equal(out.color, good)
+
+
+def test_forward_raises_when_the_second_binning_gives_up_too():
+    """... and when the launch-by-launch binning reports a look-back that gave up as well, forward raises."""
     import torch
     from d3gs_research_amd.render import GaussianSplatOp
     scene = gen_scene(1, n=20000, wh=(256, 192))
     op = GaussianSplatOp(op_config(scene, 1))
     model = torch_model(scene)
-    out, ctx = op.forward(model, scene.camera(), training=True)       # sizes the pair buffers
+    out, ctx = op.forward(model, scene.camera(), training=True)
     good = out.color.clone()
     real = op._lib
-    op._lib = _LibWithRaisedSortError(real, which)
+
+    class _Lib(_LibWithRaisedSortError):
+        def d3gs_sort_status(self, ws, nbytes, m, begin, end, st_dev, st_host, stream):
+            bad = torch.ones(nbytes, dtype=torch.uint8, device="cuda")      # a workspace whose error word is set
+            self.keep = bad
+            return real.d3gs_sort_status(C.c_void_p(bad.data_ptr()), nbytes, m, begin, end, st_dev, st_host, stream)
+
+    op._lib = _Lib(real, "pairs")
     with pytest.raises(RuntimeError, match="not sorted"):
         op.forward(model, scene.camera(), training=True)
-    assert op._lib.calls == 1
+    assert op.recovered_views == 1
     torch.cuda.synchronize()
     op._lib = real
     out, ctx = op.forward(model, scene.camera(), training=True)       # the operator is usable afterwards
-    assert op.last_forward_fused and torch.equal(out.color, good)
+    assert torch.equal(out.color, good)
 
 
 def test_stepwise_forward_raises_when_a_sort_gave_up():

@@ -129,3 +129,136 @@ def test_sparse_bundle_merges_the_cameras_rows():
         err = (a - b[unique]).abs().reshape(-1)
         scale = float(b.abs().max())
         assert float(torch.quantile(err[:: max(1, err.numel() // 1_000_000)], 0.999)) <= 1e-4 * scale and float(err.max()) <= 1e-3 * scale, name
+
+
+@pytest.mark.parametrize("count,id_limit", [(0, 10), (1, 1), (257, 40), (100_003, 30_000), (1_000_000, 3_000_000)])
+def test_unique_ids_and_merge_rows_c_abi(count, id_limit):
+    """d3gs_unique_ids / d3gs_merge_rows (the deduplication of a sparse bundle's rows, render.py:2864-2903) against
+    numpy.unique and a sequential float32 sum of each run's rows in run order."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(0, n=16)
+    op = GaussianSplatOp(op_config(scene, 1))
+    rng = np.random.default_rng(count)
+    ids = rng.integers(0, id_limit, count).astype(np.int32)
+    unique, run_rows, run_starts = op.unique_ids(torch.from_numpy(ids).cuda(), id_limit)
+    torch.cuda.synchronize()
+    want, inverse = np.unique(ids, return_inverse=True)
+    U = want.size
+    assert np.array_equal(unique.cpu().numpy(), want)
+    if count == 0:
+        return
+    assert np.array_equal(op.last_unique_inverse.cpu().numpy(), inverse)
+    rr, rs = run_rows.cpu().numpy(), run_starts.cpu().numpy()[:U + 1]
+    assert rs[0] == 0 and rs[U] == count and (np.diff(rs) > 0).all()
+    assert np.array_equal(ids[rr], np.sort(ids, kind="stable"))
+    assert np.array_equal(rr, np.argsort(ids, kind="stable"))         # rows of equal id keep their input order
+    for width in (1, 3, 48):
+        if count * width > 4_000_000:
+            continue
+        rows = rng.standard_normal((count, width)).astype(np.float32)
+        merged = op.merge_rows(torch.from_numpy(rows).cuda(), run_rows, run_starts, U).cpu().numpy()
+        ref = np.zeros((U, width), np.float32)
+        longest = int(np.diff(rs).max())
+        for k in range(longest):                                       # k-th row of every run that has one
+            has = rs[:-1] + k < rs[1:]
+            ref[has] = ref[has] + rows[rr[rs[:-1][has] + k]]
+        assert np.array_equal(merged.view(np.uint32), ref.view(np.uint32))
+
+
+def test_sparse_bundle_with_a_camera_that_renders_no_pair():
+    """A camera can accept gaussians (their 3-sigma rect meets the image) and still end without a single (tile,
+    gaussian) pair (OBB keeps no tile of any of them): it has rows in out.radii / out.sparse_gaussian_ids but no
+    context.  The rows of the cameras behind it must still line up, its own duv rows are zero."""
+    import torch
+    from d3gs_research_amd.camera import BasicPinholeCamera
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatGradients, GaussianSplatOp
+    scene = gen_scene(1, n=4000, wh=(320, 240))
+    # three faint gaussians just left of the image as the FIRST camera sees it: their 3-sigma rect reaches into
+    # tile column 0, the ellipse of alpha >= 1/255 (opacity barely above 1/255) does not
+    z = 4.0
+    for k in range(3):
+        scene.xyz[k] = [(-164.0 - k) * z / scene.fx, (k - 1) * 20.0 * z / scene.fy, 0.0]
+        scene.scale[k] = np.log(4.0 * z / scene.fx)
+        scene.opacity[k] = np.log(0.0046 / (1 - 0.0046))
+    model = torch_model(scene)
+    mask0 = np.ones(scene.n, bool)
+    mask0[:3] = False                          # camera 0 sees only the three
+    mask = np.concatenate([mask0, np.zeros(scene.n, bool), np.zeros(scene.n, bool)])
+    tw = np.array(scene.to_world, np.float64)
+    cams = []
+    for dx in (0.0, 0.25, -0.25):
+        t = tw.copy()
+        t[0, 3] += dx
+        cams.append(BasicPinholeCamera.from_params(scene.fx, scene.fy, scene.cx, scene.cy, scene.width, scene.height, t))
+    bundle = CameraBundle.from_pinhole_cams(cams)
+    mask_t = torch.from_numpy(mask).cuda()
+    rng = np.random.default_rng(5)
+    res = {}
+    for sparse in (False, True):
+        op = GaussianSplatOp(op_config(scene, 3, sparse_mode=sparse))
+        out, ctx = op.forward(model, bundle, training=True, mask=mask_t)
+        if not res:
+            drgb = torch.from_numpy(rng.standard_normal(out.color.shape).astype(np.float32)).cuda()
+            dT = torch.zeros_like(out.T)
+        gm, duv, _ = op.backward(model, bundle, ctx, out, GaussianSplatGradients(drgb=drgb, dT=dT), return_uv_grad=True)
+        torch.cuda.synchronize()
+        res[sparse] = (op, out, ctx, gm, duv)
+    (_, out_d, _, gm_d, duv_d), (op_s, out_s, ctx_s, gm_s, duv_s) = res[False], res[True]
+    B = 3
+    items = torch.nonzero(out_d.radii > 0).squeeze(1)
+    first = items[items < scene.n]
+    assert first.numel() == 3 and ctx_s.per_camera[0] is None and ctx_s.rows_per_camera[0] == 3      # accepted, no pair
+    assert float(out_s.T[0].min()) == 1.0
+    assert torch.equal(out_s.sparse_batch_ids.long() * scene.n + out_s.sparse_gaussian_ids.long(), items)
+    assert torch.equal(out_s.color, out_d.color)
+    assert tuple(duv_s.shape) == (1, items.numel(), 2) and float(duv_s[0, :3].abs().max()) == 0.0
+    top = float(duv_d.abs().max())
+    assert float((duv_s[0] - duv_d.reshape(B * scene.n, 2)[items]).abs().max()) <= 1e-4 * top
+    unique = op_s.last_sparse_unique_ids.long()
+    seen = torch.unique(out_s.sparse_gaussian_ids[3:].long())          # the first camera contributes no gradient row
+    assert torch.equal(unique, seen)
+    for name in ("xyz", "scale", "opacity", "color_sh"):
+        a, b = getattr(gm_s, name).double(), getattr(gm_d, name).double()
+        scale = float(b.abs().max())
+        assert float((a - b[unique]).abs().max()) <= 1e-3 * scale, name
+
+
+def test_sparse_mode_with_instances(oracle):
+    """sparse_mode with instance poses: the compact pass must equal the dense instance render (bit for bit) and the
+    oracle's, and its sparse gradient the oracle's rows of the accepted gaussians."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatGradients, GaussianSplatOp
+    from helpers import oracle_params
+    from test_gpu_instances import _setup
+    scene = _narrow_scene()
+    K = 5
+    T, ids_np, model, cam = _setup(scene, K, 77)
+    T_dev = torch.from_numpy(T).cuda()
+    grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
+    res = {}
+    for sparse in (False, True):
+        op = GaussianSplatOp(op_config(scene, 4, sparse_mode=sparse))
+        for _ in range(2):
+            out, ctx = op.forward(model, cam, training=True, instance2world_T=T_dev)
+        gm, duv, _ = op.backward(model, cam, ctx, out, grads, return_uv_grad=True)
+        torch.cuda.synchronize()
+        res[sparse] = (op, out, ctx, gm, duv)
+    (op_d, out_d, ctx_d, gm_d, _), (_, out_s, ctx_s, gm_s, _) = res[False], res[True]
+    ids = out_s.sparse_gaussian_ids.long()
+    assert 0 < ids.numel() < scene.n and torch.equal(ids, torch.nonzero(out_d.radii > 0).squeeze(1))
+    for name in ("color", "T", "n_contrib"):
+        assert torch.equal(getattr(out_s, name), getattr(out_d, name)), name
+    for name in ("uvs", "conic_opacity", "rgb_gaussian", "cov2d_vecs"):
+        assert torch.equal(getattr(ctx_s, name), getattr(ctx_d, name)[ids]), name
+    _, table = op_d.instance_table(model, cam, T_dev)
+    inst = (ids_np, table.cpu().numpy())
+    P = oracle_params(oracle, scene, 4)
+    args = (scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    ref = oracle.forward(P, *args, instances=inst)
+    assert np.array_equal(out_s.color.cpu().numpy()[0].view(np.uint32), ref["color"].view(np.uint32))
+    _, pb_ref = oracle.backward(P, ref, *args, scene.drgb[0], scene.dT[0], instances=inst)
+    sel = ids.cpu().numpy()
+    for name, got in (("dxyz", gm_s.xyz), ("dscale", gm_s.scale), ("dopacity", gm_s.opacity), ("dsh", gm_s.color_sh)):
+        ok, worst, nbad = grad_close(got.cpu().numpy(), pb_ref[name][sel], rel=1e-3, abs_frac=1e-4)
+        assert ok, (name, worst, nbad)
