@@ -90,8 +90,9 @@ _SIGNATURES = {
     "d3gs_unique_ids": (C.c_int, [_VP, C.c_int32, C.c_int32, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, _VP, _VP]),
     "d3gs_merge_rows": (C.c_int, [_VP, C.c_int32, C.c_int32, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_bucket_offsets": (C.c_int, [_VP, C.c_int32, _VP, _VP]),
-    "d3gs_blend_fwd_snapshots": (C.c_int, [C.POINTER(Params)] + [_VP] * 9 + [_VP, C.c_size_t] + [_VP] * 3),
-    "d3gs_blend_bwd_per_gaussian": (C.c_int, [C.POINTER(Params)] + [_VP] * 15 + [_VP]),
+    "d3gs_snapshot_floats": (C.c_int, [C.POINTER(Params)]),
+    "d3gs_blend_fwd_snapshots": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP] * 3),
+    "d3gs_blend_bwd_per_gaussian": (C.c_int, [C.POINTER(Params)] + [_VP] * 18 + [_VP]),
     "d3gs_preprocess_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 10 + [C.c_int32, C.c_int32] + [_VP] * 6 +
                             [C.POINTER(Instances), _VP]),
     "d3gs_preprocess_bwd_camera": (C.c_int, [C.POINTER(Params), C.c_int32, C.c_int32] + [_VP] * 10 +

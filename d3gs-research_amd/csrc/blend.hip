@@ -416,9 +416,13 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
             if constexpr (kSnap) {
                 // state of this wavefront's pixels in front of list entry round * 256 + chunk * 64 (a wavefront
                 // whose pixels have all finished skips this: no gaussian from here on contributes to them)
-                if (round * kBlock + chunk * kBucket < len)
-                    snap[((size_t)bucket_offsets[tile] + round * (kBlock / kBucket) + chunk) * kBlock + tid] =
-                        make_float4(T, acc0, acc1, acc2);
+                if (round * kBlock + chunk * kBucket < len) {
+                    // one quad per pixel and bucket, two with an alpha or a depth channel (their running sums)
+                    constexpr int kQuads = (kDepth || kRgba) ? 2 : 1;
+                    float4* dst = snap + (((size_t)bucket_offsets[tile] + round * (kBlock / kBucket) + chunk) * kBlock + tid) * kQuads;
+                    dst[0] = make_float4(T, acc0, acc1, acc2);
+                    if constexpr (kQuads == 2) dst[1] = make_float4(acc3, depth_accum, 0.0f, 0.0f);
+                }
             }
             unsigned long long m = uniform_u64(s_mask[wave][chunk]);
             while (m) {
@@ -730,17 +734,27 @@ __device__ __forceinline__ float dpp_shift_in(float fresh, float v) {
 }
 constexpr int kDppWaveShr1 = 0x138;
 
+// kDepth / kRgba: a depth and an alpha channel ride along as in the default kernel (render.py:2364-2398, 2412-2415,
+// 2490-2528): their running sums are part of the pixel state handed from lane to lane, the snapshots hold them in a
+// second quad, and the depth gradient is the record's tenth value.
+template <bool kDepth, bool kRgba>
 __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
     const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
     const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
-    const int32_t* __restrict__ tile_order, const float* __restrict__ final_T, const int32_t* __restrict__ n_contrib,
-    const float* __restrict__ color, const float* __restrict__ drgb, const float* __restrict__ dT,
+    const float* __restrict__ depths, const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
+    const int32_t* __restrict__ n_contrib, const float* __restrict__ color, const float* __restrict__ final_depth,
+    const float* __restrict__ drgb, const float* __restrict__ dT, const float* __restrict__ ddepth,
     const int32_t* __restrict__ bucket_offsets, const float4* __restrict__ snap, float* __restrict__ grad_records,
     uint8_t* __restrict__ touched) {
     constexpr int kWaves = kBlock / 64;
+    constexpr bool kExtra = kDepth || kRgba;
+    constexpr int kQuads = kExtra ? 2 : 1;
+    constexpr int kChannels = kRgba ? 4 : 3;
     __shared__ float4 s_pix_grad[kBlock];    // per pixel: drgb (3), -dT * final_T
     __shared__ float4 s_pix_final[kBlock];   // per pixel: final colour (3), contributor (int bits)
+    __shared__ float4 s_pix_extra[kExtra ? kBlock : 1];   // per pixel: d alpha, d depth, final alpha, final depth
     __shared__ float4 s_snap[kWaves][kBlock];            // the bucket's snapshots: T, colour in front of the bucket
+    __shared__ float2 s_snap_extra[kExtra ? kWaves : 1][kExtra ? kBlock : 1];   // ... alpha and depth sums
     __shared__ unsigned short s_open[kWaves][kBlock];    // pixels still open at the bucket's start
     __shared__ float s_out[kWaves][kBucket][D3GS_GRAD_RECORD_FLOATS + 1];
     __shared__ int s_gid[kWaves][kBucket];
@@ -763,18 +777,30 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
         const bool inside = px < P.width && py < P.height;
         int contributor = 0;
         float4 pg = make_float4(0.0f, 0.0f, 0.0f, 0.0f), pf = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float4 pe = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (inside) {
             const size_t pid = (size_t)py * P.width + px;
             const size_t gpid = (size_t)place.batch * P.width * P.height + pid;
             contributor = min(n_contrib[gpid] + 1, len);
-            pg = make_float4(drgb[color_index(P, place.batch, pid, 0, 3)], drgb[color_index(P, place.batch, pid, 1, 3)],
-                             drgb[color_index(P, place.batch, pid, 2, 3)], (-dT[gpid]) * final_T[gpid]);
-            pf = make_float4(color[color_index(P, place.batch, pid, 0, 3)], color[color_index(P, place.batch, pid, 1, 3)],
-                             color[color_index(P, place.batch, pid, 2, 3)], 0.0f);
+            pg = make_float4(drgb[color_index(P, place.batch, pid, 0, kChannels)],
+                             drgb[color_index(P, place.batch, pid, 1, kChannels)],
+                             drgb[color_index(P, place.batch, pid, 2, kChannels)], (-dT[gpid]) * final_T[gpid]);
+            pf = make_float4(color[color_index(P, place.batch, pid, 0, kChannels)],
+                             color[color_index(P, place.batch, pid, 1, kChannels)],
+                             color[color_index(P, place.batch, pid, 2, kChannels)], 0.0f);
+            if constexpr (kRgba) {
+                pe.x = drgb[color_index(P, place.batch, pid, 3, kChannels)];
+                pe.z = color[color_index(P, place.batch, pid, 3, kChannels)];
+            }
+            if constexpr (kDepth) {
+                pe.y = ddepth[gpid];
+                pe.w = final_depth[gpid];
+            }
         }
         pf.w = __int_as_float(contributor);
         s_pix_grad[tid] = pg;
         s_pix_final[tid] = pf;
+        if constexpr (kExtra) s_pix_extra[tid] = pe;
         const int wmax = wave_max_i32(contributor);
         if (lane == 0) s_wmax[wave] = wmax;
     }
@@ -786,14 +812,18 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
     for (int bucket = wave; bucket < nbuckets; bucket += kWaves) {      // wave-uniform
         const int bstart = bucket * kBucket;
         // the bucket's snapshots, and the list of pixels still open at its start
-        const float4* sb = snap + ((size_t)bucket_offsets[tile] + bucket) * kBlock;
+        const float4* sb = snap + ((size_t)bucket_offsets[tile] + bucket) * kBlock * kQuads;
         int cnt = 0;
 #pragma unroll
         for (int q = 0; q < kBlock / 64; ++q) {
             const int p = q * 64 + lane;
             const bool open = __float_as_int(s_pix_final[p].w) > bstart;
             // a snapshot of a finished pixel may never have been written: it is not read, and not staged
-            s_snap[wave][p] = open ? sb[p] : make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+            s_snap[wave][p] = open ? sb[(size_t)p * kQuads] : make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+            if constexpr (kExtra) {
+                const float4 e = open ? sb[(size_t)p * kQuads + 1] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                s_snap_extra[wave][p] = make_float2(e.x, e.y);
+            }
             const unsigned long long bal = __ballot(open);
             if (open) s_open[wave][cnt + __popcll(bal & lt_mask)] = (unsigned short)p;
             cnt += __popcll(bal);
@@ -808,15 +838,15 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
             const int g = idx_sorted[r0 + li];
             if ((unsigned)g < (unsigned)items) {   // a corrupt index list must not become a wild read or write
                 gid = g;
-                stage_gaussian(P, g, uvs, conic_opacity, rgb_g, nullptr, tile_x0, tile_y0, &sg);
+                stage_gaussian(P, g, uvs, conic_opacity, rgb_g, kDepth ? depths : nullptr, tile_x0, tile_y0, &sg);
                 c0 = sg.r;
                 c1 = sg.g;
                 c2 = sg.b;
             }
         }
         __builtin_amdgcn_wave_barrier();    // the wavefront's own LDS writes above are read below
-        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, a4 = 0.0f, a5 = 0.0f, a6 = 0.0f, a7 = 0.0f, a8 = 0.0f;
-        float T = 1.0f, rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f;
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, a4 = 0.0f, a5 = 0.0f, a6 = 0.0f, a7 = 0.0f, a8 = 0.0f, a9 = 0.0f;
+        float T = 1.0f, rr0 = 0.0f, rr1 = 0.0f, rr2 = 0.0f, rr3 = 0.0f, rdep = 0.0f;
         const int steps = cnt > 0 ? cnt + kBucket - 1 : 0;
         for (int j = 0; j < steps; ++j) {
             // lane 0 takes up open pixel j with the state it has in front of the bucket; every other lane takes
@@ -829,6 +859,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
             rr0 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.x - sn.y : 0.0f, rr0);
             rr1 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.y - sn.z : 0.0f, rr1);
             rr2 = dpp_shift_in<kDppWaveShr1>(fresh ? fin.z - sn.w : 0.0f, rr2);
+            if constexpr (kExtra) {
+                const float2 se = s_snap_extra[wave][q];
+                const float4 fe = s_pix_extra[q];
+                if constexpr (kRgba) rr3 = dpp_shift_in<kDppWaveShr1>(fresh ? fe.z - se.x : 0.0f, rr3);
+                if constexpr (kDepth) rdep = dpp_shift_in<kDppWaveShr1>(fresh ? fe.w - se.y : 0.0f, rdep);
+            }
             const int k = j - lane;                        // which open pixel this lane holds now
             const bool holding = k >= 0 && k < cnt;
             const int p = holding ? s_open[wave][k] : 0;
@@ -851,6 +887,16 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
             rr1 = __builtin_fmaf(-w, c1, rr1);
             rr2 = __builtin_fmaf(-w, c2, rr2);
             float dl = pg.w;
+            if constexpr (kDepth) {      // the default kernel's order of terms: depth, alpha, then blue, green, red
+                const float ddep = s_pix_extra[p].y;
+                rdep = __builtin_fmaf(-w, sg.depth, rdep);
+                dl = __builtin_fmaf(ddep, __builtin_fmaf(T, sg.depth, -rdep), dl);
+                a9 += w * ddep;
+            }
+            if constexpr (kRgba) {
+                rr3 = rr3 - w;
+                dl = __builtin_fmaf(s_pix_extra[p].x, T - rr3, dl);
+            }
             dl = __builtin_fmaf(pg.z, __builtin_fmaf(T, c2, -rr2), dl);
             dl = __builtin_fmaf(pg.y, __builtin_fmaf(T, c1, -rr1), dl);
             dl = __builtin_fmaf(pg.x, __builtin_fmaf(T, c0, -rr0), dl);
@@ -879,8 +925,9 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_per_gaussian_kernel(
         row[6] = a6;
         row[7] = a7;
         row[8] = a8;
+        row[9] = a9;
 #pragma unroll
-        for (int c = 9; c < D3GS_GRAD_RECORD_FLOATS; ++c) row[c] = 0.0f;
+        for (int c = 10; c < D3GS_GRAD_RECORD_FLOATS; ++c) row[c] = 0.0f;
         s_gid[wave][lane] = gid;
         __builtin_amdgcn_wave_barrier();
         // sixteen lanes add one gaussian's record: one line-wide atomic per (tile, gaussian)
@@ -958,7 +1005,10 @@ static int launch_blend_fwd(const d3gs_params* p, const int32_t* workload_ranges
     hipLaunchKernelGGL((blend_fwd_kernel<D, A, S>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,  \
                        workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
                        color, final_T, n_contrib, final_depth, (uint4*)clear_ptr, clear_bytes / 16, bucket_offsets, snap)
-    if (snap) D3GS_LAUNCH_FWD(false, false, true);
+    if (snap) {
+        if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true, true); else D3GS_LAUNCH_FWD(true, false, true); }
+        else                 { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true, true); else D3GS_LAUNCH_FWD(false, false, true); }
+    }
     else if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_FWD(true, true, false); else D3GS_LAUNCH_FWD(true, false, false); }
     else                      { if (p->render_rgba) D3GS_LAUNCH_FWD(false, true, false); else D3GS_LAUNCH_FWD(false, false, false); }
 #undef D3GS_LAUNCH_FWD
@@ -985,30 +1035,30 @@ extern "C" int d3gs_blend_fwd(const d3gs_params* p, const int32_t* workload_rang
                             color, final_T, n_contrib, final_depth, clear_ptr, clear_bytes, nullptr, nullptr, stream);
 }
 
+extern "C" int d3gs_snapshot_floats(const d3gs_params* p) {
+    return (p && (p->render_depth || p->render_rgba)) ? 8 : 4;
+}
+
 extern "C" int d3gs_blend_fwd_snapshots(const d3gs_params* p, const int32_t* workload_ranges,
                                         const int32_t* gaussian_idx_sorted, const float* uvs, const float* conic_opacity,
-                                        const float* rgb_gaussian, const int32_t* tile_order, float* color,
-                                        float* final_T, int32_t* n_contrib, void* clear_ptr, size_t clear_bytes,
-                                        const int32_t* bucket_offsets, float* snapshots, d3gs_stream_t stream) {
+                                        const float* rgb_gaussian, const float* depths, const int32_t* tile_order,
+                                        float* color, float* final_T, int32_t* n_contrib, float* final_depth,
+                                        void* clear_ptr, size_t clear_bytes, const int32_t* bucket_offsets,
+                                        float* snapshots, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_fwd_snapshots");
     if (rc) return rc;
-    if (p->render_depth || p->render_rgba) {
-        set_error("d3gs_blend_fwd_snapshots: the per-gaussian backward covers the colour channels only "
-                  "(no render_depth / render_rgba)");
-        return D3GS_ERR_UNSUPPORTED;
-    }
     if (clear_ptr && ((((uintptr_t)clear_ptr) | clear_bytes) & 15u)) {
         set_error("d3gs_blend_fwd_snapshots: clear_ptr / clear_bytes must be multiples of 16");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !color || !final_T || !n_contrib ||
-        !bucket_offsets || !snapshots || (((uintptr_t)snapshots) & 15u)) {
+        !bucket_offsets || !snapshots || (((uintptr_t)snapshots) & 15u) || (p->render_depth && (!depths || !final_depth))) {
         set_error("d3gs_blend_fwd_snapshots: NULL buffer (snapshots must be 16-byte aligned)");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    return launch_blend_fwd(p, workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, nullptr, tile_order,
-                            color, final_T, n_contrib, nullptr, clear_ptr, clear_bytes, bucket_offsets, (float4*)snapshots,
-                            stream);
+    return launch_blend_fwd(p, workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,
+                            color, final_T, n_contrib, final_depth, clear_ptr, clear_bytes, bucket_offsets,
+                            (float4*)snapshots, stream);
 }
 
 extern "C" int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
@@ -1047,23 +1097,26 @@ extern "C" int d3gs_bucket_offsets(const int32_t* workload_ranges, int32_t num_t
 
 extern "C" int d3gs_blend_bwd_per_gaussian(const d3gs_params* p, const int32_t* workload_ranges,
                                            const int32_t* gaussian_idx_sorted, const float* uvs, const float* conic_opacity,
-                                           const float* rgb_gaussian, const int32_t* tile_order, const float* final_T,
-                                           const int32_t* n_contrib, const float* color, const float* drgb, const float* dT,
-                                           const int32_t* bucket_offsets, const float* snapshots, float* grad_records,
-                                           uint8_t* touched, d3gs_stream_t stream) {
+                                           const float* rgb_gaussian, const float* depths, const int32_t* tile_order,
+                                           const float* final_T, const int32_t* n_contrib, const float* color,
+                                           const float* final_depth, const float* drgb, const float* dT,
+                                           const float* ddepth, const int32_t* bucket_offsets, const float* snapshots,
+                                           float* grad_records, uint8_t* touched, d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_blend_bwd_per_gaussian");
     if (rc) return rc;
-    if (p->render_depth || p->render_rgba || p->use_nchw) {
-        set_error("d3gs_blend_bwd_per_gaussian: colour channels in [H,W,3] only (no render_depth / render_rgba / use_nchw)");
-        return D3GS_ERR_UNSUPPORTED;
-    }
     if (!workload_ranges || !uvs || !conic_opacity || !rgb_gaussian || !final_T || !n_contrib || !color || !drgb || !dT ||
-        !bucket_offsets || !snapshots || !grad_records || (((uintptr_t)snapshots) & 15u)) {
+        !bucket_offsets || !snapshots || !grad_records || (((uintptr_t)snapshots) & 15u) ||
+        (p->render_depth && (!depths || !final_depth || !ddepth))) {
         set_error("d3gs_blend_bwd_per_gaussian: NULL buffer (snapshots must be 16-byte aligned)");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    hipLaunchKernelGGL(blend_bwd_per_gaussian_kernel, dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                       workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, tile_order, final_T,
-                       n_contrib, color, drgb, dT, bucket_offsets, (const float4*)snapshots, grad_records, touched);
+#define D3GS_LAUNCH_PG(D, A)                                                                                          \
+    hipLaunchKernelGGL((blend_bwd_per_gaussian_kernel<D, A>), dim3(blend_grid(p)), dim3(kBlock), 0, (hipStream_t)stream, \
+                       *p, workload_ranges, gaussian_idx_sorted, uvs, conic_opacity, rgb_gaussian, depths, tile_order,  \
+                       final_T, n_contrib, color, final_depth, drgb, dT, ddepth, bucket_offsets,                       \
+                       (const float4*)snapshots, grad_records, touched)
+    if (p->render_depth) { if (p->render_rgba) D3GS_LAUNCH_PG(true, true); else D3GS_LAUNCH_PG(true, false); }
+    else                 { if (p->render_rgba) D3GS_LAUNCH_PG(false, true); else D3GS_LAUNCH_PG(false, false); }
+#undef D3GS_LAUNCH_PG
     return finish_launch("d3gs_blend_bwd_per_gaussian");
 }

@@ -253,10 +253,9 @@ class GaussianSplatOp:
                                    or c.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN),
             # builtin colours off: the kernels blend zeros in their place (render.py:262, 662, 1898-1931)
             "disable_builtin_rgb with use_nchw": c.disable_builtin_rgb and c.use_nchw,
-            # the per-gaussian backward (render.py:2319-2776) is built for the colour channels in [H,W,3]
-            "rasterize_backward_algo = PER_GAUSSIAN with render_depth / render_rgba / use_nchw / disable_builtin_rgb":
-                c.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN
-                and (c.render_depth or c.render_rgba or c.use_nchw or c.disable_builtin_rgb),
+            # the per-gaussian backward (render.py:2319-2776) needs the model's own colours in the colour channels
+            "rasterize_backward_algo = PER_GAUSSIAN with disable_builtin_rgb":
+                c.rasterize_backward_algo == RasterizeBackwardAlgo.PER_GAUSSIAN and c.disable_builtin_rgb,
             # Accepted without a code path of their own, because they change how the reference computes and not
             # what: move_opacity_in_grad_to_prep (render.py:1973-1990, 2995-3003) takes the factors opacity, -1/2
             # and -1 out of the per-pixel gradient terms and applies them once per gaussian -- the same gradient up
@@ -470,9 +469,8 @@ class GaussianSplatOp:
 
     def _snapshot_floats(self) -> int:
         """Floats per pixel and bucket of the per-gaussian backward's snapshots: T and the colour accumulated so far,
-        and with a depth or an alpha channel their sums too (render.py:1744-1759, 2412-2415)."""
-        return 4 + int(bool(self._cfg.render_depth)) + int(bool(self._cfg.render_rgba)) \
-            if (self._cfg.render_depth or self._cfg.render_rgba) else 4
+        and with a depth or an alpha channel a second quad with their sums (render.py:1744-1759, 2412-2415)."""
+        return 8 if (self._cfg.render_depth or self._cfg.render_rgba) else 4
 
     # ---------------------------------------------------------------- forward
     def forward(self, model: GaussianModelOriginBase, cameras, training: bool = False, instance2world_T=None,
@@ -1173,10 +1171,10 @@ class GaussianSplatOp:
                 bucket_offsets, snapshots = ctx.per_gaussian_snap
                 _capi.check(L.d3gs_blend_fwd_snapshots(
                     C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-                    _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order),
-                    _capi.ptr(color), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(clear),
-                    0 if clear is None else clear.numel() * 4, _capi.ptr(bucket_offsets), _capi.ptr(snapshots), s),
-                    "d3gs_blend_fwd_snapshots")
+                    _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
+                    _capi.ptr(ctx.tile_order), _capi.ptr(color), _capi.ptr(out.T), _capi.ptr(out.n_contrib),
+                    _capi.ptr(out.depth), _capi.ptr(clear), 0 if clear is None else clear.numel() * 4,
+                    _capi.ptr(bucket_offsets), _capi.ptr(snapshots), s), "d3gs_blend_fwd_snapshots")
                 return None
             _capi.check(L.d3gs_blend_fwd(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
@@ -1212,8 +1210,9 @@ class GaussianSplatOp:
             bucket_offsets, snapshots = ctx.per_gaussian_snap
             _capi.check(L.d3gs_blend_bwd_per_gaussian(
                 C.byref(P), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
-                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.tile_order), _capi.ptr(out.T),
-                _capi.ptr(out.n_contrib), _capi.ptr(color), _capi.ptr(drgb), _capi.ptr(grad.dT),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(ctx.rgb_gaussian), _capi.ptr(ctx.depths),
+                _capi.ptr(ctx.tile_order), _capi.ptr(out.T), _capi.ptr(out.n_contrib), _capi.ptr(color),
+                _capi.ptr(out.depth), _capi.ptr(drgb), _capi.ptr(grad.dT), _capi.ptr(ddepth),
                 _capi.ptr(bucket_offsets), _capi.ptr(snapshots), _capi.ptr(rec), _capi.ptr(touched), s),
                 "d3gs_blend_bwd_per_gaussian")
         else:

@@ -362,25 +362,30 @@ int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const i
  *   d3gs_bucket_offsets (K8, replaces kernel_1d("prepare_bucket_...") + cumsum_, render.py:941-950):
  *     bucket_offsets[t] = sum over tiles before t of ceil(list length / D3GS_BUCKET_SIZE), [num_tiles + 1] int32,
  *     the last entry the total; no host read-back is needed: ceil(M / D3GS_BUCKET_SIZE) + num_tiles bounds the total;
- *   d3gs_blend_fwd_snapshots: d3gs_blend_fwd (colour channels, [H,W,3]) that also stores every pixel's running
- *     state in front of each bucket: snapshots [total buckets][256][4] float32 (T, accumulated r, g, b; pixel order
- *     of the kernel's threads), the reference's T_snap / color_snap (render.py:958-959, 1744-1759).  Same image
- *     bit for bit;
- *   d3gs_blend_bwd_per_gaussian: the backward over those snapshots; arguments as d3gs_blend_bwd.  One wavefront per
- *     bucket of 64 list entries (the reference: one 32-lane warp per 32), one workgroup per tile.
+ *   d3gs_blend_fwd_snapshots: d3gs_blend_fwd (same arguments, same image bit for bit) that also stores every pixel's
+ *     running state in front of each bucket: snapshots [total buckets][256][d3gs_snapshot_floats(p)] float32, pixel
+ *     order of the kernel's threads: (T, accumulated r, g, b) and, with render_depth or render_rgba, a second quad
+ *     (accumulated alpha, accumulated depth, 0, 0) -- the reference's T_snap / color_snap and their depth / alpha
+ *     companions (render.py:958-959, 1744-1759, 2412-2415);
+ *   d3gs_blend_bwd_per_gaussian: the backward over those snapshots; arguments as d3gs_blend_bwd (depth, RGBA and
+ *     NCHW included, render.py:2364-2398, 2490-2528).  One wavefront per bucket of 64 list entries (the reference:
+ *     one 32-lane warp per 32), one workgroup per tile.
  * The gradient is the complete one, as d3gs_blend_bwd's, up to the order of the float32 sums. */
 #define D3GS_BUCKET_SIZE 64
 int d3gs_bucket_offsets(const int32_t* workload_ranges, int32_t num_tiles, int32_t* bucket_offsets, d3gs_stream_t stream);
+int d3gs_snapshot_floats(const d3gs_params* p);      /* 4, or 8 with render_depth / render_rgba */
 int d3gs_blend_fwd_snapshots(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                              const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                             const int32_t* tile_order, float* color, float* final_T, int32_t* n_contrib,
-                             void* clear_ptr, size_t clear_bytes, const int32_t* bucket_offsets, float* snapshots,
-                             d3gs_stream_t stream);
+                             const float* depths, const int32_t* tile_order, float* color, float* final_T,
+                             int32_t* n_contrib, float* final_depth, void* clear_ptr, size_t clear_bytes,
+                             const int32_t* bucket_offsets, float* snapshots, d3gs_stream_t stream);
 int d3gs_blend_bwd_per_gaussian(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
                                 const float* uvs, const float* conic_opacity, const float* rgb_gaussian,
-                                const int32_t* tile_order, const float* final_T, const int32_t* n_contrib,
-                                const float* color, const float* drgb, const float* dT, const int32_t* bucket_offsets,
-                                const float* snapshots, float* grad_records, uint8_t* touched, d3gs_stream_t stream);
+                                const float* depths, const int32_t* tile_order, const float* final_T,
+                                const int32_t* n_contrib, const float* color, const float* final_depth,
+                                const float* drgb, const float* dT, const float* ddepth,
+                                const int32_t* bucket_offsets, const float* snapshots, float* grad_records,
+                                uint8_t* touched, d3gs_stream_t stream);
 
 /* K9 — replaces kernel_1d("gs3d_preprocess_bwd_...") at render.py:2922-3369
  * (body 3217-3356).  Chain rule from K7's records (duv, dconic, dopacity, dcolor

@@ -824,8 +824,9 @@ ORC_API void orc_blend_bwd(const orc_params* P, const int32_t* ranges, const int
                     }
                     if (statemass) {
                         double state = 0.0;
-                        for (int ch = 0; ch < 3; ++ch)
+                        for (int ch = 0; ch < 3 + (P->render_rgba ? 1 : 0); ++ch)
                             state += fabs((double)dr[ch]) * fabs((double)color[color_index(P, pid, ch)]);
+                        if (P->render_depth) state += fabs((double)ddep) * fabs((double)final_depth[pid]);
                         const double per_dl = fabs((double)G / (double)one_m) * state;     // d gop / d dl, times state
                         const double geom[6] = {fabs((double)co[3] * dx), fabs((double)co[3] * dy),
                                                 fabs((double)co[3] * dx * dx), fabs((double)co[3] * dx * dy),

@@ -72,9 +72,12 @@ def k9_noise_spread(O, P, scene, ref, g_ref, pb_ref, ulps=2.0, seed=11, state_ul
              "dconic": g_ref["dconic"] + rng.standard_normal(g_ref["dconic"].shape) * m[:, 2:5],
              "dopacity": g_ref["dopacity"] + rng.standard_normal(g_ref["dopacity"].shape) * m[:, 5],
              "dcolor": g_ref["dcolor"] + rng.standard_normal(g_ref["dcolor"].shape) * m[:, 6:9]}
+    dz = None
+    if g_ref.get("dz") is not None:      # a depth channel: its gradient takes part, with its own summation noise
+        dz = (g_ref["dz"] + rng.standard_normal(g_ref["dz"].shape) * (ulps * 2.0 ** -24) * g_ref["absmass"][:, 9]).astype(np.float32)
     pert = O.preprocess_bwd(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
                             ref["radii"], ref["cov2d_vecs"], ref["sh_to_rgb_ne_0"],
-                            *(noisy[k].astype(np.float32) for k in ("duv", "dconic", "dopacity", "dcolor")))
+                            *(noisy[k].astype(np.float32) for k in ("duv", "dconic", "dopacity", "dcolor")), dz=dz)
     names = ("dxyz", "dquat", "dscale", "dopacity", "dsh")
     if tail:
         return {k: rel_err_summary(per_gaussian_rel_err(pert[k], pb_ref[k])) for k in names}

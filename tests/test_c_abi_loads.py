@@ -89,13 +89,15 @@ def test_operator_config_gate():
     from d3gs_research_amd.render import GaussianSplatOp
     GaussianSplatOp(GaussianSplatConfig())
     GaussianSplatOp(GaussianSplatConfig(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN))
+    GaussianSplatOp(GaussianSplatConfig(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN, render_depth=True,
+                                        render_rgba=True, use_nchw=True))
     GaussianSplatOp(GaussianSplatConfig(disable_builtin_rgb=True, render_rgba=True, render_depth=True,
                                         enable_anti_aliasing=True))
     GaussianSplatOp(GaussianSplatConfig(move_opacity_in_grad_to_prep=True, use_int64_tile_touched=True,
                                         enable_32bit_sort=True))
     GaussianSplatOp(GaussianSplatConfig(sparse_mode=True))
     for kw, word in ((dict(sparse_mode=True, disable_builtin_rgb=True), "sparse_mode"), (dict(render_inv_depth=True), "render_inv_depth"),
-                     (dict(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN, render_depth=True), "PER_GAUSSIAN"),
+                     (dict(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN, disable_builtin_rgb=True), "PER_GAUSSIAN"),
                      (dict(transmittance_is_double=True), "transmittance_is_double"), (dict(tile_size=(8, 8)), "tile_size"),
                      (dict(disable_builtin_rgb=True, use_nchw=True), "use_nchw")):
         with pytest.raises(NotImplementedError, match=word):
