@@ -494,8 +494,14 @@ __global__ __launch_bounds__(kBlock) void blend_fwd_kernel(const d3gs_params P, 
 // four wavefronts in LDS, and only then added to global memory: one atomic per
 // value per (tile, gaussian).
 // ---------------------------------------------------------------------------
+// Gaussians staged per round: 224 instead of the workgroup's 256 keeps the kernel's LDS (staged records + ids +
+// nine rows of sums) under 20 KiB, so that eight workgroups share a compute unit instead of seven (the plain colour
+// instantiation is told to fit the 64 vector registers that takes; it does, without spilling).  The kernel is bound by
+// how many wavefronts are there to hide each other's dependent chains: seven instead of five workgroups is worth 9-12 %.
+constexpr int kBwdStage = 224;
+
 template <bool kDepth, bool kRgba>
-__global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu((kDepth || kRgba) ? 6 : 8, 8))) void blend_bwd_kernel(
     const d3gs_params P, const int32_t* __restrict__ ranges, const int32_t* __restrict__ idx_sorted,
     const float* __restrict__ uvs, const float* __restrict__ conic_opacity, const float* __restrict__ rgb_g,
     const float* __restrict__ depths, const int32_t* __restrict__ tile_order, const float* __restrict__ final_T,
@@ -504,11 +510,11 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     float* __restrict__ grad_records, uint8_t* __restrict__ touched) {
     constexpr int kValues = kDepth ? 10 : 9;
     constexpr int kChannels = kRgba ? 4 : 3;
-    __shared__ StagedGaussian s_g[kBlock];
-    __shared__ int s_id[kBlock];
+    __shared__ StagedGaussian s_g[kBwdStage];
+    __shared__ int s_id[kBwdStage];
     // one row per value; the odd row stride puts the (up to ten) lanes of one LDS atomic instruction,
     // which address the same gaussian in consecutive rows, into different banks
-    __shared__ float s_grad[kValues][kBlock + 1];
+    __shared__ float s_grad[kValues][kBwdStage + 1];
     __shared__ int s_wmax[4];
     __shared__ unsigned long long s_mask[4][4];   // [patch][64-gaussian chunk]
 #ifdef D3GS_TIMING_ONLY_LDS_PAD
@@ -568,14 +574,15 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
     if (lane == 0) s_wmax[wave] = wave_todo;
     __syncthreads();
     const int block_todo = max(max(s_wmax[0], s_wmax[1]), max(s_wmax[2], s_wmax[3]));
-    const int rounds = (block_todo + kBlock - 1) / kBlock;
+    const int rounds = (block_todo + kBwdStage - 1) / kBwdStage;
 
     float T = 1.0f;
     for (int round = 0; round < rounds; ++round) {
         __syncthreads();  // previous round's flush has read s_grad / s_id
-        const int src = r0 + round * kBlock + tid;
+        const int src = r0 + round * kBwdStage + tid;
         uint32_t bits = 0;
-        if (src < r1 && round * kBlock + tid < block_todo) {    // entries behind the tile's last contributor: not staged
+        // entries behind the tile's last contributor are not staged
+        if (tid < kBwdStage && src < r1 && round * kBwdStage + tid < block_todo) {
             const int g = idx_sorted[src];
             if ((unsigned)g < (unsigned)items) {
                 s_id[tid] = g;
@@ -589,10 +596,12 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             }
         }
         publish_masks(bits, wave, lane, s_mask);
+        if (tid < kBwdStage) {
 #pragma unroll
-        for (int k = 0; k < kValues; ++k) s_grad[k][tid] = 0.0f;
+            for (int k = 0; k < kValues; ++k) s_grad[k][tid] = 0.0f;
+        }
         __syncthreads();
-        const int cnt = min(kBlock, wave_todo - round * kBlock);
+        const int cnt = min(kBwdStage, wave_todo - round * kBwdStage);
         for (int chunk = 0; chunk < 4 && chunk * 64 < cnt; ++chunk) {
           unsigned long long m = uniform_u64(s_mask[wave][chunk]);
           if (cnt - chunk * 64 < 64) m &= (1ull << (cnt - chunk * 64)) - 1ull;
@@ -609,11 +618,11 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
             // Per-lane conditions as 64-bit lane masks (one compare instruction each, combined with scalar
             // instructions; ordered compares, a NaN fails them as it fails the C operators they stand for).
 #ifdef D3GS_TIMING_ONLY_POWER_ONLY
-            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBlock + j, contributor, kIcmpSlt) &
+            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBwdStage + j, contributor, kIcmpSlt) &
                                               __builtin_amdgcn_fcmpf(power, 1.0e30f, kFcmpOge) &
                                               __builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOle);
 #else
-            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBlock + j, contributor, kIcmpSlt) &
+            const unsigned long long cand_m = __builtin_amdgcn_sicmp(round * kBwdStage + j, contributor, kIcmpSlt) &
                                               __builtin_amdgcn_fcmpf(power, sg.thr, kFcmpOge) &
                                               __builtin_amdgcn_fcmpf(power, 0.0f, kFcmpOle);
 #endif
@@ -685,7 +694,7 @@ __global__ __launch_bounds__(kBlock) void blend_bwd_kernel(
 #ifdef D3GS_TIMING_ONLY_NO_FLUSH
         continue;
 #endif
-        const int flush_cnt = min(kBlock, block_todo - round * kBlock);
+        const int flush_cnt = min(kBwdStage, block_todo - round * kBwdStage);
         if (tid < flush_cnt) {  // moments -> (duv, dconic) of gaussian tid, with a = -2 ha, b = -nb, c = -2 hc
             const StagedGaussian sg = s_g[tid];
             const float S1 = s_grad[0][tid], S2 = s_grad[1][tid];
