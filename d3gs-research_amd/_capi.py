@@ -42,7 +42,7 @@ class Params(C.Structure):
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
         ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
-        ("batch_size", C.c_int32), ("reserved0", C.c_int32), ("batch_cameras", C.c_void_p),
+        ("batch_size", C.c_int32), ("compact_items", C.c_int32), ("batch_cameras", C.c_void_p),
         ("atomic_add_count", C.c_void_p),
     ]
 
@@ -85,7 +85,7 @@ _SIGNATURES = {
     "d3gs_preprocess_fwd_sparse": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [C.POINTER(Instances), _VP]),
     "d3gs_sh_colors_sparse": (C.c_int, [C.POINTER(Params), _VP, _VP, C.c_int32] + [_VP] * 6 + [C.POINTER(Instances), _VP]),
     "d3gs_preprocess_bwd_sparse": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [C.c_int32, C.c_int32] + [_VP] * 6 +
-                                   [C.POINTER(Instances), _VP]),
+                                   [C.POINTER(Instances), _VP, _VP]),
     "d3gs_unique_ids_workspace_bytes": (C.c_int, [C.c_int32, C.c_int32, C.POINTER(C.c_size_t)]),
     "d3gs_unique_ids": (C.c_int, [_VP, C.c_int32, C.c_int32, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, _VP, _VP]),
     "d3gs_merge_rows": (C.c_int, [_VP, C.c_int32, C.c_int32, _VP, _VP, C.c_int32, _VP, _VP]),

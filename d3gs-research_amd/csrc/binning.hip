@@ -341,7 +341,10 @@ __global__ __launch_bounds__(kBlock) void make_keys_kernel(const d3gs_params P, 
         walk = tile_walk_setup(P, g);
         // camera b of a bundle owns the tile rows from b * tiles_y on (render.py:787, 809); the per-tile test works
         // in candidate-rect coordinates, so moving the rect's origin leaves the single camera's decisions as they are
-        const int shift = P.batch_size > 1 ? (i / P.n) * P.tiles_y : 0;
+        // (with a kept-tile record the shifted origin is in the record: sparse mode's compact rows of a bundle do
+        // not say which camera they belong to otherwise)
+        const int shift = P.batch_size <= 1 ? 0 : tile_masks ? (int)((meta >> 16) & 0xFFFFu) - walk.bminy
+                                                             : (i / P.n) * P.tiles_y;
         walk.bminy += shift;
     }
     wave_tile_emit<Key>(P.filter_algo, walk_again, walk, P.tiles_x, dbits, i, off, end, keys, vals);
@@ -685,6 +688,10 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
     if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
         !gaussian_idx) {
         set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p->compact_items > 0 && p->batch_size > 1 && !tile_masks) {
+        set_error("d3gs_make_keys: the compact rows of a bundle (compact_items) need tile_masks to name their camera");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     if ((uintptr_t)tile_masks & 15u) {     // the two words of a gaussian are read as one 16-byte load

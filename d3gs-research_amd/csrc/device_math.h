@@ -588,7 +588,10 @@ __device__ constexpr float kShC3[7] = {-0.5900435899266435f, 2.890611442640554f,
 
 // Camera bundles: a call with batch_size = B > 1 works on B * n render items, item i = b * n + g.
 __host__ __device__ __forceinline__ int batch_count(const d3gs_params& P) { return P.batch_size > 1 ? P.batch_size : 1; }
-__host__ __device__ __forceinline__ int item_count(const d3gs_params& P) { return P.n * batch_count(P); }
+// render items: gaussians x cameras of a bundle, or sparse mode's compact rows of one
+__host__ __device__ __forceinline__ int item_count(const d3gs_params& P) {
+    return P.compact_items > 0 ? P.compact_items : P.n * batch_count(P);
+}
 // Camera b of the bundle into the per-camera fields (what make_params fills for a single camera); tan_fov is
 // 0.5 * resolution / focal in float32, as the host computes it (render.py:358).
 __device__ __forceinline__ void apply_batch_camera(d3gs_params& P, int b) {

@@ -748,13 +748,14 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
     const float* __restrict__ grad_records, const uint8_t* __restrict__ touched, const int sh_mask_compat,
     const int outputs_are_zero, const int rows_per_pass, const int32_t* __restrict__ origin,
-    float* __restrict__ dxyz, float* __restrict__ dquat, float* __restrict__ dscale, float* dopacity_out,
-    float* __restrict__ dsh, float* __restrict__ dsh_base) {
+    const int32_t* __restrict__ row_batch_ids, float* __restrict__ dxyz, float* __restrict__ dquat,
+    float* __restrict__ dscale, float* dopacity_out, float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
     // one camera per launch: with a bundle, camera batch_index from the table (every per-item array comes in
-    // offset to that camera's rows by the host side of the call)
+    // offset to that camera's rows by the host side of the call); sparse mode's compact rows of a bundle name
+    // their camera row by row (row_batch_ids) instead
     d3gs_params P = P_in;
-    if (P_in.batch_size > 1) apply_batch_camera(P, batch_index);
+    if (P_in.batch_size > 1 && !row_batch_ids) apply_batch_camera(P, batch_index);
     extern __shared__ float s_rows[];                    // rows_per_pass rows of `stride` floats
     __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
     __shared__ unsigned char s_active[kSpan];
@@ -849,7 +850,11 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         __syncthreads();
         if (tid < cnt) {
             d3gs_params Pg = P;
-            if constexpr (kInstances) apply_instance(Pg, inst, origin ? origin[g] : g);      // ids are per model row
+            if constexpr (kInstances) {
+                const int b = (row_batch_ids && P_in.batch_size > 1) ? row_batch_ids[g] : 0;
+                if (row_batch_ids && P_in.batch_size > 1) apply_batch_camera(Pg, b);
+                apply_instance(Pg, inst, origin ? origin[g] : g, b);      // ids are per model row
+            }
             preprocess_bwd_one(Pg, g, in, sh_mask_compat, accumulate != 0, dxyz, dquat, dscale, dopacity_out,
                                s_rows + tid * stride, dsh_base);
         }
@@ -1077,7 +1082,8 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
                                const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0, const float* grad_records,
                                const uint8_t* touched, int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
                                float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
-                               float* dcolor_sh_base, const d3gs_instances* instances, d3gs_stream_t stream);
+                               float* dcolor_sh_base, const d3gs_instances* instances, const int32_t* row_batch_ids,
+                               d3gs_stream_t stream);
 
 extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids, const float* xyz,
                                           const float* quaternion_xyzw, const float* scale, const float* opacity,
@@ -1086,15 +1092,19 @@ extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* s
                                           int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
                                           float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
                                           float* dcolor_sh_base, const d3gs_instances* instances,
-                                          d3gs_stream_t stream) {
+                                          const int32_t* sparse_batch_ids, d3gs_stream_t stream) {
     if (!sparse_gaussian_ids && p && p->n > 0) {
         set_error("d3gs_preprocess_bwd_sparse: sparse_gaussian_ids is NULL");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
+    if (p && p->batch_size > 1 && !sparse_batch_ids) {
+        set_error("d3gs_preprocess_bwd_sparse: the compact rows of a bundle need sparse_batch_ids");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     return preprocess_bwd_impl("d3gs_preprocess_bwd_sparse", p, 0, 0, sparse_gaussian_ids, xyz, quaternion_xyzw, scale,
                                opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
                                outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
-                               instances, stream);
+                               instances, sparse_batch_ids, stream);
 }
 
 extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,
@@ -1108,7 +1118,7 @@ extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_in
     return preprocess_bwd_impl("d3gs_preprocess_bwd", p, batch_index, accumulate, nullptr, xyz, quaternion_xyzw, scale,
                                opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
                                outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
-                               instances, stream);
+                               instances, nullptr, stream);
 }
 
 // origin (sparse mode): p->n compact items, item i being row origin[i] of the model arrays; gradients are written per
@@ -1120,7 +1130,7 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
                                const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
                                int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
                                float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
-                               const d3gs_instances* instances, d3gs_stream_t stream) {
+                               const d3gs_instances* instances, const int32_t* row_batch_ids, d3gs_stream_t stream) {
     int rc = check_params(p, who);
     if (rc) return rc;
     if (batch_index < 0 || batch_index >= batch_count(*p)) {
@@ -1148,12 +1158,14 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
                        (int)batch_index, (int)accumulate, inst, xyz,                                                   \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
                        touched,                                                                                        \
-                       (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, origin, dxyz, dquaternion_xyzw,      \
+                       (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, origin, row_batch_ids, dxyz,         \
+                       dquaternion_xyzw,                                                                               \
                        dscale,                                                                                         \
                        dopacity_out,                                                                                   \
                        dcolor_sh, dcolor_sh_base)
-    if (wide) { if (inst.ids) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }
-    else      { if (inst.ids) D3GS_LAUNCH_K9(1, true); else D3GS_LAUNCH_K9(1, false); }
+    const bool per_row = inst.ids || (row_batch_ids && p->batch_size > 1);      // the instantiation that forms a camera per row
+    if (wide) { if (per_row) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }
+    else      { if (per_row) D3GS_LAUNCH_K9(1, true); else D3GS_LAUNCH_K9(1, false); }
 #undef D3GS_LAUNCH_K9
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }

@@ -117,6 +117,8 @@ class GaussianSplatOpContext:
     # sparse mode (render.py:234-238, 478-500): every per-gaussian array above has one row per ACCEPTED gaussian;
     # the gaussian of each row (int32 [V], ascending)
     sparse_gaussian_ids: torch.Tensor | None = None
+    # ... and, for a bundle rendered in one pass, the camera of each row (int32 [V])
+    sparse_batch_ids: torch.Tensor | None = None
 
 
 @dataclasses.dataclass
@@ -628,8 +630,14 @@ class GaussianSplatOp:
             if num_valid < 0:
                 raise RuntimeError("d3gs_scan_gathered: a workgroup's bounded wait on an earlier chunk ran out")
             v.n = num_valid
+            # what the kernels behind the preprocess see: V compact rows; a bundle keeps its camera count (tile ids
+            # and images carry the camera) and says that its rows are compact
             v.Pd = _capi.Params.from_buffer_copy(P)
-            v.Pd.n, v.Pd.batch_size, v.Pd.batch_cameras = num_valid, 0, None
+            v.Pd.n = num_valid
+            if batch > 1:
+                v.Pd.compact_items = num_valid
+            else:
+                v.Pd.batch_size, v.Pd.batch_cameras = 0, None
             v.sparse_gaussian_ids = torch.empty(num_valid, dtype=i32, device=dev)
             v.sparse_batch_ids = torch.empty(num_valid, dtype=i32, device=dev)
         return v
@@ -964,7 +972,8 @@ class GaussianSplatOp:
             tile_order=tile_order, grad_records=v.grad_records, grad_pool=v.grad_pool, grad_clear=v.grad_clear,
             grad_touched=v.grad_touched,
             kernel_color=v.out_color if v.no_rgb else None, instance_cameras=v.inst_cams, instance_ids=v.inst_ids,
-            batch_size=v.batch, batch_cameras=v.batch_cams, sparse_gaussian_ids=v.sparse_gaussian_ids)
+            batch_size=v.batch, batch_cameras=v.batch_cams, sparse_gaussian_ids=v.sparse_gaussian_ids,
+            sparse_batch_ids=v.sparse_batch_ids if (v.sparse and v.batch > 1) else None)
         # The view's kernel parameters, for a backward pass over the same model and cameras.  The model and the
         # cameras are remembered weakly and by what the parameters depend on: backward() rebuilds the parameters
         # when it is handed other objects, or the same ones changed in place where that can be seen.
@@ -980,11 +989,11 @@ class GaussianSplatOp:
     def _bundle_in_one_pass(self, batch, cameras) -> bool:
         """A bundle of B cameras goes through the kernels in ONE pass over B * N render items, as the reference's
         does (render.py:314-326, 787, 809, 1515-1522), unless it uses an option whose host code here is written
-        per camera (sparse mode, the fused single-stream preprocess), or the 32-bit sort when the bundle's tiles
+        per camera (the fused single-stream preprocess), or the 32-bit sort when the bundle's tiles
         outgrow its 14 tile bits (the reference asserts there, render.py:227-228).  Those bundles are rendered camera
         by camera (_forward_bundle)."""
         c = self._cfg
-        if not (self.bundle_in_one_pass and batch > 1 and self.overlap_sh_colors and not c.sparse_mode):
+        if not (self.bundle_in_one_pass and batch > 1 and (self.overlap_sh_colors or c.sparse_mode)):
             return False
         if c.enable_32bit_sort:
             width, height = cameras.image_shape_wh
@@ -1163,7 +1172,7 @@ class GaussianSplatOp:
             assert _cameras is not None, "camera needed to rebuild kernel parameters"
             P = self.make_params(model, _cameras, training)
         s = self._stream()
-        n, dev = P.n * ctx.batch_size, ctx.uvs.device        # render items
+        n, dev = int(ctx.radii.numel()), ctx.uvs.device      # render items (sparse mode: the accepted ones)
         color = ctx.kernel_color if ctx.kernel_color is not None else out.color
         if grad is None:
             clear, ctx.grad_clear = ctx.grad_clear, None
@@ -1251,10 +1260,12 @@ class GaussianSplatOp:
             P = self.make_params(model, cameras, True, ctx.batch_cameras)
         s = self._stream()
         sparse_ids = ctx.sparse_gaussian_ids
+        B = ctx.batch_size
         if sparse_ids is not None:      # the kernels see a scene of the V accepted gaussians
             P.n = int(sparse_ids.numel())
+            if B > 1:                   # ... of a bundle: compact rows, each with the camera sparse_batch_ids names
+                P.compact_items = P.n
         n, dev = P.n, model.xyz.device
-        B = ctx.batch_size
         with self._stage("blend_bwd"):
             g = self.rasterize_forward_backward(model, ctx, out, grad, training=True,
                                                 render_depth=self._cfg.render_depth, _params=P)
@@ -1286,7 +1297,8 @@ class GaussianSplatOp:
                     _capi.ptr(ctx.cov2d_vecs), _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records), _capi.ptr(g.touched),
                     int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz), _capi.ptr(dquat),
                     _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base),
-                    self._instances_arg(inst_ids, inst_cams), s), "d3gs_preprocess_bwd_sparse")
+                    self._instances_arg(inst_ids, inst_cams, B), _capi.ptr(ctx.sparse_batch_ids), s),
+                    "d3gs_preprocess_bwd_sparse")
             rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
             for b in range(B if sparse_ids is None else 0):
                 inst = self._instances_arg(inst_ids, inst_cams, B, b)      # the instance poses as camera b sees them
@@ -1301,6 +1313,17 @@ class GaussianSplatOp:
         grad_model = dataclasses.replace(model, xyz=dxyz, quaternion_xyzw=dquat, scale=dscale, opacity=dopacity,
                                          color_sh=dsh, color_sh_base=dsh_base)
         self.last_raster_grads = g
+        if sparse_ids is not None and B > 1:
+            # A sparse bundle in one pass: one row per accepted (camera, gaussian); the rows of a gaussian that
+            # several cameras accepted are merged (render.py:2864-2903) into one row per distinct gaussian, ascending
+            unique, run_rows, run_starts = self.unique_ids(sparse_ids, len(model))
+            self.last_sparse_unique_ids = unique
+            merged = {name: self.merge_rows(getattr(grad_model, name), run_rows, run_starts, int(unique.numel()))
+                      for name in ("xyz", "quaternion_xyzw", "scale", "opacity", "color_sh", "color_sh_base")
+                      if getattr(grad_model, name) is not None}
+            grad_model = dataclasses.replace(model, **merged)
+            # duv keeps one row per accepted (camera, gaussian), cameras one after the other, as out.sparse_gaussian_ids
+            return grad_model, (g.duv.reshape(1, n, 2) if return_uv_grad else None), dcustom
         if return_uv_grad:
             return grad_model, g.duv.reshape(B, n, 2), dcustom
         return grad_model, None, dcustom

@@ -107,7 +107,11 @@ typedef struct d3gs_params {
      * (render.py:316-323 loads the same from its [B,4,3] and [B,4] tensors).  batch_size 0 or 1: one camera, the
      * fields above. */
     int32_t batch_size;
-    int32_t reserved0;
+    /* Sparse mode over a bundle (no counterpart field in the reference, whose kernels take the sparse ids as extra
+     * arguments): when > 0, the per-item arrays of the entry points BEHIND K1 hold this many rows -- the accepted
+     * (camera, gaussian) items, in ascending item order -- instead of batch_size * n; the camera of a row is named by
+     * the kept-tile record (d3gs_make_keys then needs tile_masks) and by sparse_batch_ids (K9).  0: batch_size * n. */
+    int32_t compact_items;
     const float* batch_cameras;
     /* measure_atomic_add_count (config_def.py:134; render.py:1451-1453, 2145-2148, 2310-2311): when not NULL, the
      * blend backward kernels add to this device counter the number of global atomic requests they issue (one
@@ -437,7 +441,10 @@ int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_
  *   5. d3gs_preprocess_bwd_sparse: K9 over the V items; gradients are written per item, [V] rows (the rows of the
  *      model arrays are found through sparse_gaussian_ids), as the reference's sparse gradient (render.py:2918).
  * The render is the dense one bit for bit: slots ascend with the item index, so ties in the sort fall the same way.
- * `instances` (may be NULL) as in the dense entry points: instance ids are per row of the model arrays. */
+ * `instances` (may be NULL) as in the dense entry points: instance ids are per row of the model arrays.
+ * A bundle of B cameras in one pass: steps 1-3 run over the B * n items (p->batch_size = B); behind them the
+ * params carry n = V, batch_size = B (the tile ids and images keep the camera) and compact_items = V;
+ * d3gs_preprocess_bwd_sparse then takes sparse_batch_ids (NULL for one camera) to give each row its camera. */
 int d3gs_preprocess_fwd_sparse(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                                const float* opacity, const uint8_t* invalid_mask, int32_t* valid_flags,
                                const int32_t* slot_scan, int32_t* sparse_gaussian_ids, int32_t* sparse_batch_ids,
@@ -454,7 +461,7 @@ int d3gs_preprocess_bwd_sparse(const d3gs_params* p /* n = V */, const int32_t* 
                                const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
                                int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz, float* dquaternion_xyzw,
                                float* dscale, float* dopacity_out, float* dcolor_sh, float* dcolor_sh_base,
-                               const d3gs_instances* instances, d3gs_stream_t stream);
+                               const d3gs_instances* instances, const int32_t* sparse_batch_ids, d3gs_stream_t stream);
 
 /* K10 -- replaces the hash-table deduplication of a sparse bundle's gradient rows (render.py:2864-2903: insert the
  * accepted gaussian ids of all cameras, collect the distinct ones, query each row's slot, add the rows with atomics).

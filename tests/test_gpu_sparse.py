@@ -93,7 +93,10 @@ def test_sparse_inference_and_empty_view():
     assert float(out_e.T.min()) == 1.0 and float(out_e.color.abs().max()) == 0.0
 
 
-def test_sparse_bundle_merges_the_cameras_rows():
+@pytest.mark.parametrize("one_pass", [True, False])
+def test_sparse_bundle_merges_the_cameras_rows(one_pass):
+    """A sparse bundle, in one pass over the B * N items (compact rows behind K1, K9 with a camera per row) and
+    camera by camera: the dense bundle's images, its accepted items' rows, and gradients merged per gaussian."""
     import torch
     from d3gs_research_amd.render import CameraBundle, GaussianSplatGradients, GaussianSplatOp
     from test_gpu_camera_bundle import _cameras
@@ -106,7 +109,12 @@ def test_sparse_bundle_merges_the_cameras_rows():
     res = {}
     for sparse in (False, True):
         op = GaussianSplatOp(op_config(scene, 4, sparse_mode=sparse))
-        out, ctx = op.forward(model, bundle, training=True)
+        op.bundle_in_one_pass = one_pass or not sparse
+        for _ in range(2):      # the second view takes the one-call binning
+            out, ctx = op.forward(model, bundle, training=True)
+        if sparse:
+            from d3gs_research_amd.render import GaussianSplatOpBatchContext
+            assert isinstance(ctx, GaussianSplatOpBatchContext) != one_pass
         if not res:
             drgb = torch.from_numpy(rng.standard_normal(out.color.shape).astype(np.float32)).cuda()
             dT = torch.from_numpy(rng.standard_normal(out.T.shape).astype(np.float32)).cuda()
@@ -166,7 +174,8 @@ def test_unique_ids_and_merge_rows_c_abi(count, id_limit):
         assert np.array_equal(merged.view(np.uint32), ref.view(np.uint32))
 
 
-def test_sparse_bundle_with_a_camera_that_renders_no_pair():
+@pytest.mark.parametrize("one_pass", [True, False])
+def test_sparse_bundle_with_a_camera_that_renders_no_pair(one_pass):
     """A camera can accept gaussians (their 3-sigma rect meets the image) and still end without a single (tile,
     gaussian) pair (OBB keeps no tile of any of them): it has rows in out.radii / out.sparse_gaussian_ids but no
     context.  The rows of the cameras behind it must still line up, its own duv rows are zero."""
@@ -197,6 +206,7 @@ def test_sparse_bundle_with_a_camera_that_renders_no_pair():
     res = {}
     for sparse in (False, True):
         op = GaussianSplatOp(op_config(scene, 3, sparse_mode=sparse))
+        op.bundle_in_one_pass = one_pass or not sparse
         out, ctx = op.forward(model, bundle, training=True, mask=mask_t)
         if not res:
             drgb = torch.from_numpy(rng.standard_normal(out.color.shape).astype(np.float32)).cuda()
@@ -208,15 +218,21 @@ def test_sparse_bundle_with_a_camera_that_renders_no_pair():
     B = 3
     items = torch.nonzero(out_d.radii > 0).squeeze(1)
     first = items[items < scene.n]
-    assert first.numel() == 3 and ctx_s.per_camera[0] is None and ctx_s.rows_per_camera[0] == 3      # accepted, no pair
+    assert first.numel() == 3                                                  # accepted, and no pair:
+    if one_pass:
+        assert int((ctx_s.workload_ranges[:ctx_s.workload_ranges.shape[0] // B, 1] - ctx_s.workload_ranges[:ctx_s.workload_ranges.shape[0] // B, 0]).sum()) == 0
+    else:
+        assert ctx_s.per_camera[0] is None and ctx_s.rows_per_camera[0] == 3
     assert float(out_s.T[0].min()) == 1.0
     assert torch.equal(out_s.sparse_batch_ids.long() * scene.n + out_s.sparse_gaussian_ids.long(), items)
     assert torch.equal(out_s.color, out_d.color)
     assert tuple(duv_s.shape) == (1, items.numel(), 2) and float(duv_s[0, :3].abs().max()) == 0.0
+    B = 3
     top = float(duv_d.abs().max())
     assert float((duv_s[0] - duv_d.reshape(B * scene.n, 2)[items]).abs().max()) <= 1e-4 * top
     unique = op_s.last_sparse_unique_ids.long()
-    seen = torch.unique(out_s.sparse_gaussian_ids[3:].long())          # the first camera contributes no gradient row
+    # camera by camera the first camera contributes no gradient row; in one pass its three rows are there, and zero
+    seen = torch.unique(out_s.sparse_gaussian_ids.long() if one_pass else out_s.sparse_gaussian_ids[3:].long())
     assert torch.equal(unique, seen)
     for name in ("xyz", "scale", "opacity", "color_sh"):
         a, b = getattr(gm_s, name).double(), getattr(gm_d, name).double()
