@@ -743,28 +743,38 @@ __device__ __forceinline__ bool record_is_zero(const float4 ra, const float4 rb,
 
 template <int kPer, bool kInstances>
 __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
-    const d3gs_params P_in, const int batch_index, const int accumulate, const InstanceView inst, const float* __restrict__ xyz, const float* __restrict__ quat,
+    const d3gs_params P_in, const int batch_index, const int batch_last, const int accumulate_in, const InstanceView inst,
+    const float* __restrict__ xyz, const float* __restrict__ quat,
     const float* __restrict__ scale, const float* __restrict__ opacity, const float* __restrict__ sh,
-    const int32_t* __restrict__ radii, const float* __restrict__ cov2d, const uint8_t* __restrict__ ne0,
-    const float* __restrict__ grad_records, const uint8_t* __restrict__ touched, const int sh_mask_compat,
+    const int32_t* __restrict__ radii_in, const float* __restrict__ cov2d_in, const uint8_t* __restrict__ ne0_in,
+    const float* __restrict__ grad_records, const uint8_t* __restrict__ touched_in, const int sh_mask_compat,
     const int outputs_are_zero, const int rows_per_pass, const int32_t* __restrict__ origin,
     const int32_t* __restrict__ row_batch_ids, float* __restrict__ dxyz, float* __restrict__ dquat,
     float* __restrict__ dscale, float* dopacity_out, float* __restrict__ dsh, float* __restrict__ dsh_base) {
     constexpr int kSpan = kBwdBlock * kPer, kWaves = kBwdBlock / 64;
-    // one camera per launch: with a bundle, camera batch_index from the table (every per-item array comes in
-    // offset to that camera's rows by the host side of the call); sparse mode's compact rows of a bundle name
-    // their camera row by row (row_batch_ids) instead
-    d3gs_params P = P_in;
-    if (P_in.batch_size > 1 && !row_batch_ids) apply_batch_camera(P, batch_index);
+    // Cameras batch_index .. batch_last of a bundle, one after the other (render.py:2972-2989, 3180-3219 loop over
+    // the batch inside the kernel too): the per-item arrays come in pointing at camera batch_index's rows, camera c's
+    // follow (c - batch_index) * n rows further on, its parameters come from the table, and from the second camera
+    // on the gradients are added to what the workgroup itself stored for the cameras before.  Sparse mode's compact
+    // rows of a bundle name their camera row by row (row_batch_ids) instead and go through once.
     extern __shared__ float s_rows[];                    // rows_per_pass rows of `stride` floats
     __shared__ unsigned short s_list[kSpan];             // gaussians (offsets from `first`) with work
     __shared__ unsigned char s_active[kSpan];
     __shared__ int s_count[kPer * kWaves];
-    const int rowlen = P.sh_stride * 3, stride = rowlen | 1;
+    const int rowlen = P_in.sh_stride * 3, stride = rowlen | 1;
     const int first = blockIdx.x * kSpan;
-    const int nrows = min(kSpan, P.n - first);
+    const int nrows = min(kSpan, P_in.n - first);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const float4* rec4 = reinterpret_cast<const float4*>(grad_records);
+    for (int cam = batch_index; cam <= batch_last; ++cam) {
+    d3gs_params P = P_in;
+    if (P_in.batch_size > 1 && !row_batch_ids) apply_batch_camera(P, cam);
+    const size_t item0 = (size_t)(cam - batch_index) * (size_t)P_in.n;     // this camera's rows of the per-item arrays
+    const int32_t* radii = radii_in + item0;
+    const uint8_t* touched = touched_in ? touched_in + item0 : nullptr;
+    const float* cov2d = cov2d_in + 3 * item0;
+    const uint8_t* ne0 = ne0_in + item0;
+    const float4* rec4 = reinterpret_cast<const float4*>(grad_records) + 4 * item0;
+    const int accumulate = accumulate_in || cam > batch_index;
     bool active[kPer];
     unsigned long long mates[kPer];
     // all radii first, then all records: two round trips to memory instead of two per gaussian.  With the blend
@@ -851,7 +861,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         if (tid < cnt) {
             d3gs_params Pg = P;
             if constexpr (kInstances) {
-                const int b = (row_batch_ids && P_in.batch_size > 1) ? row_batch_ids[g] : 0;
+                // (the instance table starts at camera batch_index's poses)
+                const int b = (row_batch_ids && P_in.batch_size > 1) ? row_batch_ids[g] : cam - batch_index;
                 if (row_batch_ids && P_in.batch_size > 1) apply_batch_camera(Pg, b);
                 apply_instance(Pg, inst, origin ? origin[g] : g, b);      // ids are per model row
             }
@@ -861,6 +872,8 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         __syncthreads();
         bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride, accumulate != 0);
         __syncthreads();
+    }
+    __syncthreads();      // the lists are rebuilt for the next camera
     }
 }
 
@@ -1059,6 +1072,16 @@ extern "C" int d3gs_sh_colors(const d3gs_params* p, const float* xyz, const floa
     return D3GS_OK;
 }
 
+static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t batch_last,
+                               int32_t accumulate,
+                               const int32_t* origin, const float* xyz, const float* quaternion_xyzw,
+                               const float* scale, const float* opacity, const float* color_sh, const int32_t* radii,
+                               const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0, const float* grad_records,
+                               const uint8_t* touched, int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
+                               float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
+                               float* dcolor_sh_base, const d3gs_instances* instances, const int32_t* row_batch_ids,
+                               d3gs_stream_t stream);
+
 extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw,
                                    const float* scale, const float* opacity, const float* color_sh,
                                    const int32_t* radii, const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0,
@@ -1067,23 +1090,12 @@ extern "C" int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const
                                    float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
                                    float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                                    d3gs_stream_t stream) {
-    if (p && p->batch_size > 1) {
-        set_error("d3gs_preprocess_bwd: a camera bundle goes through d3gs_preprocess_bwd_camera, one call per camera");
-        return D3GS_ERR_INVALID_ARGUMENT;
-    }
-    return d3gs_preprocess_bwd_camera(p, 0, 0, xyz, quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs,
-                                      sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat, outputs_are_zero, dxyz,
-                                      dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base, instances, stream);
+    // a bundle: every camera in this one launch, the per-item arrays holding batch_size * n rows
+    return preprocess_bwd_impl("d3gs_preprocess_bwd", p, 0, p ? batch_count(*p) - 1 : 0, 0, nullptr, xyz, quaternion_xyzw,
+                               scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched,
+                               sh_mask_compat, outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh,
+                               dcolor_sh_base, instances, nullptr, stream);
 }
-
-static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t accumulate,
-                               const int32_t* origin, const float* xyz, const float* quaternion_xyzw,
-                               const float* scale, const float* opacity, const float* color_sh, const int32_t* radii,
-                               const float* cov2d_vecs, const uint8_t* sh_to_rgb_ne_0, const float* grad_records,
-                               const uint8_t* touched, int32_t sh_mask_compat, int32_t outputs_are_zero, float* dxyz,
-                               float* dquaternion_xyzw, float* dscale, float* dopacity_out, float* dcolor_sh,
-                               float* dcolor_sh_base, const d3gs_instances* instances, const int32_t* row_batch_ids,
-                               d3gs_stream_t stream);
 
 extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* sparse_gaussian_ids, const float* xyz,
                                           const float* quaternion_xyzw, const float* scale, const float* opacity,
@@ -1101,7 +1113,7 @@ extern "C" int d3gs_preprocess_bwd_sparse(const d3gs_params* p, const int32_t* s
         set_error("d3gs_preprocess_bwd_sparse: the compact rows of a bundle need sparse_batch_ids");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
-    return preprocess_bwd_impl("d3gs_preprocess_bwd_sparse", p, 0, 0, sparse_gaussian_ids, xyz, quaternion_xyzw, scale,
+    return preprocess_bwd_impl("d3gs_preprocess_bwd_sparse", p, 0, 0, 0, sparse_gaussian_ids, xyz, quaternion_xyzw, scale,
                                opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
                                outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
                                instances, sparse_batch_ids, stream);
@@ -1115,7 +1127,7 @@ extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_in
                                           float* dxyz, float* dquaternion_xyzw, float* dscale, float* dopacity_out,
                                           float* dcolor_sh, float* dcolor_sh_base, const d3gs_instances* instances,
                                           d3gs_stream_t stream) {
-    return preprocess_bwd_impl("d3gs_preprocess_bwd", p, batch_index, accumulate, nullptr, xyz, quaternion_xyzw, scale,
+    return preprocess_bwd_impl("d3gs_preprocess_bwd_camera", p, batch_index, batch_index, accumulate, nullptr, xyz, quaternion_xyzw, scale,
                                opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched, sh_mask_compat,
                                outputs_are_zero, dxyz, dquaternion_xyzw, dscale, dopacity_out, dcolor_sh, dcolor_sh_base,
                                instances, nullptr, stream);
@@ -1123,8 +1135,8 @@ extern "C" int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_in
 
 // origin (sparse mode): p->n compact items, item i being row origin[i] of the model arrays; gradients are written per
 // item.
-static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t accumulate,
-                               const int32_t* origin, const float* xyz,
+static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t batch_index, int32_t batch_last,
+                               int32_t accumulate, const int32_t* origin, const float* xyz,
                                const float* quaternion_xyzw, const float* scale, const float* opacity,
                                const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
                                const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
@@ -1133,8 +1145,8 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
                                const d3gs_instances* instances, const int32_t* row_batch_ids, d3gs_stream_t stream) {
     int rc = check_params(p, who);
     if (rc) return rc;
-    if (batch_index < 0 || batch_index >= batch_count(*p)) {
-        set_error("d3gs_preprocess_bwd_camera: batch_index %d outside the bundle of %d", batch_index, batch_count(*p));
+    if (batch_index < 0 || batch_index >= batch_count(*p) || batch_last < batch_index || batch_last >= batch_count(*p)) {
+        set_error("%s: cameras %d..%d outside the bundle of %d", who, batch_index, batch_last, batch_count(*p));
         return D3GS_ERR_INVALID_ARGUMENT;
     }
     if (p->n == 0) return D3GS_OK;
@@ -1155,7 +1167,7 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
     dim3 grid((p->n + kBwdBlock * per - 1) / (kBwdBlock * per)), block(kBwdBlock);
 #define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
     hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p,            \
-                       (int)batch_index, (int)accumulate, inst, xyz,                                                   \
+                       (int)batch_index, (int)batch_last, (int)accumulate, inst, xyz,                                                   \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
                        touched,                                                                                        \
                        (int)sh_mask_compat, (int)outputs_are_zero, rows_per_pass, origin, row_batch_ids, dxyz,         \

@@ -231,6 +231,8 @@ class GaussianSplatOp:
         self.clear_gradients_early = True
         # a CameraBundle of several cameras goes through the kernels in one pass (False: camera by camera)
         self.bundle_in_one_pass = True
+        # ... and its preprocess backward in one launch (False: one launch per camera, each adding to the last)
+        self.bundle_k9_in_one_launch = True
         # the one-call binning writes the pair count to its pinned host word with a store the host can see while
         # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
         # forward blend back by the few microseconds the stream takes to process the marker
@@ -1287,8 +1289,9 @@ class GaussianSplatOp:
             inst_ids, inst_cams = ctx.instance_ids, ctx.instance_cameras
             if inst_cams is None and instance2world_T is not None:
                 inst_ids, inst_cams = self.instance_table(model, cameras, instance2world_T)
-            # One launch per camera (the reference loops over the batch inside its kernel, render.py:2972-2989):
-            # camera b works on its own rows of the per-item arrays, the first call stores, the others add.
+            # The reference loops over the batch inside its kernel (render.py:2972-2989), and so does the library's;
+            # with bundle_k9_in_one_launch off, one launch per camera instead: camera b works on its own rows of the
+            # per-item arrays, the first call stores, the others add.
             if sparse_ids is not None:
                 # sparse gradient (render.py:2918, 3185-3213): row i belongs to gaussian sparse_gaussian_ids[i]
                 _capi.check(L.d3gs_preprocess_bwd_sparse(
@@ -1299,8 +1302,17 @@ class GaussianSplatOp:
                     _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base),
                     self._instances_arg(inst_ids, inst_cams, B), _capi.ptr(ctx.sparse_batch_ids), s),
                     "d3gs_preprocess_bwd_sparse")
+            if sparse_ids is None and (B == 1 or self.bundle_k9_in_one_launch):
+                # dense: one launch, which for a bundle works every gaussian off camera after camera
+                _capi.check(L.d3gs_preprocess_bwd(
+                    C.byref(P), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),
+                    _capi.ptr(model.scale), _capi.ptr(model.opacity), _capi.ptr(model.color_sh),
+                    _capi.ptr(ctx.radii), _capi.ptr(ctx.cov2d_vecs), _capi.ptr(ctx.sh_to_rgb_ne_0), _capi.ptr(g.records),
+                    _capi.ptr(g.touched), int(self._cfg.compat_ref_sh_mask_bitorder), int(prezeroed), _capi.ptr(dxyz),
+                    _capi.ptr(dquat), _capi.ptr(dscale), _capi.ptr(dopacity), _capi.ptr(dsh), _capi.ptr(dsh_base),
+                    self._instances_arg(inst_ids, inst_cams, B), s), "d3gs_preprocess_bwd")
             rows = lambda t, b: None if t is None else t[b * n:(b + 1) * n]
-            for b in range(B if sparse_ids is None else 0):
+            for b in range(B if (sparse_ids is None and B > 1 and not self.bundle_k9_in_one_launch) else 0):
                 inst = self._instances_arg(inst_ids, inst_cams, B, b)      # the instance poses as camera b sees them
                 _capi.check(L.d3gs_preprocess_bwd_camera(
                     C.byref(P), b, int(b > 0), _capi.ptr(model.xyz), _capi.ptr(model.quaternion_xyzw),

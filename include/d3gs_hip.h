@@ -402,7 +402,11 @@ int d3gs_blend_bwd_per_gaussian(const d3gs_params* p, const int32_t* workload_ra
  * may be NULL; no counterpart in the reference) is d3gs_blend_bwd's array of the
  * same name: gaussians it marks 0 are taken to have an all-zero record, which is
  * then not read.  The *_base pointers may be NULL.  sh_mask_compat != 0 reads the SH clamp mask with the
- * reference's reversed bit order (render.py:3344-3350). */
+ * reference's reversed bit order (render.py:3344-3350).
+ * A bundle (p->batch_size = B > 1) goes through in this one launch, as in the reference, whose kernel loops over
+ * the batch (render.py:2972-2989, 3180-3219): the per-item arrays (radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,
+ * touched) hold B * n rows, camera after camera, `instances` the B tables K1 was given, and each workgroup works
+ * its gaussians off camera by camera, adding every camera's gradient to what it stored for those before. */
 int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* quaternion_xyzw, const float* scale,
                         const float* opacity, const float* color_sh, const int32_t* radii, const float* cov2d_vecs,
                         const uint8_t* sh_to_rgb_ne_0, const float* grad_records, const uint8_t* touched,
@@ -414,7 +418,9 @@ int d3gs_preprocess_bwd(const d3gs_params* p, const float* xyz, const float* qua
  * p->batch_size = B > 1 the call works on camera batch_index, taken from p->batch_cameras, and every per-item
  * array (radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records, touched) points at that camera's n rows.  accumulate != 0
  * adds to the six gradient arrays instead of storing (gaussians without work are left alone): the gradient of a
- * bundle is B calls, the first storing (or adding to cleared arrays), the others accumulating.  With
+ * bundle is then B calls, the first storing (or adding to cleared arrays), the others accumulating (what
+ * d3gs_preprocess_bwd does for a bundle inside one launch; this entry serves callers that hold the cameras' arrays
+ * apart, or that add a camera to gradients they already have).  With
  * batch_size <= 1, batch_index 0 and accumulate 0 this is d3gs_preprocess_bwd.  `instances` is the table of this
  * camera alone ([num_instances][12], the batch_index-th of the B tables K1 was given). */
 int d3gs_preprocess_bwd_camera(const d3gs_params* p, int32_t batch_index, int32_t accumulate, const float* xyz,

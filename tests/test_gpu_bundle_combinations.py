@@ -43,6 +43,7 @@ def test_one_pass_equals_camera_by_camera(seed):
     for one_pass in (True, False):
         op = GaussianSplatOp(op_config(scene, 4, **over))
         op.bundle_in_one_pass = one_pass
+        op.bundle_k9_in_one_launch = bool(seed % 2)      # the preprocess backward: one launch, or one per camera
         out, ctx = op.forward(model, bundle, training=not f["infer"], instance2world_T=T_dev, custom_features=feat,
                               mask=mask)
         gm = duv = dcf = None
