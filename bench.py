@@ -170,6 +170,9 @@ def main():
     ap.add_argument("--op-set", action="append", default=[], metavar="ATTR=0|1",
                     help="set a boolean switch of the operator for an A/B run, e.g. "
                          "overlap_sh_colors=0, poll_pair_count=0, fused_binning=0 (repeatable); the headline runs with the defaults")
+    ap.add_argument("--custom-features", type=int, default=0, metavar="F",
+                    help="carry F seeded custom feature channels per gaussian through every view, forward and backward "
+                         "(a different workload, for profiling the feature kernels: not the headline; no CPU baseline)")
     ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="only run a plain 256 MiB -> 256 MiB elementwise copy 5 times (reference reading for "
@@ -207,11 +210,19 @@ def main():
     model = scene_model(scene, "cuda:0")
     grads = GaussianSplatGradients(drgb=torch.from_numpy(scene.drgb).cuda(), dT=torch.from_numpy(scene.dT).cuda())
 
+    feat = None
+    if args.custom_features > 0:
+        gen = torch.Generator(device="cuda:0").manual_seed(5)
+        feat = torch.randn((scene.n, args.custom_features), device="cuda:0", generator=gen)
+        grads.dcustom_features = torch.randn((1, scene.height, scene.width, args.custom_features), device="cuda:0",
+                                             generator=gen)
+        args.no_cpu_baseline = True
+
     pair_counts = []
 
     def step(i=0):
         c = cams[i % len(cams)]
-        out, ctx = op.forward(model, c, training=True)
+        out, ctx = op.forward(model, c, training=True, custom_features=feat)
         pair_counts.append(op.last_num_rendered)
         if ctx is None:      # nothing of the scene in this view
             return out, None
@@ -236,7 +247,7 @@ def main():
     # view): the pair count changes from view to view, the pair buffers are sized from the previous view's count and
     # a view that outgrows them is binned again
     views8 = None
-    if args.views == 1:
+    if args.views == 1 and feat is None:
         cams8 = [cam] + orbit_cameras(scene, 7)
         counts8 = []
 
@@ -378,6 +389,7 @@ def main():
     line = {
         "metric": "fwd+bwd raster ms/view, 1M Gaussians @1080p, 1 MI355X" if args.config == 2
         else f"fwd+bwd raster ms/view, config {args.config}",
+        **({"note": f"with {args.custom_features} custom feature channels: not the headline workload"} if feat is not None else {}),
         "value": round(ms_per_step, 4), "unit": "ms/view", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
@@ -386,7 +398,8 @@ def main():
                    "rasterize_backward_algo": args.backward_algo, "pairs_M": int(M),
                    "pairs_per_gaussian": round(M / N, 3), "tiles": T_tiles, "tile_list_length": tile_lists,
                    "gaussians_with_gradient": active, "views": views_info,
-                   **({"op_set": args.op_set} if args.op_set else {})},
+                   **({"op_set": args.op_set} if args.op_set else {}),
+                   **({"custom_features": args.custom_features} if feat is not None else {})},
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
         "gpu_stage_sum_ms": round(gpu_sum, 4),
         "stages": stages,

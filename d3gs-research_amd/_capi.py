@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 31
+ABI_VERSION = 32
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
 BUCKET_SIZE = 64          # D3GS_BUCKET_SIZE
@@ -82,6 +82,8 @@ _SIGNATURES = {
     "d3gs_tile_ranges_u32": (C.c_int, [_VP, C.c_int64, _VP, _VP, C.c_int32, _VP, _VP]),
     "d3gs_blend_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [_VP, C.c_size_t] + [_VP]),
     "d3gs_blend_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 16 + [_VP]),
+    "d3gs_blend_features_fwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 5 + [C.c_int32, _VP, _VP, _VP]),
+    "d3gs_blend_features_bwd": (C.c_int, [C.POINTER(Params)] + [_VP] * 5 + [C.c_int32] + [_VP] * 7 + [_VP]),
     "d3gs_preprocess_fwd_sparse": (C.c_int, [C.POINTER(Params)] + [_VP] * 17 + [C.POINTER(Instances), _VP]),
     "d3gs_sh_colors_sparse": (C.c_int, [C.POINTER(Params), _VP, _VP, C.c_int32] + [_VP] * 6 + [C.POINTER(Instances), _VP]),
     "d3gs_preprocess_bwd_sparse": (C.c_int, [C.POINTER(Params)] + [_VP] * 11 + [C.c_int32, C.c_int32] + [_VP] * 6 +

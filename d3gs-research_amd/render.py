@@ -233,6 +233,9 @@ class GaussianSplatOp:
         self.bundle_in_one_pass = True
         # ... and its preprocess backward in one launch (False: one launch per camera, each adding to the last)
         self.bundle_k9_in_one_launch = True
+        # custom feature channels through the library's feature kernels (False: three at a time through the colour
+        # kernels, one forward and one backward blend per triple)
+        self.feature_kernels = True
         # the one-call binning writes the pair count to its pinned host word with a store the host can see while
         # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
         # forward blend back by the few microseconds the stream takes to process the marker
@@ -1123,10 +1126,18 @@ class GaussianSplatOp:
             yield k, min(3, F - k), tri
 
     def _blend_custom_features(self, P, ctx, out, feat):
+        """The feature image [B, H, W, F]: the library's feature kernels (up to 16 channels beside one evaluation of
+        alpha), or with ``feature_kernels`` off three channels at a time through the colour kernel."""
         L, s = self._lib, self._stream()
         Q = self._feature_params(P)
         B, H, W = out.T.shape        # a bundle in one pass: B images, feature rows of the B * N render items
         res = torch.empty((B, H, W, feat.shape[1]), dtype=torch.float32, device=feat.device)
+        if self.feature_kernels:
+            _capi.check(L.d3gs_blend_features_fwd(
+                C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(feat.detach()), int(feat.shape[1]), _capi.ptr(ctx.tile_order),
+                _capi.ptr(res), s), "d3gs_blend_features_fwd")
+            return res
         T2, nc2 = torch.empty_like(out.T), torch.empty_like(out.n_contrib)
         for k, w, tri in self._feature_triples(feat.detach()):
             img = torch.empty((B, H, W, 3), dtype=torch.float32, device=feat.device)
@@ -1145,6 +1156,14 @@ class GaussianSplatOp:
         feat = ctx.custom_features.detach()
         n, F = feat.shape
         B, H, W = out.T.shape
+        if self.feature_kernels:
+            dfeat = torch.zeros((n, F), dtype=torch.float32, device=feat.device)
+            _capi.check(L.d3gs_blend_features_bwd(
+                C.byref(Q), _capi.ptr(ctx.workload_ranges), _capi.ptr(ctx.gaussian_idx_sorted), _capi.ptr(ctx.uvs),
+                _capi.ptr(ctx.conic_opacity), _capi.ptr(feat), int(F), _capi.ptr(ctx.tile_order),
+                _capi.ptr(out.n_contrib), _capi.ptr(out.custom_features.detach().contiguous()), _capi.ptr(dfeat_img),
+                _capi.ptr(rec), _capi.ptr(dfeat), _capi.ptr(touched), s), "d3gs_blend_features_bwd")
+            return dfeat
         dfeat = torch.empty((n, F), dtype=torch.float32, device=feat.device)
         zero_dT = torch.zeros_like(out.T)
         for k, w, tri in self._feature_triples(feat):

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 31
+#define D3GS_ABI_VERSION 32
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -359,6 +359,29 @@ int d3gs_blend_bwd(const d3gs_params* p, const int32_t* workload_ranges, const i
                    const int32_t* tile_order, const float* final_T, const int32_t* n_contrib, const float* color,
                    const float* final_depth, const float* drgb, const float* dT, const float* ddepth,
                    float* grad_records, uint8_t* touched, d3gs_stream_t stream);
+
+/* Custom feature channels (render.py:241-246, 1536-1538, 1571-1573, 1718-1721, 1892-1895, 1920-1923, 1952-1955,
+ * 1969-1972, 2113-2117, 2268-2270; the reference compiles the channel count into its rasterize kernel): features
+ * [items][num_features] are blended like a colour over the lists of a finished forward pass.
+ *   d3gs_blend_features_fwd   feature_image [B][H][W][num_features] = sum_i T_i alpha_i f_i, the raw sums (no
+ *                             background, no clamp), with the weights of d3gs_blend_fwd pixel for pixel; up to 16
+ *                             channels per launch.
+ *   d3gs_blend_features_bwd   given n_contrib of the forward pass, the blended feature_image and its gradient
+ *                             dfeature_image: adds the channels' share of the geometry gradient to columns 0..5 of
+ *                             grad_records (D3GS_GRAD_DUV, _DCONIC, _DOPACITY: the records d3gs_blend_bwd adds the
+ *                             colour's share to, in either order), marks `touched` (may be NULL) like d3gs_blend_bwd,
+ *                             and adds dL/dfeatures to dfeatures [items][num_features] (zero-fill it first); up to
+ *                             14 channels per launch, their terms of dL/dalpha summed before the one division by
+ *                             1 - alpha (render.py:1952-1955).
+ * p: the fields the blend reads (sizes, tiles, alpha_eps, transmittance_eps, batch); num_features = 0 does nothing. */
+int d3gs_blend_features_fwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                            const float* uvs, const float* conic_opacity, const float* features, int32_t num_features,
+                            const int32_t* tile_order, float* feature_image, d3gs_stream_t stream);
+int d3gs_blend_features_bwd(const d3gs_params* p, const int32_t* workload_ranges, const int32_t* gaussian_idx_sorted,
+                            const float* uvs, const float* conic_opacity, const float* features, int32_t num_features,
+                            const int32_t* tile_order, const int32_t* n_contrib, const float* feature_image,
+                            const float* dfeature_image, float* grad_records, float* dfeatures, uint8_t* touched,
+                            d3gs_stream_t stream);
 
 /* The per-gaussian backward, config rasterize_backward_algo = PER_GAUSSIAN (config_def.py:72-74, 149-151;
  * render.py:940-962, 1577-1583, 1744-1759, 2319-2776): a second algorithm for K7's gradient in which lanes are

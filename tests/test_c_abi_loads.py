@@ -34,7 +34,7 @@ def test_params_struct_matches_header_layout():
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 31
+    assert L.d3gs_abi_version() == 32
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
     # depth-sort key width: float bits of z_far minus those of z_near, or the 18 depth-step bits
