@@ -66,6 +66,13 @@ def test_error_codes_without_compute():
     assert L.d3gs_blend_fwd(C.byref(P), *odd) == -1 and b"multiples of 16" in L.d3gs_last_error_string()
     P.sh_degree, P.sh_stride = 3, 4
     assert L.d3gs_blend_fwd(C.byref(P), *nul) == -1 and b"sh_stride" in L.d3gs_last_error_string()
+    # the feature kernels: nothing to do without channels, NULL buffers refused with them
+    P.sh_stride = 16
+    assert L.d3gs_blend_features_fwd(C.byref(P), None, None, None, None, None, 0, None, None, None) == 0
+    assert L.d3gs_blend_features_fwd(C.byref(P), None, None, None, None, None, 3, None, None, None) == -1
+    assert b"NULL" in L.d3gs_last_error_string()
+    assert L.d3gs_blend_features_bwd(C.byref(P), *([None] * 5), -1, *([None] * 8)) == -1
+    assert b"num_features" in L.d3gs_last_error_string()
     n = C.c_size_t(0)
     assert L.d3gs_sort_workspace_bytes(1000, 0, 65, C.byref(n)) == -1
     assert L.d3gs_sort_workspace_bytes(1000, 0, 45, C.byref(n)) == 0 and n.value > 0
