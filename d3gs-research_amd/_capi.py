@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 32
+ABI_VERSION = 33
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
 BUCKET_SIZE = 64          # D3GS_BUCKET_SIZE
@@ -42,7 +42,7 @@ class Params(C.Structure):
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
         ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
-        ("batch_size", C.c_int32), ("compact_items", C.c_int32), ("batch_cameras", C.c_void_p),
+        ("render_inv_depth", C.c_int32), ("batch_size", C.c_int32), ("compact_items", C.c_int32), ("batch_cameras", C.c_void_p),
         ("atomic_add_count", C.c_void_p),
     ]
 

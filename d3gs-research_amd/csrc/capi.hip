@@ -37,7 +37,13 @@ extern "C" int d3gs_depth_key_bits(const d3gs_params* p) {
     if (!p) return 32;
     if (p->enable_32bit_sort) return d3gs::kDepthStepBits;
     union { float f; uint32_t u; } far_bits;
-    far_bits.f = p->z_far;
+    // largest stored value of an accepted gaussian: z_far, or with render_inv_depth 1 / z_near
+    if (p->render_inv_depth) {
+        if (!(p->z_near > 0.0f)) return 32;
+        far_bits.f = 1.0f / p->z_near;
+    } else {
+        far_bits.f = p->z_far;
+    }
     const uint32_t base = d3gs::depth_key_base(*p);
     if (!(p->z_far > 0.0f) || far_bits.u < base) return 1;    // nothing is accepted: every key is 0
     const int bits = d3gs_higher_msb(far_bits.u - base);

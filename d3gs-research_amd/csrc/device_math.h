@@ -632,13 +632,17 @@ __device__ __forceinline__ uint32_t reference_depth_bits(const d3gs_params& P, f
 // of z_near fit d3gs_depth_key_bits() bits (27 for the default planes, three 9-bit digits instead of four
 // 8-bit ones); rejected gaussians (depth written as 0) get key 0.
 __host__ __device__ __forceinline__ uint32_t depth_key_base(const d3gs_params& P) {
-    union { float f; uint32_t u; } near_bits;
-    near_bits.f = P.z_near;
-    return P.z_near > 0.0f ? near_bits.u : 0u;
+    union { float f; uint32_t u; } low;
+    // smallest stored value of an accepted gaussian: z_near, or with render_inv_depth 1 / z_far (division rounds
+    // monotonically, so 1 / z of every z <= z_far is at least that)
+    low.f = P.render_inv_depth ? (P.z_far > 0.0f ? 1.0f / P.z_far : 0.0f) : P.z_near;
+    return low.f > 0.0f ? low.u : 0u;
 }
-__device__ __forceinline__ uint32_t depth_sort_key(const d3gs_params& P, float z) {
-    if (P.enable_32bit_sort) return reference_depth_bits(P, z);
-    return z >= P.z_near && z > 0.0f ? __float_as_uint(z) - depth_key_base(P) : 0u;
+// v: the value K1 stores in `depths` (z, or 1 / z with render_inv_depth; 0 for a rejected gaussian)
+__device__ __forceinline__ uint32_t depth_sort_key(const d3gs_params& P, float v) {
+    if (P.enable_32bit_sort) return reference_depth_bits(P, v);
+    const uint32_t bits = __float_as_uint(v), base = depth_key_base(P);
+    return v > 0.0f && bits >= base ? bits - base : 0u;
 }
 
 }  // namespace d3gs

@@ -260,8 +260,10 @@ __global__ __launch_bounds__(kPrepBlock) void preprocess_fwd_kernel(
     }
     {
     const int i = out_i;
-    depths[i] = z;
-    if (depth_sort_keys) depth_sort_keys[i] = depth_sort_key(P, z);
+    // render.py:582: the depth, or its inverse (a rejected gaussian's stays 0)
+    const float stored = (P.render_inv_depth && valid) ? 1.0f / z : z;
+    depths[i] = stored;
+    if (depth_sort_keys) depth_sort_keys[i] = depth_sort_key(P, stored);
     radii[i] = (int)radius;
     *reinterpret_cast<float2*>(uvs + 2 * i) = make_float2(u, v);
     *reinterpret_cast<float4*>(conic_opacity + 4 * i) = make_float4(con0, con1, con2, op);
@@ -424,6 +426,7 @@ __device__ __forceinline__ void preprocess_bwd_one(
     float gu = ra.x * P.fx, gv = ra.y * P.fy;
     float zi = 1.0f / z, zi2 = 1.0f / (z * z);
     float dzin = P.render_depth ? rc.y : 0.0f;
+    if (P.render_inv_depth) dzin = (-dzin) / (z * z);      // the record holds dL/d(1/z) (render.py:1965, 3051, 3283)
     float dpc[3] = {gu * zi, gv * zi, (dzin + ((-gu) * pc[0]) * zi2) + ((-gv) * pc[1]) * zi2};
 
     // conic -> cov2d backward (gs3d.py:571-586)

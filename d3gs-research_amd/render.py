@@ -10,8 +10,9 @@ ahead-of-time HIP library through ``_capi`` on torch's current stream.
 Scope: single cameras and camera bundles (one pass over B x N render items), every
 early filter (OBB_DFVT computed as the OBB tile set), RGB / RGBA / depth / custom
 feature channels in NHWC or NCHW, instances, sparse mode, both backward algorithms.
-The few options outside that scope (``render_inv_depth``, ``transmittance_is_double``,
-tile sizes other than 16 x 16, ``prep_user_inputs``) raise ``NotImplementedError``.
+``render_inv_depth`` keeps the reference's behaviour (1 / z is also what the lists are sorted by).
+The few options outside that scope (``transmittance_is_double``, tile sizes other than
+16 x 16, ``prep_user_inputs``) raise ``NotImplementedError``.
 """
 from __future__ import annotations
 
@@ -249,9 +250,6 @@ class GaussianSplatOp:
         c = self._cfg
         unsupported = {
             "tile_size != (16, 16)": tuple(c.tile_size) != (16, 16),
-            # the reference stores 1/z in the buffer it also sorts by (render.py:582, 773), which blends
-            # back to front: not reproduced
-            "render_inv_depth": c.render_inv_depth,
             "transmittance_is_double": c.transmittance_is_double,
             # sparse mode is built for the plain colour path (the reference itself excludes custom features there,
             # render.py:238)
@@ -441,6 +439,9 @@ class GaussianSplatOp:
         P.render_depth, P.render_rgba = int(c.render_depth), int(c.render_rgba)
         P.use_nchw, P.enable_anti_aliasing = int(c.use_nchw), int(c.enable_anti_aliasing)
         P.enable_32bit_sort, P.depth_32bit_prec = int(c.enable_32bit_sort), float(c.depth_32bit_prec)
+        # 1 / z in the depth buffer (render.py:582); as in the reference that buffer also gives the sort key its depth
+        # part (render.py:773), so the lists then run from the far end to the near one
+        P.render_inv_depth = int(c.render_inv_depth)
         if c.enable_32bit_sort:
             assert P.tiles_x * P.tiles_y * max(P.batch_size, 1) < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
         return P

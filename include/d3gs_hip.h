@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 32
+#define D3GS_ABI_VERSION 33
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -97,6 +97,11 @@ typedef struct d3gs_params {
                                      of the float bits (render.py:767-770, 853-854): gaussians of a tile that fall into
                                      the same depth step are blended in index order.  At most 2^14 tiles. */
     float depth_32bit_prec;       /* config_def.py:91, default 0.001 */
+    int32_t render_inv_depth;     /* config_def.py:95; render.py:582, 773, 1965, 3051, 3283: K1 stores 1 / z in `depths`
+                                     where it stores z otherwise.  The sort key's depth part is taken from that same
+                                     buffer, as in the reference, so the lists come out in descending camera depth and
+                                     the blend runs over them in that order; the depth channel blends 1 / z, the blend
+                                     backward's dz is dL/d(1/z), and K9 turns it into -dz / z^2. */
     /* Camera bundle (render.py:129-150, 314-326): batch_size = B > 1 renders B cameras of one image size in one
      * pass over B * n "render items", item i = b * n + g being gaussian g seen by camera b.  The model arrays keep
      * n rows; everything K1 writes (and the reject mask it reads) has B * n rows; tile ids carry the camera,
@@ -131,7 +136,8 @@ int d3gs_higher_msb(uint32_t n);
 /* Number of significant bits of the depth-sort keys that d3gs_preprocess_fwd writes to depth_sort_keys (no
  * counterpart in the reference): accepted depths lie in [z_near, z_far], so the key is the depth's float bits
  * minus those of z_near -- the same order in fewer bits (27 for the default planes 0.2 and 1e4) -- or, with
- * enable_32bit_sort, the 18-bit depth step.  The depth sort runs on bits [0, d3gs_depth_key_bits(p)). */
+ * enable_32bit_sort, the 18-bit depth step; with render_inv_depth the stored 1 / z lies in [1 / z_far, 1 / z_near]
+ * and the key is its float bits minus those of 1 / z_far.  The depth sort runs on bits [0, d3gs_depth_key_bits(p)). */
 int d3gs_depth_key_bits(const d3gs_params* p);
 
 /* Instance rendering (render.py:207-220, 346-356): a gaussian with instance_ids[i] = k >= 0 belongs to object

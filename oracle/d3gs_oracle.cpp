@@ -100,6 +100,8 @@ struct orc_params {
     int32_t enable_anti_aliasing;  // opacity scaled by sqrt(det / det_lowpass) (render.py:391-407)
     int32_t enable_32bit_sort;     // key = (tile << 18) | (uint32(depth / prec) & 0x3FFFF) (render.py:767-770, 820)
     float depth_32bit_prec;        // config_def.py:91
+    int32_t render_inv_depth;      // K1 stores 1 / z where it stores z otherwise (render.py:582): the buffer is also the
+                                   // sort key's depth part (render.py:773), so the lists come out in descending z
 };
 
 // ---------------------------------------------------------------------------
@@ -537,7 +539,7 @@ ORC_API int orc_preprocess_fwd(const orc_params* P0, const float* xyz, const flo
         int cnt = tile_walk(P, g, [](int, int) {});
         radii[i] = (int)radius;
         tiles_touched[i] = cnt;
-        depths[i] = z;
+        depths[i] = P->render_inv_depth ? 1.0f / z : z;   // render.py:582
         uvs[2 * i] = u;
         uvs[2 * i + 1] = v;
         conic_opacity[4 * i + 0] = con0;
@@ -923,6 +925,7 @@ ORC_API void orc_preprocess_bwd(const orc_params* P0, const float* xyz, const fl
         float gu = duv[2 * i] * P->fx, gv = duv[2 * i + 1] * P->fy;
         float zi = 1.0f / z, zi2 = 1.0f / (z * z);
         float dzin = dz ? dz[i] : 0.0f;
+        if (P->render_inv_depth) dzin = (-dzin) / (pc[2] * pc[2]);   // dz is dL/d(1/z) then (render.py:1965, 3051, 3283)
         float dpc[3] = {gu * zi, gv * zi, (dzin + ((-gu) * pc[0]) * zi2) + ((-gv) * pc[1]) * zi2};
 
         // conic -> cov2d backward (gs3d.py:571-586)

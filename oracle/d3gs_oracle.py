@@ -34,6 +34,7 @@ class OracleParams(C.Structure):
         ("scale_global", C.c_float), ("bg", C.c_float * 3), ("fused_activation", C.c_int32),
         ("render_depth", C.c_int32), ("render_rgba", C.c_int32), ("use_nchw", C.c_int32),
         ("enable_anti_aliasing", C.c_int32), ("enable_32bit_sort", C.c_int32), ("depth_32bit_prec", C.c_float),
+        ("render_inv_depth", C.c_int32),
     ]
 
 
@@ -78,7 +79,7 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
                 radii_eigen_eps=0.1, clamp_factor=1.3, std_sigma=3.0, lowpass=0.3, alpha_eps=1.0 / 255.0,
                 transmittance_eps=1e-4, scale_global=1.0, bg=(0.0, 0.0, 0.0), fused_activation=True,
                 render_depth=False, render_rgba=False, use_nchw=False, enable_anti_aliasing=False,
-                enable_32bit_sort=False, depth_32bit_prec=0.001) -> OracleParams:
+                enable_32bit_sort=False, depth_32bit_prec=0.001, render_inv_depth=False) -> OracleParams:
     """cam2world_T is the 4x3 matrix ``to_world[:3].T`` (render.py:205-206)."""
     P = OracleParams()
     P.n, P.width, P.height = int(n), int(width), int(height)
@@ -103,6 +104,7 @@ def make_params(*, n, width, height, focal_xy, principal_point, cam2world_T, sh_
     P.render_depth, P.render_rgba = int(bool(render_depth)), int(bool(render_rgba))
     P.use_nchw, P.enable_anti_aliasing = int(bool(use_nchw)), int(bool(enable_anti_aliasing))
     P.enable_32bit_sort, P.depth_32bit_prec = int(bool(enable_32bit_sort)), float(depth_32bit_prec)
+    P.render_inv_depth = int(bool(render_inv_depth))
     if P.enable_32bit_sort:
         assert P.tiles_x * P.tiles_y < 2 ** 14, "32bit sort only support 14 bits tile idx"   # render.py:227-228
     return P

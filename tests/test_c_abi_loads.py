@@ -27,14 +27,14 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_params_struct_matches_header_layout():
     from d3gs_research_amd import _capi
-    # 10 int32 + 6 float + 9 + 3 + 10 float + 3 float + 6 int32 + 1 float + 2 int32 + two pointers
-    assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3 + 6 + 1 + 2) + 16
+    # 10 int32 + 6 float + 9 + 3 + 10 float + 3 float + 6 int32 + 1 float + 3 int32, padding to 8, two pointers
+    assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3 + 6 + 1 + 3) + 4 + 16
 
 
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 32
+    assert L.d3gs_abi_version() == 33
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
     # depth-sort key width: float bits of z_far minus those of z_near, or the 18 depth-step bits
@@ -103,7 +103,8 @@ def test_operator_config_gate():
     GaussianSplatOp(GaussianSplatConfig(move_opacity_in_grad_to_prep=True, use_int64_tile_touched=True,
                                         enable_32bit_sort=True))
     GaussianSplatOp(GaussianSplatConfig(sparse_mode=True))
-    for kw, word in ((dict(sparse_mode=True, disable_builtin_rgb=True), "sparse_mode"), (dict(render_inv_depth=True), "render_inv_depth"),
+    GaussianSplatOp(GaussianSplatConfig(render_inv_depth=True, render_depth=True))
+    for kw, word in ((dict(sparse_mode=True, disable_builtin_rgb=True), "sparse_mode"),
                      (dict(rasterize_backward_algo=RasterizeBackwardAlgo.PER_GAUSSIAN, disable_builtin_rgb=True), "PER_GAUSSIAN"),
                      (dict(transmittance_is_double=True), "transmittance_is_double"), (dict(tile_size=(8, 8)), "tile_size"),
                      (dict(disable_builtin_rgb=True, use_nchw=True), "use_nchw")):

@@ -39,8 +39,9 @@ def _quat_to_R(q):
         torch.stack([2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)], -1)], -2)
 
 
-def _render_f64(scene, params, member, order, anti_aliasing=False, feat=None):
+def _render_f64(scene, params, member, order, anti_aliasing=False, feat=None, inv_depth=False):
     """Dense float64 forward: `member[p, j]` says gaussian order[j] is in pixel p's tile list.
+    inv_depth: the depth channel blends 1 / z.
     Returns colour, T, blended depth and blended alpha (the sum of the weights), and the blended
     custom features when `feat` [N, F] is given."""
     xyz, quat, scale, opac, sh = params
@@ -97,7 +98,7 @@ def _render_f64(scene, params, member, order, anti_aliasing=False, feat=None):
         use = live & ~stop & (power.detach() <= 0)
         w = torch.where(use, alpha * Tcur, torch.zeros_like(Tcur))
         col = col + w[:, None] * rgb[g]
-        dep = dep + w * z[g]
+        dep = dep + (w / z[g] if inv_depth else w * z[g])
         asum = asum + w
         if feat is not None:
             fimg = fimg + w[:, None] * feat[g]
@@ -119,13 +120,20 @@ def _setup(seed_cfg=0, n=96, wh=(48, 32), filt=0, sh_cfg=None):
     return scene
 
 
-def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False, feat=None, feat_image=None, dfeat=None):
+def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False, feat=None, feat_image=None, dfeat=None,
+               far_to_near=False):
     """Float64 autograd gradients of sum(color*drgb) + sum(T*dT) (+ sum(depth*ddepth))
     (+ sum(features*dfeat)) w.r.t. the raw model tensors (and the custom features, last in the list).
     A four-channel drgb also weights the blended alpha."""
     # global depth order (stable) and per-pixel tile-list membership from the oracle's binning
     valid = np.flatnonzero(ref["radii"] > 0)
     order = valid[np.argsort(ref["depths"][valid].view(np.uint32), kind="stable")]
+    if far_to_near:
+        # render_inv_depth: the order is not taken from the oracle's depth buffer but from the camera-space z
+        # itself, descending (what sorting by 1 / z amounts to), and the depth channel blends 1 / z
+        tw = np.asarray(scene.to_world, np.float64)
+        z = (scene.xyz[valid].astype(np.float64) - tw[:3, 3]) @ tw[:3, 2]
+        order = valid[np.argsort(-z, kind="stable")]
     pos = {g: j for j, g in enumerate(order.tolist())}
     tiles_x = (scene.width + 15) // 16
     member = np.zeros((scene.height * scene.width, len(order)), bool)
@@ -142,7 +150,8 @@ def _f64_grads(scene, ref, drgb, dT, ddepth=None, anti_aliasing=False, feat=None
         col, Tfin, dep, asum, fimg = _render_f64(scene, params[:5], torch.from_numpy(member), order.tolist(),
                                                  anti_aliasing, params[5])
     else:
-        col, Tfin, dep, asum = _render_f64(scene, params, torch.from_numpy(member), order.tolist(), anti_aliasing)
+        col, Tfin, dep, asum = _render_f64(scene, params, torch.from_numpy(member), order.tolist(), anti_aliasing,
+                                           inv_depth=far_to_near)
     # the float64 forward agrees with the oracle's float32 forward (no threshold flips on this scene)
     assert np.abs(col.detach().numpy() - ref["color"][..., :3]).max() <= 2e-5
     assert np.abs(Tfin.detach().numpy() - ref["T"]).max() <= 1e-5
@@ -298,6 +307,46 @@ def test_channels_and_anti_aliasing_match_float64_autograd(oracle, aa, depth, rg
     grads = _f64_grads(scene, ref, drgb, dT, ddepth, aa)
     for i, name in enumerate(["dxyz", "dquat", "dscale", "dopacity", "dsh"]):
         _close(pb[name], grads[i], name)
+
+
+def test_inverse_depth_matches_float64_autograd_over_far_to_near_lists(oracle):
+    """render_inv_depth (config_def.py:95; render.py:582, 773, 1965, 3051, 3283): K1 stores 1 / z, the sort key takes
+    its depth part from that buffer, so every list runs from the far end to the near one; the depth channel blends
+    1 / z and K9 turns dL/d(1/z) into -dz / z^2.  Pinned by the dense float64 restatement run over the gaussians
+    in descending camera-space z (computed here from the scene, not from the oracle's buffers) with 1 / z as the
+    depth channel: image, T, depth image and every model gradient; and the plain render of the same scene is a
+    different image (the order matters)."""
+    scene = _setup()
+    P = oracle_params(oracle, scene, 0)
+    P.render_depth, P.render_inv_depth = 1, 1
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    P0 = oracle_params(oracle, scene, 0)
+    P0.render_depth = 1
+    ref0 = oracle.forward(P0, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    seen = ref0["radii"] > 0
+    assert np.array_equal(ref["radii"], ref0["radii"]) and np.array_equal(ref["tiles_touched"], ref0["tiles_touched"])
+    assert np.array_equal(ref["depths"][seen], (np.float32(1.0) / ref0["depths"][seen]).astype(np.float32))
+    assert np.abs(ref["color"] - ref0["color"]).max() > 1e-2
+    # inside every tile list the camera depth never grows
+    z0 = ref0["depths"]
+    for r0, r1 in ref["workload_ranges"]:
+        zs = z0[ref["gaussian_idx_sorted"][r0:r1]]
+        assert np.all(zs[1:] <= zs[:-1])
+    rng = np.random.default_rng(14)
+    drgb = rng.standard_normal((scene.height, scene.width, 3)).astype(np.float32)
+    dT = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    ddepth = rng.standard_normal((scene.height, scene.width)).astype(np.float32)
+    g, pb = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                            drgb, dT, ddepth=ddepth)
+    grads = _f64_grads(scene, ref, drgb, dT, ddepth, far_to_near=True)
+    for i, name in enumerate(["dxyz", "dquat", "dscale", "dopacity", "dsh"]):
+        _close(pb[name], grads[i], name)
+    # the depth gradient alone (nothing but ddepth): what -dz / z^2 carries into dxyz
+    zeros3, zeros1 = np.zeros_like(drgb), np.zeros_like(dT)
+    _, pb_d = oracle.backward(P, ref, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh,
+                              zeros3, zeros1, ddepth=ddepth)
+    grads_d = _f64_grads(scene, ref, zeros3, zeros1, ddepth, far_to_near=True)
+    _close(pb_d["dxyz"], grads_d[0], "dxyz from the depth channel alone")
 
 
 @pytest.mark.parametrize("F,depth", [(2, False), (3, False), (7, True)])
