@@ -744,7 +744,7 @@ __device__ __forceinline__ bool record_is_zero(const float4 ra, const float4 rb,
            rb.z == 0.0f && rb.w == 0.0f && rc.x == 0.0f && rc.y == 0.0f;
 }
 
-template <int kPer, bool kInstances>
+template <int kPer, bool kInstances, bool kMany>
 __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const d3gs_params P_in, const int batch_index, const int batch_last, const int accumulate_in, const InstanceView inst,
     const float* __restrict__ xyz, const float* __restrict__ quat,
@@ -768,7 +768,9 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
     const int first = blockIdx.x * kSpan;
     const int nrows = min(kSpan, P_in.n - first);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int cam = batch_index; cam <= batch_last; ++cam) {
+    // (kMany = false: the one camera batch_index, straight-line code, the kernel's parameters stay where the
+    // compiler keeps kernel arguments)
+    auto one_camera = [&](const int cam) {
     d3gs_params P = P_in;
     if (P_in.batch_size > 1 && !row_batch_ids) apply_batch_camera(P, cam);
     const size_t item0 = (size_t)(cam - batch_index) * (size_t)P_in.n;     // this camera's rows of the per-item arrays
@@ -876,7 +878,14 @@ __global__ __launch_bounds__(kBwdBlock) void preprocess_bwd_kernel(
         bwd_rows_copy<false>(dsh, s_rows, s_list + base, cnt, first, rowlen, stride, accumulate != 0);
         __syncthreads();
     }
-    __syncthreads();      // the lists are rebuilt for the next camera
+    };
+    if constexpr (kMany) {
+        for (int cam = batch_index; cam <= batch_last; ++cam) {
+            one_camera(cam);
+            __syncthreads();      // the lists are rebuilt for the next camera
+        }
+    } else {
+        one_camera(batch_index);
     }
 }
 
@@ -1168,8 +1177,8 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
     const bool wide = p->n >= 512 * kBwdBlock * 4;
     const int per = wide ? 4 : 1;
     dim3 grid((p->n + kBwdBlock * per - 1) / (kBwdBlock * per)), block(kBwdBlock);
-#define D3GS_LAUNCH_K9(PER, INST)                                                                                     \
-    hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST>), grid, block, lds_bytes, (hipStream_t)stream, *p,            \
+#define D3GS_LAUNCH_K9(PER, INST, MANY)                                                                                     \
+    hipLaunchKernelGGL((preprocess_bwd_kernel<PER, INST, MANY>), grid, block, lds_bytes, (hipStream_t)stream, *p,      \
                        (int)batch_index, (int)batch_last, (int)accumulate, inst, xyz,                                                   \
                        quaternion_xyzw, scale, opacity, color_sh, radii, cov2d_vecs, sh_to_rgb_ne_0, grad_records,     \
                        touched,                                                                                        \
@@ -1179,8 +1188,14 @@ static int preprocess_bwd_impl(const char* who, const d3gs_params* p, int32_t ba
                        dopacity_out,                                                                                   \
                        dcolor_sh, dcolor_sh_base)
     const bool per_row = inst.ids || (row_batch_ids && p->batch_size > 1);      // the instantiation that forms a camera per row
-    if (wide) { if (per_row) D3GS_LAUNCH_K9(4, true); else D3GS_LAUNCH_K9(4, false); }
-    else      { if (per_row) D3GS_LAUNCH_K9(1, true); else D3GS_LAUNCH_K9(1, false); }
+    const bool many = batch_last > batch_index;
+    if (wide) {
+        if (many) { if (per_row) D3GS_LAUNCH_K9(4, true, true); else D3GS_LAUNCH_K9(4, false, true); }
+        else      { if (per_row) D3GS_LAUNCH_K9(4, true, false); else D3GS_LAUNCH_K9(4, false, false); }
+    } else {
+        if (many) { if (per_row) D3GS_LAUNCH_K9(1, true, true); else D3GS_LAUNCH_K9(1, false, true); }
+        else      { if (per_row) D3GS_LAUNCH_K9(1, true, false); else D3GS_LAUNCH_K9(1, false, false); }
+    }
 #undef D3GS_LAUNCH_K9
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_preprocess_bwd: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
