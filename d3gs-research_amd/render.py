@@ -1496,3 +1496,12 @@ def rasterize_gaussians(model: GaussianModelOriginBase, cameras, op: GaussianSpl
                                     instance2world_T)
     return GaussianSplatOutput(color=res[0], depth=res[1], custom_features=res[2], T=res[3], n_contrib=res[4],
                                radii=res[5])
+
+
+def __getattr__(name):
+    # render.py:3840-3891 lives beside rasterize_gaussians in the reference; here it is defined with the
+    # time-dependent model family it serves (pvg.py imports this module, hence the late lookup)
+    if name == "rasterize_gaussians_dynamic":
+        from .pvg import rasterize_gaussians_dynamic
+        return rasterize_gaussians_dynamic
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

@@ -110,3 +110,11 @@ def test_operator_config_gate():
                      (dict(disable_builtin_rgb=True, use_nchw=True), "use_nchw")):
         with pytest.raises(NotImplementedError, match=word):
             GaussianSplatOp(GaussianSplatConfig(**kw))
+
+
+def test_reference_entry_points_are_importable_from_the_render_module():
+    """Callers of the reference import these names from its render module (render.py:3783, 3840)."""
+    from d3gs_research_amd.render import (CameraBundle, GaussianSplatGradients, GaussianSplatOp,  # noqa: F401
+                                          GaussianSplatOutput, rasterize_gaussians, rasterize_gaussians_dynamic)
+    from d3gs_research_amd import pvg
+    assert rasterize_gaussians_dynamic is pvg.rasterize_gaussians_dynamic
