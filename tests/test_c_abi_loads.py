@@ -31,6 +31,25 @@ def test_params_struct_matches_header_layout():
     assert C.sizeof(_capi.Params) == 4 * (10 + 6 + 9 + 3 + 10 + 3 + 6 + 1 + 3) + 4 + 16
 
 
+def test_params_fields_follow_the_header_in_name_and_order():
+    """The ctypes mirror of d3gs_params lists the header's fields, in the header's order, with the header's types."""
+    from d3gs_research_amd import _capi
+    text = open(os.path.join(ROOT, "include", "d3gs_hip.h")).read()
+    body = text[text.index("typedef struct d3gs_params {"):text.index("} d3gs_params;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    declared = []
+    for ctype, names in re.findall(r"^\s*(int32_t|float|const float\*|uint32_t\*)\s+([^;]+);", body, flags=re.M):
+        for name in names.split(","):
+            m = re.match(r"\s*(\w+)(?:\[(\d+)\])?\s*$", name)
+            declared.append((m.group(1), ctype, int(m.group(2) or 0)))
+    kinds = {"int32_t": C.c_int32, "float": C.c_float, "const float*": C.c_void_p, "uint32_t*": C.c_void_p}
+    want = [(n, kinds[t] * k if k else kinds[t]) for n, t, k in declared]
+    got = list(_capi.Params._fields_)
+    assert [n for n, _ in got] == [n for n, _ in want]
+    for (n, a), (_, b) in zip(got, want):
+        assert C.sizeof(a) == C.sizeof(b) and (a is b or getattr(a, "_length_", 0) == getattr(b, "_length_", 0)), n
+
+
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
