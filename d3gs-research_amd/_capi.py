@@ -15,13 +15,13 @@ _CSRC = os.path.join(_HERE, "csrc")
 # D3GS_HIP_LIBRARY overrides the in-tree location (a library installed elsewhere)
 LIB_PATH = os.environ.get("D3GS_HIP_LIBRARY") or os.path.join(_CSRC, "libd3gs_hip.so")
 
-ABI_VERSION = 33
+ABI_VERSION = 34
 GRAD_RECORD_FLOATS = 16   # D3GS_GRAD_RECORD_FLOATS
 BATCH_CAMERA_FLOATS = 16  # D3GS_BATCH_CAMERA_FLOATS
 BUCKET_SIZE = 64          # D3GS_BUCKET_SIZE
 ERR_SORT_LOOKBACK = -5    # D3GS_ERR_SORT_LOOKBACK
 COUNT_SCAN_GAVE_UP, COUNT_SORT_GAVE_UP, COUNT_PENDING = -1, -2, -3
-BIN_WORKSPACES_ARE_ZERO, BIN_HOST_COUNT_AT_END = 1, 2
+BIN_WORKSPACES_ARE_ZERO, BIN_HOST_COUNT_AT_END, BIN_KEYS_16BIT = 1, 2, 4
 MAX_PAIRS = (1 << 31) - 1024     # D3GS_MAX_PAIRS
 SCAN_NOALLOC_MAX_N = 1 << 24   # D3GS_SCAN_NOALLOC_MAX_N
 

@@ -393,6 +393,9 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
         if constexpr (sizeof(Key) == 4) {
             const uint4 v = *reinterpret_cast<const uint4*>(keys + i0);   // i0 is a multiple of 4
             k[0] = v.x; k[1] = v.y; k[2] = v.z; k[3] = v.w;
+        } else if constexpr (sizeof(Key) == 2) {
+            const uint2 v = *reinterpret_cast<const uint2*>(keys + i0);   // four 16-bit keys
+            k[0] = (Key)(v.x & 0xFFFFu); k[1] = (Key)(v.x >> 16); k[2] = (Key)(v.y & 0xFFFFu); k[3] = (Key)(v.y >> 16);
         } else {
 #pragma unroll
             for (int j = 0; j < kRangeItems; ++j) k[j] = keys[i0 + j];
@@ -677,16 +680,18 @@ extern "C" int d3gs_scan_tiles(int32_t* tiles_touched, int32_t n, void* workspac
     return rc;
 }
 
-extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
-                              const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
-                              const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
-                              uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
+// keys: (tile << 32) | depth bits; tile_keys / tile_keys16: the tile id alone in 32 or 16 bits.  Exactly one is given.
+static int make_keys_impl(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                          const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                          const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                          uint32_t* tile_keys, uint16_t* tile_keys16, int32_t* gaussian_idx, int64_t m,
+                          d3gs_stream_t stream) {
     int rc = check_params(p, "d3gs_make_keys");
     if (rc) return rc;
     if (m < 0) { set_error("d3gs_make_keys: m < 0"); return D3GS_ERR_INVALID_ARGUMENT; }
     if (p->n == 0 || m == 0) return D3GS_OK;
-    if (!radii || !uvs || !conic_opacity || !depths || !offsets || (!keys && !tile_keys) || (keys && tile_keys) ||
-        !gaussian_idx) {
+    const int given = (keys != nullptr) + (tile_keys != nullptr) + (tile_keys16 != nullptr);
+    if (!radii || !uvs || !conic_opacity || !depths || !offsets || given != 1 || !gaussian_idx) {
         set_error("d3gs_make_keys: NULL buffer (exactly one of keys / tile_keys must be given)");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
@@ -698,18 +703,42 @@ extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const 
         set_error("d3gs_make_keys: tile_masks must be 16-byte aligned");
         return D3GS_ERR_INVALID_ARGUMENT;
     }
+    if (tile_keys16 && (long long)p->tiles_x * p->tiles_y * batch_count(*p) > (1ll << 16)) {
+        set_error("d3gs_make_keys: 16-bit tile ids need at most 2^16 tiles");
+        return D3GS_ERR_INVALID_ARGUMENT;
+    }
     const dim3 grid((item_count(*p) + kBlock - 1) / kBlock), block(kBlock);
     if (keys)
         hipLaunchKernelGGL(make_keys_kernel<uint64_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
                            depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,
                            keys, gaussian_idx, (long long)m);
-    else
+    else if (tile_keys)
         hipLaunchKernelGGL(make_keys_kernel<uint32_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
                            depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,
                            tile_keys, gaussian_idx, (long long)m);
+    else
+        hipLaunchKernelGGL(make_keys_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, *p, radii, uvs, conic_opacity,
+                           depths, offsets, gaussian_order, ordered_depth_keys, (const unsigned long long*)tile_masks,
+                           tile_keys16, gaussian_idx, (long long)m);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { set_error("d3gs_make_keys: launch failed: %s", hipGetErrorString(e)); return D3GS_ERR_LAUNCH; }
     return D3GS_OK;
+}
+
+extern "C" int d3gs_make_keys(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                              const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                              const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint64_t* keys,
+                              uint32_t* tile_keys, int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
+    return make_keys_impl(p, radii, uvs, conic_opacity, depths, offsets, gaussian_order, ordered_depth_keys, tile_masks,
+                          keys, tile_keys, nullptr, gaussian_idx, m, stream);
+}
+
+int d3gs::make_tile_keys_u16(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                             const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                             const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint16_t* tile_keys,
+                             int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream) {
+    return make_keys_impl(p, radii, uvs, conic_opacity, depths, offsets, gaussian_order, ordered_depth_keys, tile_masks,
+                          nullptr, nullptr, tile_keys, gaussian_idx, m, stream);
 }
 
 extern "C" int d3gs_depth_keys(const float* depths, int32_t n, uint64_t* keys, int32_t* gaussian_idx,
@@ -774,6 +803,15 @@ extern "C" int d3gs_tile_ranges(const uint64_t* keys_sorted, int64_t m, int32_t*
 }
 
 namespace d3gs {
+int tile_ranges_u16_with_status(const uint16_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
+                                int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
+                                const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
+                                int64_t* total_host, bool publish_host, d3gs_stream_t stream) {
+    return tile_ranges_impl<uint16_t>("d3gs_bin_pairs (tile ranges)", tile_keys_sorted, m, m_device, workload_ranges,
+                                      num_tiles, tile_order, stream,
+                                      BinStatus{{sort_error_a, sort_error_b}, total_dev, total_host,
+                                                publish_host && total_host != nullptr});
+}
 int tile_ranges_u32_with_status(const uint32_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
                                 int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
                                 const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,

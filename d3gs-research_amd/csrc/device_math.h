@@ -620,6 +620,22 @@ int tile_ranges_u32_with_status(const uint32_t* tile_keys_sorted, int64_t m, con
                                 const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
                                 int64_t* total_host, bool publish_host, d3gs_stream_t stream);
 
+// value of the sorts' workspace_is_zero argument
+constexpr int kSortWorkspaceIsZero = 1;
+// The one-call binning on 16-bit tile ids (binning.hip, radix_sort.hip): key expansion, pair sort and tile ranges
+// over uint16 keys; arguments as the 32-bit entry points'.
+int make_tile_keys_u16(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
+                       const float* depths, const int32_t* offsets, const int32_t* gaussian_order,
+                       const uint32_t* ordered_depth_keys, const uint64_t* tile_masks, uint16_t* tile_keys,
+                       int32_t* gaussian_idx, int64_t m, d3gs_stream_t stream);
+int sort_pairs_u16(uint16_t* keys_a, uint16_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                   size_t workspace_bytes, int64_t m, const int64_t* m_device, int workspace_is_zero, int end_bit,
+                   int* result_in_b_host, d3gs_stream_t stream);
+int tile_ranges_u16_with_status(const uint16_t* tile_keys_sorted, int64_t m, const int64_t* m_device,
+                                int32_t* workload_ranges, int32_t num_tiles, int32_t* tile_order,
+                                const uint32_t* sort_error_a, const uint32_t* sort_error_b, int64_t* total_dev,
+                                int64_t* total_host, bool publish_host, d3gs_stream_t stream);
+
 // Depth part of the reference's sort key (render.py:767-775): the float bits (positive floats order like their
 // bit patterns), or with enable_32bit_sort the depth in steps of depth_32bit_prec, truncated to 18 bits.
 __device__ __forceinline__ uint32_t reference_depth_bits(const d3gs_params& P, float z) {

@@ -123,21 +123,27 @@ __global__ __launch_bounds__(kHistThreads) void os_hist_kernel(const Key* __rest
     // body of the input goes in 16-byte loads, two in flight (the bytes a CU has under way set its rate here);
     // the last few keys, and an input that is not 16-byte aligned, go one key at a time, four in flight.
     long long i = (long long)blockIdx.x * kHistThreads + threadIdx.x;
-    if constexpr (sizeof(Key) == 4) {
+    if constexpr (sizeof(Key) <= 4) {
         if ((reinterpret_cast<uintptr_t>(keys) & 15u) == 0) {
+            constexpr int kPerQuad = 16 / (int)sizeof(Key);       // keys in a 16-byte load: four, or eight 16-bit ones
             const uint4* quads = reinterpret_cast<const uint4*>(keys);
-            const long long nq = m / 4;
+            const long long nq = m / kPerQuad;
+            auto count_quad = [&](const uint4& a) {
+                if constexpr (sizeof(Key) == 4) {
+                    count(a.x); count(a.y); count(a.z); count(a.w);
+                } else {
+                    count((Key)(a.x & 0xFFFFu)); count((Key)(a.x >> 16)); count((Key)(a.y & 0xFFFFu)); count((Key)(a.y >> 16));
+                    count((Key)(a.z & 0xFFFFu)); count((Key)(a.z >> 16)); count((Key)(a.w & 0xFFFFu)); count((Key)(a.w >> 16));
+                }
+            };
             long long q = i;
             for (; q + stride < nq; q += 2 * stride) {
                 const uint4 a = quads[q], b = quads[q + stride];
-                count(a.x); count(a.y); count(a.z); count(a.w);
-                count(b.x); count(b.y); count(b.z); count(b.w);
+                count_quad(a);
+                count_quad(b);
             }
-            for (; q < nq; q += stride) {
-                const uint4 a = quads[q];
-                count(a.x); count(a.y); count(a.z); count(a.w);
-            }
-            i += nq * 4;      // the up to three keys behind the last whole quad
+            for (; q < nq; q += stride) count_quad(quads[q]);
+            i += nq * kPerQuad;      // the few keys behind the last whole quad
         }
     }
     for (; i + 3 * stride < m; i += 4 * stride) {
@@ -491,6 +497,16 @@ extern "C" int d3gs_sort_pairs(uint64_t* keys_a, uint64_t* keys_b, int32_t* vals
                                d3gs_stream_t stream) {
     return sort_pairs_impl<uint64_t>("d3gs_sort_pairs", 64, keys_a, keys_b, vals_a, vals_b, workspace, workspace_bytes, m,
                                      nullptr, 0, 0, begin_bit, end_bit, result_in_b_host, stream);
+}
+
+// The pair sort of the one-call binning on 16-bit tile ids (at most 2^16 tiles): the same kernels over keys half as
+// wide, a quarter less to move per pass.
+int d3gs::sort_pairs_u16(uint16_t* keys_a, uint16_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,
+                         size_t workspace_bytes, int64_t m, const int64_t* m_device, int workspace_is_zero, int end_bit,
+                         int* result_in_b_host, d3gs_stream_t stream) {
+    return sort_pairs_impl<uint16_t>("d3gs_bin_pairs (pair sort, 16-bit tile ids)", 16, keys_a, keys_b, vals_a, vals_b,
+                                     workspace, workspace_bytes, m, m_device, 0, workspace_is_zero, 0, end_bit,
+                                     result_in_b_host, stream);
 }
 
 extern "C" int d3gs_sort_pairs_u32(uint32_t* keys_a, uint32_t* keys_b, int32_t* vals_a, int32_t* vals_b, void* workspace,

@@ -237,6 +237,8 @@ class GaussianSplatOp:
         # custom feature channels through the library's feature kernels (False: three at a time through the colour
         # kernels, one forward and one backward blend per triple)
         self.feature_kernels = True
+        # the one-call binning carries the pairs' tile ids as 16-bit keys when the view has at most 2^16 tiles
+        self.narrow_tile_keys = True
         # the one-call binning writes the pair count to its pinned host word with a store the host can see while
         # the stream runs on, and the host polls that word: an event recorded behind the binning would hold the
         # forward blend back by the few microseconds the stream takes to process the marker
@@ -279,6 +281,8 @@ class GaussianSplatOp:
         sorted tile keys and gaussian indices (parity tests compare them with the oracle's)."""
         assert self._last_sorted is not None, "set D3GS_KEEP_SORTED_KEYS=1 before importing the package"
         tile_keys, idx, depths = self._last_sorted
+        if tile_keys.dtype == torch.int16:      # the one-call binning's 16-bit tile ids
+            tile_keys = tile_keys.long() & 0xFFFF
         if self._cfg.enable_32bit_sort:     # render.py:767-770, 820: (tile << 18) | depth steps
             steps = (depths / torch.tensor(self._cfg.depth_32bit_prec, dtype=torch.float32, device=depths.device))
             return (tile_keys.long() << 18) | (steps.long()[idx.long()] & 0x3FFFF)
@@ -820,6 +824,8 @@ class GaussianSplatOp:
             at = lambda off: C.c_void_p(base + 4 * off)
             v.total = torch.empty(1, dtype=torch.int64, device=dev)
             order_in_b, pairs_in_b = C.c_int(0), C.c_int(0)
+            # tile ids that fit 16 bits travel through key expansion, pair sort and ranges as 16-bit keys
+            narrow = bool(self.narrow_tile_keys and v.num_tiles <= (1 << 16))
             # Polling gains a few microseconds per view; a view whose binning takes milliseconds (hundreds of millions
             # of pairs) waits on an event instead, which costs it nothing by comparison and keeps the host thread free.
             v.polled = bool(self.poll_pair_count and n > 0 and cap <= POLL_MAX_PAIRS)
@@ -831,7 +837,8 @@ class GaussianSplatOp:
                 at(o_ord_b), _capi.ptr(v.zero_ws_n), v.zero_ws_n.numel(), at(o_offs), _capi.ptr(v.zero_scan_ws),
                 v.zero_scan_ws.numel(), _capi.ptr(v.total), C.c_void_p(v.slot.count_host.data_ptr()), cap, at(o_tk_a),
                 at(o_tk_b), at(o_ix_a), at(o_ix_b), _capi.ptr(v.zero_ws_m), v.zero_ws_m.numel(), _capi.ptr(v.zero_ranges),
-                at(o_order), _capi.BIN_WORKSPACES_ARE_ZERO | (_capi.BIN_HOST_COUNT_AT_END if v.polled else 0),
+                at(o_order), _capi.BIN_WORKSPACES_ARE_ZERO | (_capi.BIN_HOST_COUNT_AT_END if v.polled else 0)
+                | (_capi.BIN_KEYS_16BIT if narrow else 0),
                 C.byref(order_in_b), C.byref(pairs_in_b), s), "d3gs_bin_pairs")
             if not v.polled:
                 v.count_ready = torch.cuda.Event()
@@ -841,7 +848,8 @@ class GaussianSplatOp:
             v.gaussian_order = pool[o_ord_b:o_ord_b + n] if order_in_b.value else pool[o_ord_a:o_ord_a + n]
             v.counts_ordered = pool[o_offs:o_offs + n]
             o_tk, o_ix = (o_tk_b, o_ix_b) if pairs_in_b.value else (o_tk_a, o_ix_a)
-            v.fused_result = (pool[o_tk:o_tk + cap], pool[o_ix:o_ix + cap], pool[o_order:o_order + v.num_tiles])
+            tile_keys = pool[o_tk:o_tk + cap].view(torch.int16)[:cap] if narrow else pool[o_tk:o_tk + cap]
+            v.fused_result = (tile_keys, pool[o_ix:o_ix + cap], pool[o_order:o_order + v.num_tiles])
             return
         # The reference sorts all M pairs on the whole (tile, depth) key (render.py:845-887).  The depth
         # digits only depend on the gaussian, so the same stable order comes from sorting the N

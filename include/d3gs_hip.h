@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define D3GS_ABI_VERSION 33
+#define D3GS_ABI_VERSION 34
 
 #define D3GS_OK 0
 #define D3GS_ERR_INVALID_ARGUMENT (-1)
@@ -308,9 +308,13 @@ int d3gs_tile_ranges_u32(const uint32_t* tile_keys_sorted, int64_t m, const int6
  * of the call (it needs tile_order != NULL or a workspace to run), with the count or the status in its place, as
  * a system-scope release store: a caller that sets the word to D3GS_COUNT_PENDING before the call can poll it
  * from the host while the stream runs on, where waiting on an event would put a marker into the stream ahead of
- * the kernels that follow.  workload_ranges must be zero on entry. */
+ * the kernels that follow.  With D3GS_BIN_KEYS_16BIT (at most 2^16 tiles in the call) the pair keys are 16-bit tile
+ * ids: tile_keys_a / tile_keys_b are then read and written as uint16[capacity] (the front half of the buffers) and
+ * the sorted keys are found there in that form; the sorted gaussian indices, the ranges and the order are the same.
+ * workload_ranges must be zero on entry. */
 #define D3GS_BIN_WORKSPACES_ARE_ZERO 1
 #define D3GS_BIN_HOST_COUNT_AT_END 2
+#define D3GS_BIN_KEYS_16BIT 4
 int d3gs_bin_pairs(const d3gs_params* p, const int32_t* radii, const float* uvs, const float* conic_opacity,
                    const float* depths, const int32_t* tiles_touched, const uint64_t* tile_masks,
                    uint32_t* depth_keys_a, uint32_t* depth_keys_b, int32_t* order_a, int32_t* order_b,

@@ -53,7 +53,7 @@ def test_params_fields_follow_the_header_in_name_and_order():
 def test_abi_version_and_msb():
     from d3gs_research_amd import _capi
     L = _capi.lib()
-    assert L.d3gs_abi_version() == 33
+    assert L.d3gs_abi_version() == 34
     # devsort.py:131-149: bit length; the sort's end bit for the benchmark tile grids
     assert [L.d3gs_higher_msb(v) for v in (0, 1, 64, 1024, 8160, 32400)] == [0, 1, 7, 11, 13, 15]
     # depth-sort key width: float bits of z_far minus those of z_near, or the 18 depth-step bits
@@ -92,6 +92,14 @@ def test_error_codes_without_compute():
     assert b"NULL" in L.d3gs_last_error_string()
     assert L.d3gs_blend_features_bwd(C.byref(P), *([None] * 5), -1, *([None] * 8)) == -1
     assert b"num_features" in L.d3gs_last_error_string()
+    # 16-bit tile ids are refused for a call with more than 2^16 tiles (before anything is launched)
+    big = _capi.Params()
+    big.n, big.width, big.height, big.tiles_x, big.tiles_y, big.sh_stride = 4, 16 * 300, 16 * 300, 300, 300, 1
+    flags_out = C.c_int(0), C.c_int(0)
+    total = C.c_int64(0)
+    args = [None] * 10 + [None, 0, None, None, 0, C.addressof(total), None, 0] + [None] * 4 + [None, 0, None, None]
+    rc = L.d3gs_bin_pairs(C.byref(big), *args, _capi.BIN_KEYS_16BIT, C.byref(flags_out[0]), C.byref(flags_out[1]), None)
+    assert rc == -1 and b"2^16 tiles" in L.d3gs_last_error_string()
     n = C.c_size_t(0)
     assert L.d3gs_sort_workspace_bytes(1000, 0, 65, C.byref(n)) == -1
     assert L.d3gs_sort_workspace_bytes(1000, 0, 45, C.byref(n)) == 0 and n.value > 0

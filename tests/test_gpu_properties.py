@@ -5,7 +5,7 @@ integer / forward output, and linearity of the backward in the incoming gradient
 import numpy as np
 import pytest
 
-from helpers import gen_scene, op_config, torch_model
+from helpers import gen_scene, op_config, oracle_params, torch_model
 
 pytestmark = pytest.mark.gpu
 NONE, AABB, OBB, DFVT = 0, 1, 3, 4
@@ -183,6 +183,32 @@ def test_every_optional_acceleration_off_gives_the_same_result():
             # a gaussian without gradient has exactly none on both paths
             assert torch.equal(a.reshape(scene.n, -1).abs().sum(1) == 0, b.reshape(scene.n, -1).abs().sum(1) == 0), name
         assert float((u1 - u2).abs().max()) <= 1e-4 * float(u2.abs().max())
+
+
+@pytest.mark.parametrize("cfg_id,n,wh", [(1, 30000, (320, 200)), (4, 20000, (1280, 720))])
+def test_sixteen_bit_tile_keys_sort_like_thirty_two_bit_ones(oracle, cfg_id, n, wh):
+    """The one-call binning carries tile ids as 16-bit keys when the view has at most 2^16 tiles: sorted keys,
+    sorted indices, ranges and image are those of the 32-bit keys and of the oracle, bit for bit."""
+    import torch
+    from d3gs_research_amd.render import GaussianSplatOp
+    scene = gen_scene(cfg_id, n=n, wh=wh)
+    P = oracle_params(oracle, scene, DFVT)
+    ref = oracle.forward(P, scene.xyz, scene.quaternion_xyzw, scene.scale, scene.opacity, scene.color_sh)
+    model = torch_model(scene)
+    seen = {}
+    for narrow in (True, False):
+        op = GaussianSplatOp(op_config(scene, DFVT))
+        op.narrow_tile_keys = narrow
+        for _ in range(2):
+            out, ctx = op.forward(model, scene.camera(), training=True)
+        assert op.last_forward_fused
+        assert (op._last_sorted[0].dtype == torch.int16) == narrow
+        keys = op._last_keys_sorted.cpu().numpy().view(np.uint64)
+        assert np.array_equal(keys, ref["keys_sorted"])
+        assert np.array_equal(ctx.gaussian_idx_sorted.cpu().numpy(), ref["gaussian_idx_sorted"])
+        assert np.array_equal(ctx.workload_ranges.cpu().numpy(), ref["workload_ranges"])
+        seen[narrow] = out
+    assert torch.equal(seen[True].color, seen[False].color) and torch.equal(seen[True].n_contrib, seen[False].n_contrib)
 
 
 def test_runs_on_the_callers_stream():
