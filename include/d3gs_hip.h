@@ -205,7 +205,7 @@ int d3gs_scan_gathered(const int32_t* src, int32_t src_n, const int32_t* index, 
 /* d3gs_scan_gathered without a workspace argument, for callers that cannot allocate one.  It has no counterpart
  * in the reference (whose `cumsum_` allocates its temporary storage inside torch); it is meant for code under HIP
  * graph capture, tight serving loops and harnesses that forbid hipMalloc.  The look-back's status words live in
- * a file-scope device array of the library (64 KiB + 256 B per GPU, held until the process ends), so n is limited
+ * a file-scope device array of the library (32 KiB + 256 B per GPU, held until the process ends), so n is limited
  * to D3GS_SCAN_NOALLOC_MAX_N elements (a larger n returns D3GS_ERR_WORKSPACE_TOO_SMALL).  The call allocates and
  * frees nothing; it clears the part of the array it uses with a fill kernel on `stream` and then runs the same
  * kernel as d3gs_scan_gathered: same outputs bit for bit.  The array is resolved for the device that is
