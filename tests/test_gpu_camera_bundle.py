@@ -202,3 +202,32 @@ def test_bundle_with_custom_features(one_pass, no_rgb):
             assert top == 0.0 and float(err.max()) == 0.0      # no SH colours: no gradient reaches the coefficients
             continue
         assert float(torch.quantile(err, 0.999)) <= 1e-4 * top and float(err.max()) <= 1e-3 * top, k
+
+
+@pytest.mark.parametrize("cameras,narrow", [(6, True), (9, False)])
+def test_bundle_with_many_tiles(cameras, narrow):
+    """Bundles whose tile ids pass 2^15 and 2^16: 6 cameras at 1920x1080 are 48 960 tiles (16-bit pair keys in the
+    one-call binning, the upper half of their range in use), 9 cameras 73 440 (the keys stay 32-bit).  Each camera's
+    image must be its own single-camera render."""
+    import torch
+    from d3gs_research_amd.camera import BasicPinholeCamera
+    from d3gs_research_amd.render import CameraBundle, GaussianSplatOp
+    scene = gen_scene(2, n=20000, wh=(1920, 1080))
+    cams = []
+    for k in range(cameras):
+        tw = np.array(scene.to_world, np.float64)
+        tw[:3, :3] = tw[:3, :3] @ Rotation.from_euler("xyz", (0.03 * k, -0.05 * k, 0.02 * k)).as_matrix()
+        tw[:3, 3] += (0.1 * k, -0.05 * k, 0.0)
+        cams.append(BasicPinholeCamera.from_params(scene.fx, scene.fy, scene.cx, scene.cy, scene.width, scene.height, tw))
+    bundle = CameraBundle.from_pinhole_cams(cams)
+    model = torch_model(scene)
+    op = GaussianSplatOp(op_config(scene, 4))
+    for _ in range(2):      # the second view takes the one-call binning
+        out, _ = op.forward(model, bundle, training=False)
+    assert op.last_forward_fused and (op._last_sorted[0].dtype == torch.int16) == narrow
+    tile_ids = op._last_keys_sorted >> 32
+    assert int(tile_ids.max()) >= (cameras - 1) * 8160 and bool((tile_ids[1:] >= tile_ids[:-1]).all())
+    single = GaussianSplatOp(op_config(scene, 4))
+    for b in (0, cameras // 2, cameras - 1):
+        one, _ = single.forward(model, cams[b], training=False)
+        assert torch.equal(one.color[0], out.color[b]) and torch.equal(one.n_contrib[0], out.n_contrib[b]), b
