@@ -403,6 +403,10 @@ def main():
         "gaussians_per_s": round(N / (ms_per_step * 1e-3), 1),
         "gpu_stage_sum_ms": round(gpu_sum, 4),
         "stages": stages,
+        # (the stage pass issues the binning launch by launch, with 32-bit pair keys; the timed views go through the
+        # one-call binning, whose pair keys are 16-bit tile ids when the view has at most 2^16 tiles)
+        "stages_note": "stage timers on: binning launch by launch, 32-bit pair keys; timed views: one library call, "
+                       + ("16" if (op.narrow_tile_keys and T_tiles <= 65536) else "32") + "-bit pair keys",
         "roofline": roofline,
         "hbm_whole_view": hbm_whole_view,
         "views8": views8,
