@@ -129,6 +129,46 @@ def save_3dgs_origin_model(model: GaussianModelOriginBase, path: str) -> None:
         f.write(np.ascontiguousarray(table).tobytes())
 
 
+def nearest_neighbour_distances(points: np.ndarray, k: int = 3) -> np.ndarray:
+    """Distances [N, k] from every point to its k nearest other points (what the reference's ``simple_knn`` returns,
+    d3sim/algos/d3gs/ops.py:185-214).  A k-d tree on the host: this runs once, when a model is initialised."""
+    from scipy.spatial import cKDTree
+    pts = np.ascontiguousarray(points, np.float64)
+    assert pts.ndim == 2 and pts.shape[1] == 3 and pts.shape[0] > k, "points must be [N, 3] with N > k"
+    dist, _ = cKDTree(pts).query(pts, k=k + 1)     # the nearest hit of a point is the point itself
+    return dist[:, 1:].astype(np.float32)
+
+
+def points_to_gaussian_init_scale(points: torch.Tensor) -> torch.Tensor:
+    """tools.py:64-69: the log of the root mean square distance to the three nearest neighbours, the same on every
+    axis, as the initial (raw) scale [N, 3]."""
+    knn = torch.from_numpy(nearest_neighbour_distances(points.detach().cpu().numpy(), 3)).to(points.device)
+    dist2 = torch.clamp_min(torch.square(knn).mean(1), 0.0000001)
+    return torch.log(torch.sqrt(dist2))[..., None].repeat(1, 3)
+
+
+def init_original_3dgs_model(model: GaussianModelOriginBase, points: np.ndarray, points_rgb: np.ndarray) -> None:
+    """tools.py:71-90: the original recipe's start from a point cloud, written into an allocated model in place:
+    positions = points, DC colour from the points' rgb in [0, 1], scale from the neighbour distances, identity
+    rotations, opacity 0.1 (as a logit), SH degree 0."""
+    with torch.no_grad():
+        assert model.xyz.shape[0] == points.shape[0]
+        dev = model.xyz.device
+        pts = torch.from_numpy(points.astype(np.float32)).to(dev).contiguous()
+        dc = rgb_to_sh(torch.from_numpy(points_rgb.astype(np.float32)).to(dev))
+        if model.color_sh_base is None:
+            model.color_sh[:, 0] = dc
+        else:
+            model.color_sh_base[:] = dc
+        model.scale[:] = points_to_gaussian_init_scale(pts)
+        quat = torch.zeros((pts.shape[0], 4), device=dev)
+        quat[:, 3] = 1
+        model.quaternion_xyzw[:] = quat
+        model.opacity[:] = inverse_sigmoid(0.1 * torch.ones(pts.shape[0], dtype=torch.float32, device=dev))
+        model.cur_sh_degree = 0
+        model.xyz[:] = pts
+
+
 def get_expon_lr_func(lr_init, lr_final, lr_delay_steps=0, lr_delay_mult=1.0, max_steps=1000000):
     """tools.py:92-126: log-linear interpolation from lr_init to lr_final with an optional sine warm-up."""
     def helper(step):
@@ -162,3 +202,35 @@ def create_origin_3dgs_optimizer(model: GaussianModelOriginBase, optim_cfg, spat
                                  lr_delay_mult=optim_cfg.position_lr_delay_mult,
                                  max_steps=optim_cfg.position_lr_max_steps)
     return optim, schedule
+
+
+def create_origin_xyz_scheduler(optim_cfg, batch_size: int, spatial_lr_scale: float):
+    """tools.py:175-181: the position schedule for a step over ``batch_size`` views (rates scaled by its root)."""
+    bs_scale = math.sqrt(batch_size)
+    return get_expon_lr_func(lr_init=optim_cfg.position_lr_init * spatial_lr_scale * bs_scale,
+                             lr_final=optim_cfg.position_lr_final * spatial_lr_scale * bs_scale,
+                             lr_delay_mult=optim_cfg.position_lr_delay_mult,
+                             max_steps=optim_cfg.position_lr_max_steps)
+
+
+def create_origin_3dgs_optimizers(model: GaussianModelOriginBase, optim_cfg, batch_size: int, spatial_lr_scale: float,
+                                  fused: bool = True):
+    """tools.py:146-173: one optimizer per parameter group for steps over ``batch_size`` views: rates scaled by
+    sqrt(batch_size), eps by its inverse, and the betas of ``batch_size`` single-view steps folded into one,
+    1 - batch_size (1 - beta).  The reference instantiates its own fused Adam kernel per group; here each group gets a
+    ``torch.optim.Adam`` (``fused`` asks for torch's fused implementation).  Returns ({name: optimizer}, schedule)."""
+    bs_scale = math.sqrt(batch_size)
+    groups = [("xyz", model.xyz, optim_cfg.position_lr_init * spatial_lr_scale * bs_scale)]
+    if model.color_sh_base is not None:
+        groups.append(("color_sh_base", model.color_sh_base, optim_cfg.feature_lr * bs_scale))
+    groups += [("color_sh", model.color_sh, optim_cfg.feature_lr * bs_scale / 20.0),
+               ("opacity", model.opacity, optim_cfg.opacity_lr * bs_scale),
+               ("scale", model.scale, optim_cfg.scaling_lr * bs_scale),
+               ("quaternion_xyzw", model.quaternion_xyzw, optim_cfg.rotation_lr * bs_scale)]
+    betas = (1 - batch_size * (1 - 0.9), 1 - batch_size * (1 - 0.999))
+    optimizers = {}
+    for name, tensor, lr in groups:
+        use_fused = bool(fused and tensor.is_cuda)
+        optimizers[name] = torch.optim.Adam([{"params": [tensor], "lr": lr, "name": name}], lr=lr, eps=1e-15 / bs_scale,
+                                            betas=betas, fused=use_fused)
+    return optimizers, create_origin_xyz_scheduler(optim_cfg, batch_size, spatial_lr_scale)
