@@ -152,6 +152,40 @@ class GaussianStrategyOrigin(config_def.Strategy):
             state.max_radii.copy_(torch.maximum(state.max_radii, r.max(0).values))
 
     @torch.no_grad()
+    def update_v1(self, state: GaussianTrainState, out, duv: torch.Tensor):
+        """origin/strategy.py:45-73, the earlier form: duv [..., N, 2] and out.radii of the same leading shape; the
+        gradient is scaled to NDC by (width / 2, height / 2) without the batch factor, and every (view, gaussian)
+        with a positive radius adds its length and one count to the gaussian."""
+        width, height = out.image_shape_wh
+        n = state.duv_ndc_length.shape[0]
+        scale = torch.tensor([width / 2.0, height / 2.0], dtype=duv.dtype, device=duv.device)
+        length = torch.linalg.norm(duv * scale, dim=-1).reshape(-1, n)
+        radii = out.radii.reshape(-1, n)
+        seen = radii > 0
+        state.duv_ndc_length += (length * seen).sum(0)
+        state.count += seen.sum(0).to(state.count.dtype)
+        if self.refine_scale2d_stop_iter > 0:
+            r = torch.where(seen, radii.to(torch.float32) / float(max(width, height)), torch.zeros((), device=duv.device))
+            state.max_radii.copy_(torch.maximum(state.max_radii, r.max(0).values))
+
+    @torch.no_grad()
+    def update_v2(self, state: GaussianTrainState, out, duv: torch.Tensor, batch_size: int = 1):
+        """origin/strategy.py:125-157: one state row per row of duv (duv.reshape(-1, 2) and out.radii flat have the
+        state's length); the gradient of a mean over ``batch_size`` views is scaled back by it."""
+        width, height = out.image_shape_wh
+        flat = duv.reshape(-1, 2)
+        radii = out.radii.reshape(-1)
+        assert flat.shape[0] == radii.shape[0] == state.duv_ndc_length.shape[0] == state.count.shape[0]
+        scale = torch.tensor([0.5 * width * batch_size, 0.5 * height * batch_size], dtype=duv.dtype, device=duv.device)
+        length = torch.linalg.norm(flat * scale, dim=-1)
+        seen = radii > 0
+        state.duv_ndc_length += length * seen
+        state.count += seen.to(state.count.dtype)
+        if self.refine_scale2d_stop_iter > 0:
+            r = torch.where(seen, radii.to(torch.float32) / float(max(width, height)), torch.zeros((), device=duv.device))
+            state.max_radii.copy_(torch.maximum(state.max_radii, r))
+
+    @torch.no_grad()
     def refine_gs(self, model: GaussianModelOriginBase, optimizers, state: GaussianTrainState, step: int,
                   generator: torch.Generator | None = None):
         """origin/strategy.py:160-364: clone small gaussians with a high screen-space gradient, split

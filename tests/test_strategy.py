@@ -39,6 +39,25 @@ def test_update_accumulates_ndc_gradient_length():
     assert state.max_radii.tolist() == pytest.approx([5 / 200, 0.0, 20 / 200])
 
 
+def test_the_two_other_update_forms():
+    """origin/strategy.py:45-73 (no batch factor, per view and gaussian) and 125-157 (one state row per row of duv)."""
+    W, H = 200, 100
+    radii = torch.tensor([5, 0, 7, 0, 0, 20], dtype=torch.int32)
+    duv = torch.tensor([[[3e-3, 4e-3], [1.0, 1.0], [0.0, 1e-3]], [[9.0, 9.0], [2.0, 2.0], [6e-3, 8e-3]]])
+    out = GaussianSplatOutput(custom_features=None, T=torch.zeros(2, H, W), color=torch.zeros(2, H, W, 3), radii=radii)
+    st = GaussianStrategyOrigin(refine_scale2d_stop_iter=10)
+    state = GaussianTrainState.create(3)
+    st.update_v1(state, out, duv)       # scale (W / 2, H / 2) = (100, 50)
+    assert state.duv_ndc_length.tolist() == pytest.approx([math.hypot(0.3, 0.2), 0.0, 0.05 + math.hypot(0.6, 0.4)])
+    assert state.count.tolist() == [1.0, 0.0, 2.0]
+    assert state.max_radii.tolist() == pytest.approx([5 / 200, 0.0, 20 / 200])
+    flat = GaussianTrainState.create(6)
+    st.update_v2(flat, out, duv, batch_size=2)       # scale (0.5 W B, 0.5 H B) = (200, 100), one row per (view, gaussian)
+    assert flat.duv_ndc_length.tolist() == pytest.approx([math.hypot(0.6, 0.4), 0.0, 0.1, 0.0, 0.0, math.hypot(1.2, 0.8)])
+    assert flat.count.tolist() == [1.0, 0.0, 1.0, 0.0, 0.0, 1.0]
+    assert flat.max_radii.tolist() == pytest.approx([5 / 200, 0.0, 7 / 200, 0.0, 0.0, 20 / 200])
+
+
 def _toy(fused=True):
     # 0: high gradient, small  -> cloned        1: high gradient, large -> split (parent removed)
     # 2: transparent           -> pruned        3: quiet               -> kept
