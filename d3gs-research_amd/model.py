@@ -82,6 +82,54 @@ class GaussianModelOriginBase:
         kw = {k: v.to(device) for k, v in self.get_proxy_field_dict().items()}
         return dataclasses.replace(self, **kw)
 
+    @property
+    def color_sh_act(self) -> torch.Tensor:
+        return self.color_sh
+
+    @property
+    def color_sh_base_act(self) -> torch.Tensor | None:
+        return self.color_sh_base
+
+    # constructors (origin/model.py:158-246)
+    @classmethod
+    def _allocate(cls, make, N: int, max_num_degree: int, split: bool, dtype, device, opacity=None):
+        coefficients = (max_num_degree + 1) * (max_num_degree + 1) - (1 if split else 0)
+        return cls(xyz=make(N, 3, dtype=dtype, device=device), quaternion_xyzw=make(N, 4, dtype=dtype, device=device),
+                   scale=make(N, 3, dtype=dtype, device=device),
+                   opacity=opacity if opacity is not None else make(N, dtype=dtype, device=device),
+                   color_sh_base=make(N, 3, dtype=dtype, device=device) if split else None,
+                   color_sh=make(N, coefficients, 3, dtype=dtype, device=device), cur_sh_degree=0)
+
+    @classmethod
+    def empty(cls, N: int, max_num_degree: int, split: bool = False, dtype: torch.dtype = torch.float32,
+              device: torch.device | str = "cuda"):
+        """origin/model.py:158-178: uninitialised tensors for N gaussians with SH up to ``max_num_degree``; ``split``
+        keeps the DC coefficient in ``color_sh_base``."""
+        return cls._allocate(torch.empty, N, max_num_degree, split, dtype, device)
+
+    @classmethod
+    def zeros(cls, N: int, max_num_degree: int, split: bool = False, dtype: torch.dtype = torch.float32,
+              device: torch.device | str = "cpu", opacity: torch.Tensor | None = None):
+        """origin/model.py:208-229 (``opacity`` lets a caller hand in storage it already has)."""
+        return cls._allocate(torch.zeros, N, max_num_degree, split, dtype, device, opacity)
+
+    @classmethod
+    def zeros_like_debug(cls, model: "GaussianModelOriginBase", opacity: torch.Tensor | None = None):
+        """origin/model.py:231-246: zeros with the shapes of ``model``."""
+        return cls.zeros(len(model), model.color_sh_degree, model.color_sh_base is not None, model.xyz.dtype,
+                         model.xyz.device, opacity)
+
+    @classmethod
+    def create_from_points(cls, points, points_rgb, device: torch.device | str = "cuda"):
+        """The original recipe's start from a point cloud (origin/model.py:180-206, ``create_from_dataset`` applied
+        to the dataset's ``dataset_point_cloud.xyz`` / ``.rgb``; dataset readers are not part of this package):
+        degree-3 storage with a split DC term, initialised by ``tools.init_original_3dgs_model``."""
+        from . import tools
+        model = cls.empty(points.shape[0], 3, True, device=device)
+        model.color_sh.zero_()
+        tools.init_original_3dgs_model(model, points, points_rgb)
+        return model
+
 
 @dataclasses.dataclass(kw_only=True)
 class GaussianModelOriginFused(GaussianModelOriginBase):

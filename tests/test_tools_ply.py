@@ -144,3 +144,22 @@ def test_optimizers_for_steps_over_several_views():
     m2 = GaussianModelOriginFused(xyz=torch.zeros(n, 3), quaternion_xyzw=torch.zeros(n, 4), scale=torch.zeros(n, 3),
                                   opacity=torch.zeros(n), color_sh=torch.zeros(n, 16, 3), color_sh_base=None)
     assert "color_sh_base" not in tools.create_origin_3dgs_optimizers(m2, cfg, 1, 1.0, fused=False)[0]
+
+
+def test_model_constructors():
+    """origin/model.py:158-246: empty / zeros / zeros_like_debug shapes, and the start from a point cloud."""
+    for split in (False, True):
+        m = GaussianModelOriginFused.zeros(7, 2, split)
+        assert m.color_sh.shape == (7, 9 - int(split), 3) and (m.color_sh_base is not None) == split
+        assert m.color_sh_degree == 2 and m.cur_sh_degree == 0 and len(m) == 7 and float(m.xyz.abs().max()) == 0.0
+        e = GaussianModelOrigin.empty(5, 3, split, device="cpu")
+        assert e.color_sh.shape == (5, 16 - int(split), 3) and e.opacity.shape == (5,) and e.quaternion_xyzw.shape == (5, 4)
+        op = torch.ones(7)
+        z = GaussianModelOriginFused.zeros_like_debug(m, opacity=op)
+        assert z.opacity is op and z.color_sh.shape == m.color_sh.shape and (z.color_sh_base is not None) == split
+    rng = np.random.default_rng(5)
+    pts, rgb = rng.standard_normal((50, 3)).astype(np.float32), rng.random((50, 3)).astype(np.float32)
+    m = GaussianModelOriginFused.create_from_points(pts, rgb, device="cpu")
+    assert m.color_sh.shape == (50, 15, 3) and float(m.color_sh.abs().max()) == 0.0 and m.cur_sh_degree == 0
+    assert np.array_equal(m.xyz.numpy(), pts) and np.allclose(m.color_sh_base.numpy() * tools.SH_C0 + 0.5, rgb, atol=1e-6)
+    assert m.color_sh_act is m.color_sh and m.color_sh_base_act is m.color_sh_base
