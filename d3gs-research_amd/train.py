@@ -15,7 +15,7 @@ from . import config_def
 from .model import GaussianModelOriginBase
 from .render import CameraBundle, GaussianSplatOp, GaussianSplatOutput, rasterize_gaussians
 from .strategy import GaussianStrategyOrigin, GaussianTrainState
-from .tools import create_origin_3dgs_optimizer
+from .tools import create_origin_3dgs_optimizer, create_origin_3dgs_optimizers
 
 
 def l1_loss(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
@@ -75,17 +75,28 @@ class Trainer:
         self.op = op
         model.act_applied = False
         model.set_requires_grad(True)
-        self.optim, self.xyz_schedule = create_origin_3dgs_optimizer(
-            model, self.cfg.optim, scene_scale if spatial_lr_scale is None else spatial_lr_scale)
+        lr_scale = scene_scale if spatial_lr_scale is None else spatial_lr_scale
+        if self.cfg.batch_size > 1:
+            # steps over several views (train.py:46-52): the schedules shrink by the batch size, and every
+            # parameter group gets its own optimizer with rates, eps and betas scaled for it (tools.py:146-173)
+            self.cfg.rescale_steps_by_batch_size(self.cfg.batch_size)
+            self.optim, self.xyz_schedule = create_origin_3dgs_optimizers(model, self.cfg.optim, self.cfg.batch_size,
+                                                                          lr_scale)
+        else:
+            self.optim, self.xyz_schedule = create_origin_3dgs_optimizer(model, self.cfg.optim, lr_scale)
         self.strategy = GaussianStrategyOrigin.from_config(self.cfg.strategy)
         self.state = GaussianTrainState.create(len(model), scene_scale, device=model.xyz.device)
         self.step = 0
 
+    def _optimizers(self):
+        return list(self.optim.values()) if isinstance(self.optim, dict) else [self.optim]
+
     def _set_position_lr(self):
         lr = self.xyz_schedule(self.step)
-        for group in self.optim.param_groups:
-            if group["name"] == "xyz":
-                group["lr"] = lr
+        for optim in self._optimizers():
+            for group in optim.param_groups:
+                if group["name"] == "xyz":
+                    group["lr"] = lr
 
     def train_step(self, cameras, gt_image: torch.Tensor, generator: torch.Generator | None = None) -> StepResult:
         """cameras: one camera or a CameraBundle; gt_image: [B, 3, H, W] in [0, 1]."""
@@ -98,8 +109,9 @@ class Trainer:
         color = out.color if self.op.is_nchw else out.color.permute(0, 3, 1, 2).contiguous()
         loss = photometric_loss(color[:, :3], gt_image, cfg.lambda_dssim)
         loss.backward()
-        self.optim.step()
-        self.optim.zero_grad(set_to_none=True)
+        for optim in self._optimizers():
+            optim.step()
+            optim.zero_grad(set_to_none=True)
         done = self.step + 1
         res = StepResult(float(loss.detach()), out)
         if done < st.refine_stop_iter and holder.grad is not None:

@@ -76,9 +76,11 @@ def test_trainer_with_densification_and_opacity_reset():
         model.xyz += 0.02 * torch.randn(model.xyz.shape, generator=g, device="cuda")
         model.opacity -= 1.0
         model.color_sh *= 0.5
+    # steps over two views: the trainer halves the schedules (train.py:46-52) and gives every parameter group its own
+    # optimizer with the rates, eps and betas of such steps (tools.py:146-173)
     cfg = config_def.Train(batch_size=2)
-    cfg.strategy.refine_start_iter, cfg.strategy.refine_every, cfg.strategy.refine_stop_iter = 10, 20, 70
-    cfg.strategy.reset_opacity_every = 50
+    cfg.strategy.refine_start_iter, cfg.strategy.refine_every, cfg.strategy.refine_stop_iter = 20, 40, 140
+    cfg.strategy.reset_opacity_every = 100
     cfg.strategy.grow_grad2d = 2e-5
     trainer = Trainer(model, op, cfg, scene_scale=2.0)
     n0, losses, events = len(model), [], []
@@ -94,5 +96,8 @@ def test_trainer_with_densification_and_opacity_reset():
     assert [e[0] for e in events] == ["refine", "refine", "reset", "refine"]          # steps 20, 40, 50, 60
     assert len(model) != n0 and trainer.state.count.shape[0] == len(model)
     assert min(losses[40:49]) < 0.8 * losses[0]                                       # before the opacity reset
-    for group in trainer.optim.param_groups:
-        assert group["params"][0] is getattr(model, group["name"])
+    assert cfg.strategy.refine_every == 20 and cfg.strategy.reset_opacity_every == 50 and isinstance(trainer.optim, dict)
+    for name, optim in trainer.optim.items():
+        (group,) = optim.param_groups
+        assert group["name"] == name and group["params"][0] is getattr(model, name)
+        assert group["betas"] == pytest.approx((0.8, 0.998))
