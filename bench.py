@@ -173,6 +173,8 @@ def main():
     ap.add_argument("--custom-features", type=int, default=0, metavar="F",
                     help="carry F seeded custom feature channels per gaussian through every view, forward and backward "
                          "(a different workload, for profiling the feature kernels: not the headline; no CPU baseline)")
+    ap.add_argument("--gaussians", type=int, default=0, help="override the configuration's gaussian count (not the headline)")
+    ap.add_argument("--image", type=str, default="", metavar="WxH", help="override the configuration's image size (not the headline)")
     ap.add_argument("--cpu-n", type=int, default=0, help="gaussians in the CPU-baseline sample (0 = full workload)")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="only run a plain 256 MiB -> 256 MiB elementwise copy 5 times (reference reading for "
@@ -198,7 +200,9 @@ def main():
     from d3gs_research_amd.synthetic import gen_scene, scene_config, scene_model
 
     filt = EarlyFilterAlgo[args.filter]
-    scene = gen_scene(args.config)
+    resized = bool(args.gaussians or args.image)
+    scene = gen_scene(args.config, n=args.gaussians or None,
+                      wh=tuple(int(v) for v in args.image.lower().split("x")) if args.image else None)
     cam = scene.camera()
     cams = [cam] + orbit_cameras(scene, args.views - 1)
     op = GaussianSplatOp(scene_config(scene, filt, rasterize_backward_algo=RasterizeBackwardAlgo[args.backward_algo]))
@@ -320,7 +324,7 @@ def main():
     # at the rate their mix allows for their whole duration (roofline.valu below) while moving a fraction of a byte
     # per evaluated pair, so they are "valu"; the HBM fraction asked for is reported all the same.
     roofline = {"bound": "valu" if dom in ("blend_fwd", "blend_bwd", "preprocess") else "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": committed_traffic_bytes(dom, args.config),
+                "frac": round(achieved / HBM_PEAK_GBS, 5), "traffic": None if resized else committed_traffic_bytes(dom, args.config),
                 "traffic_source": f"profiles/config{args.config}_all_kernels.txt (rocprofv3 --pmc, not this run)",
                 "pair_evals_per_s": round(256.0 * M / (stages[dom]["ms"] * 1e-3), 1),
                 # what a plain device-to-device copy reaches on this box (read + written bytes per second)
@@ -329,7 +333,7 @@ def main():
     # rate at which the dominant kernel retires vector instructions (count from the committed counter summary, time
     # from this run) against 256 CUs x 4 SIMDs x 2.4 GHz / 4 cycles per wave64 instruction.  Plain FP32 operations
     # issue in half that time on this chip, so the ratio can exceed 1; its ceiling for this kernel's mix is about 1.3.
-    valu = committed_valu_instructions(dom, args.config)
+    valu = None if resized else committed_valu_instructions(dom, args.config)
     if valu is not None:
         rate = valu / (stages[dom]["ms"] * 1e-3)
         roofline["valu"] = {"wave_instructions_per_launch": valu, "per_s": round(rate, 1),
@@ -337,7 +341,7 @@ def main():
     # The whole view against the HBM roofline: measured traffic of every kernel on the path (committed counter
     # summary) over this run's time per view.
     hbm_whole_view = None
-    whole = committed_whole_view_traffic(args.config)
+    whole = None if resized else committed_whole_view_traffic(args.config)
     if whole is not None and filt.name == "OBB_DFVT" and args.backward_algo == "DEFAULT":
         gbs = (whole[0] + whole[1]) / (ms_per_step * 1e-3) / 1e9
         hbm_whole_view = {"read_bytes": whole[0], "written_bytes": whole[1], "traffic_bytes": whole[0] + whole[1],
@@ -387,8 +391,8 @@ def main():
                                   + ("" if single is None else "; single_thread_ms: one view on one thread")}
 
     line = {
-        "metric": "fwd+bwd raster ms/view, 1M Gaussians @1080p, 1 MI355X" if args.config == 2
-        else f"fwd+bwd raster ms/view, config {args.config}",
+        "metric": "fwd+bwd raster ms/view, 1M Gaussians @1080p, 1 MI355X" if (args.config == 2 and not resized)
+        else f"fwd+bwd raster ms/view, config {args.config}" + (" with another gaussian count or image size" if resized else ""),
         **({"note": f"with {args.custom_features} custom feature channels: not the headline workload"} if feat is not None else {}),
         "value": round(ms_per_step, 4), "unit": "ms/view", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
