@@ -380,12 +380,14 @@ __device__ __forceinline__ uint32_t key_tile(Key k) {
     else return (uint32_t)k;
 }
 
-constexpr int kRangeItems = 4;   // consecutive keys per thread (one 16-byte load of 32-bit keys)
+// consecutive keys per thread: one 16-byte load (four 32-bit keys, eight 16-bit ones)
+template <typename Key> constexpr int range_items() { return sizeof(Key) == 2 ? 8 : 4; }
 
 template <typename Key>
 __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restrict__ keys, long long m,
                                                               const long long* __restrict__ m_device,
                                                               int32_t* __restrict__ ranges, int num_tiles) {
+    constexpr int kRangeItems = range_items<Key>();
     if (m_device) m = min(m, max(*m_device, 0ll));   // m is then the capacity of the key buffer
     const long long i0 = ((long long)blockIdx.x * kBlock + threadIdx.x) * kRangeItems;
     if (i0 >= m) return;
@@ -396,8 +398,13 @@ __global__ __launch_bounds__(kBlock) void tile_ranges_kernel(const Key* __restri
             const uint4 v = *reinterpret_cast<const uint4*>(keys + i0);   // i0 is a multiple of 4
             k[0] = v.x; k[1] = v.y; k[2] = v.z; k[3] = v.w;
         } else if constexpr (sizeof(Key) == 2) {
-            const uint2 v = *reinterpret_cast<const uint2*>(keys + i0);   // four 16-bit keys
-            k[0] = (Key)(v.x & 0xFFFFu); k[1] = (Key)(v.x >> 16); k[2] = (Key)(v.y & 0xFFFFu); k[3] = (Key)(v.y >> 16);
+            const uint4 v = *reinterpret_cast<const uint4*>(keys + i0);   // i0 is a multiple of 8
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                k[2 * j] = (Key)(w[j] & 0xFFFFu);
+                k[2 * j + 1] = (Key)(w[j] >> 16);
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < kRangeItems; ++j) k[j] = keys[i0 + j];
@@ -780,7 +787,7 @@ static int tile_ranges_impl(const char* who, const Key* keys_sorted, int64_t m, 
     }
     if (m > 0)
         hipLaunchKernelGGL(tile_ranges_kernel<Key>,
-                           dim3((unsigned)((m + (long long)kBlock * kRangeItems - 1) / ((long long)kBlock * kRangeItems))), dim3(kBlock), 0,
+                           dim3((unsigned)((m + (long long)kBlock * range_items<Key>() - 1) / ((long long)kBlock * range_items<Key>()))), dim3(kBlock), 0,
                            (hipStream_t)stream, keys_sorted, (long long)m, (const long long*)m_device, workload_ranges,
                            (int)num_tiles);
     if (tile_order && num_tiles > 0) {
